@@ -1,0 +1,75 @@
+"""Build the gfx950 chain library (`libditto_chain.so`) in-tree with hipcc.
+
+Usage: ``python -m ditto_amd.build`` (or ``__graft_entry__.build()``).  Objects are
+compiled in parallel, one hipcc process per translation unit, then linked into
+``ditto_amd/csrc/libditto_chain.so``.
+"""
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+
+CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIB = os.path.join(CSRC, "libditto_chain.so")
+OBJ_DIR = os.path.join(CSRC, "build")
+
+# -packed-fp32-ops is switched off: packed fp32 VALU forms are not wanted in these kernels.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+# (object name, source, extra defines)
+UNITS = [
+    ("api", "api.hip", []),
+    ("fp_f16_cast", "bmm_chain_fp_inst.hip",
+     ["-DDITTO_INST_T=f16", "-DDITTO_INST_INTER=0", "-DDITTO_INST_NAME=launch_f16_cast"]),
+    ("fp_f16_softmax", "bmm_chain_fp_inst.hip",
+     ["-DDITTO_INST_T=f16", "-DDITTO_INST_INTER=2", "-DDITTO_INST_NAME=launch_f16_softmax"]),
+    ("fp_bf16_cast", "bmm_chain_fp_inst.hip",
+     ["-DDITTO_INST_T=bf16", "-DDITTO_INST_INTER=0", "-DDITTO_INST_NAME=launch_bf16_cast"]),
+    ("fp_bf16_softmax", "bmm_chain_fp_inst.hip",
+     ["-DDITTO_INST_T=bf16", "-DDITTO_INST_INTER=2", "-DDITTO_INST_NAME=launch_bf16_softmax"]),
+]
+
+
+def _hipcc():
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; the chain library needs ROCm to build")
+    return exe
+
+
+def _compile(unit):
+    name, src, defs = unit
+    obj = os.path.join(OBJ_DIR, name + ".o")
+    cmd = [_hipcc(), *HIPCC_FLAGS, *defs, "-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, " ".join(cmd), r.stderr))
+    return obj
+
+
+def build(verbose=True, jobs=None):
+    """Compile every translation unit and link the shared library.  Always rebuilds."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(_compile, UNITS))
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n%s" % r.stderr)
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()
+    sys.exit(0)

@@ -1,0 +1,222 @@
+// C ABI of the chain library: descriptor validation, tile choice, kernel dispatch.
+// Declarations and the reference interfaces they replace are in include/ditto_chain.h.
+#include "../../include/ditto_chain.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "bmm_chain_fp.h"
+#include "chain_kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+int elem_bytes(int dt) {
+  switch (dt) {
+    case DITTO_F16:
+    case DITTO_BF16:
+      return 2;
+    case DITTO_F32:
+    case DITTO_I32:
+      return 4;
+    case DITTO_I8:
+      return 1;
+  }
+  return 0;
+}
+
+// Number of compute units of the current device (cached per thread).
+int device_cus() {
+  static thread_local int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+struct BmmPlan {
+  int family;  // 0: fp16/bf16 register-resident chain, 1: fp32 chain, 2: int8 requant chain
+  int d_pad, qt;
+  ditto_tile_param tile;
+};
+
+int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
+  if (!d) return fail(DITTO_EINVAL, "null descriptor");
+  if (d->abi_version != DITTO_CHAIN_ABI_VERSION)
+    return fail(DITTO_EINVAL, "descriptor abi_version %d, library %d", d->abi_version,
+                DITTO_CHAIN_ABI_VERSION);
+  if (d->batch <= 0 || d->M <= 0 || d->N <= 0 || d->K <= 0 || d->L <= 0)
+    return fail(DITTO_EINVAL, "batch, M, N, K, L must be positive (got %lld %lld %lld %lld %lld)",
+                (long long)d->batch, (long long)d->M, (long long)d->N, (long long)d->K,
+                (long long)d->L);
+  if (d->M > 0x7fffffff / 2 || d->L > 0x7fffffff / 2 || d->batch > 0x7fffffff / 2)
+    return fail(DITTO_EINVAL, "extent too large");
+  if (d->b_layout != DITTO_B_KL && d->b_layout != DITTO_B_LK)
+    return fail(DITTO_EINVAL, "unknown b_layout %d", d->b_layout);
+  const int in = d->in_dtype;
+  memset(plan, 0, sizeof(*plan));
+
+  if (in == DITTO_F16 || in == DITTO_BF16) {
+    if (d->acc_dtype != DITTO_F32)
+      return fail(DITTO_EUNSUPPORTED, "fp16/bf16 chains accumulate in fp32 (acc_dtype %d)", d->acc_dtype);
+    if (d->out_dtype != in && d->out_dtype != DITTO_F32)
+      return fail(DITTO_EINVAL, "out_dtype must be in_dtype or fp32");
+    if (d->inter_op != DITTO_INTER_CAST && d->inter_op != DITTO_INTER_RELU &&
+        d->inter_op != DITTO_INTER_SOFTMAX)
+      return fail(DITTO_EINVAL, "inter_op %d not valid for a floating-point chain", d->inter_op);
+    if (d->inter_op == DITTO_INTER_SOFTMAX && !(d->softmax_scale > 0.f))
+      return fail(DITTO_EINVAL, "softmax_scale must be > 0");
+    // 16-byte vector loads: extents and strides in multiples of 8 elements.
+    // (The reference builders require multiples of 16: bmm_chain.py:34-38.)
+    if (d->K % 8 || d->N % 8) return fail(DITTO_EINVAL, "K and N must be multiples of 8");
+    if (d->b_layout == DITTO_B_KL && d->L % 8)
+      return fail(DITTO_EINVAL, "L must be a multiple of 8 when B is [K][L]");
+    if (d->a_row_stride % 8 || d->b_row_stride % 8 || d->c_row_stride % 8 || d->a_batch_stride % 8 ||
+        d->b_batch_stride % 8 || d->c_batch_stride % 8)
+      return fail(DITTO_EINVAL, "input strides must be multiples of 8 elements");
+    const int out_vec = 4;
+    if (d->f_row_stride % out_vec || d->f_batch_stride % out_vec)
+      return fail(DITTO_EINVAL, "output strides must be multiples of 4 elements");
+    if (d->a_row_stride < d->K || d->c_row_stride < d->N || d->f_row_stride < d->N ||
+        d->b_row_stride < (d->b_layout == DITTO_B_KL ? d->L : d->K))
+      return fail(DITTO_EINVAL, "row stride smaller than row extent");
+    if (d->a_row_stride > 0x7fffffff || d->b_row_stride > 0x7fffffff ||
+        d->c_row_stride > 0x7fffffff || d->f_row_stride > 0x7fffffff)
+      return fail(DITTO_EINVAL, "row stride too large");
+    const long long dmax = d->K > d->N ? d->K : d->N;
+    if (dmax > 128)
+      return fail(DITTO_EUNSUPPORTED, "max(K,N)=%lld: register-resident chain supports up to 128", dmax);
+    plan->family = 0;
+    plan->d_pad = dmax <= 64 ? 64 : 128;
+    const int cus = need_device ? device_cus() : 256;
+    const long long blocks_qt2 = ((d->M + 255) / 256) * d->batch;
+    plan->qt = (blocks_qt2 >= 2LL * cus) ? 2 : 1;
+    const int bm = 128 * plan->qt;
+    ditto_tile_param& t = plan->tile;
+    t.block_threads = 256;
+    t.block_m = bm;
+    t.block_l = ditto::kBN;
+    t.block_n = (int)d->N;
+    t.head_pad = plan->d_pad;
+    const bool kl = d->b_layout == DITTO_B_KL;
+    t.lds_bytes = plan->d_pad == 64 ? (kl ? ditto::bmm_chain_lds_bytes<64, true>() : ditto::bmm_chain_lds_bytes<64, false>())
+                                    : (kl ? ditto::bmm_chain_lds_bytes<128, true>() : ditto::bmm_chain_lds_bytes<128, false>());
+    t.grid_x = (int)(((d->M + bm - 1) / bm) * d->batch);
+    t.grid_y = t.grid_z = 1;
+    t.variant = plan->d_pad * 10 + plan->qt;
+    return DITTO_OK;
+  }
+  return fail(DITTO_EUNSUPPORTED, "no chain kernel for in_dtype %d", in);
+}
+
+}  // namespace
+
+extern "C" {
+
+int ditto_chain_abi_version(void) { return DITTO_CHAIN_ABI_VERSION; }
+
+const char* ditto_last_error(void) { return g_err; }
+
+int ditto_bmm_chain_select_tile(const ditto_bmm_chain_desc* desc, ditto_tile_param* out) {
+  BmmPlan plan;
+  int rc = plan_bmm(desc, &plan, false);
+  if (rc != DITTO_OK) return rc;
+  if (!out) return fail(DITTO_EINVAL, "null output");
+  *out = plan.tile;
+  return DITTO_OK;
+}
+
+size_t ditto_bmm_chain_workspace_bytes(const ditto_bmm_chain_desc* desc) {
+  (void)desc;
+  return 0;
+}
+
+int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void* b, const void* c,
+                        const void* aux, void* f, void* workspace, size_t workspace_bytes,
+                        void* stream) {
+  (void)workspace;
+  (void)workspace_bytes;
+  (void)aux;
+  BmmPlan plan;
+  int rc = plan_bmm(d, &plan, true);
+  if (rc != DITTO_OK) return rc;
+  if (!a || !b || !c || !f) return fail(DITTO_EINVAL, "null data pointer");
+  if (!aligned(a, 16) || !aligned(b, 16) || !aligned(c, 16) || !aligned(f, 16))
+    return fail(DITTO_EINVAL, "data pointers must be 16-byte aligned");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+
+  if (plan.family == 0) {
+    ditto::BmmChainArgs args;
+    args.a = a;
+    args.b = b;
+    args.c = c;
+    args.f = f;
+    args.a_bs = d->a_batch_stride;
+    args.b_bs = d->b_batch_stride;
+    args.c_bs = d->c_batch_stride;
+    args.f_bs = d->f_batch_stride;
+    args.a_rs = (int)d->a_row_stride;
+    args.b_rs = (int)d->b_row_stride;
+    args.c_rs = (int)d->c_row_stride;
+    args.f_rs = (int)d->f_row_stride;
+    args.M = (int)d->M;
+    args.N = (int)d->N;
+    args.K = (int)d->K;
+    args.L = (int)d->L;
+    args.batch = (int)d->batch;
+    args.mblocks = (int)((d->M + plan.tile.block_m - 1) / plan.tile.block_m);
+    args.scale_log2 = d->softmax_scale * 1.4426950408889634f;
+    args.relu = d->inter_op == DITTO_INTER_RELU;
+    args.out_f32 = d->out_dtype == DITTO_F32;
+    const bool kl = d->b_layout == DITTO_B_KL;
+    const bool sm = d->inter_op == DITTO_INTER_SOFTMAX;
+    hipError_t e;
+    if (d->in_dtype == DITTO_F16)
+      e = sm ? ditto::launch_f16_softmax(plan.d_pad, plan.qt, kl, args, st)
+             : ditto::launch_f16_cast(plan.d_pad, plan.qt, kl, args, st);
+    else
+      e = sm ? ditto::launch_bf16_softmax(plan.d_pad, plan.qt, kl, args, st)
+             : ditto::launch_bf16_cast(plan.d_pad, plan.qt, kl, args, st);
+    if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
+    return DITTO_OK;
+  }
+  return fail(DITTO_EUNSUPPORTED, "no kernel family %d", plan.family);
+}
+
+int ditto_conv_chain_select_tile(const ditto_conv_chain_desc* desc, ditto_tile_param* out) {
+  (void)desc;
+  (void)out;
+  return fail(DITTO_EUNSUPPORTED, "conv chain kernel not built");
+}
+
+size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
+  (void)desc;
+  return 0;
+}
+
+int ditto_conv_chain_run(const ditto_conv_chain_desc* desc, const void* x, const void* w1,
+                         const void* w2, void* y, void* workspace, size_t workspace_bytes,
+                         void* stream) {
+  (void)desc; (void)x; (void)w1; (void)w2; (void)y; (void)workspace; (void)workspace_bytes; (void)stream;
+  return fail(DITTO_EUNSUPPORTED, "conv chain kernel not built");
+}
+
+}  // extern "C"

@@ -1,0 +1,15 @@
+// Launchers defined in the per-variant translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "bmm_chain_fp.h"
+
+namespace ditto {
+
+// bmm_chain_fp_inst.hip, one object per (element type, inter-op)
+hipError_t launch_f16_cast(int d_pad, int qt, bool b_kl, const BmmChainArgs& args, hipStream_t stream);
+hipError_t launch_f16_softmax(int d_pad, int qt, bool b_kl, const BmmChainArgs& args, hipStream_t stream);
+hipError_t launch_bf16_cast(int d_pad, int qt, bool b_kl, const BmmChainArgs& args, hipStream_t stream);
+hipError_t launch_bf16_softmax(int d_pad, int qt, bool b_kl, const BmmChainArgs& args, hipStream_t stream);
+
+}  // namespace ditto

@@ -1,0 +1,115 @@
+// Shared device/host helpers for the gfx950 chain kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ditto {
+
+typedef _Float16 f16;
+typedef __bf16 bf16;
+
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(2))) int i32x2;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(16))) int i32x16;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+
+#define DITTO_LDS __attribute__((address_space(3)))
+
+// Per-element-type traits: vector types and the gfx950 MFMA that consumes them.
+//   32x32x16: A lane l holds A[l%32][8*(l/32)+0..7], B lane l holds B[8*(l/32)+0..7][l%32],
+//             acc[r] = C[8*(r/4) + 4*(l/32) + r%4][l%32].
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<f16> {
+  typedef f16x8 v8;
+  typedef f16x4 v4;
+  typedef f16x2 v2;
+  static __device__ __forceinline__ f32x16 mfma32(v8 a, v8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(v8 a, v8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <>
+struct Elem<bf16> {
+  typedef bf16x8 v8;
+  typedef bf16x4 v4;
+  typedef bf16x2 v2;
+  static __device__ __forceinline__ f32x16 mfma32(v8 a, v8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(v8 a, v8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+// Round-to-nearest-even conversion of two fp32 values to a packed pair of T.
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::v2 cvt2(float a, float b) {
+  f32x2 v = {a, b};
+  return __builtin_convertvector(v, typename Elem<T>::v2);
+}
+
+// LDS transpose read (gfx950 ds_read_b64_tr_b16).  Within each group of 16
+// lanes, lane i receives for j=0..3 the 16-bit element (i%4) of the 64-bit
+// word addressed by lane 4*j + i/4 of the same group.  If lane s of a group
+// points at Mat[r0 + s/4][c0 + 4*(s%4)] of a row-major 16-bit matrix, lane i
+// receives Mat[r0 + 0..3][c0 + i]: a 4x16 block read column-wise.
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::v4 lds_read_tr4(const T* p) {
+  s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DITTO_LDS s16x4*)p);
+  return __builtin_bit_cast(typename Elem<T>::v4, r);
+}
+
+template <typename V4, typename V8>
+__device__ __forceinline__ V8 concat4(V4 lo, V4 hi) {
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Exchange across the two half-waves.  v_permlane32_swap a, b swaps a[32..63] with
+// b[0..31]; started from a == b == x it leaves (a, b) = (x[l], x[l+32]) in lanes 0..31
+// and (x[l-32], x[l]) in lanes 32..63, i.e. every lane holds its own value and its
+// partner's.  Issued as inline asm: the compiler's builtin folds the two results into
+// one value when both operands start equal.  The s_nop covers the VALU-write ->
+// permlane-read hazard the compiler would otherwise pad itself.
+__device__ __forceinline__ void pair_both(float x, float& a, float& b) {
+  a = x;
+  b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float pair_max(float x) {
+  float a, b;
+  pair_both(x, a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  float a, b;
+  pair_both(x, a, b);
+  return a + b;
+}
+
+// Workgroups are dealt round-robin to the 8 XCDs (each with a private L2) by
+// linear id.  Remap so that ids that are neighbours in the logical order (and
+// share operands) land on the same XCD.
+__device__ __forceinline__ unsigned xcd_remap(unsigned bid, unsigned nblk) {
+  const unsigned NX = 8;
+  if (nblk % NX != 0) return bid;
+  return (bid % NX) * (nblk / NX) + bid / NX;
+}
+
+}  // namespace ditto

@@ -1,0 +1,160 @@
+/*
+ * ditto_chain.h — C ABI of the MI355X (gfx950) fused operator-chain library.
+ *
+ * This is the boundary a Ditto maintainer binds in place of the TVM PackedFunc
+ * that `tvm.build(sch, layer.schedule_tensors, "cuda")` returns for a
+ * hyper_fusion chain (reference: benchmark/chimera/cuda/bmm_softmax_bmm_cuda.py:26,239,256;
+ * src/runtime/graph_runtime.cc:149).  The reference call is
+ * `func(*inputs, *outputs)` with destination passing: the caller owns every
+ * buffer and the callee allocates nothing the caller can see.  The same holds
+ * here: all data pointers are DEVICE pointers owned by the caller; the library
+ * enqueues one kernel on the given HIP stream and returns without
+ * synchronising.  Nothing is thrown across this boundary: every entry point
+ * returns 0 on success or a negative DITTO_E* code, and ditto_last_error()
+ * returns the calling thread's last message.
+ *
+ * Plain C: no HIP or torch types appear in the signatures (a stream is passed
+ * as void*, i.e. a hipStream_t; NULL is the default stream).
+ */
+#ifndef DITTO_CHAIN_H_
+#define DITTO_CHAIN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DITTO_CHAIN_ABI_VERSION 1
+
+/* error codes */
+#define DITTO_OK 0
+#define DITTO_EINVAL (-1)      /* descriptor / shape / alignment not valid          */
+#define DITTO_EUNSUPPORTED (-2)/* valid chain, but no kernel for this dtype / shape */
+#define DITTO_EHIP (-3)        /* a HIP runtime call failed                         */
+#define DITTO_EWORKSPACE (-4)  /* workspace too small                               */
+
+/* element types (reference: the in_dtype / acc_dtype strings of the chain
+ * builders, benchmark/chimera/cuda/bmm_bmm_cuda.py:273-288) */
+typedef enum ditto_dtype {
+  DITTO_F16 = 0,
+  DITTO_BF16 = 1,
+  DITTO_F32 = 2,
+  DITTO_I8 = 3,
+  DITTO_I32 = 4
+} ditto_dtype;
+
+/* The op on the single path between the two contractions
+ * (reference: TensorizeHyperFusionState::inter_path, src/auto_tensorize/hyper_fusion.cc:51-216). */
+typedef enum ditto_inter_op {
+  DITTO_INTER_CAST = 0,    /* mid = cast_in(acc)                      bmm_bmm_cuda.py:114-118           */
+  DITTO_INTER_RELU = 1,    /* mid = cast_in(max(acc,0))               conv_relu_conv_relu_fuse_hw_cuda.py:134-142 */
+  DITTO_INTER_SOFTMAX = 2, /* mid = softmax(scale*acc) over L, online  bmm_chain.py:63-103 (exp + ones column + divide) */
+  DITTO_INTER_REQUANT = 3  /* mid = sat_i8(rne(acc * 2^-shift[col]))   int8 chain, BASELINE config 5     */
+} ditto_inter_op;
+
+/* How the second operand of the first contraction is laid out in memory. */
+typedef enum ditto_b_layout {
+  DITTO_B_KL = 0, /* B[batch][K][L], L contiguous: the reference's placeholder layout
+                     (bmm_bmm_cuda.py:87, bmm_chain.py:29-31 `key[batch,K,L]`)          */
+  DITTO_B_LK = 1  /* B stored as [batch][L][K], K contiguous: a transposed view of the
+                     above (what self_attention.py:55-57 transposes FROM); no copy made */
+} ditto_b_layout;
+
+/*
+ * Batched two-contraction chain  F[b] = epilogue( inter( A[b]·B[b] ) · C[b] ).
+ * Names follow the reference builders: A[batch,M,K], B[batch,K,L], C[batch,L,N],
+ * F[batch,M,N] (bmm_bmm_cuda.py:69-149, bmm_chain.py:5-105).
+ * Strides are in ELEMENTS.  Rows must be contiguous (innermost stride 1).
+ */
+typedef struct ditto_bmm_chain_desc {
+  int32_t abi_version;   /* DITTO_CHAIN_ABI_VERSION */
+  int32_t in_dtype;      /* ditto_dtype of A, B, C                                    */
+  int32_t acc_dtype;     /* DITTO_F32 (fp) or DITTO_I32 (int8)                         */
+  int32_t out_dtype;     /* in_dtype (reference: F cast to in_dtype) or acc_dtype      */
+  int32_t inter_op;      /* ditto_inter_op                                            */
+  int32_t b_layout;      /* ditto_b_layout                                            */
+  int64_t batch, M, N, K, L;
+  int64_t a_batch_stride, a_row_stride; /* A[b][m][k] = a + b*abs + m*ars + k          */
+  int64_t b_batch_stride, b_row_stride; /* KL: B[b][k][l] = b + b*bbs + k*brs + l
+                                           LK: B[b][k][l] = b + b*bbs + l*brs + k      */
+  int64_t c_batch_stride, c_row_stride; /* C[b][l][n]                                  */
+  int64_t f_batch_stride, f_row_stride; /* F[b][m][n]                                  */
+  float softmax_scale;   /* DITTO_INTER_SOFTMAX only; the reference uses 1.0           */
+  int32_t requant_shift_uniform; /* DITTO_INTER_REQUANT: if >=0, every column uses this
+                                    power-of-two shift and `aux` may be NULL           */
+} ditto_bmm_chain_desc;
+
+/*
+ * conv -> conv chain on plain NCHW tensors (reference forms:
+ * testing/hyper_fusion/conv_relu_conv_relu_fuse_hw_cuda.py:17-262 for NCHW,
+ * benchmark/chimera/cuda/conv3x3_conv1x1_cuda.py:77-172 for the chain; shape
+ * tuple as python_test/auto_tensorize/test_hyper_fusion.py:51-192).
+ *   X[N][C0][H][W], W1[C1][C0][R1][S1], W2[C2][C1][R2][S2] -> Y[N][C2][P2][Q2]
+ */
+typedef struct ditto_conv_chain_desc {
+  int32_t abi_version;
+  int32_t in_dtype, acc_dtype, out_dtype;
+  int32_t inter_op;      /* DITTO_INTER_CAST or DITTO_INTER_RELU */
+  int32_t relu_out;      /* 1: ReLU after the second convolution too */
+  int64_t N, C0, H, W;
+  int64_t C1, R1, S1, pad1, stride1;
+  int64_t C2, R2, S2, pad2, stride2;
+} ditto_conv_chain_desc;
+
+/* Tile choice reported back to the host; the static per-shape table replaces
+ * CUDATensorizeParam and its search (hyper_fusion.cc:586-607,
+ * chimera_integrate.py:298-449). */
+typedef struct ditto_tile_param {
+  int32_t block_threads;  /* threads per workgroup (multiple of 64)              */
+  int32_t block_m;        /* rows of the chain output one workgroup owns         */
+  int32_t block_l;        /* extent of the intermediate processed per step       */
+  int32_t block_n;        /* columns of the chain output one workgroup owns      */
+  int32_t head_pad;       /* K and N padded to this inside the kernel (0: n/a)   */
+  int32_t lds_bytes;      /* dynamic LDS per workgroup                           */
+  int32_t grid_x, grid_y, grid_z;
+  int32_t variant;        /* kernel variant id, for logs                         */
+} ditto_tile_param;
+
+/* ---- entry points ------------------------------------------------------- */
+
+/* Library / ABI version (DITTO_CHAIN_ABI_VERSION of the build). */
+int ditto_chain_abi_version(void);
+
+/* Last error message of the calling thread ("" if none). */
+const char* ditto_last_error(void);
+
+/* Tile the library would use for this chain; also validates the descriptor.
+ * Replaces the parameter choice of chimera_integrate.py:452-478. */
+int ditto_bmm_chain_select_tile(const ditto_bmm_chain_desc* desc, ditto_tile_param* out);
+int ditto_conv_chain_select_tile(const ditto_conv_chain_desc* desc, ditto_tile_param* out);
+
+/* Bytes of device workspace the run call needs (0 for every chain today; the
+ * reference's generated code allocates an fp32 E_frag[B,M,ext_N] internally,
+ * evaluation/asplos/ncu_summary_chimera_bmm_softmax_bmm.txt:8). */
+size_t ditto_bmm_chain_workspace_bytes(const ditto_bmm_chain_desc* desc);
+size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc);
+
+/*
+ * Run one fused chain: replaces `func(A, B, C, F)` of the built PackedFunc
+ * (bmm_bmm_cuda.py:256, bmm_softmax_bmm_cuda.py:256).
+ *   a, b, c : inputs (device), read-only
+ *   aux     : DITTO_INTER_REQUANT: int32 shift[L] per intermediate column
+ *             (mid = sat_i8(rne(acc / 2^shift))), else NULL
+ *   f       : output (device), must not alias an input
+ */
+int ditto_bmm_chain_run(const ditto_bmm_chain_desc* desc, const void* a, const void* b,
+                        const void* c, const void* aux, void* f, void* workspace,
+                        size_t workspace_bytes, void* stream);
+
+/* Run one fused conv->conv chain: replaces `func(Img, W1, W2, Out)`
+ * (conv3x3_conv1x1_cuda.py:296-305). */
+int ditto_conv_chain_run(const ditto_conv_chain_desc* desc, const void* x, const void* w1,
+                         const void* w2, void* y, void* workspace, size_t workspace_bytes,
+                         void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DITTO_CHAIN_H_ */
