@@ -1,0 +1,221 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused operator chains on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-also]
+
+A "step" is one call of the fused chain on one batch of synthetic input that is already
+resident in HBM.  The headline workload is the long-sequence BMM -> softmax -> BMM chain
+(bf16, 64 x (4096 x 128)): the MFMA-bound configuration on which the ">= 50 % of dense MFMA
+peak" target is stated.  The other configurations are timed briefly and reported under
+"also".  One JSON line is printed.
+
+Timing protocol (mirrors the reference's ``time_evaluator(..., min_repeat_ms=600)`` use,
+benchmark/chimera/cuda/bmm_softmax_bmm_cuda.py:39): W untimed warm-up calls, then exactly K
+calls between two HIP events recorded on the launch stream, bracketed by device
+synchronisation.  FLOPs are the algorithmic ``2*batch*M*L*(K+N)`` (the reference counts
+``batch*M*L*(K+N)`` MACs, benchmark/chimera/cpu/bmm_bmm_cpu.py:281); softmax, casts and
+padding count zero.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published peaks (dense)
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "i8": 5000.0, "f32": 157.3}
+PEAK_HBM_GBS = 8000.0
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a copy
+# kernel of known size; see the summaries under profiles/.  None where not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+WORKLOADS = {
+    # name: kind, dtype, dims
+    "attn_bf16_b64_s4096_d128": dict(kind="softmax", dtype="bfloat16", batch=64, M=4096, N=128, K=128, L=4096,
+                                     scale=128 ** -0.5, bound="mfma",
+                                     desc="BMM-softmax-BMM, batch 4x16 heads, seq 4096, head dim 128, bf16"),
+    "attn_f16_b96_s512_d64": dict(kind="softmax", dtype="float16", batch=96, M=512, N=64, K=64, L=512,
+                                  scale=0.125, bound="hbm",
+                                  desc="BMM-softmax-BMM, BERT-base: batch 8x12 heads, seq 512, head dim 64, fp16"),
+    "gemm_chain_f16_b1_512x64x64x64": dict(kind="cast", dtype="float16", batch=1, M=512, N=64, K=64, L=64,
+                                           scale=1.0, bound="hbm",
+                                           desc="GEMM chain (A.B).D at the shape of the CPU plumbing case, fp16"),
+}
+DEFAULT_WORKLOAD = "attn_bf16_b64_s4096_d128"
+SHORT = {"bfloat16": "bf16", "float16": "f16", "int8": "i8", "float32": "f32"}
+
+
+def flops_of(w):
+    return 2.0 * w["batch"] * w["M"] * w["L"] * (w["K"] + w["N"])
+
+
+def bytes_of(w):
+    eb = 2
+    return eb * w["batch"] * (w["M"] * w["K"] + w["K"] * w["L"] + w["L"] * w["N"] + w["M"] * w["N"])
+
+
+def make_inputs(w, dev):
+    import torch
+
+    g = torch.Generator().manual_seed(0)
+    dt = {"bfloat16": torch.bfloat16, "float16": torch.float16}[w["dtype"]]
+    std = 1.0 if w["kind"] == "softmax" else 0.25
+    a = (torch.randn(w["batch"], w["M"], w["K"], generator=g) * std).to(dt).to(dev)
+    c = (torch.randn(w["batch"], w["L"], w["N"], generator=g) * std).to(dt).to(dev)
+    if w["kind"] == "softmax":
+        # keys are stored [batch, L, K]; the chain's B operand is the transposed view
+        b = torch.randn(w["batch"], w["L"], w["K"], generator=g).to(dt).to(dev).transpose(1, 2)
+    else:
+        b = (torch.randn(w["batch"], w["K"], w["L"], generator=g) * std).to(dt).to(dev)
+    f = torch.empty(w["batch"], w["M"], w["N"], dtype=dt, device=dev)
+    return a, b, c, f
+
+
+def time_gpu(w, steps, warmup, dev):
+    """(ms per step over the synchronised wall clock, ms per launch from HIP events)."""
+    import torch
+
+    from ditto_amd import chain
+
+    a, b, c, f = make_inputs(w, dev)
+    desc = chain.bmm_chain_desc(a, b, c, f, w["kind"], w["scale"])
+    call = lambda: chain.run_bmm_chain(a, b, c, f, desc=desc)  # noqa: E731
+    for _ in range(max(warmup, 1)):
+        call()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        call()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = e0.elapsed_time(e1) / steps
+    tile = chain.select_tile(desc).to_json()
+    return wall_ms, ev_ms, tile
+
+
+def cpu_baseline(w, budget_s=12.0):
+    """The fused CPU loop nest (the checker's restatement of the reference's TensorizeCPU nest)
+    on a bounded sample of the same workload: whole batch entries, one after another, until
+    ``budget_s`` of CPU time is used.  fp32 arithmetic, OpenMP over the host cores."""
+    import numpy as np
+
+    from oracle import oracle as orc
+
+    rng = np.random.default_rng(0)
+    M, N, K, L = w["M"], w["N"], w["K"], w["L"]
+    per_entry = 2.0 * M * L * (K + N)
+    done, elapsed = 0, 0.0
+    out = np.empty((1, M, N), dtype=np.float32)
+    # one untimed entry warms the thread pool and the code
+    A = rng.standard_normal((1, M, K), dtype=np.float32)
+    B = rng.standard_normal((1, K, L), dtype=np.float32)
+    C = rng.standard_normal((1, L, N), dtype=np.float32)
+    inter = "softmax" if w["kind"] == "softmax" else w["kind"]
+    orc.bmm_chain_fused_f32(A, B, C, inter=inter, scale=w["scale"], mb=48, lb=256, out=out)
+    while done < w["batch"] and elapsed < budget_s:
+        A = rng.standard_normal((1, M, K), dtype=np.float32)  # fresh data: nothing is cache-resident
+        B = rng.standard_normal((1, K, L), dtype=np.float32)
+        C = rng.standard_normal((1, L, N), dtype=np.float32)
+        t0 = time.perf_counter()
+        orc.bmm_chain_fused_f32(A, B, C, inter=inter, scale=w["scale"], mb=48, lb=256, out=out)
+        elapsed += time.perf_counter() - t0
+        done += 1
+        if elapsed > 0 and done >= 3 and elapsed / done * (done + 1) > 2.5 * budget_s:
+            break
+    return {
+        "value": per_entry * done / elapsed / 1e12,
+        "unit": "TFLOP/s",
+        "cores": orc.num_threads(),
+        "kind": "port",
+        "sample": "%d of %d batch entries of the same chain in fp32 through the fused CPU loop nest "
+                  "(oracle_bmm_chain_fused_f32), %.1f s" % (done, w["batch"], elapsed),
+    }
+
+
+def run_one(name, steps, warmup, dev):
+    w = WORKLOADS[name]
+    wall_ms, ev_ms, tile = time_gpu(w, steps, warmup, dev)
+    fl, by = flops_of(w), bytes_of(w)
+    short = SHORT[w["dtype"]]
+    tflops = fl / (ev_ms * 1e-3) / 1e12
+    if w["bound"] == "mfma":
+        roof = {"bound": "mfma", "achieved": tflops, "peak": PEAK_TFLOPS[short], "unit": "TFLOP/s",
+                "frac": tflops / PEAK_TFLOPS[short]}
+    else:
+        gbs = by / (ev_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS}
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
+    roof["algorithmic_flops"] = fl
+    roof["algorithmic_bytes"] = by
+    roof["kernel_ms"] = ev_ms
+    return w, wall_ms, ev_ms, tile, roof
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-also", action="store_true", help="skip the brief runs of the other configurations")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the chains shard over batch entries with no "
+                 "exchange step; see DESIGN.md); --gpus %d is not supported" % args.gpus)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a HIP device")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    w, wall_ms, ev_ms, tile, roof = run_one(args.workload, args.steps, args.warmup, dev)
+    fl = flops_of(w)
+    value = fl / (wall_ms * 1e-3) / 1e12
+    short = SHORT[w["dtype"]]
+    line = {
+        "metric": "fused_chain_tflops",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall_ms,
+        "us_per_call": ev_ms * 1e3,
+        "pct_of_mfma_peak": 100.0 * (fl / (ev_ms * 1e-3) / 1e12) / PEAK_TFLOPS[short],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": short,
+        "data": "synthetic",
+        "config": {"workload": args.workload, "description": w["desc"], "batch": w["batch"], "M": w["M"],
+                   "N": w["N"], "K": w["K"], "L": w["L"], "tile": tile},
+        "roofline": roof,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(w)
+    if not args.no_also:
+        also = {}
+        for name in WORKLOADS:
+            if name == args.workload:
+                continue
+            ow, owall, oev, otile, oroof = run_one(name, 200, 20, dev)
+            also[name] = {"us_per_call": oev * 1e3, "tflops": flops_of(ow) / (oev * 1e-3) / 1e12,
+                          "roofline": {k: oroof[k] for k in ("bound", "achieved", "peak", "unit", "frac")}}
+        line["also"] = also
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,14 @@
+"""MI355X-native fused operator chains behind Ditto's hyper_fusion front-end.
+
+    import ditto_amd as ditto
+    from ditto_amd import auto_compute as ac, auto_tensorize as at, hardware as hw
+
+The sub-packages keep the reference's names (``auto_compute``, ``auto_tensorize``,
+``hardware``); ``ditto_amd.build`` stands where ``tvm.build`` is called on the scheduled
+chain.  The compute runs in ``csrc/libditto_chain.so`` (hand-written gfx950 kernels behind the
+C ABI of ``include/ditto_chain.h``); there is no CPU or PyTorch fallback.
+"""
+from . import auto_compute, auto_tensorize, hardware, te  # noqa: F401
+from .module import ChainFunction, build  # noqa: F401
+
+__all__ = ["auto_compute", "auto_tensorize", "hardware", "te", "build", "ChainFunction"]

@@ -127,7 +127,7 @@ def load():
             return _lib
         if not os.path.exists(LIB_PATH):
             raise ChainLibraryError(
-                "%s not found: build it with `python -m ditto_amd.build` (needs hipcc). "
+                "%s not found: build it with `python -m ditto_amd.build_ext` (needs hipcc). "
                 "There is no CPU or PyTorch fallback for the fused chains." % LIB_PATH
             )
         lib = ctypes.CDLL(LIB_PATH)

@@ -1,0 +1,3 @@
+from .bmm_chain import (BatchGemmGemm, BatchGemmGemmMMA, BatchGemmSoftmaxGemm,
+                        BatchGemmSoftmaxGemmMMA)
+from .conv_chain import Conv3x3Conv1x1, conv_chain, conv_relu_conv

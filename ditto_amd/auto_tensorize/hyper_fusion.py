@@ -1,0 +1,262 @@
+"""Chain descriptors and the "tensorize" step that turns a described chain into a kernel
+choice (reference: python/ditto/auto_tensorize/hyper_fusion.py:21-302,
+src/auto_tensorize/hyper_fusion.cc:24-216, 586-607, 1494-1603).
+
+In the reference ``tensorize_cuda`` returns a ``te.Schedule`` that TVM then lowers; here it
+returns a ``ChainSchedule``: the recognised chain (which contraction pair, which inter-path
+op, which epilogue, shapes and dtypes) that ``ditto_amd.build`` binds to one hand-written
+gfx950 kernel through the C ABI.  The 13-integer ``CUDATensorizeParam`` is accepted for
+source compatibility; the tile actually used comes from the library's per-shape table
+(``ditto_bmm_chain_select_tile``), which replaces the reference's parameter search.
+"""
+from dataclasses import dataclass
+from typing import Dict, List
+
+from .. import te
+from ..auto_compute.graph import Layer
+from ..hardware import HardwareParam
+
+
+@dataclass
+class FusionChoice:
+    first_op: te.Operation
+    second_op: te.Operation
+    ordered_iters: List[te.IterVar]
+    attach_pos: int
+
+    def __str__(self):
+        return "FusionChoice(axis=%s, pos=%d)" % (self.ordered_iters, self.attach_pos)
+
+
+def fusion_choice(first_op, second_op, ordered_iters, attach_pos):
+    return FusionChoice(first_op, second_op, list(ordered_iters), int(attach_pos))
+
+
+@dataclass
+class MatchInfo:
+    axis: List[te.IterVar]
+    intrin: object
+    impl: str = ""
+
+    def __str__(self):
+        return "MatchInfo(axis=%s, intrin=%s)" % (self.axis, self.intrin)
+
+
+def match_info(axis, intrin, impl=""):
+    return MatchInfo(list(axis), intrin, impl)
+
+
+class TensorizeHyperFusionState:
+    """Partition of the layer DAG around the two contractions: prologues of each, the single
+    path between them, and the epilogue (hyper_fusion.cc:51-216)."""
+
+    def __init__(self, layer: Layer, fuse_choice: FusionChoice, match_info: Dict[te.Operation, MatchInfo]):
+        self.layer = layer
+        self.first_op = fuse_choice.first_op
+        self.second_op = fuse_choice.second_op
+        if not fuse_choice.attach_pos < len(fuse_choice.ordered_iters):
+            raise ValueError("attach_pos %d out of range of %d ordered iters"
+                             % (fuse_choice.attach_pos, len(fuse_choice.ordered_iters)))
+        self.fused_spatial_outer_iters, self.fused_reduce_outer_iters = [], []
+        for iv in fuse_choice.ordered_iters[: fuse_choice.attach_pos + 1]:
+            if iv.iter_type == te.DATA_PAR:
+                self.fused_spatial_outer_iters.append(iv)
+            elif iv.iter_type == te.COMM_REDUCE:
+                self.fused_reduce_outer_iters.append(iv)
+            else:
+                raise ValueError("Unexpected iter_type %s." % iv.iter_type)
+        self.first_op_prologue, self.second_op_prologue = [], []
+        self.inter_path, self.epilogue = [], []
+        if len(layer.ops) != 1:
+            raise ValueError("a fused chain has exactly one output op, got %d" % len(layer.ops))
+
+        prefix = {}
+        found = {"first": False, "second": False}
+
+        def helper(op):
+            if not isinstance(op, te.ComputeOp):
+                return False, False
+            if op in prefix or (op is self.first_op and found["first"]) or (op is self.second_op and found["second"]):
+                raise ValueError("The same op %s is visited multiple times.\n"
+                                 "The given layer is not a tree structure." % op.name)
+            met_first = met_second = False
+            if op is self.first_op:
+                for inp in op.input_tensors:
+                    f, s = helper(inp.op)
+                    if f or s or found["first"] or found["second"]:
+                        raise ValueError("the first contraction must not consume a contraction")
+                    if inp.op in prefix:
+                        self.first_op_prologue.append(prefix[inp.op])
+                found["first"] = True
+                met_first = True
+            elif op is self.second_op:
+                first_in_producer = False
+                for inp in op.input_tensors:
+                    f, s = helper(inp.op)
+                    if s or found["second"]:
+                        raise ValueError("the second contraction appears twice")
+                    first_in_producer |= f
+                    if inp.op in prefix:
+                        if f:
+                            if self.inter_path:
+                                raise ValueError("Multiple paths from first op to second op.")
+                            self.inter_path = prefix[inp.op]
+                        else:
+                            self.second_op_prologue.append(prefix[inp.op])
+                if not first_in_producer:
+                    raise ValueError("First op is not the producer of second op.")
+                found["second"] = True
+                met_second = True
+            else:
+                chain = []
+                for inp in op.input_tensors:
+                    f, s = helper(inp.op)
+                    met_first |= f
+                    met_second |= s
+                    chain.extend(prefix.get(inp.op, []))
+                prefix[op] = chain + [op]
+            return met_first, met_second
+
+        helper(layer.ops[0])
+        if layer.ops[0] in prefix:
+            self.epilogue = prefix[layer.ops[0]]
+        if not (found["first"] and found["second"]):
+            raise ValueError("the layer does not contain both contraction ops of the fusion choice")
+        if self.first_op not in match_info or self.second_op not in match_info:
+            raise ValueError("match_info must cover both contraction ops")
+        self.tensorize_iters = {op: mi.axis for op, mi in match_info.items()}
+        self.tensorize_intrinsics = {op: mi.intrin for op, mi in match_info.items()}
+        self.tensorize_impl = {op: mi.impl for op, mi in match_info.items()}
+
+    def __str__(self):
+        return "TensorizeHyperFusionState(layer=%s)" % self.layer.name
+
+    def summary(self, verbose=False):
+        ret = "TensorizeHyperFusionState Summary:\n==================================\n"
+        ret += "First op: %s\nSecond op: %s\n" % (self.first_op.name, self.second_op.name)
+        if verbose:
+            line = "----------------------------------\n"
+            ret += line + "First op prologue:\n" + line
+            for v in self.first_op_prologue:
+                ret += "[" + " ".join(o.name for o in v) + " ]\n"
+            ret += line + "Second op prologue:\n" + line
+            for v in self.second_op_prologue:
+                ret += "[" + " ".join(o.name for o in v) + " ]\n"
+            ret += line + "Inter Path:\n[" + " ".join(o.name for o in self.inter_path) + " ]\n"
+            ret += line + "Epilogue:\n[" + " ".join(o.name for o in self.epilogue) + " ]\n"
+            ret += line + "Fused outer spatial iters: %s\n" % self.fused_spatial_outer_iters
+            ret += "Fused outer reduce iters: %s\n" % self.fused_reduce_outer_iters
+        ret += "==================================\n"
+        return ret
+
+
+def tensorize_hyper_fusion_state(layer, fuse_choice, match_info):
+    return TensorizeHyperFusionState(layer, fuse_choice, match_info)
+
+
+@dataclass
+class CUDATensorizeParam:
+    warp_size: int = 32
+    ty_size: int = 4
+    tz_size: int = 2
+    input_vector_len: int = 4
+    serial_y: int = 2
+    serial_z: int = 1
+    block_rx: int = 4
+    block_ry: int = 1
+    block_rz: int = 4
+    warp_rx: int = 1
+    warp_ry: int = 4
+    warp_rz: int = 1
+    unroll_steps: int = 1500
+
+    def to_json(self):
+        # the same eleven keys the reference serialises (hyper_fusion.py:143-156)
+        keys = ["warp_size", "ty_size", "tz_size", "input_vector_len", "serial_y", "serial_z", "block_rx",
+                "warp_rx", "block_ry", "warp_ry", "unroll_steps"]
+        return {k: getattr(self, k) for k in keys}
+
+    def __str__(self):
+        return str(self.to_json())
+
+
+def cuda_tensorize_param(warp_size=32, ty_size=4, tz_size=2, input_vector_len=4, serial_y=2, serial_z=1,
+                         block_rx=4, block_ry=1, block_rz=4, warp_rx=1, warp_ry=4, warp_rz=1, unroll_steps=1500):
+    return CUDATensorizeParam(warp_size, ty_size, tz_size, input_vector_len, serial_y, serial_z, block_rx,
+                              block_ry, block_rz, warp_rx, warp_ry, warp_rz, unroll_steps)
+
+
+@dataclass
+class ChainSchedule:
+    """What ``tensorize_cuda`` / ``tensorize_hip`` returns: the recognised chain."""
+    layer: Layer
+    state: TensorizeHyperFusionState
+    kind: str            # "bmm_chain" | "conv_chain"
+    inter_op: str        # "cast" | "relu" | "softmax"
+    in_dtype: str
+    acc_dtype: str
+    out_dtype: str
+    dims: dict
+    softmax_scale: float = 1.0
+    relu_out: bool = False
+    hw_param: HardwareParam = None
+    tensorize_param: CUDATensorizeParam = None
+
+
+def _kinds(ops):
+    return [op.kind for op in ops]
+
+
+def _recognise(layer, state):
+    first, second = state.first_op, state.second_op
+    if first.kind != "contract" or second.kind != "contract":
+        raise ValueError("The fusion and tensorize decisions are not valid.")
+    inter = _kinds(state.inter_path)
+    epi = _kinds(state.epilogue)
+    out_t = layer.ops[0].output(0)
+    if first.attrs.get("conv"):
+        # conv -> (cast|relu) -> pad -> conv -> (cast|relu)
+        if len(inter) != 2 or inter[0] not in ("cast", "relu") or inter[1] != "pad":
+            raise ValueError("unsupported inter path %s for a conv chain" % inter)
+        if epi not in (["unpack_cast"], ["relu_cast"]):
+            raise ValueError("unsupported epilogue %s for a conv chain" % epi)
+        img = first.input_tensors[0].op.input_tensors[0]  # pad1 <- Img
+        w1, w2 = first.input_tensors[1], second.input_tensors[1]
+        N, C0, H, W = img.shape
+        C1, _, R1, S1 = w1.shape
+        C2, _, R2, S2 = w2.shape
+        dims = dict(N=N, C0=C0, H=H, W=W, C1=C1, R1=R1, S1=S1, pad1=first.attrs["padding"],
+                    stride1=first.attrs["stride"], C2=C2, R2=R2, S2=S2, pad2=second.attrs["padding"],
+                    stride2=second.attrs["stride"])
+        return dict(kind="conv_chain", inter_op=inter[0], dims=dims, relu_out=epi == ["relu_cast"],
+                    in_dtype=img.dtype, acc_dtype=first.output(0).dtype, out_dtype=out_t.dtype, softmax_scale=1.0)
+    # batched GEMM chain: dims from the layer's input placeholders
+    A, B, C = layer.inputs[:3] if len(layer.inputs) >= 3 else (layer.inputs + layer.weights)[:3]
+    batch, M, K = A.shape
+    L, N = B.shape[2], C.shape[2]
+    dims = dict(batch=batch, M=M, N=N, K=K, L=L)
+    if inter == ["exp"]:
+        pro = [k for chain in state.second_op_prologue for k in _kinds(chain)]
+        pads = [op for chain in state.second_op_prologue for op in chain if op.kind == "pad"]
+        if pro != ["pad"] or pads[0].attrs.get("pad_value") != 1 or epi != ["unpack_divide"]:
+            raise ValueError("an exp inter path needs the ones-column operand and the divide epilogue "
+                             "(got prologue %s, epilogue %s)" % (pro, epi))
+        return dict(kind="bmm_chain", inter_op="softmax", dims=dims, relu_out=False, in_dtype=A.dtype,
+                    acc_dtype=first.output(0).dtype, out_dtype=out_t.dtype,
+                    softmax_scale=state.inter_path[0].attrs.get("scale", 1.0))
+    if inter in (["cast"], ["relu"]) and epi == ["unpack_cast"]:
+        return dict(kind="bmm_chain", inter_op=inter[0], dims=dims, relu_out=False, in_dtype=A.dtype,
+                    acc_dtype=first.output(0).dtype, out_dtype=out_t.dtype, softmax_scale=1.0)
+    raise ValueError("The fusion and tensorize decisions are not valid (inter path %s, epilogue %s)." % (inter, epi))
+
+
+def tensorize_hip(layer, state, hip_param=None, tensorize_param=None):
+    """Bind a described chain to its gfx950 kernel family.  Raises ``ValueError`` for chains
+    the path does not cover, where the reference raises ``TVMError`` from a failed CHECK."""
+    info = _recognise(layer, state)
+    return ChainSchedule(layer=layer, state=state, hw_param=hip_param, tensorize_param=tensorize_param, **info)
+
+
+def tensorize_cuda(layer, state, cuda_param=None, tensorize_param=None):
+    """Same entry point and argument list as the reference's (hyper_fusion.py:191-197)."""
+    return tensorize_hip(layer, state, cuda_param, tensorize_param)

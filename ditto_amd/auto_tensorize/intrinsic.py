@@ -1,0 +1,120 @@
+"""Matrix-core contracts (reference: python/ditto/auto_tensorize/intrinsic.py:252-272 for
+``cuda_wmma``, :37-48 for ``intrinsic_match``; src/auto_tensorize/intrinsic.cc:9-32).
+
+``cuda_wmma`` keeps its signature; on this target it describes the same 16x16x16 logical
+tile, which the gfx950 kernels execute with MFMA.  ``hip_mfma`` names the hardware tile
+directly."""
+from dataclasses import dataclass
+from typing import List
+
+from .. import te
+from .pattern import IsCubic
+
+# gfx950 dense MFMA tiles: (M, N, K) per input type
+MFMA_SHAPES = {
+    "float16": [(32, 32, 16), (16, 16, 32)],
+    "bfloat16": [(32, 32, 16), (16, 16, 32)],
+    "int8": [(32, 32, 32), (16, 16, 64)],
+    "float32": [(32, 32, 2), (16, 16, 4)],
+}
+_ACC = {"float16": ("float32",), "bfloat16": ("float32",), "int8": ("int32",), "float32": ("float32",)}
+
+
+@dataclass(frozen=True)
+class TensorIntrin:
+    name: str
+    M: int
+    N: int
+    K: int
+    in_dtype: str
+    out_dtype: str
+    scope: str = ""
+
+
+@dataclass(frozen=True)
+class PackedIntrinsic:
+    load_intrinsics: tuple
+    compute_intrinsic: TensorIntrin
+    store_intrinsic: TensorIntrin
+    load_scopes: tuple
+    compute_scope: str
+    store_scope: str
+
+    def __str__(self):
+        return "PackedIntrinsic(load=%s; compute=%s; store=%s)" % (
+            [i.name for i in self.load_intrinsics], self.compute_intrinsic.name, self.store_intrinsic.name)
+
+
+def packed_intrinsic(loads, compute, store, load_scopes, compute_scope, store_scope):
+    return PackedIntrinsic(tuple(loads), compute, store, tuple(load_scopes), compute_scope, store_scope)
+
+
+def cuda_wmma(M=16, N=16, K=16, in_dtype="float16", out_dtype="float32", scope="global"):
+    """The tensor-core contract of the reference: A/B tiles loaded row-major, accumulator
+    fragment zero-filled, multiply-accumulated, stored row-major to ``scope``."""
+    loads = [TensorIntrin("load_a", M, N, K, in_dtype, in_dtype, "shared"),
+             TensorIntrin("load_b", M, N, K, in_dtype, in_dtype, "shared")]
+    compute = TensorIntrin("gemm", M, N, K, in_dtype, out_dtype)
+    store = TensorIntrin("store", M, N, K, out_dtype, out_dtype, scope)
+    return packed_intrinsic(loads, compute, store, ["wmma.matrix_a", "wmma.matrix_b"], "wmma.accumulator",
+                            "wmma.accumulator")
+
+
+def hip_mfma(M=32, N=32, K=16, in_dtype="float16", out_dtype="float32", scope="vgpr"):
+    """A gfx950 MFMA tile.  Operands come from VGPRs (loaded from LDS), the accumulator stays
+    in VGPRs/AGPRs: ``scope`` is "vgpr" for the first contraction of a chain (its result is
+    consumed in registers) and "global" for the second."""
+    if in_dtype not in MFMA_SHAPES:
+        raise ValueError("no MFMA for input type %s" % in_dtype)
+    if (M, N, K) not in MFMA_SHAPES[in_dtype]:
+        raise ValueError("no %dx%dx%d MFMA for %s; have %s" % (M, N, K, in_dtype, MFMA_SHAPES[in_dtype]))
+    if out_dtype not in _ACC[in_dtype]:
+        raise ValueError("MFMA on %s accumulates in %s, not %s" % (in_dtype, _ACC[in_dtype][0], out_dtype))
+    loads = [TensorIntrin("lds_read_a", M, N, K, in_dtype, in_dtype, "lds"),
+             TensorIntrin("lds_read_b", M, N, K, in_dtype, in_dtype, "lds")]
+    compute = TensorIntrin("mfma_%dx%dx%d" % (M, N, K), M, N, K, in_dtype, out_dtype)
+    store = TensorIntrin("store", M, N, K, out_dtype, out_dtype, scope)
+    return packed_intrinsic(loads, compute, store, ["mfma.a", "mfma.b"], "mfma.accumulator", "mfma.accumulator")
+
+
+def intrinsic_match(target: te.Tensor, packed_intrin: PackedIntrinsic, restrictions: List[str] = ()):
+    """Iteration variables of ``target`` that map onto the intrinsic's (i, j, k).
+
+    Returns a list of choices; callers take ``[0]`` = ``[mi, ni, rki]``
+    (bmm_bmm_cuda.py:182-188).  With "InnerMost" the innermost spatial variable owned by each
+    input and the innermost shared reduce variable are chosen; with "SameRange" their extents
+    must equal the intrinsic's tile (for a 16^3 ``cuda_wmma`` tile; MFMA tiles are matched on
+    divisibility, since the kernels re-tile the packed 16-blocks themselves).
+    """
+    op = target.op if isinstance(target, te.Tensor) else target
+    if not IsCubic(op):
+        return []
+    intr = packed_intrin.compute_intrinsic
+    n_in = len(op.accesses)
+
+    def owned_by(i):
+        return [iv for iv in op.axis
+                if any(v is iv for v in op.accesses[i][1])
+                and not any(any(v is iv for v in op.accesses[j][1]) for j in range(n_in) if j != i)]
+
+    a_owned, b_owned = owned_by(0), owned_by(1)
+    shared = [iv for iv in op.reduce_axis if all(any(v is iv for v in acc[1]) for acc in op.accesses)]
+    if not a_owned or not b_owned or not shared:
+        return []
+    choices = []
+    a_cands = a_owned[::-1] if "InnerMost" in restrictions else a_owned
+    b_cands = b_owned[::-1] if "InnerMost" in restrictions else b_owned
+    k_cands = shared[::-1] if "InnerMost" in restrictions else shared
+    for mi in a_cands:
+        for ni in b_cands:
+            for ki in k_cands:
+                if "SameRange" in restrictions:
+                    is_wmma = intr.name == "gemm"
+                    ok = ((mi.extent, ni.extent, ki.extent) == (intr.M, intr.N, intr.K)) if is_wmma else (
+                        mi.extent % 16 == 0 and ni.extent % 16 == 0 and ki.extent % 16 == 0)
+                    if not ok:
+                        continue
+                choices.append([mi, ni, ki])
+                if "InnerMost" in restrictions:
+                    return choices
+    return choices

