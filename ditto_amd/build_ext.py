@@ -21,6 +21,9 @@ HIPCC_FLAGS = [
     "-std=c++17",
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # let MFMA read and write its accumulator in arch VGPRs where the allocator can: the
+    # inter-path op works on the accumulator, so AGPR-resident results cost a copy per use
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument",
 ]
 

@@ -38,6 +38,7 @@ constexpr int kInterCast = 0;
 constexpr int kInterSoftmax = 2;
 
 constexpr int kBN = 64;  // L step
+constexpr float kLazy = 8.0f;  // log2 of the slack allowed before the running maximum is raised
 constexpr int kNW = 4;   // waves per workgroup
 
 // Row stride (elements) of a row-major 16-bit LDS tile that is read with transpose
@@ -213,24 +214,27 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
         for (int i = 0; i < 2; ++i)
 #pragma unroll
           for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[i][j][r]);
-        mx = pair_max(mx);
-        const float mnew = fmaxf(mrow[j], mx * c2);
-        const float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);
-        mrow[j] = mnew;
-        float rs = 0.f;
+        mx = pair_max(mx) * c2;
+        // Lazy rescale: the running maximum only has to bound the scores well enough that
+        // exp2 cannot overflow, so it is raised (and the accumulators rescaled) only when
+        // some row of the wave exceeds it by more than 2^kLazy.  Rows keep a stale maximum
+        // otherwise; the final division by the row sum cancels it exactly.
+        if (__builtin_amdgcn_ballot_w64(mx > mrow[j] + kLazy) != 0) {
+          const float mnew = fmaxf(mrow[j], mx);
+          const float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);
+          mrow[j] = mnew;
+          lsum[j] *= alpha;
+#pragma unroll
+          for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[t][j][r] *= alpha;
+        }
+        const float mcur = mrow[j];
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i][j][r], c2, -mnew));
-            s[i][j][r] = e;
-            rs += e;
-          }
-        lsum[j] = lsum[j] * alpha + rs;
-#pragma unroll
-        for (int t = 0; t < D / 32; ++t)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) o[t][j][r] *= alpha;
+          for (int r = 0; r < 16; ++r)
+            s[i][j][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i][j][r], c2, -mcur));
       }
     } else if (p.relu) {
 #pragma unroll
@@ -254,6 +258,14 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
         typename Elem<T>::v2 p1 = cvt2<T>(s[i][j][r0 + 2], s[i][j][r0 + 3]);
         typename Elem<T>::v2 p2 = cvt2<T>(s[i][j][r0 + 4], s[i][j][r0 + 5]);
         typename Elem<T>::v2 p3 = cvt2<T>(s[i][j][r0 + 6], s[i][j][r0 + 7]);
+        if (INTER == kInterSoftmax) {
+          // the row sum is taken over the ROUNDED probabilities, i.e. exactly the values
+          // that enter the second contraction
+          lsum[j] = Elem<T>::add_pair(p0, lsum[j]);
+          lsum[j] = Elem<T>::add_pair(p1, lsum[j]);
+          lsum[j] = Elem<T>::add_pair(p2, lsum[j]);
+          lsum[j] = Elem<T>::add_pair(p3, lsum[j]);
+        }
         V8 v = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
         pf[j] = v;
       }

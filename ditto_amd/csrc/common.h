@@ -43,6 +43,11 @@ struct Elem<f16> {
   static __device__ __forceinline__ f32x4 mfma16(v8 a, v8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
+  // acc + p[0] + p[1] in one instruction (v_dot2c_f32_f16 against a pair of ones)
+  static __device__ __forceinline__ float add_pair(v2 p, float acc) {
+    const v2 ones = {(f16)1.0f, (f16)1.0f};
+    return __builtin_amdgcn_fdot2(p, ones, acc, false);
+  }
 };
 
 template <>
@@ -55,6 +60,10 @@ struct Elem<bf16> {
   }
   static __device__ __forceinline__ f32x4 mfma16(v8 a, v8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float add_pair(v2 p, float acc) {
+    const v2 ones = {(bf16)1.0f, (bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(p, ones, acc, false);
   }
 };
 
