@@ -45,7 +45,7 @@ class BmmChainDesc(ctypes.Structure):
         ("f_batch_stride", ctypes.c_int64),
         ("f_row_stride", ctypes.c_int64),
         ("softmax_scale", ctypes.c_float),
-        ("requant_shift_uniform", ctypes.c_int32),
+        ("requant_scale", ctypes.c_float),
     ]
 
 

@@ -30,6 +30,7 @@ HIPCC_FLAGS = [
 # (object name, source, extra defines)
 UNITS = [
     ("api", "api.hip", []),
+    ("gemm_chain_i8", "gemm_chain_i8.hip", []),
     ("fp_f16_cast", "bmm_chain_fp_inst.hip",
      ["-DDITTO_INST_T=f16", "-DDITTO_INST_INTER=0", "-DDITTO_INST_NAME=launch_f16_cast"]),
     ("fp_f16_softmax", "bmm_chain_fp_inst.hip",

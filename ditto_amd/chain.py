@@ -49,7 +49,7 @@ def _as3d(t, name):
     return t
 
 
-def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_shift=-1):
+def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=1.0):
     """Fill a ``ditto_bmm_chain_desc`` from tensors A[b,M,K], B[b,K,L], C[b,L,N], F[b,M,N].
 
     B may be a transposed view of a ``[b, L, K]`` tensor (stride 1 along K); it is then
@@ -90,7 +90,7 @@ def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_shift
     d.c_batch_stride, d.c_row_stride = C.stride(0), C.stride(1)
     d.f_batch_stride, d.f_row_stride = F.stride(0), F.stride(1)
     d.softmax_scale = float(softmax_scale)
-    d.requant_shift_uniform = int(requant_shift)
+    d.requant_scale = float(requant_scale)
     return d
 
 
@@ -105,15 +105,20 @@ def select_tile(desc):
     return tile
 
 
-def run_bmm_chain(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_shift=-1, aux=None, desc=None):
-    """F[b] = epilogue(inter(A[b] . B[b]) . C[b]) as ONE kernel on the current stream."""
+def run_bmm_chain(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=1.0, aux=None, desc=None):
+    """F[b] = epilogue(inter(A[b] . B[b]) . C[b]) as ONE kernel on the current stream.
+
+    ``aux``: for ``inter_op="requant"`` an fp32 tensor of L per-column scales (``None``: use
+    ``requant_scale`` for every column)."""
     lib = _lib.load()
     dev = _check_device(A, B, C, F)
     if desc is None:
-        desc = bmm_chain_desc(A, B, C, F, inter_op, softmax_scale, requant_shift)
+        desc = bmm_chain_desc(A, B, C, F, inter_op, softmax_scale, requant_scale)
     aux_ptr = None
     if aux is not None:
         _check_device(A, aux)
+        if aux.dtype != torch.float32 or not aux.is_contiguous() or aux.numel() != desc.L:
+            raise ValueError("aux must be a contiguous fp32 tensor of L = %d scales" % desc.L)
         aux_ptr = aux.data_ptr()
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream

@@ -124,6 +124,39 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     t.variant = plan->d_pad * 10 + plan->qt;
     return DITTO_OK;
   }
+  if (in == DITTO_I8) {
+    if (d->acc_dtype != DITTO_I32 || d->out_dtype != DITTO_I32)
+      return fail(DITTO_EINVAL, "the int8 chain accumulates and outputs int32");
+    if (d->inter_op != DITTO_INTER_REQUANT)
+      return fail(DITTO_EUNSUPPORTED, "the int8 chain needs inter_op = DITTO_INTER_REQUANT");
+    if (d->b_layout != DITTO_B_KL) return fail(DITTO_EUNSUPPORTED, "the int8 chain takes B as [K][L]");
+    if (d->K % 16 || d->L % 16 || d->N % 16)
+      return fail(DITTO_EINVAL, "K, L and N must be multiples of 16 for the int8 chain");
+    if (d->a_row_stride % 16 || d->b_row_stride % 16 || d->c_row_stride % 16 || d->a_batch_stride % 16 ||
+        d->b_batch_stride % 16 || d->c_batch_stride % 16)
+      return fail(DITTO_EINVAL, "int8 input strides must be multiples of 16 elements");
+    if (d->a_row_stride < d->K || d->b_row_stride < d->L || d->c_row_stride < d->N || d->f_row_stride < d->N)
+      return fail(DITTO_EINVAL, "row stride smaller than row extent");
+    if (d->a_row_stride > 0x7fffffff || d->b_row_stride > 0x7fffffff || d->c_row_stride > 0x7fffffff ||
+        d->f_row_stride > 0x7fffffff || d->K > 0x7fffffff / 2 || d->N > 0x7fffffff / 2)
+      return fail(DITTO_EINVAL, "extent or row stride too large");
+    const long long Lp = (d->L + 255) / 256 * 256;
+    const int lds = ditto::i8_chain_lds_bytes_host((int)Lp);
+    if (lds > 160 * 1024)
+      return fail(DITTO_EUNSUPPORTED, "L=%lld: the requantised row block does not fit in LDS", (long long)d->L);
+    plan->family = 2;
+    ditto_tile_param& t = plan->tile;
+    t.block_threads = 256;
+    t.block_m = 64;
+    t.block_l = (int)Lp;
+    t.block_n = 256;
+    t.head_pad = 0;
+    t.lds_bytes = lds;
+    t.grid_x = (int)(((d->M + 63) / 64) * d->batch);
+    t.grid_y = t.grid_z = 1;
+    t.variant = 8064;
+    return DITTO_OK;
+  }
   return fail(DITTO_EUNSUPPORTED, "no chain kernel for in_dtype %d", in);
 }
 
@@ -195,6 +228,34 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     else
       e = sm ? ditto::launch_bf16_softmax(plan.d_pad, plan.qt, kl, args, st)
              : ditto::launch_bf16_cast(plan.d_pad, plan.qt, kl, args, st);
+    if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
+    return DITTO_OK;
+  }
+  if (plan.family == 2) {
+    if (aux && !aligned(aux, 4)) return fail(DITTO_EINVAL, "aux (scale vector) must be 4-byte aligned");
+    ditto::I8ChainArgs args;
+    args.a = static_cast<const int8_t*>(a);
+    args.b = static_cast<const int8_t*>(b);
+    args.d = static_cast<const int8_t*>(c);
+    args.scale = static_cast<const float*>(aux);
+    args.scale_uniform = d->requant_scale;
+    args.e = static_cast<int32_t*>(f);
+    args.a_bs = d->a_batch_stride;
+    args.b_bs = d->b_batch_stride;
+    args.d_bs = d->c_batch_stride;
+    args.e_bs = d->f_batch_stride;
+    args.a_rs = (int)d->a_row_stride;
+    args.b_rs = (int)d->b_row_stride;
+    args.d_rs = (int)d->c_row_stride;
+    args.e_rs = (int)d->f_row_stride;
+    args.M = (int)d->M;
+    args.N = (int)d->N;
+    args.K = (int)d->K;
+    args.L = (int)d->L;
+    args.batch = (int)d->batch;
+    args.mblocks = (int)((d->M + 63) / 64);
+    args.Lp = plan.tile.block_l;
+    hipError_t e = ditto::launch_gemm_chain_i8(args, st);
     if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
     return DITTO_OK;
   }

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include "bmm_chain_fp.h"
+#include "gemm_chain_i8.h"
 
 namespace ditto {
 

@@ -1,0 +1,26 @@
+// Arguments and launcher of the int8 requantised GEMM chain kernel (gemm_chain_i8.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ditto {
+
+struct I8ChainArgs {
+  const int8_t* a;
+  const int8_t* b;
+  const int8_t* d;
+  const float* scale;   // [L] or null
+  float scale_uniform;  // used when scale == null
+  int32_t* e;
+  long long a_bs, b_bs, d_bs, e_bs;  // batch strides, elements
+  int a_rs, b_rs, d_rs, e_rs;        // row strides, elements
+  int M, N, K, L, batch;
+  int mblocks;
+  int Lp;  // L rounded up to the weight-chunk width
+};
+
+// dynamic LDS bytes of the kernel for a given padded L
+int i8_chain_lds_bytes_host(int Lp);
+hipError_t launch_gemm_chain_i8(const I8ChainArgs& args, hipStream_t stream);
+
+}  // namespace ditto

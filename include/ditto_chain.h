@@ -51,7 +51,8 @@ typedef enum ditto_inter_op {
   DITTO_INTER_CAST = 0,    /* mid = cast_in(acc)                      bmm_bmm_cuda.py:114-118           */
   DITTO_INTER_RELU = 1,    /* mid = cast_in(max(acc,0))               conv_relu_conv_relu_fuse_hw_cuda.py:134-142 */
   DITTO_INTER_SOFTMAX = 2, /* mid = softmax(scale*acc) over L, online  bmm_chain.py:63-103 (exp + ones column + divide) */
-  DITTO_INTER_REQUANT = 3  /* mid = sat_i8(rne(acc * 2^-shift[col]))   int8 chain, BASELINE config 5     */
+  DITTO_INTER_REQUANT = 3  /* mid = sat_i8(rne(acc * scale[col]))      int8 chain; not in the reference,
+                              whose int8 chain wraps with astype("int8") (bmm_bmm_cuda.py:116)   */
 } ditto_inter_op;
 
 /* How the second operand of the first contraction is laid out in memory. */
@@ -82,8 +83,7 @@ typedef struct ditto_bmm_chain_desc {
   int64_t c_batch_stride, c_row_stride; /* C[b][l][n]                                  */
   int64_t f_batch_stride, f_row_stride; /* F[b][m][n]                                  */
   float softmax_scale;   /* DITTO_INTER_SOFTMAX only; the reference uses 1.0           */
-  int32_t requant_shift_uniform; /* DITTO_INTER_REQUANT: if >=0, every column uses this
-                                    power-of-two shift and `aux` may be NULL           */
+  float requant_scale;   /* DITTO_INTER_REQUANT: scale of every column when `aux` is NULL */
 } ditto_bmm_chain_desc;
 
 /*
@@ -140,8 +140,9 @@ size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc);
  * Run one fused chain: replaces `func(A, B, C, F)` of the built PackedFunc
  * (bmm_bmm_cuda.py:256, bmm_softmax_bmm_cuda.py:256).
  *   a, b, c : inputs (device), read-only
- *   aux     : DITTO_INTER_REQUANT: int32 shift[L] per intermediate column
- *             (mid = sat_i8(rne(acc / 2^shift))), else NULL
+ *   aux     : DITTO_INTER_REQUANT: fp32 scale[L], one per intermediate column:
+ *             mid = saturate_to_[-128,127](round_to_nearest_even((float)acc * scale[l]));
+ *             NULL to use desc->requant_scale for every column.  Other chains: NULL
  *   f       : output (device), must not alias an input
  */
 int ditto_bmm_chain_run(const ditto_bmm_chain_desc* desc, const void* a, const void* b,

@@ -1,0 +1,106 @@
+"""Bit-exact parity of the int8 requantised GEMM chain against the exact-integer checker."""
+import numpy as np
+import pytest
+import torch
+
+from ditto_amd import chain
+
+pytestmark = pytest.mark.gpu
+
+
+def run_i8(A, B, D, scale=None, uniform=None):
+    dev = "cuda:0"
+    a, b, d = (torch.from_numpy(np.ascontiguousarray(x)).to(dev) for x in (A, B, D))
+    M, N = A.shape[-2], D.shape[-1]
+    shape = (A.shape[0], M, N) if A.ndim == 3 else (M, N)
+    e = torch.full(shape, -7, dtype=torch.int32, device=dev)
+    aux = None if scale is None else torch.from_numpy(scale).to(dev)
+    chain.run_bmm_chain(a, b, d, e, "requant", requant_scale=uniform if uniform is not None else 1.0, aux=aux)
+    torch.cuda.synchronize()
+    return e.cpu().numpy()
+
+
+@pytest.mark.parametrize("shape", [
+    # M, K, L, N
+    (64, 64, 256, 256),
+    (128, 128, 256, 512),
+    (100, 96, 48, 80),       # ragged M, L below one chunk, N below one chunk
+    (200, 1024, 256, 1024),  # the full K / L / N of the quantised configuration, fewer rows
+    (64, 64, 512, 272),      # two L chunks
+    (37, 16, 16, 16),        # smallest legal extents
+])
+def test_i8_chain_bit_exact(oracle, shape):
+    M, K, L, N = shape
+    A, B, D, scale = oracle.make_i8_chain_inputs(M, K, L, N, seed=M + N)
+    want = oracle.gemm_chain_i8(A, B, D, scale)[0]
+    got = run_i8(A, B, D, scale)
+    assert got.dtype == np.int32 and np.array_equal(got, want)
+    # uniform scale through the descriptor gives the same result as the vector
+    assert np.array_equal(run_i8(A, B, D, None, uniform=2.0 ** -10), want)
+
+
+def test_i8_chain_per_column_scales_and_saturation(oracle):
+    M, K, L, N = 96, 256, 64, 48
+    A, B, D, _ = oracle.make_i8_chain_inputs(M, K, L, N, seed=5)
+    rng = np.random.default_rng(1)
+    scale = (2.0 ** -rng.integers(6, 14, L)).astype(np.float32)
+    scale[::7] = np.float32(0.0123)  # not a power of two: exercises the fp32 multiply + RNE
+    want, mid = oracle.gemm_chain_i8(A, B, D, scale, return_mid=True)
+    assert (mid == 127).any() and (mid == -128).any()  # both saturation ends are hit
+    assert np.array_equal(run_i8(A, B, D, scale), want[0])
+
+
+def test_i8_chain_ties_round_to_even(oracle):
+    # A = row of ones times B = multiples of 512 gives exact .5 ties at scale 2^-10
+    M, K, L, N = 64, 16, 16, 16
+    A = np.zeros((M, K), np.int8); A[:, 0] = 1
+    B = np.zeros((K, L), np.int8)
+    D = np.eye(L, N, dtype=np.int8)
+    A[:, 1] = 4; B[1, :] = 127          # 508
+    A[:, 2] = 4; B[2, :] = np.arange(1, 17)  # 4*(1..16): with 508 -> 512, 516, ...
+    scale = np.full(L, 2.0 ** -10, np.float32)
+    want = oracle.gemm_chain_i8(A, B, D, scale)[0]
+    got = run_i8(A, B, D, scale)
+    assert np.array_equal(got, want)
+    assert got[0, 0] == 0  # 512 / 1024 = 0.5 rounds to even 0
+
+
+def test_i8_chain_batched_and_full_rows(oracle):
+    rng = np.random.default_rng(2)
+    batch, M, K, L, N = 3, 70, 64, 32, 64
+    A = rng.integers(-127, 128, (batch, M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (batch, K, L), dtype=np.int8)
+    D = rng.integers(-127, 128, (batch, L, N), dtype=np.int8)
+    scale = np.full(L, 2.0 ** -9, np.float32)
+    want = oracle.gemm_chain_i8(A, B, D, scale)
+    assert np.array_equal(run_i8(A, B, D, scale), want)
+
+
+def test_i8_chain_full_size_properties(oracle):
+    # BASELINE size: A[8192,1024], B[1024,256], D[256,1024].  The exact oracle runs on a row
+    # sample; the whole output is checked through linearity in D: E(D1 + D2) = E(D1) + E(D2)
+    M, K, L, N = 8192, 1024, 256, 1024
+    A, B, D, scale = oracle.make_i8_chain_inputs(M, K, L, N, seed=0)
+    got = run_i8(A, B, D, scale)
+    rows = np.r_[0:64, 4000:4064, 8128:8192]
+    want = oracle.gemm_chain_i8(A[rows], B, D, scale)[0]
+    assert np.array_equal(got[rows], want)
+    D1 = (D // 2).astype(np.int8)
+    D2 = (D - D1).astype(np.int8)
+    assert np.array_equal(run_i8(A, B, D1, scale) + run_i8(A, B, D2, scale), got)
+
+
+def test_i8_chain_rejects_bad_descriptors():
+    dev = "cuda:0"
+    a = torch.zeros(64, 64, dtype=torch.int8, device=dev)
+    b = torch.zeros(64, 32, dtype=torch.int8, device=dev)
+    d = torch.zeros(32, 64, dtype=torch.int8, device=dev)
+    e = torch.zeros(64, 64, dtype=torch.int32, device=dev)
+    with pytest.raises(NotImplementedError):
+        chain.run_bmm_chain(a, b, d, e, "cast")
+    with pytest.raises(ValueError):
+        chain.run_bmm_chain(a[:, :60], b[:60], d, e, "requant")
+    with pytest.raises(ValueError):
+        chain.run_bmm_chain(a, b, d, e, "requant", aux=torch.ones(5, device=dev))
+    with pytest.raises(ValueError):
+        chain.run_bmm_chain(a, b, d, e.float(), "requant")
