@@ -160,6 +160,83 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
   return fail(DITTO_EUNSUPPORTED, "no chain kernel for in_dtype %d", in);
 }
 
+struct ConvPlan {
+  int c1_tiles;
+  ditto::ConvChainArgs args;
+  ditto_tile_param tile;
+};
+
+int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan) {
+  if (!d) return fail(DITTO_EINVAL, "null descriptor");
+  if (d->abi_version != DITTO_CHAIN_ABI_VERSION)
+    return fail(DITTO_EINVAL, "descriptor abi_version %d, library %d", d->abi_version, DITTO_CHAIN_ABI_VERSION);
+  if (d->in_dtype != DITTO_F16 && d->in_dtype != DITTO_BF16)
+    return fail(DITTO_EUNSUPPORTED, "conv chains are built for fp16 / bf16 (in_dtype %d)", d->in_dtype);
+  if (d->acc_dtype != DITTO_F32) return fail(DITTO_EUNSUPPORTED, "conv chains accumulate in fp32");
+  if (d->out_dtype != d->in_dtype && d->out_dtype != DITTO_F32)
+    return fail(DITTO_EINVAL, "out_dtype must be in_dtype or fp32");
+  if (d->inter_op != DITTO_INTER_CAST && d->inter_op != DITTO_INTER_RELU)
+    return fail(DITTO_EINVAL, "inter_op %d not valid for a conv chain", d->inter_op);
+  if (d->N <= 0 || d->C0 <= 0 || d->H <= 0 || d->W <= 0 || d->C1 <= 0 || d->C2 <= 0 || d->R1 <= 0 ||
+      d->S1 <= 0 || d->R2 <= 0 || d->S2 <= 0 || d->stride1 <= 0 || d->stride2 <= 0 || d->pad1 < 0 || d->pad2 < 0)
+    return fail(DITTO_EINVAL, "conv extents must be positive and paddings non-negative");
+  if (d->R2 != 1 || d->S2 != 1 || d->pad2 != 0 || d->stride2 != 1)
+    return fail(DITTO_EUNSUPPORTED,
+                "the fused conv chain needs a 1x1, stride 1, unpadded second convolution (got %lldx%lld)",
+                (long long)d->R2, (long long)d->S2);
+  if (d->C1 % 8) return fail(DITTO_EINVAL, "C1 must be a multiple of 8");
+  if (d->C1 > 256) return fail(DITTO_EUNSUPPORTED, "C1=%lld: at most 256 intermediate channels", (long long)d->C1);
+  if (d->R1 > 7 || d->S1 > 7) return fail(DITTO_EUNSUPPORTED, "first filter larger than 7x7");
+  const long long P = (d->H + 2 * d->pad1 - d->R1) / d->stride1 + 1;
+  const long long Q = (d->W + 2 * d->pad1 - d->S1) / d->stride1 + 1;
+  if (d->H + 2 * d->pad1 < d->R1 || d->W + 2 * d->pad1 < d->S1 || P <= 0 || Q <= 0)
+    return fail(DITTO_EINVAL, "empty convolution output");
+  if (d->N * d->C0 * d->H * d->W > 0x7fffffffLL * 4 || d->N * d->C2 * P * Q > 0x7fffffffLL * 4 ||
+      d->H > 65535 || d->W > 65535 || d->N > 65535 || d->C0 > 65535 || d->C2 > 65535)
+    return fail(DITTO_EINVAL, "tensor too large");
+  memset(plan, 0, sizeof(*plan));
+  const int c1t = d->C1 <= 32 ? 1 : d->C1 <= 64 ? 2 : d->C1 <= 128 ? 4 : 8;
+  const int pxw = c1t == 8 ? 1 : 2;
+  const int slots = 128 * pxw;
+  ditto::ConvChainArgs& a = plan->args;
+  a.N = (int)d->N; a.C0 = (int)d->C0; a.H = (int)d->H; a.W = (int)d->W;
+  a.C1 = (int)d->C1; a.R = (int)d->R1; a.S = (int)d->S1; a.pad = (int)d->pad1; a.stride = (int)d->stride1;
+  a.C2 = (int)d->C2; a.P = (int)P; a.Q = (int)Q;
+  a.TW = (int)(Q < slots ? Q : slots);
+  a.TH = slots / a.TW;
+  if (a.TH > P) a.TH = (int)P;
+  // shrink the tile until the halo tile and the weight chunk fit in LDS
+  const int RS = a.R * a.S;
+  int lds = 0;
+  for (;;) {
+    a.rows_in = (a.TH - 1) * a.stride + a.R;
+    a.cols_in = (a.TW - 1) * a.stride + a.S;
+    lds = ditto::conv_chain_lds_bytes(a.rows_in, a.cols_in, RS, 32 * c1t);
+    if (lds <= 150 * 1024) break;
+    if (a.TH > 1) a.TH = (a.TH + 1) / 2;
+    else if (a.TW > 16) a.TW = (a.TW + 1) / 2;
+    else return fail(DITTO_EUNSUPPORTED, "conv chain tile does not fit in LDS");
+  }
+  a.tiles_h = (int)((P + a.TH - 1) / a.TH);
+  a.tiles_w = (int)((Q + a.TW - 1) / a.TW);
+  a.relu_mid = d->inter_op == DITTO_INTER_RELU;
+  a.relu_out = d->relu_out != 0;
+  a.out_f32 = d->out_dtype == DITTO_F32;
+  plan->c1_tiles = c1t;
+  ditto_tile_param& t = plan->tile;
+  t.block_threads = 256;
+  t.block_m = a.TH * a.TW;   // output pixels per workgroup
+  t.block_l = 32 * c1t;      // intermediate channels held in registers
+  t.block_n = (int)d->C2;
+  t.head_pad = ditto::kConvCh;
+  t.lds_bytes = lds;
+  t.grid_x = a.N * a.tiles_h * a.tiles_w;
+  t.grid_y = a.TH;
+  t.grid_z = a.TW;
+  t.variant = 3000 + c1t * 10 + pxw;
+  return DITTO_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -263,9 +340,12 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
 }
 
 int ditto_conv_chain_select_tile(const ditto_conv_chain_desc* desc, ditto_tile_param* out) {
-  (void)desc;
-  (void)out;
-  return fail(DITTO_EUNSUPPORTED, "conv chain kernel not built");
+  ConvPlan plan;
+  int rc = plan_conv(desc, &plan);
+  if (rc != DITTO_OK) return rc;
+  if (!out) return fail(DITTO_EINVAL, "null output");
+  *out = plan.tile;
+  return DITTO_OK;
 }
 
 size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
@@ -273,11 +353,26 @@ size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
   return 0;
 }
 
-int ditto_conv_chain_run(const ditto_conv_chain_desc* desc, const void* x, const void* w1,
-                         const void* w2, void* y, void* workspace, size_t workspace_bytes,
-                         void* stream) {
-  (void)desc; (void)x; (void)w1; (void)w2; (void)y; (void)workspace; (void)workspace_bytes; (void)stream;
-  return fail(DITTO_EUNSUPPORTED, "conv chain kernel not built");
+int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const void* w1, const void* w2,
+                         void* y, void* workspace, size_t workspace_bytes, void* stream) {
+  (void)workspace;
+  (void)workspace_bytes;
+  ConvPlan plan;
+  int rc = plan_conv(d, &plan);
+  if (rc != DITTO_OK) return rc;
+  if (!x || !w1 || !w2 || !y) return fail(DITTO_EINVAL, "null data pointer");
+  if (!aligned(x, 2) || !aligned(w1, 2) || !aligned(w2, 8) || !aligned(y, 4))
+    return fail(DITTO_EINVAL, "misaligned data pointer");
+  ditto::ConvChainArgs a = plan.args;
+  a.x = x;
+  a.w1 = w1;
+  a.w2 = w2;
+  a.y = y;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  hipError_t e = d->in_dtype == DITTO_F16 ? ditto::launch_conv_f16(plan.c1_tiles, a, st)
+                                          : ditto::launch_conv_bf16(plan.c1_tiles, a, st);
+  if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
+  return DITTO_OK;
 }
 
 }  // extern "C"

@@ -1,0 +1,118 @@
+"""GPU parity of the fused conv -> conv chain against the CPU checker (NCHW, fp16 / bf16)."""
+import numpy as np
+import pytest
+import torch
+
+from ditto_amd import chain
+from tests.gpu_util import errors, to_dev, TORCH_DTYPES
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, REL_L2, REL_L2_BF16_QUANT = 1e-2, 1e-3, 3e-3
+
+
+def run_conv(X, W1, W2, dtype, pad1=1, stride1=1, inter="cast", relu_out=False, out_dtype=None):
+    x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
+    N, _, H, W = X.shape
+    R, S = W1.shape[2:]
+    P = (H + 2 * pad1 - R) // stride1 + 1
+    Q = (W + 2 * pad1 - S) // stride1 + 1
+    y = torch.full((N, W2.shape[0], P, Q), float("nan"), device=x.device, dtype=TORCH_DTYPES[out_dtype or dtype])
+    chain.run_conv_chain(x, w1, w2, y, pad1, stride1, 0, 1, inter, relu_out)
+    torch.cuda.synchronize()
+    return y.float().cpu().numpy()
+
+
+CASES = [
+    # N, C0, H, W, C1, R, pad, stride, C2
+    (2, 64, 56, 56, 64, 3, 1, 1, 256),   # the chain of the workload definition, 2 images
+    (1, 16, 12, 20, 32, 3, 1, 1, 40),    # small, C2 not a multiple of 32
+    (2, 24, 17, 23, 64, 3, 1, 2, 64),    # odd extents, stride 2, C0 not a multiple of 16
+    (1, 64, 28, 28, 128, 3, 1, 1, 64),   # Darknet-19 row of the reference's table (scaled down)
+    (1, 32, 14, 14, 256, 3, 1, 1, 128),  # 256 intermediate channels
+    (2, 64, 56, 56, 64, 1, 0, 1, 64),    # conv1x1 -> conv1x1 (modified ResNet-50 row)
+    (1, 8, 9, 140, 16, 3, 1, 1, 16),     # wider than one tile
+    (1, 16, 30, 30, 24, 5, 2, 1, 32),    # 5x5 first filter, C1 padded to 32
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_conv_chain_vs_oracle(oracle, case, dtype):
+    N, C0, H, W, C1, R, pad, stride, C2 = case
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, R, 1, dtype, seed=C0 + C1, w_std=0.05)
+    want32 = oracle.conv_chain_f32(X, W1, W2, pad, stride, 0, 1, round_mid=dtype)
+    got32 = run_conv(X, W1, W2, dtype, pad, stride, out_dtype="float32")
+    assert np.isfinite(got32).all()
+    mx, rel = errors(got32, want32)
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
+    got = run_conv(X, W1, W2, dtype, pad, stride)
+    assert np.array_equal(got, oracle.np_round_to(got32, dtype))
+    mx, rel = errors(got, oracle.np_round_to(want32, dtype))
+    assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (mx, rel)
+
+
+def test_conv_relu_conv_relu_vs_torch(oracle):
+    # the reference's GPU check: conv3x3 -> ReLU -> conv -> ReLU vs torch conv2d, uniform(-1,1)
+    # inputs, rtol = atol = 0.1 (testing/hyper_fusion/conv_relu_conv_relu_fuse_hw_cuda.py:750-793);
+    # here with a 1x1 second convolution and the workload tolerance
+    rng = np.random.default_rng(4)
+    N, C0, H, W, C1, C2 = 2, 32, 16, 16, 64, 64
+    X = oracle.np_round_to(rng.uniform(-1, 1, (N, C0, H, W)).astype(np.float32), "float16")
+    W1 = oracle.np_round_to(rng.uniform(-1, 1, (C1, C0, 3, 3)).astype(np.float32) * 0.1, "float16")
+    W2 = oracle.np_round_to(rng.uniform(-1, 1, (C2, C1, 1, 1)).astype(np.float32) * 0.1, "float16")
+    got = run_conv(X, W1, W2, "float16", inter="relu", relu_out=True, out_dtype="float32")
+    t = torch.nn.functional
+    mid = t.conv2d(torch.from_numpy(X).double(), torch.from_numpy(W1).double(), padding=1).clamp_min(0)
+    mid = mid.float().half().double()
+    want = t.conv2d(mid, torch.from_numpy(W2).double()).clamp_min(0).numpy()
+    assert (got >= 0).all()
+    assert np.allclose(got, want, rtol=0.1, atol=0.1)
+    mx, rel = errors(got, want)
+    assert mx <= MAX_ABS and rel <= REL_L2
+    want_o = oracle.conv_chain_f32(X, W1, W2, relu_mid=True, relu_out=True, round_mid="float16")
+    assert errors(got, want_o)[1] <= REL_L2
+
+
+def test_conv_chain_delta_filter(oracle):
+    # a 3x3 filter with a single one shifts the image; the 1x1 then mixes channels exactly
+    rng = np.random.default_rng(6)
+    X = oracle.np_round_to(rng.integers(-4, 5, (1, 16, 10, 12)).astype(np.float32), "float16")
+    W1 = np.zeros((16, 16, 3, 3), np.float32)
+    for c in range(16):
+        W1[c, c, 2, 0] = 1.0  # y[p][q] = x[p+1][q-1]
+    W2 = rng.integers(-2, 3, (8, 16, 1, 1)).astype(np.float32)
+    got = run_conv(X, W1, W2, "float16", out_dtype="float32")
+    shifted = np.zeros_like(X)
+    shifted[:, :, :-1, 1:] = X[:, :, 1:, :-1]
+    want = np.einsum("kc,nchw->nkhw", W2[:, :, 0, 0], shifted)
+    assert np.array_equal(got, want)  # small integers: exact
+
+
+def test_conv_chain_full_size_linearity(oracle):
+    # the full configuration (N=32, 64 -> 64 3x3 on 56x56, then 64 -> 256): checked against the
+    # checker on two images and through linearity in W2 on all of them
+    N, C0, H, W, C1, C2 = 32, 64, 56, 56, 64, 256
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, 3, 1, "float16", seed=0)
+    got = run_conv(X, W1, W2, "float16", out_dtype="float32")
+    sel = [0, 31]
+    want = oracle.conv_chain_f32(X[sel], W1, W2, round_mid="float16")
+    mx, rel = errors(got[sel], want)
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
+    W2a = oracle.np_round_to(W2 * 0.5, "float16")
+    W2b = W2 - W2a
+    assert np.array_equal(oracle.np_round_to(W2b, "float16"), W2b)
+    s = run_conv(X, W1, W2a, "float16", out_dtype="float32") + run_conv(X, W1, W2b, "float16", out_dtype="float32")
+    assert errors(s, got)[1] <= 1e-5
+
+
+def test_conv_chain_rejects_unsupported():
+    dev = "cuda:0"
+    x = torch.zeros(1, 16, 8, 8, device=dev, dtype=torch.float16)
+    w1 = torch.zeros(16, 16, 3, 3, device=dev, dtype=torch.float16)
+    w2 = torch.zeros(16, 16, 3, 3, device=dev, dtype=torch.float16)
+    y = torch.zeros(1, 16, 8, 8, device=dev, dtype=torch.float16)
+    with pytest.raises(NotImplementedError, match="1x1"):
+        chain.run_conv_chain(x, w1, w2, y, 1, 1, 1, 1)
+    with pytest.raises(ValueError):
+        chain.run_conv_chain(x, w1, w2[:, :, :1, :1].contiguous(), y[:, :8].contiguous(), 1, 1, 0, 1)
