@@ -46,23 +46,63 @@ WORKLOADS = {
                                            scale=1.0, bound="hbm",
                                            desc="GEMM chain (A.B).D at the shape of the CPU plumbing case, fp16"),
 }
+WORKLOADS.update({
+    "conv_chain_f16_n32_c64_56x56_k64_k256": dict(
+        kind="conv", dtype="float16", N=32, C0=64, H=56, W=56, C1=64, R=3, pad=1, stride=1, C2=256, bound="hbm",
+        desc="conv3x3(64->64, s1 p1) -> conv1x1(64->256) on 32x56x56, NCHW fp16"),
+    "gemm_chain_i8_8192x1024x256x1024": dict(
+        kind="requant", dtype="int8", batch=1, M=8192, K=1024, L=256, N=1024, scale=2.0 ** -10, bound="hbm",
+        desc="int8 A[8192,1024].B[1024,256] -> requantise(2^-10, RNE, saturate) -> .D[256,1024], int32 out"),
+})
 DEFAULT_WORKLOAD = "attn_bf16_b64_s4096_d128"
 SHORT = {"bfloat16": "bf16", "float16": "f16", "int8": "i8", "float32": "f32"}
 
 
 def flops_of(w):
+    if w["kind"] == "conv":
+        P = (w["H"] + 2 * w["pad"] - w["R"]) // w["stride"] + 1
+        Q = (w["W"] + 2 * w["pad"] - w["R"]) // w["stride"] + 1
+        return 2.0 * w["N"] * P * Q * (w["C0"] * w["C1"] * w["R"] * w["R"] + w["C1"] * w["C2"])
     return 2.0 * w["batch"] * w["M"] * w["L"] * (w["K"] + w["N"])
 
 
 def bytes_of(w):
+    """Algorithmic bytes: every input read once, the output written once."""
+    if w["kind"] == "conv":
+        P = (w["H"] + 2 * w["pad"] - w["R"]) // w["stride"] + 1
+        Q = (w["W"] + 2 * w["pad"] - w["R"]) // w["stride"] + 1
+        return 2 * (w["N"] * w["C0"] * w["H"] * w["W"] + w["C1"] * w["C0"] * w["R"] * w["R"] + w["C2"] * w["C1"]
+                    + w["N"] * w["C2"] * P * Q)
+    if w["kind"] == "requant":
+        return w["batch"] * (w["M"] * w["K"] + w["K"] * w["L"] + w["L"] * w["N"] + 4 * w["M"] * w["N"])
     eb = 2
     return eb * w["batch"] * (w["M"] * w["K"] + w["K"] * w["L"] + w["L"] * w["N"] + w["M"] * w["N"])
 
 
-def make_inputs(w, dev):
+def make_call(w, dev):
+    """Synthetic inputs resident on the device and a zero-argument callable that runs one step."""
     import torch
 
+    from ditto_amd import chain
+
     g = torch.Generator().manual_seed(0)
+    if w["kind"] == "conv":
+        x = torch.randn(w["N"], w["C0"], w["H"], w["W"], generator=g).half().to(dev)
+        w1 = (torch.randn(w["C1"], w["C0"], w["R"], w["R"], generator=g) * 0.05).half().to(dev)
+        w2 = (torch.randn(w["C2"], w["C1"], 1, 1, generator=g) * 0.05).half().to(dev)
+        P = (w["H"] + 2 * w["pad"] - w["R"]) // w["stride"] + 1
+        Q = (w["W"] + 2 * w["pad"] - w["R"]) // w["stride"] + 1
+        y = torch.empty(w["N"], w["C2"], P, Q, dtype=torch.float16, device=dev)
+        desc = chain.conv_chain_desc(x, w1, w2, y, w["pad"], w["stride"], 0, 1, "cast", False)
+        return (lambda: chain.run_conv_chain(x, w1, w2, y, desc=desc)), desc
+    if w["kind"] == "requant":
+        a = torch.randint(-127, 128, (w["M"], w["K"]), generator=g, dtype=torch.int8).to(dev)
+        b = torch.randint(-127, 128, (w["K"], w["L"]), generator=g, dtype=torch.int8).to(dev)
+        d = torch.randint(-127, 128, (w["L"], w["N"]), generator=g, dtype=torch.int8).to(dev)
+        scale = torch.full((w["L"],), w["scale"], dtype=torch.float32, device=dev)
+        e = torch.empty(w["M"], w["N"], dtype=torch.int32, device=dev)
+        desc = chain.bmm_chain_desc(a, b, d, e, "requant")
+        return (lambda: chain.run_bmm_chain(a, b, d, e, aux=scale, desc=desc)), desc
     dt = {"bfloat16": torch.bfloat16, "float16": torch.float16}[w["dtype"]]
     std = 1.0 if w["kind"] == "softmax" else 0.25
     a = (torch.randn(w["batch"], w["M"], w["K"], generator=g) * std).to(dt).to(dev)
@@ -73,7 +113,8 @@ def make_inputs(w, dev):
     else:
         b = (torch.randn(w["batch"], w["K"], w["L"], generator=g) * std).to(dt).to(dev)
     f = torch.empty(w["batch"], w["M"], w["N"], dtype=dt, device=dev)
-    return a, b, c, f
+    desc = chain.bmm_chain_desc(a, b, c, f, w["kind"], w["scale"])
+    return (lambda: chain.run_bmm_chain(a, b, c, f, desc=desc)), desc
 
 
 def time_gpu(w, steps, warmup, dev):
@@ -82,9 +123,7 @@ def time_gpu(w, steps, warmup, dev):
 
     from ditto_amd import chain
 
-    a, b, c, f = make_inputs(w, dev)
-    desc = chain.bmm_chain_desc(a, b, c, f, w["kind"], w["scale"])
-    call = lambda: chain.run_bmm_chain(a, b, c, f, desc=desc)  # noqa: E731
+    call, desc = make_call(w, dev)
     for _ in range(max(warmup, 1)):
         call()
     torch.cuda.synchronize()
@@ -199,11 +238,11 @@ def main():
         "vs_baseline": None,
         "dtype": short,
         "data": "synthetic",
-        "config": {"workload": args.workload, "description": w["desc"], "batch": w["batch"], "M": w["M"],
-                   "N": w["N"], "K": w["K"], "L": w["L"], "tile": tile},
+        "config": dict({"workload": args.workload, "description": w["desc"], "tile": tile},
+                       **{k: v for k, v in w.items() if k not in ("kind", "dtype", "desc", "bound", "scale")}),
         "roofline": roof,
     }
-    if not args.no_cpu:
+    if not args.no_cpu and w["kind"] in ("softmax", "cast", "relu"):
         line["cpu_baseline"] = cpu_baseline(w)
     if not args.no_also:
         also = {}

@@ -1,0 +1,37 @@
+"""BMM -> softmax -> BMM chain driver (reference: benchmark/chimera/cuda/bmm_softmax_bmm_cuda.py)."""
+from ditto_amd import auto_compute as ac
+
+from . import common
+
+example_text = """
+ example:
+    python -m ditto_amd.drivers.bmm_softmax_bmm --in_dtype float16 --acc_dtype float32 --begin 0 --num 1
+"""
+shapes = common.BMM_SHAPES
+
+
+def main(batch=12, M=512, N=64, K=64, L=512, in_dtype="float16", acc_dtype="float32", sm="gfx950",
+         only_once=False, scale=1.0):
+    ins, outs = ac.nn.functional.BatchGemmSoftmaxGemm(batch=batch, M=M, N=N, K=K, L=L, in_dtype=in_dtype,
+                                                      acc_dtype=acc_dtype, scale=scale)
+    try:
+        layer, sch = common.describe_bmm_chain(ins, outs, in_dtype, acc_dtype, sm)
+    except Exception as error:
+        print("chain failed:", type(error).__name__, error)
+        return common.SENTINEL_COST
+    args = common.random_args(layer, in_dtype, 3)
+    return common.evaluate(sch, layer, args, only_once)
+
+
+if __name__ == "__main__":
+    parser = common.base_parser(example_text, len(shapes), with_ai=False)
+    args = parser.parse_args()
+    if common.check_dtypes(args):
+        costs = []
+        for ss in shapes[args.begin: args.begin + args.num]:
+            B, M, N, K, L = ss
+            costs.append((ss, main(B, M, N, K, L, args.in_dtype, args.acc_dtype, args.sm, args.only_once)))
+        print("B,M,N,K,L,in_dtype,acc_dtype,sm,cost")
+        for cc in costs:
+            print(f"{cc[0][0]},{cc[0][1]},{cc[0][2]},{cc[0][3]},{cc[0][4]},{args.in_dtype},{args.acc_dtype},"
+                  f"{args.sm},{cc[1]}")

@@ -1,0 +1,50 @@
+"""The per-chain drivers keep the reference's flags, shape tables, CSV header and cost unit
+(benchmark/chimera/cuda/bmm_bmm_cuda.py:304-397, conv3x3_conv1x1_cuda.py:331-337)."""
+import subprocess
+import sys
+
+import pytest
+
+from ditto_amd.drivers import bmm_bmm, bmm_softmax_bmm, common, conv3x3_conv1x1
+
+
+def test_shape_tables_match_reference():
+    assert len(common.BMM_SHAPES) == 12
+    assert common.BMM_SHAPES[1] == (12, 512, 64, 64, 512)      # Bert-Base
+    assert common.BMM_SHAPES[6] == (12, 208, 64, 64, 208)      # ViT-Base/16: uround(196, 16)
+    assert common.BMM_SHAPES[9] == (1, 512, 64, 64, 256)       # Mixer-Small/32-S: uround(49, 16)
+    assert common.CONV3X3_CONV1X1_SHAPES[2] == (64, 56, 56, 128, 64, 1, 1)
+    assert common.cal_ai(12, 512, 64, 64, 512) == (256.0, 512 * 64 / 576)
+
+
+def test_cli_ai_and_unsupported_dtype():
+    out = subprocess.run([sys.executable, "-m", "ditto_amd.drivers.bmm_bmm", "--ai", "--begin", "1", "--num", "1"],
+                         capture_output=True, text=True, check=True).stdout
+    assert out.strip() == "(12, 512, 64, 64, 512) 256.0 56.888888888888886"
+    out = subprocess.run([sys.executable, "-m", "ditto_amd.drivers.bmm_softmax_bmm", "--in_dtype", "float64",
+                          "--acc_dtype", "float64", "--num", "1"], capture_output=True, text=True, check=True).stdout
+    assert "Data type not supported" in out and "cost" not in out
+
+
+def test_descriptor_failure_gives_sentinel_cost():
+    # N not a multiple of 16: the builder's assert is turned into the sentinel cost, not an exception
+    # (the reference swallows failures of its measurement worker the same way, bmm_bmm_cuda.py:58-64)
+    assert conv3x3_conv1x1.main(1, 16, 8, 8, 12, 16) == common.SENTINEL_COST
+
+
+@pytest.mark.gpu
+def test_drivers_run_one_row_each(capsys):
+    assert bmm_bmm.main(*common.BMM_SHAPES[9], only_once=True) == -1
+    cost = bmm_softmax_bmm.main(*common.BMM_SHAPES[3])
+    assert 0 < cost < 5.0  # milliseconds
+    C, H, W, K1, K2, s1, s2 = common.CONV3X3_CONV1X1_SHAPES[2]
+    cost = conv3x3_conv1x1.main(1, C, H, W, K1, K2, s1, s2)
+    assert 0 < cost < 5.0
+
+
+@pytest.mark.gpu
+def test_cli_csv_format():
+    out = subprocess.run([sys.executable, "-m", "ditto_amd.drivers.bmm_softmax_bmm", "--begin", "3", "--num", "1",
+                          "--only_once"], capture_output=True, text=True, check=True).stdout.strip().splitlines()
+    assert out[-2] == "B,M,N,K,L,in_dtype,acc_dtype,sm,cost"
+    assert out[-1] == "12,256,64,64,256,float16,float32,gfx950,-1"
