@@ -32,7 +32,13 @@ PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a copy
 # kernel of known size; see the summaries under profiles/.  None where not measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # FETCH_SIZE reads half of a plain copy's bytes on this device (scale factor 2.00), WRITE_SIZE all of them
+    "attn_bf16_b64_s4096_d128": int((192.21 + 64.00) * 2 ** 20),
+    "attn_f16_b96_s512_d64": int((18.10 + 6.00) * 2 ** 20),
+    "conv_chain_f16_n32_c64_56x56_k64_k256": int((13.21 + 50.11) * 2 ** 20),
+    "gemm_chain_i8_8192x1024x256x1024": int((12.18 + 32.00) * 2 ** 20),
+}
 
 WORKLOADS = {
     # name: kind, dtype, dims
@@ -207,6 +213,9 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-also", action="store_true", help="skip the brief runs of the other configurations")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="also launch one plain device copy of MIB MiB (read MIB, write MIB): a dispatch of known "
+                         "traffic against which rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the chains shard over batch entries with no "
@@ -218,6 +227,13 @@ def main():
         sys.exit("bench.py needs a HIP device")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.copy_probe > 0:
+        src = torch.ones(args.copy_probe << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     w, wall_ms, ev_ms, tile, roof = run_one(args.workload, args.steps, args.warmup, dev)
     fl = flops_of(w)
