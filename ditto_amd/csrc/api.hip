@@ -101,6 +101,12 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     if (d->a_row_stride > 0x7fffffff || d->b_row_stride > 0x7fffffff ||
         d->c_row_stride > 0x7fffffff || d->f_row_stride > 0x7fffffff)
       return fail(DITTO_EINVAL, "row stride too large");
+    // one batch entry of B and of C is addressed through a 32-bit buffer offset
+    {
+      const long long b_rows = d->b_layout == DITTO_B_KL ? d->K : d->L;
+      if (b_rows * d->b_row_stride * 2 >= 0x7fffffffLL || d->L * d->c_row_stride * 2 >= 0x7fffffffLL)
+        return fail(DITTO_EUNSUPPORTED, "a batch entry of B or C exceeds 2 GiB");
+    }
     const long long dmax = d->K > d->N ? d->K : d->N;
     if (dmax > 128)
       return fail(DITTO_EUNSUPPORTED, "max(K,N)=%lld: register-resident chain supports up to 128", dmax);
@@ -117,8 +123,8 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     t.block_n = (int)d->N;
     t.head_pad = plan->d_pad;
     const bool kl = d->b_layout == DITTO_B_KL;
-    t.lds_bytes = plan->d_pad == 64 ? (kl ? ditto::bmm_chain_lds_bytes<64, true>() : ditto::bmm_chain_lds_bytes<64, false>())
-                                    : (kl ? ditto::bmm_chain_lds_bytes<128, true>() : ditto::bmm_chain_lds_bytes<128, false>());
+    (void)kl;
+    t.lds_bytes = plan->d_pad == 64 ? ditto::bmm_chain_lds_bytes<64>() : ditto::bmm_chain_lds_bytes<128>();
     t.grid_x = (int)(((d->M + bm - 1) / bm) * d->batch);
     t.grid_y = t.grid_z = 1;
     t.variant = plan->d_pad * 10 + plan->qt;

@@ -11,10 +11,19 @@
 // accumulator registers already have the layout of the second contraction's
 // B operand (F^T = C^T.P^T): the intermediate never leaves VGPRs.
 //
-// Work split: a workgroup of 4 waves owns 128*QT rows of A for one batch entry; each
-// wave owns 32*QT rows and keeps their A fragments in VGPRs for the whole kernel.
-// The L axis is walked in steps of 64: B and C tiles are staged through LDS (double
-// buffered, one barrier per step) and shared by the 4 waves.
+// Work split: a workgroup of 4 waves (one per SIMD) owns 128*QT rows of A for one batch
+// entry; each wave owns 32*QT rows and keeps their A fragments in VGPRs for the whole
+// kernel.  The L axis is walked in steps of 64.  B and C tiles go from global memory
+// straight into LDS (buffer_load ... lds, 16 bytes per lane, no staging registers; rows and
+// columns outside the matrices read as zero through the buffer range check), double
+// buffered, one barrier per step, shared by the 4 waves.  Tiles are stored unpadded with the
+// 16-byte chunk index of each row XOR-swizzled so that both the plain 16-byte row reads and
+// the transposing reads (ds_read_b64_tr_b16) are bank-conflict free.
+//
+// Software pipeline (one wave per SIMD, so overlap must come from within the wave): while
+// the MFMA pipe computes the scores of step i+1, the VALU exponentiates the scores of step
+// i; while it accumulates P(i).C(i), the VALU packs P(i) and takes the row maximum of step
+// i+1.  The two score buffers alternate by unrolling the step loop twice.
 #pragma once
 #include "common.h"
 
@@ -37,41 +46,51 @@ struct BmmChainArgs {
 constexpr int kInterCast = 0;
 constexpr int kInterSoftmax = 2;
 
-constexpr int kBN = 64;  // L step
+constexpr int kBN = 64;        // L step
+constexpr int kNW = 4;         // waves per workgroup
 constexpr float kLazy = 8.0f;  // log2 of the slack allowed before the running maximum is raised
-constexpr int kNW = 4;   // waves per workgroup
 
-// Row stride (elements) of a row-major 16-bit LDS tile that is read with transpose
-// reads: 4 consecutive rows x 64 B must fall into different banks, which holds when
-// the stride in bytes is 64 mod 128.
-__host__ __device__ constexpr int tr_stride(int cols) { return (cols % 64 == 32) ? cols : cols + 32; }
-// Row stride of a tile read with plain 16-byte row reads (one row per lane).
-__host__ __device__ constexpr int row_stride(int cols) { return cols + 8; }
-
-template <int D, bool B_KL>
+template <int D>
 __host__ __device__ constexpr int bmm_chain_lds_bytes() {
-  const int btile = B_KL ? D * tr_stride(kBN) : kBN * row_stride(D);
-  const int ctile = kBN * tr_stride(D);
-  return 2 * (btile + ctile) * 2;
+  return (3 + 2) * kBN * D * 2;  // three B tiles, two C tiles, 16-bit elements
+}
+
+// XOR applied to the 16-byte chunk index of a row of an unpadded LDS tile.
+//   row-read tiles (one 16-byte read per lane, consecutive lanes = consecutive rows):
+//     16 consecutive rows must hit 16 different chunk slots of a 256-byte bank window
+//   transpose-read tiles (ds_read_b64_tr_b16: 16 lanes read 4 rows x 32 bytes):
+//     4 consecutive rows x 4 chunks must hit different slots
+template <int CPR>  // chunks per row: 16 (256-byte rows) or 8 (128-byte rows)
+__device__ __forceinline__ int swz_rowread(int row) {
+  return CPR == 16 ? (row & 15) : ((row ^ (row >> 3)) & 7);
+}
+template <int CPR>
+__device__ __forceinline__ int swz_trread(int row) {
+  return CPR == 16 ? 4 * (row & 3) : 4 * ((row >> 1) & 1);
 }
 
 template <typename T, int D, int QT, int INTER, bool B_KL>
 __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
+  // The body uses device-only types (buffer resources); the host pass only needs the stub.
+#if defined(__HIP_DEVICE_COMPILE__)
   typedef typename Elem<T>::v8 V8;
   typedef typename Elem<T>::v4 V4;
+  typedef typename Elem<T>::v2 V2;
   constexpr int BM = kNW * 32 * QT;
-  constexpr int BSTR = B_KL ? tr_stride(kBN) : row_stride(D);
-  constexpr int BTILE = B_KL ? D * BSTR : kBN * BSTR;
-  constexpr int CSTR = tr_stride(D);
-  constexpr int CTILE = kBN * CSTR;
-  constexpr int NCH = kBN * D / 8 / 256;  // 16-byte chunks per thread per tile
-  static_assert(NCH >= 1 && (kBN * D / 8) % 256 == 0, "tile must split evenly over 256 threads");
+  constexpr int TILE = kBN * D;                 // elements per staged tile (B and C alike)
+  constexpr int B_RB = B_KL ? kBN * 2 : D * 2;  // bytes per LDS row of the B tile
+  constexpr int B_CPR = B_RB / 16;
+  constexpr int C_RB = D * 2;
+  constexpr int C_CPR = C_RB / 16;
+  constexpr int NLD = TILE * 2 / 1024 / kNW;    // direct-load instructions per wave per tile
+  static_assert(NLD >= 1, "tile too small");
 
-  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  T* const Bs = reinterpret_cast<T*>(smem_raw);  // [2][BTILE]
-  T* const Cs = Bs + 2 * BTILE;                  // [2][CTILE]
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  // B tiles [3][TILE] at byte 0, C tiles [2][TILE] at byte 3*TILE*2
+  constexpr int C_BASE = 3 * TILE * 2;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31, g = lane >> 5;
   const int i16 = lane & 15, h = (lane >> 4) & 1;
 
@@ -79,10 +98,76 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
   const int mb = lid % p.mblocks;
   const int bz = lid / p.mblocks;
   const T* __restrict__ Ag = reinterpret_cast<const T*>(p.a) + (long long)bz * p.a_bs;
-  const T* __restrict__ Bg = reinterpret_cast<const T*>(p.b) + (long long)bz * p.b_bs;
-  const T* __restrict__ Cg = reinterpret_cast<const T*>(p.c) + (long long)bz * p.c_bs;
+  const T* Bg = reinterpret_cast<const T*>(p.b) + (long long)bz * p.b_bs;
+  const T* Cg = reinterpret_cast<const T*>(p.c) + (long long)bz * p.c_bs;
   const int m_wave = mb * BM + wave * 32 * QT;
   const int M = p.M, N = p.N, K = p.K, L = p.L;
+
+  // ---- buffer resources over this batch entry's B and C (reads past the end return 0)
+  const unsigned b_bytes = (unsigned)(B_KL ? ((long long)(K - 1) * p.b_rs + L) : ((long long)(L - 1) * p.b_rs + K)) * 2u;
+  const unsigned c_bytes = (unsigned)((long long)(L - 1) * p.c_rs + N) * 2u;
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(Bg), 0, b_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(Cg), 0, c_bytes, 0x00020000);
+
+  // ---- per-lane source offsets of the direct loads.  Load q of this wave fills the LDS
+  // bytes [1024*(NLD*wave + q), +1024): lane -> (row, physical chunk) -> swizzled source.
+  int b_voff[NLD], c_voff[NLD];
+  int b_col[NLD];  // B_KL only: first l column (within the tile) the lane loads
+#pragma unroll
+  for (int q = 0; q < NLD; ++q) {
+    const int gi = NLD * wave + q;
+    {
+      const int row = gi * (64 / B_CPR) + lane / B_CPR, pc = lane % B_CPR;
+      if (B_KL) {
+        const int cl = pc ^ swz_trread<B_CPR>(row);  // rows are k, columns l
+        b_col[q] = cl * 8;
+        b_voff[q] = row < K ? (row * p.b_rs + cl * 8) * 2 : (int)b_bytes;
+      } else {
+        const int cl = pc ^ swz_rowread<B_CPR>(row);  // rows are l, columns k
+        b_col[q] = 0;
+        b_voff[q] = cl * 8 < K ? (row * p.b_rs + cl * 8) * 2 : (int)b_bytes;
+      }
+    }
+    {
+      const int row = gi * (64 / C_CPR) + lane / C_CPR, pc = lane % C_CPR;
+      const int cl = pc ^ swz_trread<C_CPR>(row);
+      c_voff[q] = cl * 8 < N ? (row * p.c_rs + cl * 8) * 2 : (int)c_bytes;
+    }
+  }
+  auto load_b = [&](int tile, int buf) {
+    const int l0 = tile * kBN;
+    const int soff = B_KL ? l0 * 2 : l0 * p.b_rs * 2;
+#pragma unroll
+    for (int q = 0; q < NLD; ++q) {
+      // the whole offset goes into the per-lane operand: it is what the range check sees
+      int vo = b_voff[q] + soff;
+      if (B_KL) vo = (l0 + b_col[q] < L) ? vo : (int)b_bytes;  // columns past L are inside the buffer
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          b_rsrc, (DITTO_LDS void*)(smem_raw + (buf * TILE) * 2 + 1024 * (NLD * wave + q)), 16, vo, 0, 0, 0);
+    }
+  };
+  auto load_c = [&](int tile, int buf) {
+    const int soff = tile * kBN * p.c_rs * 2;
+#pragma unroll
+    for (int q = 0; q < NLD; ++q)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          c_rsrc, (DITTO_LDS void*)(smem_raw + C_BASE + (buf * TILE) * 2 + 1024 * (NLD * wave + q)), 16,
+          c_voff[q] + soff, 0, 0, 0);
+  };
+
+  // ---- per-lane LDS read offsets (bytes, within one tile)
+  // B operand of step st, L-tile i (A operand of D^T = B^T.A^T: rows l, 8 consecutive k)
+  //   row-read layout: row 32i+ln, logical chunk 2st+g      -> (2st) ^ (g ^ swz(ln))
+  //   tr-read  layout: rows k = 16st+8g+(i16>>2)+{0,4}, chunk 4i+2h+((i16&3)>>1), +8*(i16&1)
+  const int b_rd = B_KL ? ((8 * g + (i16 >> 2)) * B_RB + (2 * h + ((i16 & 3) >> 1)) * 16 + 8 * (i16 & 1))
+                        : (ln * B_RB);
+  int b_x[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) b_x[i] = B_KL ? swz_trread<B_CPR>(i16 >> 2) : (g ^ swz_rowread<B_CPR>(32 * i + ln));
+  // C operand of step u, N-tile t (A operand of F^T = C^T.P^T: rows n, k = l permuted):
+  //   rows l = 16u + 4g + (i16>>2) + {0,8}, chunk 4t + 2h + ((i16&3)>>1), +8*(i16&1)
+  const int c_rd = (4 * g + (i16 >> 2)) * C_RB + (2 * h + ((i16 & 3) >> 1)) * 16 + 8 * (i16 & 1);
+  const int c_x = swz_trread<C_CPR>(i16 >> 2);
 
   // ---- A fragments (B operand of D^T = B^T.A^T): lane holds A[row][16s + 8g .. +7]
   V8 af[QT][D / 16];
@@ -98,44 +183,6 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
     }
   }
 
-  // ---- global -> register staging of one (B, C) tile pair
-  V8 breg[NCH], creg[NCH];
-  auto load_tiles = [&](int l0) {
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const int ch = tid + 256 * c;
-      V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (B_KL) {
-        const int k = ch / (kBN / 8), l = l0 + (ch % (kBN / 8)) * 8;
-        if (k < K && l < L) v = *reinterpret_cast<const V8*>(Bg + (long long)k * p.b_rs + l);
-      } else {
-        const int l = l0 + ch / (D / 8), k = (ch % (D / 8)) * 8;
-        if (l < L && k < K) v = *reinterpret_cast<const V8*>(Bg + (long long)l * p.b_rs + k);
-      }
-      breg[c] = v;
-      V8 w = {0, 0, 0, 0, 0, 0, 0, 0};
-      {
-        const int l = l0 + ch / (D / 8), n = (ch % (D / 8)) * 8;
-        if (l < L && n < N) w = *reinterpret_cast<const V8*>(Cg + (long long)l * p.c_rs + n);
-      }
-      creg[c] = w;
-    }
-  };
-  auto store_tiles = [&](int buf) {
-    T* bs = Bs + buf * BTILE;
-    T* cs = Cs + buf * CTILE;
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const int ch = tid + 256 * c;
-      if (B_KL) {
-        *reinterpret_cast<V8*>(bs + (ch / (kBN / 8)) * BSTR + (ch % (kBN / 8)) * 8) = breg[c];
-      } else {
-        *reinterpret_cast<V8*>(bs + (ch / (D / 8)) * BSTR + (ch % (D / 8)) * 8) = breg[c];
-      }
-      *reinterpret_cast<V8*>(cs + (ch / (D / 8)) * CSTR + (ch % (D / 8)) * 8) = creg[c];
-    }
-  };
-
   // ---- accumulators of F^T: o[t][j][r] = F^T[32t + 8(r/4) + 4g + r%4][32j + ln]
   f32x16 o[D / 32][QT];
 #pragma unroll
@@ -144,143 +191,172 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
     for (int j = 0; j < QT; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[t][j][r] = 0.f;
-  float mrow[QT], lsum[QT];
+  float mrow[QT], lsum[QT], mxn[QT];
 #pragma unroll
   for (int j = 0; j < QT; ++j) {
     mrow[j] = -INFINITY;
     lsum[j] = 0.f;
+    mxn[j] = -INFINITY;
   }
   const float c2 = p.scale_log2;
-
   const int ntiles = (L + kBN - 1) / kBN;
-  load_tiles(0);
-  store_tiles(0);
+  const bool ragged = (L % kBN) != 0;
+
+  // Scores are produced and consumed in HALF steps of 32 rows of the L tile: s[j] is the
+  // transposed score tile (32 l x 32 m) of A-row tile j.
+  // first contraction of one half step: s[j] = (B^T rows 32i..32i+31) . (A^T tile j)
+  auto s_half = [&](f32x16 (&s)[QT], const char* bs, int i, int st) {
+    V8 bf;
+    if (B_KL) {
+      const char* q = bs + b_rd + 16 * st * B_RB + (((4 * i) ^ b_x[i]) * 16);
+      V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
+      V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(q + 4 * B_RB));
+      bf = concat4<V4, V8>(lo, hi);
+    } else {
+      bf = *reinterpret_cast<const V8*>(bs + b_rd + 32 * i * B_RB + (((2 * st) ^ b_x[i]) * 16));
+    }
+#pragma unroll
+    for (int j = 0; j < QT; ++j) {
+      if (st == 0) {
+        const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        s[j] = Elem<T>::mfma32(bf, af[j][st], z);
+      } else {
+        s[j] = Elem<T>::mfma32(bf, af[j][st], s[j]);
+      }
+    }
+  };
+  // scores of rows past L are masked out (softmax only; other chains see zero operands)
+  auto mask_tail = [&](f32x16 (&s)[QT], int l0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int l = l0 + 8 * (r >> 2) + 4 * g + (r & 3);
+      if (l >= L) {
+#pragma unroll
+        for (int j = 0; j < QT; ++j) s[j][r] = -INFINITY;
+      }
+    }
+  };
+  // scaled row maximum of a finished half tile (pair of half-waves combined)
+  auto row_max = [&](f32x16 (&s)[QT]) {
+#pragma unroll
+    for (int j = 0; j < QT; ++j) {
+      float mx = s[j][0];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[j][r]);
+      mxn[j] = pair_max(mx) * c2;
+    }
+  };
+  // Lazy rescale: the running maximum only has to bound the scores well enough that exp2
+  // cannot overflow, so it is raised (and the accumulators rescaled) only when some row of
+  // the wave exceeds it by more than 2^kLazy.  Rows keep a stale maximum otherwise; the
+  // final division by the row sum cancels it exactly.
+  auto maybe_rescale = [&]() {
+#pragma unroll
+    for (int j = 0; j < QT; ++j) {
+      if (__builtin_amdgcn_ballot_w64(mxn[j] > mrow[j] + kLazy) != 0) {
+        const float mnew = fmaxf(mrow[j], mxn[j]);
+        const float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);
+        mrow[j] = mnew;
+        lsum[j] *= alpha;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[t][j][r] *= alpha;
+      }
+    }
+  };
+  // exponentials of registers [r0, r0 + n) of the half tile
+  auto exp_slice = [&](f32x16 (&s)[QT], int r0, int n) {
+#pragma unroll
+    for (int j = 0; j < QT; ++j)
+#pragma unroll
+      for (int e = 0; e < n; ++e)
+        s[j][r0 + e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r0 + e], c2, -mrow[j]));
+  };
+  // second contraction, 16 rows of the L tile: o[t][j] += (C^T tile t, rows 16u..) . (P^T).
+  // Half-wave g supplies rows 16u + 4g + {0..3} and 16u + 8 + 4g + {0..3}: registers
+  // 8(u%2) .. 8(u%2)+7 of the half tile, the accumulator layout of s.
+  auto pv_step = [&](f32x16 (&s)[QT], const char* cs, int u) {
+    V8 pf[QT];
+#pragma unroll
+    for (int j = 0; j < QT; ++j) {
+      const int r0 = 8 * (u & 1);
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        v[e] = s[j][r0 + e];
+        if (INTER != kInterSoftmax && p.relu) v[e] = fmaxf(v[e], 0.f);
+      }
+      V2 p0 = cvt2<T>(v[0], v[1]), p1 = cvt2<T>(v[2], v[3]), p2 = cvt2<T>(v[4], v[5]), p3 = cvt2<T>(v[6], v[7]);
+      if constexpr (INTER == kInterSoftmax) {
+        // the row sum is taken over the ROUNDED probabilities, i.e. exactly the values that
+        // enter the second contraction
+        lsum[j] = Elem<T>::add_pair(p0, lsum[j]);
+        lsum[j] = Elem<T>::add_pair(p1, lsum[j]);
+        lsum[j] = Elem<T>::add_pair(p2, lsum[j]);
+        lsum[j] = Elem<T>::add_pair(p3, lsum[j]);
+      }
+      V8 w = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+      pf[j] = w;
+    }
+#pragma unroll
+    for (int t = 0; t < D / 32; ++t) {
+      const char* q = cs + c_rd + 16 * u * C_RB + (((4 * t) ^ c_x) * 16);
+      V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
+      V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(q + 8 * C_RB));
+      V8 cf = concat4<V4, V8>(lo, hi);
+#pragma unroll
+      for (int j = 0; j < QT; ++j) o[t][j] = Elem<T>::mfma32(cf, pf[j], o[t][j]);
+    }
+  };
+
+  // One pipelined half step: consumes the finished scores `cur` (half hh of L tile `it`) and
+  // produces `nxt`, the scores of the following half (half 1 of the same tile, or half 0 of
+  // tile it+1).  Past the last tile the MFMAs run on a resident but stale B buffer and their
+  // result is dropped, which keeps the half step one straight-line block whose MFMA and VALU
+  // streams the scheduler can interleave.
+  auto half_step = [&](f32x16 (&cur)[QT], f32x16 (&nxt)[QT], int it, int hh) {
+    const int nt = hh ? it + 1 : it;  // tile of the next half
+    const char* bs_next = smem_raw + ((nt % 3) * TILE) * 2;
+    const char* cs_cur = smem_raw + C_BASE + ((it & 1) * TILE) * 2;
+    if constexpr (INTER == kInterSoftmax) maybe_rescale();
+    constexpr int NST = D / 16, PER = 16 / NST;  // MFMA groups and score registers per group
+#pragma unroll
+    for (int st = 0; st < NST; ++st) {
+      s_half(nxt, bs_next, hh ^ 1, st);
+      if constexpr (INTER == kInterSoftmax) exp_slice(cur, PER * st, PER);
+    }
+    pv_step(cur, cs_cur, 2 * hh);
+    pv_step(cur, cs_cur, 2 * hh + 1);
+    if constexpr (INTER == kInterSoftmax) {
+      if (ragged && nt == ntiles - 1) mask_tail(nxt, nt * kBN + 32 * (hh ^ 1));
+      row_max(nxt);
+    }
+  };
+
+  // ---- prologue: B(0), C(0), B(1) in flight; scores of the first half
+  load_b(0, 0);
+  load_c(0, 0);
+  load_b(1, 1);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+  f32x16 sa[QT], sb[QT];
+#pragma unroll
+  for (int st = 0; st < D / 16; ++st) s_half(sa, smem_raw, 0, st);
+  if constexpr (INTER == kInterSoftmax) {
+    if (ragged && ntiles == 1) mask_tail(sa, 0);
+    row_max(sa);
+  }
 
   for (int it = 0; it < ntiles; ++it) {
-    const int buf = it & 1;
-    const int l0 = it * kBN;
-    if (it + 1 < ntiles) load_tiles(l0 + kBN);
-    const T* bs = Bs + buf * BTILE;
-    const T* cs = Cs + buf * CTILE;
-
-    // ---- first contraction, transposed: s[i][j] = (B^T tile i) . (A^T tile j)
-    f32x16 s[2][QT];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < QT; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[i][j][r] = 0.f;
-#pragma unroll
-    for (int st = 0; st < D / 16; ++st) {
-      V8 bf[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        if (B_KL) {
-          // rows of the LDS tile are k, columns are l: transpose read
-          const T* q = bs + (16 * st + 8 * g + (i16 >> 2)) * BSTR + 32 * i + 16 * h + 4 * (i16 & 3);
-          V4 lo = lds_read_tr4<T>(q);
-          V4 hi = lds_read_tr4<T>(q + 4 * BSTR);
-          bf[i] = concat4<V4, V8>(lo, hi);
-        } else {
-          bf[i] = *reinterpret_cast<const V8*>(bs + (32 * i + ln) * BSTR + 16 * st + 8 * g);
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < QT; ++j) s[i][j] = Elem<T>::mfma32(bf[i], af[j][st], s[i][j]);
-    }
-
-    // ---- inter-path op on the accumulator registers
-    if (INTER == kInterSoftmax) {
-      if (l0 + kBN > L) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int l = l0 + 32 * i + 8 * (r >> 2) + 4 * g + (r & 3);
-            if (l >= L) {
-#pragma unroll
-              for (int j = 0; j < QT; ++j) s[i][j][r] = -INFINITY;
-            }
-          }
-      }
-#pragma unroll
-      for (int j = 0; j < QT; ++j) {
-        float mx = s[0][j][0];
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[i][j][r]);
-        mx = pair_max(mx) * c2;
-        // Lazy rescale: the running maximum only has to bound the scores well enough that
-        // exp2 cannot overflow, so it is raised (and the accumulators rescaled) only when
-        // some row of the wave exceeds it by more than 2^kLazy.  Rows keep a stale maximum
-        // otherwise; the final division by the row sum cancels it exactly.
-        if (__builtin_amdgcn_ballot_w64(mx > mrow[j] + kLazy) != 0) {
-          const float mnew = fmaxf(mrow[j], mx);
-          const float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);
-          mrow[j] = mnew;
-          lsum[j] *= alpha;
-#pragma unroll
-          for (int t = 0; t < D / 32; ++t)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o[t][j][r] *= alpha;
-        }
-        const float mcur = mrow[j];
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            s[i][j][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i][j][r], c2, -mcur));
-      }
-    } else if (p.relu) {
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < QT; ++j)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[i][j][r] = fmaxf(s[i][j][r], 0.f);
-    }
-
-    // ---- second contraction: o[t][j] += (C^T tile t, l step u) . (P^T tile j, l step u)
-    // l step u covers tile rows 16u..16u+15; half-wave g supplies rows
-    // 16u + 4g + {0..3} and 16u + 8 + 4g + {0..3} (the accumulator layout of s).
-#pragma unroll
-    for (int u = 0; u < kBN / 16; ++u) {
-      V8 pf[QT];
-#pragma unroll
-      for (int j = 0; j < QT; ++j) {
-        const int i = u >> 1, r0 = 8 * (u & 1);
-        typename Elem<T>::v2 p0 = cvt2<T>(s[i][j][r0 + 0], s[i][j][r0 + 1]);
-        typename Elem<T>::v2 p1 = cvt2<T>(s[i][j][r0 + 2], s[i][j][r0 + 3]);
-        typename Elem<T>::v2 p2 = cvt2<T>(s[i][j][r0 + 4], s[i][j][r0 + 5]);
-        typename Elem<T>::v2 p3 = cvt2<T>(s[i][j][r0 + 6], s[i][j][r0 + 7]);
-        if (INTER == kInterSoftmax) {
-          // the row sum is taken over the ROUNDED probabilities, i.e. exactly the values
-          // that enter the second contraction
-          lsum[j] = Elem<T>::add_pair(p0, lsum[j]);
-          lsum[j] = Elem<T>::add_pair(p1, lsum[j]);
-          lsum[j] = Elem<T>::add_pair(p2, lsum[j]);
-          lsum[j] = Elem<T>::add_pair(p3, lsum[j]);
-        }
-        V8 v = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
-        pf[j] = v;
-      }
-#pragma unroll
-      for (int t = 0; t < D / 32; ++t) {
-        const T* q = cs + (16 * u + 4 * g + (i16 >> 2)) * CSTR + 32 * t + 16 * h + 4 * (i16 & 3);
-        V4 lo = lds_read_tr4<T>(q);
-        V4 hi = lds_read_tr4<T>(q + 8 * CSTR);
-        V8 cf = concat4<V4, V8>(lo, hi);
-#pragma unroll
-        for (int j = 0; j < QT; ++j) o[t][j] = Elem<T>::mfma32(cf, pf[j], o[t][j]);
-      }
-    }
-
-    if (it + 1 < ntiles) store_tiles(buf ^ 1);
+    // loads two tiles ahead: B(it+2) replaces B(it-1), C(it+1) replaces C(it-1); both were
+    // released by the barrier that ended tile it-1.  Tiles past the end are entirely out of
+    // range and load zeros.
+    load_b(it + 2, (it + 2) % 3);
+    load_c(it + 1, (it + 1) & 1);
+    half_step(sa, sb, it, 0);
+    half_step(sb, sa, it, 1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
 
@@ -288,7 +364,7 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
 #pragma unroll
   for (int j = 0; j < QT; ++j) {
     float inv = 1.f;
-    if (INTER == kInterSoftmax) inv = 1.f / pair_sum(lsum[j]);
+    if constexpr (INTER == kInterSoftmax) inv = 1.f / pair_sum(lsum[j]);
     const int row = m_wave + 32 * j + ln;
     if (row >= M) continue;
 #pragma unroll
@@ -304,18 +380,21 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
           f32x4 w = {v0, v1, v2, v3};
           *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.f) + off) = w;
         } else {
-          typename Elem<T>::v2 a0 = cvt2<T>(v0, v1), a1 = cvt2<T>(v2, v3);
+          V2 a0 = cvt2<T>(v0, v1), a1 = cvt2<T>(v2, v3);
           V4 w = {a0[0], a0[1], a1[0], a1[1]};
           *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.f) + off) = w;
         }
       }
   }
+#else
+  (void)p;
+#endif
 }
 
 // Host-side launcher for one instantiation.
 template <typename T, int D, int QT, int INTER, bool B_KL>
 hipError_t launch_bmm_chain(const BmmChainArgs& args, hipStream_t stream) {
-  constexpr int lds = bmm_chain_lds_bytes<D, B_KL>();
+  constexpr int lds = bmm_chain_lds_bytes<D>();
   auto kern = bmm_chain_kernel<T, D, QT, INTER, B_KL>;
   static thread_local int configured_dev = -1;
   int dev = 0;
