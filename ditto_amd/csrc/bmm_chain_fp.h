@@ -204,27 +204,6 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
 
   // Scores are produced and consumed in HALF steps of 32 rows of the L tile: s[j] is the
   // transposed score tile (32 l x 32 m) of A-row tile j.
-  // first contraction of one half step: s[j] = (B^T rows 32i..32i+31) . (A^T tile j)
-  auto s_half = [&](f32x16 (&s)[QT], const char* bs, int i, int st) {
-    V8 bf;
-    if (B_KL) {
-      const char* q = bs + b_rd + 16 * st * B_RB + (((4 * i) ^ b_x[i]) * 16);
-      V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
-      V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(q + 4 * B_RB));
-      bf = concat4<V4, V8>(lo, hi);
-    } else {
-      bf = *reinterpret_cast<const V8*>(bs + b_rd + 32 * i * B_RB + (((2 * st) ^ b_x[i]) * 16));
-    }
-#pragma unroll
-    for (int j = 0; j < QT; ++j) {
-      if (st == 0) {
-        const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        s[j] = Elem<T>::mfma32(bf, af[j][st], z);
-      } else {
-        s[j] = Elem<T>::mfma32(bf, af[j][st], s[j]);
-      }
-    }
-  };
   // scores of rows past L are masked out (softmax only; other chains see zero operands)
   auto mask_tail = [&](f32x16 (&s)[QT], int l0) {
 #pragma unroll
@@ -273,11 +252,28 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
       for (int e = 0; e < n; ++e)
         s[j][r0 + e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r0 + e], c2, -mrow[j]));
   };
-  // second contraction, 16 rows of the L tile: o[t][j] += (C^T tile t, rows 16u..) . (P^T).
-  // Half-wave g supplies rows 16u + 4g + {0..3} and 16u + 8 + 4g + {0..3}: registers
-  // 8(u%2) .. 8(u%2)+7 of the half tile, the accumulator layout of s.
-  auto pv_step = [&](f32x16 (&s)[QT], const char* cs, int u) {
-    V8 pf[QT];
+  // ---- operand fragments read from LDS
+  // B fragment of MFMA group st for rows 32i..32i+31 of the L tile in buffer `bs`
+  auto b_frag = [&](const char* bs, int i, int st) -> V8 {
+    if (B_KL) {
+      const char* q = bs + b_rd + 16 * st * B_RB + (((4 * i) ^ b_x[i]) * 16);
+      V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
+      V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(q + 4 * B_RB));
+      return concat4<V4, V8>(lo, hi);
+    }
+    return *reinterpret_cast<const V8*>(bs + b_rd + 32 * i * B_RB + (((2 * st) ^ b_x[i]) * 16));
+  };
+  // C fragment of N tile t for rows 16u..16u+15 of the L tile
+  auto c_frag = [&](const char* cs, int u, int t) -> V8 {
+    const char* q = cs + c_rd + 16 * u * C_RB + (((4 * t) ^ c_x) * 16);
+    V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
+    V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(q + 8 * C_RB));
+    return concat4<V4, V8>(lo, hi);
+  };
+  // P fragment (B operand of the second contraction) of 16 rows of the L tile: registers
+  // 8(u%2) .. 8(u%2)+7 of the half tile, cast; the row sum is taken over the ROUNDED
+  // probabilities, i.e. exactly the values that enter the second contraction
+  auto p_frag = [&](f32x16 (&s)[QT], int u, V8 (&pf)[QT]) {
 #pragma unroll
     for (int j = 0; j < QT; ++j) {
       const int r0 = 8 * (u & 1);
@@ -289,8 +285,6 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
       }
       V2 p0 = cvt2<T>(v[0], v[1]), p1 = cvt2<T>(v[2], v[3]), p2 = cvt2<T>(v[4], v[5]), p3 = cvt2<T>(v[6], v[7]);
       if constexpr (INTER == kInterSoftmax) {
-        // the row sum is taken over the ROUNDED probabilities, i.e. exactly the values that
-        // enter the second contraction
         lsum[j] = Elem<T>::add_pair(p0, lsum[j]);
         lsum[j] = Elem<T>::add_pair(p1, lsum[j]);
         lsum[j] = Elem<T>::add_pair(p2, lsum[j]);
@@ -299,38 +293,73 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
       V8 w = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
       pf[j] = w;
     }
-#pragma unroll
-    for (int t = 0; t < D / 32; ++t) {
-      const char* q = cs + c_rd + 16 * u * C_RB + (((4 * t) ^ c_x) * 16);
-      V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
-      V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(q + 8 * C_RB));
-      V8 cf = concat4<V4, V8>(lo, hi);
-#pragma unroll
-      for (int j = 0; j < QT; ++j) o[t][j] = Elem<T>::mfma32(cf, pf[j], o[t][j]);
-    }
   };
 
   // One pipelined half step: consumes the finished scores `cur` (half hh of L tile `it`) and
   // produces `nxt`, the scores of the following half (half 1 of the same tile, or half 0 of
   // tile it+1).  Past the last tile the MFMAs run on a resident but stale B buffer and their
-  // result is dropped, which keeps the half step one straight-line block whose MFMA and VALU
-  // streams the scheduler can interleave.
+  // result is dropped, which keeps the half step straight-line code.
+  //
+  // The half step is a sequence of NG MFMA groups, each fed by one LDS fragment: D/16 groups
+  // of the first contraction (scores of the next half) followed by D/16 groups of the second
+  // (2 sixteen-row steps x D/32 column tiles).  Fragments are fetched kAhead groups before
+  // they are used so that the LDS latency is covered by the MFMAs of the groups in between;
+  // the exponentials of `cur` are spread over the first-contraction groups.
+  constexpr int NS = D / 16, NG = 2 * NS, kAhead = 2;
   auto half_step = [&](f32x16 (&cur)[QT], f32x16 (&nxt)[QT], int it, int hh) {
     const int nt = hh ? it + 1 : it;  // tile of the next half
     const char* bs_next = smem_raw + ((nt % 3) * TILE) * 2;
     const char* cs_cur = smem_raw + C_BASE + ((it & 1) * TILE) * 2;
     if constexpr (INTER == kInterSoftmax) maybe_rescale();
-    constexpr int NST = D / 16, PER = 16 / NST;  // MFMA groups and score registers per group
+    V8 fr[NG];
+    auto fetch = [&](int k) {
+      fr[k] = k < NS ? b_frag(bs_next, hh ^ 1, k) : c_frag(cs_cur, 2 * hh + (k - NS) / (D / 32), (k - NS) % (D / 32));
+    };
 #pragma unroll
-    for (int st = 0; st < NST; ++st) {
-      s_half(nxt, bs_next, hh ^ 1, st);
-      if constexpr (INTER == kInterSoftmax) exp_slice(cur, PER * st, PER);
+    for (int k = 0; k < kAhead; ++k) fetch(k);
+    V8 pf[QT];
+#pragma unroll
+    for (int k = 0; k < NG; ++k) {
+      if (k + kAhead < NG) fetch(k + kAhead);
+      __builtin_amdgcn_sched_barrier(0);
+      if (k < NS) {
+#pragma unroll
+        for (int j = 0; j < QT; ++j) {
+          if (k == 0) {
+            const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            nxt[j] = Elem<T>::mfma32(fr[k], af[j][k], z);
+          } else {
+            nxt[j] = Elem<T>::mfma32(fr[k], af[j][k], nxt[j]);
+          }
+        }
+        if constexpr (INTER == kInterSoftmax) exp_slice(cur, (16 / NS) * k, 16 / NS);
+      } else {
+        const int u = 2 * hh + (k - NS) / (D / 32), t = (k - NS) % (D / 32);
+        if (t == 0) p_frag(cur, u, pf);
+#pragma unroll
+        for (int j = 0; j < QT; ++j) o[t][j] = Elem<T>::mfma32(fr[k], pf[j], o[t][j]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    pv_step(cur, cs_cur, 2 * hh);
-    pv_step(cur, cs_cur, 2 * hh + 1);
     if constexpr (INTER == kInterSoftmax) {
       if (ragged && nt == ntiles - 1) mask_tail(nxt, nt * kBN + 32 * (hh ^ 1));
       row_max(nxt);
+    }
+  };
+  // scores of the very first half (prologue)
+  auto first_half = [&](f32x16 (&s)[QT]) {
+#pragma unroll
+    for (int st = 0; st < NS; ++st) {
+      const V8 bf = b_frag(smem_raw, 0, st);
+#pragma unroll
+      for (int j = 0; j < QT; ++j) {
+        if (st == 0) {
+          const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+          s[j] = Elem<T>::mfma32(bf, af[j][st], z);
+        } else {
+          s[j] = Elem<T>::mfma32(bf, af[j][st], s[j]);
+        }
+      }
     }
   };
 
@@ -341,8 +370,7 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   f32x16 sa[QT], sb[QT];
-#pragma unroll
-  for (int st = 0; st < D / 16; ++st) s_half(sa, smem_raw, 0, st);
+  first_half(sa);
   if constexpr (INTER == kInterSoftmax) {
     if (ragged && ntiles == 1) mask_tail(sa, 0);
     row_max(sa);
