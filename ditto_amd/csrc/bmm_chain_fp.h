@@ -43,6 +43,11 @@ struct BmmChainArgs {
   int out_f32;       // write F as fp32 instead of T
 };
 
+template <int V>
+struct IntC {
+  static constexpr int value = V;
+};
+
 constexpr int kInterCast = 0;
 constexpr int kInterSoftmax = 2;
 
@@ -52,7 +57,7 @@ constexpr float kLazy = 8.0f;  // log2 of the slack allowed before the running m
 
 template <int D>
 __host__ __device__ constexpr int bmm_chain_lds_bytes() {
-  return (3 + 2) * kBN * D * 2;  // three B tiles, two C tiles, 16-bit elements
+  return (4 + 2) * kBN * D * 2;  // four B tiles, two C tiles, 16-bit elements
 }
 
 // XOR applied to the 16-byte chunk index of a row of an unpadded LDS tile.
@@ -86,8 +91,10 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
   static_assert(NLD >= 1, "tile too small");
 
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
-  // B tiles [3][TILE] at byte 0, C tiles [2][TILE] at byte 3*TILE*2
-  constexpr int C_BASE = 3 * TILE * 2;
+  // B tiles [4][TILE] at byte 0, C tiles [2][TILE] at byte 4*TILE*2.  Tile t of B lives in
+  // buffer t%4 and tile t of C in buffer t%2; the tile loop is unrolled four times so that every
+  // buffer address is a compile-time constant and folds into the LDS instructions' offsets.
+  constexpr int C_BASE = 4 * TILE * 2;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -106,8 +113,9 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
   // ---- buffer resources over this batch entry's B and C (reads past the end return 0)
   const unsigned b_bytes = (unsigned)(B_KL ? ((long long)(K - 1) * p.b_rs + L) : ((long long)(L - 1) * p.b_rs + K)) * 2u;
   const unsigned c_bytes = (unsigned)((long long)(L - 1) * p.c_rs + N) * 2u;
-  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(Bg), 0, b_bytes, 0x00020000);
-  const __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(Cg), 0, c_bytes, 0x00020000);
+  const i32x4 b_rsrc = make_rsrc(Bg, b_bytes);
+  const i32x4 c_rsrc = make_rsrc(Cg, c_bytes);
+  const unsigned lds0 = (unsigned)(size_t)(DITTO_LDS char*)smem_raw;  // LDS byte address of the tiles
 
   // ---- per-lane source offsets of the direct loads.  Load q of this wave fills the LDS
   // bytes [1024*(NLD*wave + q), +1024): lane -> (row, physical chunk) -> swizzled source.
@@ -142,17 +150,14 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
       // the whole offset goes into the per-lane operand: it is what the range check sees
       int vo = b_voff[q] + soff;
       if (B_KL) vo = (l0 + b_col[q] < L) ? vo : (int)b_bytes;  // columns past L are inside the buffer
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          b_rsrc, (DITTO_LDS void*)(smem_raw + (buf * TILE) * 2 + 1024 * (NLD * wave + q)), 16, vo, 0, 0, 0);
+      lds_dma_16(b_rsrc, (unsigned)vo, lds0 + (buf * TILE) * 2 + 1024 * (NLD * wave + q));
     }
   };
   auto load_c = [&](int tile, int buf) {
     const int soff = tile * kBN * p.c_rs * 2;
 #pragma unroll
     for (int q = 0; q < NLD; ++q)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          c_rsrc, (DITTO_LDS void*)(smem_raw + C_BASE + (buf * TILE) * 2 + 1024 * (NLD * wave + q)), 16,
-          c_voff[q] + soff, 0, 0, 0);
+      lds_dma_16(c_rsrc, (unsigned)(c_voff[q] + soff), lds0 + C_BASE + (buf * TILE) * 2 + 1024 * (NLD * wave + q));
   };
 
   // ---- per-lane LDS read offsets (bytes, within one tile)
@@ -161,13 +166,20 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
   //   tr-read  layout: rows k = 16st+8g+(i16>>2)+{0,4}, chunk 4i+2h+((i16&3)>>1), +8*(i16&1)
   const int b_rd = B_KL ? ((8 * g + (i16 >> 2)) * B_RB + (2 * h + ((i16 & 3) >> 1)) * 16 + 8 * (i16 & 1))
                         : (ln * B_RB);
-  int b_x[2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i) b_x[i] = B_KL ? swz_trread<B_CPR>(i16 >> 2) : (g ^ swz_rowread<B_CPR>(32 * i + ln));
   // C operand of step u, N-tile t (A operand of F^T = C^T.P^T: rows n, k = l permuted):
   //   rows l = 16u + 4g + (i16>>2) + {0,8}, chunk 4t + 2h + ((i16&3)>>1), +8*(i16&1)
   const int c_rd = (4 * g + (i16 >> 2)) * C_RB + (2 * h + ((i16 & 3) >> 1)) * 16 + 8 * (i16 & 1);
-  const int c_x = swz_trread<C_CPR>(i16 >> 2);
+  // Per-lane byte addresses, loop invariant; everything else is a compile-time offset.
+  constexpr int NS = D / 16;
+  int b_ad[2][NS], c_ad[D / 32];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int x = B_KL ? swz_trread<B_CPR>(i16 >> 2) : (g ^ swz_rowread<B_CPR>(32 * i + ln));
+#pragma unroll
+    for (int st = 0; st < NS; ++st) b_ad[i][st] = b_rd + (B_KL ? ((4 * i) ^ x) : ((2 * st) ^ x)) * 16;
+  }
+#pragma unroll
+  for (int t = 0; t < D / 32; ++t) c_ad[t] = c_rd + ((4 * t) ^ swz_trread<C_CPR>(i16 >> 2)) * 16;
 
   // ---- A fragments (B operand of D^T = B^T.A^T): lane holds A[row][16s + 8g .. +7]
   V8 af[QT][D / 16];
@@ -250,22 +262,26 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
     for (int j = 0; j < QT; ++j)
 #pragma unroll
       for (int e = 0; e < n; ++e)
+#ifdef DITTO_X_NOEXP
+        s[j][r0 + e] = __builtin_fmaf(s[j][r0 + e], c2, -mrow[j]);
+#else
         s[j][r0 + e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r0 + e], c2, -mrow[j]));
+#endif
   };
   // ---- operand fragments read from LDS
-  // B fragment of MFMA group st for rows 32i..32i+31 of the L tile in buffer `bs`
-  auto b_frag = [&](const char* bs, int i, int st) -> V8 {
+  // B fragment of MFMA group st for rows 32i..32i+31 of the L tile at byte offset `off`
+  auto b_frag = [&](int off, int i, int st) -> V8 {
     if (B_KL) {
-      const char* q = bs + b_rd + 16 * st * B_RB + (((4 * i) ^ b_x[i]) * 16);
+      const char* q = smem_raw + b_ad[i][st] + (off + 16 * st * B_RB);
       V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
       V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(q + 4 * B_RB));
       return concat4<V4, V8>(lo, hi);
     }
-    return *reinterpret_cast<const V8*>(bs + b_rd + 32 * i * B_RB + (((2 * st) ^ b_x[i]) * 16));
+    return *reinterpret_cast<const V8*>(smem_raw + b_ad[i][st] + (off + 32 * i * B_RB));
   };
-  // C fragment of N tile t for rows 16u..16u+15 of the L tile
-  auto c_frag = [&](const char* cs, int u, int t) -> V8 {
-    const char* q = cs + c_rd + 16 * u * C_RB + (((4 * t) ^ c_x) * 16);
+  // C fragment of N tile t for rows 16u..16u+15 of the L tile at byte offset `off`
+  auto c_frag = [&](int off, int u, int t) -> V8 {
+    const char* q = smem_raw + c_ad[t] + (off + 16 * u * C_RB);
     V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
     V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(q + 8 * C_RB));
     return concat4<V4, V8>(lo, hi);
@@ -305,14 +321,18 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
   // (2 sixteen-row steps x D/32 column tiles).  Fragments are fetched kAhead groups before
   // they are used so that the LDS latency is covered by the MFMAs of the groups in between;
   // the exponentials of `cur` are spread over the first-contraction groups.
-  constexpr int NS = D / 16, NG = 2 * NS, kAhead = 2;
-  auto half_step = [&](f32x16 (&cur)[QT], f32x16 (&nxt)[QT], int it, int hh) {
+  constexpr int NG = 2 * NS, kAhead = 2;
+  auto half_step = [&](f32x16 (&cur)[QT], f32x16 (&nxt)[QT], int it, auto bi_c, auto hh_c) {
+    constexpr int BI = decltype(bi_c)::value, hh = decltype(hh_c)::value;  // B buffer of tile it; half
     const int nt = hh ? it + 1 : it;  // tile of the next half
-    const char* bs_next = smem_raw + ((nt % 3) * TILE) * 2;
-    const char* cs_cur = smem_raw + C_BASE + ((it & 1) * TILE) * 2;
+    constexpr int bs_next = ((hh ? (BI + 1) & 3 : BI) * TILE) * 2;
+    constexpr int cs_cur = C_BASE + ((BI & 1) * TILE) * 2;
     if constexpr (INTER == kInterSoftmax) maybe_rescale();
     V8 fr[NG];
     auto fetch = [&](int k) {
+#ifdef DITTO_X_NOLDS
+      if (k >= 2) { fr[k] = fr[k & 1]; return; }
+#endif
       fr[k] = k < NS ? b_frag(bs_next, hh ^ 1, k) : c_frag(cs_cur, 2 * hh + (k - NS) / (D / 32), (k - NS) % (D / 32));
     };
 #pragma unroll
@@ -350,7 +370,7 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
   auto first_half = [&](f32x16 (&s)[QT]) {
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
-      const V8 bf = b_frag(smem_raw, 0, st);
+      const V8 bf = b_frag(0, 0, st);
 #pragma unroll
       for (int j = 0; j < QT; ++j) {
         if (st == 0) {
@@ -376,16 +396,27 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
     row_max(sa);
   }
 
-  for (int it = 0; it < ntiles; ++it) {
-    // loads two tiles ahead: B(it+2) replaces B(it-1), C(it+1) replaces C(it-1); both were
-    // released by the barrier that ended tile it-1.  Tiles past the end are entirely out of
-    // range and load zeros.
-    load_b(it + 2, (it + 2) % 3);
-    load_c(it + 1, (it + 1) & 1);
-    half_step(sa, sb, it, 0);
-    half_step(sb, sa, it, 1);
+  // One L tile: loads two tiles ahead (B(it+2) replaces B(it-2), C(it+1) replaces C(it-1); both
+  // were released by earlier barriers; tiles past the end are entirely out of range and load
+  // zeros), then the two pipelined half steps, then the barrier that publishes the loads.
+  auto tile_step = [&](int it, auto bi_c) {
+    constexpr int BI = decltype(bi_c)::value;
+#ifndef DITTO_X_NOLOAD
+    load_b(it + 2, (BI + 2) & 3);
+    load_c(it + 1, (BI + 1) & 1);
+#endif
+    half_step(sa, sb, it, bi_c, IntC<0>{});
+    half_step(sb, sa, it, bi_c, IntC<1>{});
+#ifndef DITTO_X_NOBAR
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+#endif
+  };
+  for (int it = 0; it < ntiles; it += 4) {
+    tile_step(it, IntC<0>{});
+    if (it + 1 < ntiles) tile_step(it + 1, IntC<1>{});
+    if (it + 2 < ntiles) tile_step(it + 2, IntC<2>{});
+    if (it + 3 < ntiles) tile_step(it + 3, IntC<3>{});
   }
 
   // ---- epilogue: normalise (softmax), cast, store 4 contiguous columns per lane

@@ -112,6 +112,28 @@ __device__ __forceinline__ float pair_sum(float x) {
   return a + b;
 }
 
+// Direct global -> LDS load of 16 bytes per lane (buffer_load_dwordx4 ... lds): lane l's data
+// lands at LDS byte address lds_base + 16*l; reads whose offset is at or past the resource's
+// num_records return zero.  Issued as inline asm so that the compiler does not track it: its
+// own bookkeeping would make every later LDS read wait for ALL outstanding loads (it cannot
+// prove that the tile being filled and the tile being read are different), which serialises
+// the prefetch.  The caller must s_waitcnt vmcnt(0) (and barrier) before reading the tile.
+__device__ __forceinline__ void lds_dma_16(i32x4 rsrc, unsigned voffset, unsigned lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %0, %1, 0 offen lds"
+      :
+      : "v"(voffset), "s"(rsrc), "s"(lds_base)
+      : "memory", "m0");
+}
+// raw buffer resource (stride 0, range checked against `bytes`) as four dwords
+__device__ __forceinline__ i32x4 make_rsrc(const void* base, unsigned bytes) {
+  const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+  i32x4 r = {(int)(unsigned)a, (int)(unsigned)((a >> 32) & 0xffff), (int)bytes, 0x00020000};
+  return r;
+}
+
 // Workgroups are dealt round-robin to the 8 XCDs (each with a private L2) by
 // linear id.  Remap so that ids that are neighbours in the logical order (and
 // share operands) land on the same XCD.
