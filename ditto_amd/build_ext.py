@@ -25,6 +25,7 @@ HIPCC_FLAGS = [
     # inter-path op works on the accumulator, so AGPR-resident results cost a copy per use
     "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument",
+    "-Wno-inline-asm",
 ]
 
 # The row maximum of the online softmax is only a stabiliser: without NaN-quieting the compiler

@@ -6,6 +6,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "bmm_chain_fp.h"
@@ -304,13 +305,15 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     args.out_f32 = d->out_dtype == DITTO_F32;
     const bool kl = d->b_layout == DITTO_B_KL;
     const bool sm = d->inter_op == DITTO_INTER_SOFTMAX;
+    static const bool fold_env = getenv("DITTO_FOLD_SCALE") ? atoi(getenv("DITTO_FOLD_SCALE")) != 0 : false;
+    const bool fold = sm && fold_env;
     hipError_t e;
     if (d->in_dtype == DITTO_F16)
-      e = sm ? ditto::launch_f16_softmax(plan.d_pad, plan.qt, kl, args, st)
-             : ditto::launch_f16_cast(plan.d_pad, plan.qt, kl, args, st);
+      e = sm ? ditto::launch_f16_softmax(plan.d_pad, plan.qt, kl, fold, args, st)
+             : ditto::launch_f16_cast(plan.d_pad, plan.qt, kl, false, args, st);
     else
-      e = sm ? ditto::launch_bf16_softmax(plan.d_pad, plan.qt, kl, args, st)
-             : ditto::launch_bf16_cast(plan.d_pad, plan.qt, kl, args, st);
+      e = sm ? ditto::launch_bf16_softmax(plan.d_pad, plan.qt, kl, fold, args, st)
+             : ditto::launch_bf16_cast(plan.d_pad, plan.qt, kl, false, args, st);
     if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
     return DITTO_OK;
   }

@@ -74,8 +74,8 @@ __device__ __forceinline__ int swz_trread(int row) {
   return CPR == 16 ? 4 * (row & 3) : 4 * ((row >> 1) & 1);
 }
 
-template <typename T, int D, int QT, int INTER, bool B_KL>
-__global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
+template <typename T, int D, int QT, int INTER, bool B_KL, bool FOLD>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void bmm_chain_kernel(BmmChainArgs p) {
   // The body uses device-only types (buffer resources); the host pass only needs the stub.
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef typename Elem<T>::v8 V8;
@@ -142,22 +142,26 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
       c_voff[q] = cl * 8 < N ? (row * p.c_rs + cl * 8) * 2 : (int)c_bytes;
     }
   }
-  auto load_b = [&](int tile, int buf) {
+  // direct load q (of NLD) of this wave for B tile `tile` into buffer `buf`
+  auto load_b1 = [&](int tile, int buf, int q) __attribute__((always_inline)) {
     const int l0 = tile * kBN;
     const int soff = B_KL ? l0 * 2 : l0 * p.b_rs * 2;
-#pragma unroll
-    for (int q = 0; q < NLD; ++q) {
-      // the whole offset goes into the per-lane operand: it is what the range check sees
-      int vo = b_voff[q] + soff;
-      if (B_KL) vo = (l0 + b_col[q] < L) ? vo : (int)b_bytes;  // columns past L are inside the buffer
-      lds_dma_16(b_rsrc, (unsigned)vo, lds0 + (buf * TILE) * 2 + 1024 * (NLD * wave + q));
-    }
+    // the whole offset goes into the per-lane operand: it is what the range check sees
+    int vo = b_voff[q] + soff;
+    if (B_KL) vo = (l0 + b_col[q] < L) ? vo : (int)b_bytes;  // columns past L are inside the buffer
+    lds_dma_16(b_rsrc, (unsigned)vo, lds0 + (buf * TILE) * 2 + 1024 * (NLD * wave + q));
   };
-  auto load_c = [&](int tile, int buf) {
+  auto load_c1 = [&](int tile, int buf, int q) __attribute__((always_inline)) {
     const int soff = tile * kBN * p.c_rs * 2;
+    lds_dma_16(c_rsrc, (unsigned)(c_voff[q] + soff), lds0 + C_BASE + (buf * TILE) * 2 + 1024 * (NLD * wave + q));
+  };
+  auto load_b = [&](int tile, int buf) __attribute__((always_inline)) {
 #pragma unroll
-    for (int q = 0; q < NLD; ++q)
-      lds_dma_16(c_rsrc, (unsigned)(c_voff[q] + soff), lds0 + C_BASE + (buf * TILE) * 2 + 1024 * (NLD * wave + q));
+    for (int q = 0; q < NLD; ++q) load_b1(tile, buf, q);
+  };
+  auto load_c = [&](int tile, int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q = 0; q < NLD; ++q) load_c1(tile, buf, q);
   };
 
   // ---- per-lane LDS read offsets (bytes, within one tile)
@@ -191,6 +195,11 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
       const int col = 16 * s + 8 * g;
       V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
       if (row < M && col < K) v = *reinterpret_cast<const V8*>(Ag + (long long)row * p.a_rs + col);
+      if constexpr (FOLD) {
+        // softmax scale (in the exp2 domain) folded into the A operand
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (T)((float)v[e] * p.scale_log2);
+      }
       af[j][s] = v;
     }
   }
@@ -203,12 +212,21 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
     for (int j = 0; j < QT; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[t][j][r] = 0.f;
+  // Softmax state per A-row tile j (one row per lane pair): running maximum mrow (exp2 domain),
+  // partial row sum lsum, and mxn = row maximum of the half tile about to be consumed.
+  //   !FOLD: scores are raw dot products; mxn is absolute (scaled); p = exp2(s*c2 - mrow).
+  //   FOLD : the A fragments carry the scale and the score MFMAs start from -mrow (negm), so
+  //          the accumulator already holds s*c2 - mrow and p = exp2(acc): one VALU op per
+  //          score; mxn is relative to the mrow the tile was computed with.
   float mrow[QT], lsum[QT], mxn[QT];
+  f32x16 negm[QT];
 #pragma unroll
   for (int j = 0; j < QT; ++j) {
-    mrow[j] = -INFINITY;
+    mrow[j] = FOLD ? 0.f : -INFINITY;
     lsum[j] = 0.f;
-    mxn[j] = -INFINITY;
+    mxn[j] = FOLD ? 0.f : -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) negm[j][r] = 0.f;
   }
   const float c2 = p.scale_log2;
   const int ntiles = (L + kBN - 1) / kBN;
@@ -217,7 +235,7 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
   // Scores are produced and consumed in HALF steps of 32 rows of the L tile: s[j] is the
   // transposed score tile (32 l x 32 m) of A-row tile j.
   // scores of rows past L are masked out (softmax only; other chains see zero operands)
-  auto mask_tail = [&](f32x16 (&s)[QT], int l0) {
+  auto mask_tail = [&](f32x16 (&s)[QT], int l0) __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int l = l0 + 8 * (r >> 2) + 4 * g + (r & 3);
@@ -228,49 +246,64 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
     }
   };
   // scaled row maximum of a finished half tile (pair of half-waves combined)
-  auto row_max = [&](f32x16 (&s)[QT]) {
+  auto row_max = [&](f32x16 (&s)[QT]) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < QT; ++j) {
       float mx = s[j][0];
 #pragma unroll
       for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[j][r]);
-      mxn[j] = pair_max(mx) * c2;
+      mxn[j] = FOLD ? pair_max(mx) : pair_max(mx) * c2;
     }
   };
   // Lazy rescale: the running maximum only has to bound the scores well enough that exp2
   // cannot overflow, so it is raised (and the accumulators rescaled) only when some row of
   // the wave exceeds it by more than 2^kLazy.  Rows keep a stale maximum otherwise; the
   // final division by the row sum cancels it exactly.
-  auto maybe_rescale = [&]() {
+  auto maybe_rescale = [&](f32x16 (&cur)[QT]) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < QT; ++j) {
-      if (__builtin_amdgcn_ballot_w64(mxn[j] > mrow[j] + kLazy) != 0) {
-        const float mnew = fmaxf(mrow[j], mxn[j]);
-        const float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);
-        mrow[j] = mnew;
-        lsum[j] *= alpha;
+      if constexpr (FOLD) {
+        if (__builtin_amdgcn_ballot_w64(mxn[j] > kLazy) != 0) {
+          const float up = fmaxf(mxn[j], 0.f);  // rows below their maximum keep it
+          const float alpha = __builtin_amdgcn_exp2f(-up);
+          mrow[j] += up;
+          lsum[j] *= alpha;
 #pragma unroll
-        for (int t = 0; t < D / 32; ++t)
+          for (int r = 0; r < 16; ++r) {
+            cur[j][r] -= up;  // these scores were computed against the old maximum
+            negm[j][r] = -mrow[j];
+          }
 #pragma unroll
-          for (int r = 0; r < 16; ++r) o[t][j][r] *= alpha;
+          for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[t][j][r] *= alpha;
+        }
+      } else {
+        if (__builtin_amdgcn_ballot_w64(mxn[j] > mrow[j] + kLazy) != 0) {
+          const float mnew = fmaxf(mrow[j], mxn[j]);
+          const float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);
+          mrow[j] = mnew;
+          lsum[j] *= alpha;
+#pragma unroll
+          for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[t][j][r] *= alpha;
+        }
       }
     }
   };
   // exponentials of registers [r0, r0 + n) of the half tile
-  auto exp_slice = [&](f32x16 (&s)[QT], int r0, int n) {
+  auto exp_slice = [&](f32x16 (&s)[QT], int r0, int n) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < QT; ++j)
 #pragma unroll
       for (int e = 0; e < n; ++e)
-#ifdef DITTO_X_NOEXP
-        s[j][r0 + e] = __builtin_fmaf(s[j][r0 + e], c2, -mrow[j]);
-#else
-        s[j][r0 + e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r0 + e], c2, -mrow[j]));
-#endif
+        s[j][r0 + e] = FOLD ? __builtin_amdgcn_exp2f(s[j][r0 + e])
+                            : __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r0 + e], c2, -mrow[j]));
   };
   // ---- operand fragments read from LDS
   // B fragment of MFMA group st for rows 32i..32i+31 of the L tile at byte offset `off`
-  auto b_frag = [&](int off, int i, int st) -> V8 {
+  auto b_frag = [&](int off, int i, int st) __attribute__((always_inline)) -> V8 {
     if (B_KL) {
       const char* q = smem_raw + b_ad[i][st] + (off + 16 * st * B_RB);
       V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
@@ -280,7 +313,7 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
     return *reinterpret_cast<const V8*>(smem_raw + b_ad[i][st] + (off + 32 * i * B_RB));
   };
   // C fragment of N tile t for rows 16u..16u+15 of the L tile at byte offset `off`
-  auto c_frag = [&](int off, int u, int t) -> V8 {
+  auto c_frag = [&](int off, int u, int t) __attribute__((always_inline)) -> V8 {
     const char* q = smem_raw + c_ad[t] + (off + 16 * u * C_RB);
     V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
     V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(q + 8 * C_RB));
@@ -289,7 +322,7 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
   // P fragment (B operand of the second contraction) of 16 rows of the L tile: registers
   // 8(u%2) .. 8(u%2)+7 of the half tile, cast; the row sum is taken over the ROUNDED
   // probabilities, i.e. exactly the values that enter the second contraction
-  auto p_frag = [&](f32x16 (&s)[QT], int u, V8 (&pf)[QT]) {
+  auto p_frag = [&](f32x16 (&s)[QT], int u, V8 (&pf)[QT]) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < QT; ++j) {
       const int r0 = 8 * (u & 1);
@@ -322,42 +355,58 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
   // they are used so that the LDS latency is covered by the MFMAs of the groups in between;
   // the exponentials of `cur` are spread over the first-contraction groups.
   constexpr int NG = 2 * NS, kAhead = 2;
-  auto half_step = [&](f32x16 (&cur)[QT], f32x16 (&nxt)[QT], int it, auto bi_c, auto hh_c) {
+  auto half_step = [&](f32x16 (&cur)[QT], f32x16 (&nxt)[QT], int it, auto bi_c, auto hh_c) __attribute__((always_inline)) {
     constexpr int BI = decltype(bi_c)::value, hh = decltype(hh_c)::value;  // B buffer of tile it; half
     const int nt = hh ? it + 1 : it;  // tile of the next half
     constexpr int bs_next = ((hh ? (BI + 1) & 3 : BI) * TILE) * 2;
     constexpr int cs_cur = C_BASE + ((BI & 1) * TILE) * 2;
-    if constexpr (INTER == kInterSoftmax) maybe_rescale();
+    if constexpr (INTER == kInterSoftmax) maybe_rescale(cur);
     V8 fr[NG];
-    auto fetch = [&](int k) {
+    auto fetch = [&](int k) __attribute__((always_inline)) {
 #ifdef DITTO_X_NOLDS
       if (k >= 2) { fr[k] = fr[k & 1]; return; }
 #endif
-      fr[k] = k < NS ? b_frag(bs_next, hh ^ 1, k) : c_frag(cs_cur, 2 * hh + (k - NS) / (D / 32), (k - NS) % (D / 32));
+      // second contraction groups run N tile by N tile, two sixteen-row steps each
+      fr[k] = k < NS ? b_frag(bs_next, hh ^ 1, k) : c_frag(cs_cur, 2 * hh + (k - NS) % 2, (k - NS) / 2);
     };
 #pragma unroll
     for (int k = 0; k < kAhead; ++k) fetch(k);
-    V8 pf[QT];
+    V8 pf[2][QT];
 #pragma unroll
     for (int k = 0; k < NG; ++k) {
       if (k + kAhead < NG) fetch(k + kAhead);
+#ifndef DITTO_X_NOLOAD
+      if (hh == 0) {
+        // the direct loads for two tiles ahead are spread over the groups of the first half
+        // step (a burst of them would hold up the wave's single instruction stream)
+        constexpr int NL2 = 2 * NLD, EVERY = NG / NL2 > 0 ? NG / NL2 : 1;
+        if (k % EVERY == 0 && k / EVERY < NL2) {
+          const int q = k / EVERY;
+          if (q < NLD) load_b1(it + 2, (BI + 2) & 3, q);
+          else load_c1(it + 1, (BI + 1) & 1, q - NLD);
+        }
+      }
+#endif
       __builtin_amdgcn_sched_barrier(0);
       if (k < NS) {
 #pragma unroll
         for (int j = 0; j < QT; ++j) {
           if (k == 0) {
             const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            nxt[j] = Elem<T>::mfma32(fr[k], af[j][k], z);
+            nxt[j] = Elem<T>::mfma32(fr[k], af[j][k], FOLD ? negm[j] : z);
           } else {
             nxt[j] = Elem<T>::mfma32(fr[k], af[j][k], nxt[j]);
           }
         }
         if constexpr (INTER == kInterSoftmax) exp_slice(cur, (16 / NS) * k, 16 / NS);
       } else {
-        const int u = 2 * hh + (k - NS) / (D / 32), t = (k - NS) % (D / 32);
-        if (t == 0) p_frag(cur, u, pf);
+        const int uu = (k - NS) % 2, t = (k - NS) / 2;
+        if (k == NS) {
+          p_frag(cur, 2 * hh, pf[0]);
+          p_frag(cur, 2 * hh + 1, pf[1]);
+        }
 #pragma unroll
-        for (int j = 0; j < QT; ++j) o[t][j] = Elem<T>::mfma32(fr[k], pf[j], o[t][j]);
+        for (int j = 0; j < QT; ++j) o[t][j] = Elem<T>::mfma32(fr[k], pf[uu][j], o[t][j]);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -367,7 +416,7 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
     }
   };
   // scores of the very first half (prologue)
-  auto first_half = [&](f32x16 (&s)[QT]) {
+  auto first_half = [&](f32x16 (&s)[QT]) __attribute__((always_inline)) {
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
       const V8 bf = b_frag(0, 0, st);
@@ -394,17 +443,26 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
   if constexpr (INTER == kInterSoftmax) {
     if (ragged && ntiles == 1) mask_tail(sa, 0);
     row_max(sa);
+    if constexpr (FOLD) {
+      // start from the exact maximum of the first half (whatever its sign)
+#pragma unroll
+      for (int j = 0; j < QT; ++j) {
+        mrow[j] = mxn[j];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          sa[j][r] -= mxn[j];
+          negm[j][r] = -mxn[j];
+        }
+        mxn[j] = 0.f;
+      }
+    }
   }
 
   // One L tile: loads two tiles ahead (B(it+2) replaces B(it-2), C(it+1) replaces C(it-1); both
   // were released by earlier barriers; tiles past the end are entirely out of range and load
   // zeros), then the two pipelined half steps, then the barrier that publishes the loads.
-  auto tile_step = [&](int it, auto bi_c) {
+  auto tile_step = [&](int it, auto bi_c) __attribute__((always_inline)) {
     constexpr int BI = decltype(bi_c)::value;
-#ifndef DITTO_X_NOLOAD
-    load_b(it + 2, (BI + 2) & 3);
-    load_c(it + 1, (BI + 1) & 1);
-#endif
     half_step(sa, sb, it, bi_c, IntC<0>{});
     half_step(sb, sa, it, bi_c, IntC<1>{});
 #ifndef DITTO_X_NOBAR
@@ -451,10 +509,10 @@ __global__ __launch_bounds__(256) void bmm_chain_kernel(BmmChainArgs p) {
 }
 
 // Host-side launcher for one instantiation.
-template <typename T, int D, int QT, int INTER, bool B_KL>
+template <typename T, int D, int QT, int INTER, bool B_KL, bool FOLD>
 hipError_t launch_bmm_chain(const BmmChainArgs& args, hipStream_t stream) {
   constexpr int lds = bmm_chain_lds_bytes<D>();
-  auto kern = bmm_chain_kernel<T, D, QT, INTER, B_KL>;
+  auto kern = bmm_chain_kernel<T, D, QT, INTER, B_KL, FOLD>;
   static thread_local int configured_dev = -1;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);

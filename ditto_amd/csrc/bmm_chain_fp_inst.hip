@@ -5,13 +5,16 @@
 
 namespace ditto {
 
-hipError_t DITTO_INST_NAME(int d_pad, int qt, bool b_kl, const BmmChainArgs& args, hipStream_t stream) {
+hipError_t DITTO_INST_NAME(int d_pad, int qt, bool b_kl, bool fold, const BmmChainArgs& args, hipStream_t stream) {
   typedef DITTO_INST_T T;
   constexpr int I = DITTO_INST_INTER;
 #define DITTO_CASE(DP, Q)                                                          \
   if (d_pad == DP && qt == Q) {                                                    \
-    return b_kl ? launch_bmm_chain<T, DP, Q, I, true>(args, stream)                \
-                : launch_bmm_chain<T, DP, Q, I, false>(args, stream);              \
+    if (I == kInterSoftmax && fold)                                                \
+      return b_kl ? launch_bmm_chain<T, DP, Q, I, true, I == kInterSoftmax>(args, stream)   \
+                  : launch_bmm_chain<T, DP, Q, I, false, I == kInterSoftmax>(args, stream); \
+    return b_kl ? launch_bmm_chain<T, DP, Q, I, true, false>(args, stream)         \
+                : launch_bmm_chain<T, DP, Q, I, false, false>(args, stream);       \
   }
   DITTO_CASE(64, 1)
   DITTO_CASE(64, 2)
