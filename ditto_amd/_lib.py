@@ -46,6 +46,8 @@ class BmmChainDesc(ctypes.Structure):
         ("f_row_stride", ctypes.c_int64),
         ("softmax_scale", ctypes.c_float),
         ("requant_scale", ctypes.c_float),
+        ("tile_variant", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
     ]
 
 

@@ -49,11 +49,12 @@ def _as3d(t, name):
     return t
 
 
-def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=1.0):
+def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=1.0, tile_variant=0):
     """Fill a ``ditto_bmm_chain_desc`` from tensors A[b,M,K], B[b,K,L], C[b,L,N], F[b,M,N].
 
     B may be a transposed view of a ``[b, L, K]`` tensor (stride 1 along K); it is then
-    consumed in place (``DITTO_B_LK``).
+    consumed in place (``DITTO_B_LK``).  ``tile_variant`` forces a kernel variant (an id that
+    ``select_tile`` reports); 0 leaves the choice to the library's per-shape table.
     """
     A, B, C, F = _as3d(A, "A"), _as3d(B, "B"), _as3d(C, "C"), _as3d(F, "F")
     batch, M, K = A.shape
@@ -91,6 +92,8 @@ def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale
     d.f_batch_stride, d.f_row_stride = F.stride(0), F.stride(1)
     d.softmax_scale = float(softmax_scale)
     d.requant_scale = float(requant_scale)
+    d.tile_variant = int(tile_variant)
+    d.reserved = 0
     return d
 
 
@@ -105,7 +108,8 @@ def select_tile(desc):
     return tile
 
 
-def run_bmm_chain(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=1.0, aux=None, desc=None):
+def run_bmm_chain(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=1.0, aux=None, desc=None,
+                  tile_variant=0):
     """F[b] = epilogue(inter(A[b] . B[b]) . C[b]) as ONE kernel on the current stream.
 
     ``aux``: for ``inter_op="requant"`` an fp32 tensor of L per-column scales (``None``: use
@@ -113,7 +117,7 @@ def run_bmm_chain(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=
     lib = _lib.load()
     dev = _check_device(A, B, C, F)
     if desc is None:
-        desc = bmm_chain_desc(A, B, C, F, inter_op, softmax_scale, requant_scale)
+        desc = bmm_chain_desc(A, B, C, F, inter_op, softmax_scale, requant_scale, tile_variant)
     aux_ptr = None
     if aux is not None:
         _check_device(A, aux)

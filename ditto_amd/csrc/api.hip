@@ -9,7 +9,7 @@
 #include <cstdlib>
 #include <cstring>
 
-#include "bmm_chain_fp.h"
+#include "bmm_chain_fp8.h"
 #include "chain_kernels.h"
 
 namespace {
@@ -64,6 +64,8 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
   if (d->abi_version != DITTO_CHAIN_ABI_VERSION)
     return fail(DITTO_EINVAL, "descriptor abi_version %d, library %d", d->abi_version,
                 DITTO_CHAIN_ABI_VERSION);
+  if (d->reserved != 0) return fail(DITTO_EINVAL, "descriptor field `reserved` must be 0");
+  if (d->tile_variant < 0) return fail(DITTO_EINVAL, "tile_variant must be 0 or a variant id");
   if (d->batch <= 0 || d->M <= 0 || d->N <= 0 || d->K <= 0 || d->L <= 0)
     return fail(DITTO_EINVAL, "batch, M, N, K, L must be positive (got %lld %lld %lld %lld %lld)",
                 (long long)d->batch, (long long)d->M, (long long)d->N, (long long)d->K,
@@ -114,18 +116,36 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     plan->family = 0;
     plan->d_pad = dmax <= 64 ? 64 : 128;
     const int cus = need_device ? device_cus() : 256;
-    const long long blocks_qt2 = ((d->M + 255) / 256) * d->batch;
-    plan->qt = (blocks_qt2 >= 2LL * cus) ? 2 : 1;
-    const int bm = 128 * plan->qt;
+    // Variant table (measured on MI355X, bf16 attention shapes).  With n8 = number of 256-row
+    // workgroups: the eight-wave kernel (two waves per SIMD) wins once n8 fills 3/4 of the CUs;
+    // below that the four-wave kernel with 128-row workgroups spreads over more CUs.  For
+    // head_pad 128 and n8 >= 2 CUs the two are within noise and the four-wave, 256-row kernel
+    // (half the LDS fragment traffic) is kept.
+    const long long n8 = ((d->M + 255) / 256) * d->batch;
+    if (n8 * 4 >= 3LL * cus && !(plan->d_pad == 128 && n8 >= 2LL * cus))
+      plan->qt = 8;
+    else
+      plan->qt = (n8 >= 2LL * cus) ? 2 : 1;
+    if (d->tile_variant != 0) {
+      const int q = d->tile_variant % 10;
+      if (d->tile_variant / 10 != plan->d_pad || (q != 1 && q != 2 && q != 8))
+        return fail(DITTO_EINVAL, "tile_variant %d cannot run this shape (head_pad %d; q must be 1, 2 or 8)",
+                    d->tile_variant, plan->d_pad);
+      plan->qt = q;
+    }
+    const bool kl = d->b_layout == DITTO_B_KL;
+    const int bm = plan->qt == 8 ? 256 : 128 * plan->qt;
     ditto_tile_param& t = plan->tile;
-    t.block_threads = 256;
+    t.block_threads = plan->qt == 8 ? 512 : 256;
     t.block_m = bm;
     t.block_l = ditto::kBN;
     t.block_n = (int)d->N;
     t.head_pad = plan->d_pad;
-    const bool kl = d->b_layout == DITTO_B_KL;
-    (void)kl;
-    t.lds_bytes = plan->d_pad == 64 ? ditto::bmm_chain_lds_bytes<64>() : ditto::bmm_chain_lds_bytes<128>();
+    if (plan->qt == 8)
+      t.lds_bytes = plan->d_pad == 64 ? (kl ? ditto::bmm_chain8_lds_bytes<64, true>() : ditto::bmm_chain8_lds_bytes<64, false>())
+                                      : (kl ? ditto::bmm_chain8_lds_bytes<128, true>() : ditto::bmm_chain8_lds_bytes<128, false>());
+    else
+      t.lds_bytes = plan->d_pad == 64 ? ditto::bmm_chain_lds_bytes<64>() : ditto::bmm_chain_lds_bytes<128>();
     t.grid_x = (int)(((d->M + bm - 1) / bm) * d->batch);
     t.grid_y = t.grid_z = 1;
     t.variant = plan->d_pad * 10 + plan->qt;
@@ -137,6 +157,7 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     if (d->inter_op != DITTO_INTER_REQUANT)
       return fail(DITTO_EUNSUPPORTED, "the int8 chain needs inter_op = DITTO_INTER_REQUANT");
     if (d->b_layout != DITTO_B_KL) return fail(DITTO_EUNSUPPORTED, "the int8 chain takes B as [K][L]");
+    if (d->tile_variant != 0) return fail(DITTO_EINVAL, "the int8 chain has a single variant (tile_variant must be 0)");
     if (d->K % 16 || d->L % 16 || d->N % 16)
       return fail(DITTO_EINVAL, "K, L and N must be multiples of 16 for the int8 chain");
     if (d->a_row_stride % 16 || d->b_row_stride % 16 || d->c_row_stride % 16 || d->a_batch_stride % 16 ||
@@ -305,15 +326,13 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     args.out_f32 = d->out_dtype == DITTO_F32;
     const bool kl = d->b_layout == DITTO_B_KL;
     const bool sm = d->inter_op == DITTO_INTER_SOFTMAX;
-    static const bool fold_env = getenv("DITTO_FOLD_SCALE") ? atoi(getenv("DITTO_FOLD_SCALE")) != 0 : false;
-    const bool fold = sm && fold_env;
     hipError_t e;
     if (d->in_dtype == DITTO_F16)
-      e = sm ? ditto::launch_f16_softmax(plan.d_pad, plan.qt, kl, fold, args, st)
-             : ditto::launch_f16_cast(plan.d_pad, plan.qt, kl, false, args, st);
+      e = sm ? ditto::launch_f16_softmax(plan.d_pad, plan.qt, kl, args, st)
+             : ditto::launch_f16_cast(plan.d_pad, plan.qt, kl, args, st);
     else
-      e = sm ? ditto::launch_bf16_softmax(plan.d_pad, plan.qt, kl, fold, args, st)
-             : ditto::launch_bf16_cast(plan.d_pad, plan.qt, kl, false, args, st);
+      e = sm ? ditto::launch_bf16_softmax(plan.d_pad, plan.qt, kl, args, st)
+             : ditto::launch_bf16_cast(plan.d_pad, plan.qt, kl, args, st);
     if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
     return DITTO_OK;
   }

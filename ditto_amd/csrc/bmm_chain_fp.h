@@ -74,7 +74,7 @@ __device__ __forceinline__ int swz_trread(int row) {
   return CPR == 16 ? 4 * (row & 3) : 4 * ((row >> 1) & 1);
 }
 
-template <typename T, int D, int QT, int INTER, bool B_KL, bool FOLD>
+template <typename T, int D, int QT, int INTER, bool B_KL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void bmm_chain_kernel(BmmChainArgs p) {
   // The body uses device-only types (buffer resources); the host pass only needs the stub.
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -195,11 +195,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       const int col = 16 * s + 8 * g;
       V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
       if (row < M && col < K) v = *reinterpret_cast<const V8*>(Ag + (long long)row * p.a_rs + col);
-      if constexpr (FOLD) {
-        // softmax scale (in the exp2 domain) folded into the A operand
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = (T)((float)v[e] * p.scale_log2);
-      }
       af[j][s] = v;
     }
   }
@@ -213,20 +208,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[t][j][r] = 0.f;
   // Softmax state per A-row tile j (one row per lane pair): running maximum mrow (exp2 domain),
-  // partial row sum lsum, and mxn = row maximum of the half tile about to be consumed.
-  //   !FOLD: scores are raw dot products; mxn is absolute (scaled); p = exp2(s*c2 - mrow).
-  //   FOLD : the A fragments carry the scale and the score MFMAs start from -mrow (negm), so
-  //          the accumulator already holds s*c2 - mrow and p = exp2(acc): one VALU op per
-  //          score; mxn is relative to the mrow the tile was computed with.
+  // partial row sum lsum, and mxn = scaled row maximum of the half tile about to be consumed.
+  // Scores are raw dot products; p = exp2(s*c2 - mrow).
   float mrow[QT], lsum[QT], mxn[QT];
-  f32x16 negm[QT];
 #pragma unroll
   for (int j = 0; j < QT; ++j) {
-    mrow[j] = FOLD ? 0.f : -INFINITY;
+    mrow[j] = -INFINITY;
     lsum[j] = 0.f;
-    mxn[j] = FOLD ? 0.f : -INFINITY;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) negm[j][r] = 0.f;
+    mxn[j] = -INFINITY;
   }
   const float c2 = p.scale_log2;
   const int ntiles = (L + kBN - 1) / kBN;
@@ -252,7 +241,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       float mx = s[j][0];
 #pragma unroll
       for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[j][r]);
-      mxn[j] = FOLD ? pair_max(mx) : pair_max(mx) * c2;
+      mxn[j] = pair_max(mx) * c2;
     }
   };
   // Lazy rescale: the running maximum only has to bound the scores well enough that exp2
@@ -262,33 +251,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   auto maybe_rescale = [&](f32x16 (&cur)[QT]) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < QT; ++j) {
-      if constexpr (FOLD) {
-        if (__builtin_amdgcn_ballot_w64(mxn[j] > kLazy) != 0) {
-          const float up = fmaxf(mxn[j], 0.f);  // rows below their maximum keep it
-          const float alpha = __builtin_amdgcn_exp2f(-up);
-          mrow[j] += up;
-          lsum[j] *= alpha;
+      if (__builtin_amdgcn_ballot_w64(mxn[j] > mrow[j] + kLazy) != 0) {
+        const float mnew = fmaxf(mrow[j], mxn[j]);
+        const float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);
+        mrow[j] = mnew;
+        lsum[j] *= alpha;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            cur[j][r] -= up;  // these scores were computed against the old maximum
-            negm[j][r] = -mrow[j];
-          }
+        for (int t = 0; t < D / 32; ++t)
 #pragma unroll
-          for (int t = 0; t < D / 32; ++t)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o[t][j][r] *= alpha;
-        }
-      } else {
-        if (__builtin_amdgcn_ballot_w64(mxn[j] > mrow[j] + kLazy) != 0) {
-          const float mnew = fmaxf(mrow[j], mxn[j]);
-          const float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);
-          mrow[j] = mnew;
-          lsum[j] *= alpha;
-#pragma unroll
-          for (int t = 0; t < D / 32; ++t)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o[t][j][r] *= alpha;
-        }
+          for (int r = 0; r < 16; ++r) o[t][j][r] *= alpha;
       }
     }
   };
@@ -298,8 +269,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int j = 0; j < QT; ++j)
 #pragma unroll
       for (int e = 0; e < n; ++e)
-        s[j][r0 + e] = FOLD ? __builtin_amdgcn_exp2f(s[j][r0 + e])
-                            : __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r0 + e], c2, -mrow[j]));
+        s[j][r0 + e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][r0 + e], c2, -mrow[j]));
   };
   // ---- operand fragments read from LDS
   // B fragment of MFMA group st for rows 32i..32i+31 of the L tile at byte offset `off`
@@ -363,9 +333,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     if constexpr (INTER == kInterSoftmax) maybe_rescale(cur);
     V8 fr[NG];
     auto fetch = [&](int k) __attribute__((always_inline)) {
-#ifdef DITTO_X_NOLDS
-      if (k >= 2) { fr[k] = fr[k & 1]; return; }
-#endif
       // second contraction groups run N tile by N tile, two sixteen-row steps each
       fr[k] = k < NS ? b_frag(bs_next, hh ^ 1, k) : c_frag(cs_cur, 2 * hh + (k - NS) % 2, (k - NS) / 2);
     };
@@ -375,7 +342,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
     for (int k = 0; k < NG; ++k) {
       if (k + kAhead < NG) fetch(k + kAhead);
-#ifndef DITTO_X_NOLOAD
       if (hh == 0) {
         // the direct loads for two tiles ahead are spread over the groups of the first half
         // step (a burst of them would hold up the wave's single instruction stream)
@@ -386,14 +352,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           else load_c1(it + 1, (BI + 1) & 1, q - NLD);
         }
       }
-#endif
       __builtin_amdgcn_sched_barrier(0);
       if (k < NS) {
 #pragma unroll
         for (int j = 0; j < QT; ++j) {
           if (k == 0) {
             const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            nxt[j] = Elem<T>::mfma32(fr[k], af[j][k], FOLD ? negm[j] : z);
+            nxt[j] = Elem<T>::mfma32(fr[k], af[j][k], z);
           } else {
             nxt[j] = Elem<T>::mfma32(fr[k], af[j][k], nxt[j]);
           }
@@ -443,19 +408,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   if constexpr (INTER == kInterSoftmax) {
     if (ragged && ntiles == 1) mask_tail(sa, 0);
     row_max(sa);
-    if constexpr (FOLD) {
-      // start from the exact maximum of the first half (whatever its sign)
-#pragma unroll
-      for (int j = 0; j < QT; ++j) {
-        mrow[j] = mxn[j];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          sa[j][r] -= mxn[j];
-          negm[j][r] = -mxn[j];
-        }
-        mxn[j] = 0.f;
-      }
-    }
   }
 
   // One L tile: loads two tiles ahead (B(it+2) replaces B(it-2), C(it+1) replaces C(it-1); both
@@ -465,10 +417,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     constexpr int BI = decltype(bi_c)::value;
     half_step(sa, sb, it, bi_c, IntC<0>{});
     half_step(sb, sa, it, bi_c, IntC<1>{});
-#ifndef DITTO_X_NOBAR
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-#endif
   };
   for (int it = 0; it < ntiles; it += 4) {
     tile_step(it, IntC<0>{});
@@ -509,10 +459,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 }
 
 // Host-side launcher for one instantiation.
-template <typename T, int D, int QT, int INTER, bool B_KL, bool FOLD>
+template <typename T, int D, int QT, int INTER, bool B_KL>
 hipError_t launch_bmm_chain(const BmmChainArgs& args, hipStream_t stream) {
   constexpr int lds = bmm_chain_lds_bytes<D>();
-  auto kern = bmm_chain_kernel<T, D, QT, INTER, B_KL, FOLD>;
+  auto kern = bmm_chain_kernel<T, D, QT, INTER, B_KL>;
   static thread_local int configured_dev = -1;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);

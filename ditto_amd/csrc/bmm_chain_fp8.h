@@ -1,0 +1,404 @@
+// Eight-wave variant of the fused two-contraction chain (see bmm_chain_fp.h for the chain,
+// the transposed formulation and the operand layouts).
+//
+// A wave of the four-wave kernel issues one instruction stream per SIMD: while an MFMA
+// occupies its issue slot nothing else of that wave can issue, so at most two or three VALU
+// instructions hide under each MFMA and the softmax (about four per MFMA) does not.  Here a
+// workgroup has EIGHT waves, two per SIMD, each owning 32 rows of A with at most 256
+// registers: the hardware interleaves the two instruction streams, so one wave's
+// exponentials run under the other wave's MFMAs without any software pipelining.
+//
+// The price is LDS traffic: with 32 rows per wave every operand fragment read from LDS feeds
+// a single MFMA.  16-byte row reads sustain that (256 B/clk per CU), the transposing read
+// ds_read_b64_tr_b16 (about 100 B/clk) does not.  So every tile whose contraction index is
+// the row index (C always, B in [K][L] layout) is transposed ONCE per workgroup: the wave
+// that owns a fragment reads it with the transposing read and writes it back "fragment
+// major" (1 KB per fragment, lane l at byte 16*l), after which all eight waves fetch it with
+// plain, conflict-free 16-byte reads.
+//
+// Pipeline per L tile `it` (one barrier per tile):
+//   direct loads   B(it+2) (row-read layout) or B(it+3) (raw, [K][L] layout), C(it+2) (raw)
+//   transposition  raw C(it+1) -> fragment-major C(it+1); raw B(it+2) -> fragment-major B(it+2)
+//   compute        waves 0-3: S(it) = B(it)^T.A^T, inter op, F^T += C(it)^T.P(it)^T
+//                  waves 4-7: inter op on S(it), F^T += C(it)^T.P(it)^T, S(it+1)
+#pragma once
+#include "bmm_chain_fp.h"
+
+namespace ditto {
+
+template <int D, bool B_KL>
+__host__ __device__ constexpr int bmm_chain8_lds_bytes() {
+  return ((B_KL ? 6 : 4) + 4) * kBN * D * 2;
+}
+
+template <typename T, int D, int INTER, bool B_KL>
+__global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef typename Elem<T>::v8 V8;
+  typedef typename Elem<T>::v4 V4;
+  typedef typename Elem<T>::v2 V2;
+  constexpr int NW = 8, BM = NW * 32;
+  constexpr int TB = kBN * D * 2;               // bytes per tile
+  constexpr int B_RB = B_KL ? kBN * 2 : D * 2;  // bytes per LDS row of a B tile as loaded
+  constexpr int B_CPR = B_RB / 16;
+  constexpr int C_RB = D * 2;
+  constexpr int C_CPR = C_RB / 16;
+  constexpr int NS = D / 16;                    // MFMA k steps of the first contraction per 32 rows
+  constexpr int NT = D / 32;                    // column tiles of the second contraction
+  constexpr int NFRAG = 2 * NS;                 // fragments per tile (B and C alike)
+  constexpr int NLD = TB / 1024 / NW;           // direct loads per wave per tile
+  constexpr int NTR = NFRAG / NW;               // fragments each wave transposes per tile
+  static_assert(NLD >= 1 && NTR >= 1, "tile too small for eight waves");
+  // LDS map (bytes): B tiles, then raw C tiles, then fragment-major C tiles
+  constexpr int B_LOAD = 0;                             // as loaded: [4] row-read layout, or [2] raw
+  constexpr int B_FRAG = 2 * TB;                        // [4] fragment major (B_KL only)
+  constexpr int C_RAW = (B_KL ? 6 : 4) * TB;            // [2]
+  constexpr int C_FRAG = C_RAW + 2 * TB;                // [2]
+  constexpr int B_USE = B_KL ? B_FRAG : B_LOAD;         // the four buffers the first contraction reads
+
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 31, g = lane >> 5;
+  const int i16 = lane & 15, h = (lane >> 4) & 1;
+  // The two waves of a SIMD (w and w+4) run half a tile apart: the "late" wave computes the
+  // scores of tile it+1 at the END of step it, so its softmax of step it+1 runs while the
+  // other wave's MFMAs occupy the matrix pipe, and vice versa.
+  const bool late = wave >= 4;
+
+  const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int mb = lid % p.mblocks;
+  const int bz = lid / p.mblocks;
+  const T* __restrict__ Ag = reinterpret_cast<const T*>(p.a) + (long long)bz * p.a_bs;
+  const T* Bg = reinterpret_cast<const T*>(p.b) + (long long)bz * p.b_bs;
+  const T* Cg = reinterpret_cast<const T*>(p.c) + (long long)bz * p.c_bs;
+  const int m_wave = mb * BM + wave * 32;
+  const int M = p.M, N = p.N, K = p.K, L = p.L;
+
+  const unsigned b_bytes = (unsigned)(B_KL ? ((long long)(K - 1) * p.b_rs + L) : ((long long)(L - 1) * p.b_rs + K)) * 2u;
+  const unsigned c_bytes = (unsigned)((long long)(L - 1) * p.c_rs + N) * 2u;
+  const i32x4 b_rsrc = make_rsrc(Bg, b_bytes);
+  const i32x4 c_rsrc = make_rsrc(Cg, c_bytes);
+  const unsigned lds0 = (unsigned)(size_t)(DITTO_LDS char*)smem_raw;
+
+  // ---- per-lane source offsets of the direct loads (same swizzles as the four-wave kernel)
+  int b_voff[NLD], c_voff[NLD], b_col[NLD];
+#pragma unroll
+  for (int q = 0; q < NLD; ++q) {
+    const int gi = NLD * wave + q;
+    {
+      const int row = gi * (64 / B_CPR) + lane / B_CPR, pc = lane % B_CPR;
+      if (B_KL) {
+        const int cl = pc ^ swz_trread<B_CPR>(row);
+        b_col[q] = cl * 8;
+        b_voff[q] = row < K ? (row * p.b_rs + cl * 8) * 2 : (int)b_bytes;
+      } else {
+        const int cl = pc ^ swz_rowread<B_CPR>(row);
+        b_col[q] = 0;
+        b_voff[q] = cl * 8 < K ? (row * p.b_rs + cl * 8) * 2 : (int)b_bytes;
+      }
+    }
+    {
+      const int row = gi * (64 / C_CPR) + lane / C_CPR, pc = lane % C_CPR;
+      const int cl = pc ^ swz_trread<C_CPR>(row);
+      c_voff[q] = cl * 8 < N ? (row * p.c_rs + cl * 8) * 2 : (int)c_bytes;
+    }
+  }
+  auto load_b = [&](int tile, int buf) __attribute__((always_inline)) {
+    const int l0 = tile * kBN;
+    const int soff = B_KL ? l0 * 2 : l0 * p.b_rs * 2;
+#pragma unroll
+    for (int q = 0; q < NLD; ++q) {
+      int vo = b_voff[q] + soff;
+      if (B_KL) vo = (l0 + b_col[q] < L) ? vo : (int)b_bytes;
+      lds_dma_16(b_rsrc, (unsigned)vo, lds0 + B_LOAD + buf * TB + 1024 * (NLD * wave + q));
+    }
+  };
+  auto load_c = [&](int tile, int buf) __attribute__((always_inline)) {
+    const int soff = tile * kBN * p.c_rs * 2;
+#pragma unroll
+    for (int q = 0; q < NLD; ++q)
+      lds_dma_16(c_rsrc, (unsigned)(c_voff[q] + soff), lds0 + C_RAW + buf * TB + 1024 * (NLD * wave + q));
+  };
+
+  // ---- per-lane LDS read addresses (bytes within a tile), loop invariant
+  const int b_rd = B_KL ? ((8 * g + (i16 >> 2)) * B_RB + (2 * h + ((i16 & 3) >> 1)) * 16 + 8 * (i16 & 1))
+                        : (ln * B_RB);
+  const int c_rd = (4 * g + (i16 >> 2)) * C_RB + (2 * h + ((i16 & 3) >> 1)) * 16 + 8 * (i16 & 1);
+  int b_ad[2][NS], c_ad[NT];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int x = B_KL ? swz_trread<B_CPR>(i16 >> 2) : (g ^ swz_rowread<B_CPR>(32 * i + ln));
+#pragma unroll
+    for (int st = 0; st < NS; ++st) b_ad[i][st] = b_rd + (B_KL ? ((4 * i) ^ x) : ((2 * st) ^ x)) * 16;
+  }
+#pragma unroll
+  for (int t = 0; t < NT; ++t) c_ad[t] = c_rd + ((4 * t) ^ swz_trread<C_CPR>(i16 >> 2)) * 16;
+  const int frag_ad = lane * 16;
+
+  // a row-read B fragment (plain 16-byte read) and a fragment-major fragment
+  auto b_frag_row = [&](int off, int i, int st) __attribute__((always_inline)) -> V8 {
+    return *reinterpret_cast<const V8*>(smem_raw + b_ad[i][st] + (off + 32 * i * B_RB));
+  };
+  auto frag_rd = [&](int off, int f) __attribute__((always_inline)) -> V8 {
+    return *reinterpret_cast<const V8*>(smem_raw + frag_ad + (off + 1024 * f));
+  };
+  // This wave's share of the transposition of one tile: fragments NTR*wave .. +NTR-1
+  // (C fragment f = u*NT + t: rows 16u.., columns 32t..; B fragment f = i*NS + st: rows 16st..,
+  // columns 32i..).  The per-lane source addresses are wave dependent, computed once.
+  int ctr_ad[NTR], btr_ad[NTR], fw_ad[NTR];
+#pragma unroll
+  for (int q = 0; q < NTR; ++q) {
+    const int f = NTR * wave + q;
+    ctr_ad[q] = c_rd + ((4 * (f % NT)) ^ swz_trread<C_CPR>(i16 >> 2)) * 16 + 16 * (f / NT) * C_RB;
+    btr_ad[q] = B_KL ? b_rd + ((4 * (f / NS)) ^ swz_trread<B_CPR>(i16 >> 2)) * 16 + 16 * (f % NS) * B_RB : 0;
+    fw_ad[q] = frag_ad + 1024 * f;
+  }
+  auto tr_read_c = [&](int raw_off, V8* x) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q = 0; q < NTR; ++q) {
+      const char* a = smem_raw + ctr_ad[q] + raw_off;
+      V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(a));
+      V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(a + 8 * C_RB));
+      x[q] = concat4<V4, V8>(lo, hi);
+    }
+  };
+  auto tr_read_b = [&](int raw_off, V8* x) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q = 0; q < NTR; ++q) {
+      const char* a = smem_raw + btr_ad[q] + raw_off;
+      V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(a));
+      V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(a + 4 * B_RB));
+      x[q] = concat4<V4, V8>(lo, hi);
+    }
+  };
+  auto tr_write = [&](int frag_off, const V8* x) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q = 0; q < NTR; ++q) *reinterpret_cast<V8*>(smem_raw + fw_ad[q] + frag_off) = x[q];
+  };
+
+  // ---- A fragments (B operand of D^T = B^T.A^T): lane holds A[row][16s + 8g .. +7]
+  V8 af[NS];
+  {
+    const int row = m_wave + ln;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const int col = 16 * s + 8 * g;
+      V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (row < M && col < K) v = *reinterpret_cast<const V8*>(Ag + (long long)row * p.a_rs + col);
+      af[s] = v;
+    }
+  }
+
+  // ---- accumulators of F^T: o[t][r] = F^T[32t + 8(r/4) + 4g + r%4][ln]
+  f32x16 o[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
+  float mrow = -INFINITY, lsum = 0.f;
+  const float c2 = p.scale_log2;
+  const int ntiles = (L + kBN - 1) / kBN;
+  const bool ragged = (L % kBN) != 0;
+
+  // Operand fragments are fetched kAhead MFMAs ahead of their use; the scheduling barriers keep
+  // the compiler from collapsing the prefetch distance (it otherwise reuses one register set
+  // and waits for every fragment).
+  constexpr int kAhead = 4;
+  f32x16 s[2];
+  // first contraction, transposed: s[i] = (B^T rows 32i..32i+31) . A^T; MFMA k = 2*st + i
+  auto scores = [&](auto off_c) __attribute__((always_inline)) {
+    constexpr int OFF = decltype(off_c)::value;
+    auto rd = [&](int k) __attribute__((always_inline)) -> V8 {
+      return B_KL ? frag_rd(OFF, (k & 1) * NS + (k >> 1)) : b_frag_row(OFF, k & 1, k >> 1);
+    };
+    V8 fr[2 * NS];
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) fr[k] = rd(k);
+#pragma unroll
+    for (int k = 0; k < 2 * NS; ++k) {
+      if (k + kAhead < 2 * NS) fr[k + kAhead] = rd(k + kAhead);
+      __builtin_amdgcn_sched_barrier(0);
+      if (k < 2) {
+        const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        s[k & 1] = Elem<T>::mfma32(fr[k], af[k >> 1], z);
+      } else {
+        s[k & 1] = Elem<T>::mfma32(fr[k], af[k >> 1], s[k & 1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // One L tile.  J = it % 4 selects the buffers of tile it (compile time).
+  auto tile_step = [&](int it, auto j_c) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value;
+    constexpr int PAR = J & 1;
+    constexpr int CF = C_FRAG + PAR * TB;
+    // loads ahead (tiles past the end are out of range and load zeros); transposition reads
+    V8 xb[NTR], xc[NTR];
+    if (B_KL) {
+      load_b(it + 3, PAR ^ 1);
+    } else {
+      load_b(it + 2, (J + 2) % 4);
+    }
+    load_c(it + 2, PAR);
+    if (B_KL) tr_read_b(B_LOAD + PAR * TB, xb);
+    tr_read_c(C_RAW + (PAR ^ 1) * TB, xc);
+
+    if (!late) scores(IntC<B_USE + J * TB>{});
+
+    // transposition writes; first fragments of the second contraction
+    if (B_KL) tr_write(B_FRAG + ((J + 2) % 4) * TB, xb);
+    tr_write(C_FRAG + (PAR ^ 1) * TB, xc);
+    V8 fr[4 * NT];
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) fr[k] = frag_rd(CF, k);
+    __builtin_amdgcn_sched_barrier(0);
+
+    if constexpr (INTER == kInterSoftmax) {
+      if (ragged && it == ntiles - 1) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int l = it * kBN + 32 * i + 8 * (r >> 2) + 4 * g + (r & 3);
+            if (l >= L) s[i][r] = -INFINITY;
+          }
+      }
+      float mx = s[0][0];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[i][r]);
+      mx = pair_max(mx) * c2;
+      // lazy rescale: raise the running maximum only when a row of the wave exceeds it by 2^kLazy
+      if (__builtin_amdgcn_ballot_w64(mx > mrow + kLazy) != 0) {
+        const float mnew = fmaxf(mrow, mx);
+        const float alpha = __builtin_amdgcn_exp2f(mrow - mnew);
+        mrow = mnew;
+        lsum *= alpha;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[i][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i][r], c2, -mrow));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // second contraction: o[t] += (C^T tile t, rows 16u..16u+15) . (P^T); half-wave g supplies
+    // rows 16u + 4g + {0..3} and 16u + 8 + 4g + {0..3}: registers 8(u%2)..+7 of s[u/2].
+    // MFMA k = u*NT + t.
+    V8 pf;
+#pragma unroll
+    for (int k = 0; k < 4 * NT; ++k) {
+      const int u = k / NT, t = k % NT;
+      if (k + kAhead < 4 * NT) fr[k + kAhead] = frag_rd(CF, k + kAhead);
+      if (t == 0) {
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          v[e] = s[u >> 1][8 * (u & 1) + e];
+          if (INTER != kInterSoftmax && p.relu) v[e] = fmaxf(v[e], 0.f);
+        }
+        V2 p0 = cvt2<T>(v[0], v[1]), p1 = cvt2<T>(v[2], v[3]), p2 = cvt2<T>(v[4], v[5]), p3 = cvt2<T>(v[6], v[7]);
+        if constexpr (INTER == kInterSoftmax) {
+          // row sum over the ROUNDED probabilities: exactly what enters the MFMA
+          lsum = Elem<T>::add_pair(p0, lsum);
+          lsum = Elem<T>::add_pair(p1, lsum);
+          lsum = Elem<T>::add_pair(p2, lsum);
+          lsum = Elem<T>::add_pair(p3, lsum);
+        }
+        pf = V8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      o[t] = Elem<T>::mfma32(fr[k], pf, o[t]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (late && it + 1 < ntiles) scores(IntC<B_USE + ((J + 1) % 4) * TB>{});
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
+
+  // ---- prologue: first tiles in flight, first transposition(s), the late waves' first scores
+  load_b(0, 0);
+  load_b(1, 1);
+  load_c(0, 0);
+  load_c(1, 1);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  {
+    V8 x[NTR];
+    tr_read_c(C_RAW, x);
+    tr_write(C_FRAG, x);
+    if (B_KL) {
+      tr_read_b(B_LOAD, x);
+      tr_write(B_FRAG, x);
+      tr_read_b(B_LOAD + TB, x);
+      tr_write(B_FRAG + TB, x);
+      __syncthreads();
+      load_b(2, 0);
+    }
+  }
+  if (late) scores(IntC<B_USE>{});
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  for (int it = 0; it < ntiles; it += 4) {
+    tile_step(it, IntC<0>{});
+    if (it + 1 < ntiles) tile_step(it + 1, IntC<1>{});
+    if (it + 2 < ntiles) tile_step(it + 2, IntC<2>{});
+    if (it + 3 < ntiles) tile_step(it + 3, IntC<3>{});
+  }
+
+  // ---- epilogue: normalise (softmax), cast, store 4 contiguous columns per lane
+  float inv = 1.f;
+  if constexpr (INTER == kInterSoftmax) inv = 1.f / pair_sum(lsum);
+  const int row = m_wave + ln;
+  if (row < M) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int n = 32 * t + 8 * q4 + 4 * g;
+        if (n >= N) continue;
+        const float v0 = o[t][4 * q4 + 0] * inv, v1 = o[t][4 * q4 + 1] * inv;
+        const float v2 = o[t][4 * q4 + 2] * inv, v3 = o[t][4 * q4 + 3] * inv;
+        const long long off = (long long)bz * p.f_bs + (long long)row * p.f_rs + n;
+        if (p.out_f32) {
+          f32x4 w = {v0, v1, v2, v3};
+          *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.f) + off) = w;
+        } else {
+          V2 a0 = cvt2<T>(v0, v1), a1 = cvt2<T>(v2, v3);
+          V4 w = {a0[0], a0[1], a1[0], a1[1]};
+          *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.f) + off) = w;
+        }
+      }
+  }
+#else
+  (void)p;
+#endif
+}
+
+template <typename T, int D, int INTER, bool B_KL>
+hipError_t launch_bmm_chain8(const BmmChainArgs& args, hipStream_t stream) {
+  constexpr int lds = bmm_chain8_lds_bytes<D, B_KL>();
+  auto kern = bmm_chain8_kernel<T, D, INTER, B_KL>;
+  static thread_local int configured_dev = -1;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (configured_dev != dev) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return e;
+    configured_dev = dev;
+  }
+  const unsigned grid = (unsigned)args.mblocks * (unsigned)args.batch;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, args);
+  return hipGetLastError();
+}
+
+}  // namespace ditto

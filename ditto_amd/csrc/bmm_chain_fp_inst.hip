@@ -1,26 +1,30 @@
-// Instantiates the fp16/bf16 chain kernel for one (element type, inter-op) pair.
+// Instantiates the fp16/bf16 chain kernels for one (element type, inter-op) pair.
 // Compiled once per pair with -DDITTO_INST_T=<f16|bf16> -DDITTO_INST_INTER=<0|2>
 // -DDITTO_INST_NAME=<symbol> so the variants build in parallel.
-#include "bmm_chain_fp.h"
+#include "bmm_chain_fp8.h"
 
 namespace ditto {
 
-hipError_t DITTO_INST_NAME(int d_pad, int qt, bool b_kl, bool fold, const BmmChainArgs& args, hipStream_t stream) {
+// q = 1 | 2: four-wave kernel, 32*q rows per wave; q = 8: eight-wave kernel
+hipError_t DITTO_INST_NAME(int d_pad, int q, bool b_kl, const BmmChainArgs& args, hipStream_t stream) {
   typedef DITTO_INST_T T;
   constexpr int I = DITTO_INST_INTER;
-#define DITTO_CASE(DP, Q)                                                          \
-  if (d_pad == DP && qt == Q) {                                                    \
-    if (I == kInterSoftmax && fold)                                                \
-      return b_kl ? launch_bmm_chain<T, DP, Q, I, true, I == kInterSoftmax>(args, stream)   \
-                  : launch_bmm_chain<T, DP, Q, I, false, I == kInterSoftmax>(args, stream); \
-    return b_kl ? launch_bmm_chain<T, DP, Q, I, true, false>(args, stream)         \
-                : launch_bmm_chain<T, DP, Q, I, false, false>(args, stream);       \
-  }
+#define DITTO_CASE(DP, Q)                                                  \
+  if (d_pad == DP && q == Q)                                               \
+    return b_kl ? launch_bmm_chain<T, DP, Q, I, true>(args, stream)        \
+                : launch_bmm_chain<T, DP, Q, I, false>(args, stream);
+#define DITTO_CASE8(DP)                                                    \
+  if (d_pad == DP && q == 8)                                               \
+    return b_kl ? launch_bmm_chain8<T, DP, I, true>(args, stream)          \
+                : launch_bmm_chain8<T, DP, I, false>(args, stream);
   DITTO_CASE(64, 1)
   DITTO_CASE(64, 2)
   DITTO_CASE(128, 1)
   DITTO_CASE(128, 2)
+  DITTO_CASE8(64)
+  DITTO_CASE8(128)
 #undef DITTO_CASE
+#undef DITTO_CASE8
   return hipErrorInvalidValue;
 }
 

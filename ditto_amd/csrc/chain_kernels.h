@@ -9,10 +9,10 @@
 namespace ditto {
 
 // bmm_chain_fp_inst.hip, one object per (element type, inter-op)
-hipError_t launch_f16_cast(int d_pad, int qt, bool b_kl, bool fold, const BmmChainArgs& args, hipStream_t stream);
-hipError_t launch_f16_softmax(int d_pad, int qt, bool b_kl, bool fold, const BmmChainArgs& args, hipStream_t stream);
-hipError_t launch_bf16_cast(int d_pad, int qt, bool b_kl, bool fold, const BmmChainArgs& args, hipStream_t stream);
-hipError_t launch_bf16_softmax(int d_pad, int qt, bool b_kl, bool fold, const BmmChainArgs& args, hipStream_t stream);
+hipError_t launch_f16_cast(int d_pad, int q, bool b_kl, const BmmChainArgs& args, hipStream_t stream);
+hipError_t launch_f16_softmax(int d_pad, int q, bool b_kl, const BmmChainArgs& args, hipStream_t stream);
+hipError_t launch_bf16_cast(int d_pad, int q, bool b_kl, const BmmChainArgs& args, hipStream_t stream);
+hipError_t launch_bf16_softmax(int d_pad, int q, bool b_kl, const BmmChainArgs& args, hipStream_t stream);
 
 // conv_chain_inst.hip, one object per element type; c1_tiles in {1, 2, 4, 8}
 hipError_t launch_conv_f16(int c1_tiles, const ConvChainArgs& args, hipStream_t stream);

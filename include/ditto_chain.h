@@ -84,6 +84,11 @@ typedef struct ditto_bmm_chain_desc {
   int64_t f_batch_stride, f_row_stride; /* F[b][m][n]                                  */
   float softmax_scale;   /* DITTO_INTER_SOFTMAX only; the reference uses 1.0           */
   float requant_scale;   /* DITTO_INTER_REQUANT: scale of every column when `aux` is NULL */
+  int32_t tile_variant;  /* 0: the library's per-shape table picks the kernel variant; else a
+                            `ditto_tile_param.variant` id to force (the counterpart of passing
+                            an explicit CUDATensorizeParam, hyper_fusion.cc:586-607);
+                            DITTO_EINVAL if that variant cannot run the shape              */
+  int32_t reserved;      /* must be 0 */
 } ditto_bmm_chain_desc;
 
 /*
@@ -114,7 +119,9 @@ typedef struct ditto_tile_param {
   int32_t head_pad;       /* K and N padded to this inside the kernel (0: n/a)   */
   int32_t lds_bytes;      /* dynamic LDS per workgroup                           */
   int32_t grid_x, grid_y, grid_z;
-  int32_t variant;        /* kernel variant id, for logs                         */
+  int32_t variant;        /* kernel variant id: fp16/bf16 chains head_pad*10 + q, with
+                             q = 1|2: four waves owning 32*q rows each, q = 8: eight
+                             waves owning 32 rows each; other chains: see api.hip  */
 } ditto_tile_param;
 
 /* ---- entry points ------------------------------------------------------- */

@@ -22,7 +22,14 @@ REL_L2 = 1e-3
 REL_L2_BF16_QUANT = 3e-3
 
 
-def run_chain(A, B, C, dtype, inter, scale=1.0, b_layout="KL", out_dtype=None):
+def variants(K, N):
+    """0 (the library's own choice) and every kernel variant that can run the head size:
+    four waves x 32 rows, four waves x 64 rows, eight waves x 32 rows."""
+    pad = 64 if max(K, N) <= 64 else 128
+    return [0] + [pad * 10 + q for q in (1, 2, 8)]
+
+
+def run_chain(A, B, C, dtype, inter, scale=1.0, b_layout="KL", out_dtype=None, variant=0):
     """A[b,M,K], B[b,K,L], C[b,L,N] fp32 numpy (rounded to dtype) -> F numpy fp32."""
     a, c = to_dev(A, dtype), to_dev(C, dtype)
     if b_layout == "LK":  # keep B^T contiguous and hand over the transposed view
@@ -31,7 +38,7 @@ def run_chain(A, B, C, dtype, inter, scale=1.0, b_layout="KL", out_dtype=None):
         b = to_dev(B, dtype)
     f = torch.full((A.shape[0], A.shape[1], C.shape[2]), float("nan"), device=a.device,
                    dtype=TORCH_DTYPES[out_dtype or dtype])
-    chain.run_bmm_chain(a, b, c, f, inter, scale)
+    chain.run_bmm_chain(a, b, c, f, inter, scale, tile_variant=variant)
     torch.cuda.synchronize()
     return f.float().cpu().numpy()
 
@@ -56,12 +63,13 @@ def test_softmax_chain_vs_oracle(oracle, shape, dtype, b_layout):
     scale = 1.0 / np.sqrt(K)
     A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, dtype, seed=100 + M)
     want = oracle.bmm_chain_f64(A, B, C, inter="softmax", scale=scale)
-    for out_dtype in (dtype, "float32"):
-        got = run_chain(A, B, C, dtype, "softmax", scale, b_layout, out_dtype)
-        assert np.isfinite(got).all()
-        mx, rel = errors(got, want)
-        assert mx <= MAX_ABS, (mx, rel)
-        assert rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (mx, rel)
+    for variant in variants(K, N):
+        for out_dtype in (dtype, "float32"):
+            got = run_chain(A, B, C, dtype, "softmax", scale, b_layout, out_dtype, variant)
+            assert np.isfinite(got).all(), variant
+            mx, rel = errors(got, want)
+            assert mx <= MAX_ABS, (variant, mx, rel)
+            assert rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (variant, mx, rel)
 
 
 CAST_SHAPES = [
@@ -82,18 +90,21 @@ def test_cast_chain_vs_oracle(oracle, shape, dtype, inter):
     A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, dtype, seed=200 + M, std=0.25)
     # the checker rounds the intermediate to in_dtype exactly where the chain does
     want32 = oracle.bmm_chain_f64(A, B, C, inter=inter, round_mid=dtype)
-    got32 = run_chain(A, B, C, dtype, inter, out_dtype="float32")
-    mx, rel = errors(got32, want32)
-    # fp32 accumulation order differs; a rounding flip of one intermediate moves the output by
-    # about one unit of the intermediate's last place
-    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
-    got = run_chain(A, B, C, dtype, inter)
     want = oracle.np_round_to(want32, dtype)
-    mx, rel = errors(got, want)
-    assert mx <= (MAX_ABS if dtype == "float16" else 4e-2), (mx, rel)  # one bf16 ulp at |x| ~ 4 is 3e-2
-    assert rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (mx, rel)
-    # and the narrow output is the rounding of the fp32 output (same kernel, cast at the end)
-    assert np.array_equal(got, oracle.np_round_to(got32, dtype))
+    for variant in variants(K, N):
+        for b_layout in ("KL", "LK"):
+            got32 = run_chain(A, B, C, dtype, inter, 1.0, b_layout, "float32", variant)
+            mx, rel = errors(got32, want32)
+            # fp32 accumulation order differs; a rounding flip of one intermediate moves the output
+            # by about one unit of the intermediate's last place
+            assert mx <= MAX_ABS and rel <= REL_L2, (variant, b_layout, mx, rel)
+            got = run_chain(A, B, C, dtype, inter, 1.0, b_layout, None, variant)
+            mx, rel = errors(got, want)
+            # one bf16 ulp at |x| ~ 4 is 3e-2
+            assert mx <= (MAX_ABS if dtype == "float16" else 4e-2), (variant, b_layout, mx, rel)
+            assert rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (variant, b_layout, mx, rel)
+            # and the narrow output is the rounding of the fp32 output (same kernel, cast at the end)
+            assert np.array_equal(got, oracle.np_round_to(got32, dtype)), (variant, b_layout)
 
 
 def test_fused_cpu_nest_agrees_with_gpu(oracle):
@@ -105,25 +116,26 @@ def test_fused_cpu_nest_agrees_with_gpu(oracle):
     assert mx <= MAX_ABS and rel <= REL_L2
 
 
-def test_softmax_invariants_on_gpu(oracle):
+@pytest.mark.parametrize("variant", [641, 642, 648])
+def test_softmax_invariants_on_gpu(oracle, variant):
     batch, M, N, K, L = 2, 160, 64, 64, 264
     A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, "float16", seed=9)
-    base = run_chain(A, B, C, "float16", "softmax", 0.125, "LK", "float32")
+    base = run_chain(A, B, C, "float16", "softmax", 0.125, "LK", "float32", variant)
     # V = ones -> O = ones: the normaliser matches the probabilities that were multiplied
-    ones = run_chain(A, B, np.ones_like(C), "float16", "softmax", 0.125, "LK", "float32")
+    ones = run_chain(A, B, np.ones_like(C), "float16", "softmax", 0.125, "LK", "float32", variant)
     assert np.abs(ones - 1.0).max() <= 2e-3
     # permuting keys and values together leaves O unchanged (up to accumulation order)
     perm = np.random.default_rng(0).permutation(L)
     got = run_chain(A, np.ascontiguousarray(B[:, :, perm]), np.ascontiguousarray(C[:, perm, :]), "float16",
-                    "softmax", 0.125, "LK", "float32")
+                    "softmax", 0.125, "LK", "float32", variant)
     assert errors(got, base)[1] <= 5e-4
     # Q = 0 -> O = column means of V
-    zero = run_chain(np.zeros_like(A), B, C, "float16", "softmax", 0.125, "KL", "float32")
+    zero = run_chain(np.zeros_like(A), B, C, "float16", "softmax", 0.125, "KL", "float32", variant)
     assert np.abs(zero - C.mean(axis=1, keepdims=True)).max() <= 1e-3
     # large scores do not overflow (the reference's exp-without-max form does)
     Ah = A.copy()
     Ah[:, :, 0] = 60.0
-    hot = run_chain(Ah, B, C, "float16", "softmax", 1.0, "LK", "float32")
+    hot = run_chain(Ah, B, C, "float16", "softmax", 1.0, "LK", "float32", variant)
     want = oracle.bmm_chain_f64(Ah, B, C, inter="softmax", scale=1.0)
     assert np.isfinite(hot).all() and errors(hot, want)[0] <= MAX_ABS
 
@@ -147,6 +159,72 @@ def test_reference_semantics_on_reference_inputs(oracle):
     assert 0.95 < ok.mean() < 1.0
     assert np.allclose(got[ok], emul[ok], rtol=0.1, atol=0.1)
     assert errors(got[ok], emul[ok])[0] <= 5e-3
+
+
+def test_attention_full_size_fp16_heads(oracle):
+    # the fp16 configuration at its full size: 96 heads of 512 x 64, scale 1/8, every row checked
+    batch, M, N, K, L = 96, 512, 64, 64, 512
+    A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, "float16", seed=21)
+    want = oracle.bmm_chain_f64(A, B, C, inter="softmax", scale=0.125)
+    for variant in variants(K, N):
+        got = run_chain(A, B, C, "float16", "softmax", 0.125, "LK", None, variant)
+        mx, rel = errors(got, want)
+        assert mx <= MAX_ABS and rel <= REL_L2, (variant, mx, rel)
+
+
+@pytest.mark.parametrize("variant", [0, 1282, 1288])
+def test_attention_full_size_bf16_long_sequence(oracle, variant):
+    # the bf16 configuration at its full size (64 heads of 4096 x 128).  The CPU closed form over
+    # all of it would take minutes, so: every row of three heads chosen across the batch, one
+    # row block of every head, and size-independent properties over the whole output.
+    batch, S, d = 64, 4096, 128
+    scale = d ** -0.5
+    dev = "cuda:0"
+    g = torch.Generator(device="cpu").manual_seed(33)
+    q = torch.randn(batch, S, d, generator=g).to(torch.bfloat16)
+    k = torch.randn(batch, S, d, generator=g).to(torch.bfloat16)
+    v = torch.randn(batch, S, d, generator=g).to(torch.bfloat16)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    out = torch.full((batch, S, d), float("nan"), device=dev, dtype=torch.bfloat16)
+    chain.run_bmm_chain(qd, kd.transpose(1, 2), vd, out, "softmax", scale, tile_variant=variant)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    qn, kn, vn = q.float().numpy(), k.float().numpy(), v.float().numpy()
+    for h in (0, 31, 63):  # whole heads
+        want = oracle.bmm_chain_f64(qn[h:h + 1], np.ascontiguousarray(kn[h:h + 1].transpose(0, 2, 1)), vn[h:h + 1],
+                                    inter="softmax", scale=scale)
+        mx, rel = errors(got[h:h + 1], want)
+        assert mx <= MAX_ABS and rel <= REL_L2_BF16_QUANT, (h, mx, rel)
+    rows = slice(1000, 1032)  # one row block of every head (straddles no tile boundary specially)
+    want = oracle.bmm_chain_f64(np.ascontiguousarray(qn[:, rows]), np.ascontiguousarray(kn.transpose(0, 2, 1)), vn,
+                                inter="softmax", scale=scale)
+    mx, rel = errors(got[:, rows], want)
+    assert mx <= MAX_ABS and rel <= REL_L2_BF16_QUANT, (mx, rel)
+    # values all ones -> output all ones (the normaliser is the sum of what was multiplied)
+    ones = torch.ones_like(vd)
+    chain.run_bmm_chain(qd, kd.transpose(1, 2), ones, out, "softmax", scale, tile_variant=variant)
+    torch.cuda.synchronize()
+    assert (out.float() - 1.0).abs().max().item() <= 8e-3  # one bf16 ulp below 1 is 3.9e-3
+    # convexity: every output lies within the column range of V of its head
+    chain.run_bmm_chain(qd, kd.transpose(1, 2), vd, out, "softmax", scale, tile_variant=variant)
+    torch.cuda.synchronize()
+    lo = vd.float().amin(dim=1, keepdim=True)
+    hi = vd.float().amax(dim=1, keepdim=True)
+    o32 = out.float()
+    assert bool(((o32 >= lo - 1e-2) & (o32 <= hi + 1e-2)).all())
+    # rows of Q permuted -> rows of the output permuted the same way.  Not bit for bit: the
+    # running maximum is raised for all rows of a wave at once, so a row's rescale history (and
+    # with it the last bit before rounding) depends on its neighbours; a few outputs move by
+    # one bf16 unit in the last place.
+    perm = torch.randperm(S, generator=g).to(dev)
+    out2 = torch.empty_like(out)
+    chain.run_bmm_chain(qd[:, perm].contiguous(), kd.transpose(1, 2), vd, out2, "softmax", scale, tile_variant=variant)
+    torch.cuda.synchronize()
+    a, b = out2.float(), out[:, perm].float()
+    assert float((a != b).float().mean()) <= 1e-2
+    assert float((a - b).norm() / b.norm()) <= 5e-4
+    assert bool(((a - b).abs() <= 2.0 ** -7 * b.abs() + 1e-6).all())
 
 
 def test_strided_views_and_errors():
