@@ -55,7 +55,7 @@ int device_cus() {
 
 struct BmmPlan {
   int family;  // 0: fp16/bf16 register-resident chain, 1: fp32 chain, 2: int8 requant chain
-  int d_pad, qt;
+  int d_pad, qt;  // fp chains: head pad and rows-per-wave code; int8 chain: row tiles and ring depth
   ditto_tile_param tile;
 };
 
@@ -169,20 +169,34 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
         d->f_row_stride > 0x7fffffff || d->K > 0x7fffffff / 2 || d->N > 0x7fffffff / 2)
       return fail(DITTO_EINVAL, "extent or row stride too large");
     const long long Lp = (d->L + 255) / 256 * 256;
-    const int lds = ditto::i8_chain_lds_bytes_host((int)Lp);
+    if ((d->M + 64) * d->a_row_stride >= 0x7fffffffLL || d->K * d->b_row_stride >= 0x7fffffffLL ||
+        Lp * d->c_row_stride >= 0x7fffffffLL)
+      return fail(DITTO_EUNSUPPORTED, "a batch entry of A, B or C exceeds 2 GiB");
+    // 64-row workgroups halve the weight traffic per row but need twice as many rows to fill the
+    // chip; the ring of staged chunks is as deep as LDS allows (four or three stages, else two)
+    const int cus = need_device ? device_cus() : 256;
+    int mt = ((d->M + 63) / 64) * d->batch >= 2LL * cus ? 2 : 1;
+    auto fits = [&](int m, int n) { return ditto::i8_chain_lds_bytes_host((int)Lp, m, n) <= 160 * 1024; };
+    int nst = mt == 2 ? 3 : 4;
+    if (!fits(mt, nst)) nst = 2;
+    if (!fits(mt, nst)) mt = 1, nst = 4;
+    if (!fits(mt, nst)) nst = 2;
+    const int lds = ditto::i8_chain_lds_bytes_host((int)Lp, mt, nst);
     if (lds > 160 * 1024)
       return fail(DITTO_EUNSUPPORTED, "L=%lld: the requantised row block does not fit in LDS", (long long)d->L);
     plan->family = 2;
+    plan->d_pad = mt;
+    plan->qt = nst;
     ditto_tile_param& t = plan->tile;
-    t.block_threads = 256;
-    t.block_m = 64;
+    t.block_threads = 512;
+    t.block_m = 32 * mt;
     t.block_l = (int)Lp;
     t.block_n = 256;
     t.head_pad = 0;
     t.lds_bytes = lds;
-    t.grid_x = (int)(((d->M + 63) / 64) * d->batch);
+    t.grid_x = (int)(((d->M + 32 * mt - 1) / (32 * mt)) * d->batch);
     t.grid_y = t.grid_z = 1;
-    t.variant = 8064;
+    t.variant = 8000 + 10 * mt + nst;  // int8 chain: 8000 + 10 * (row tiles of 32) + ring depth
     return DITTO_OK;
   }
   return fail(DITTO_EUNSUPPORTED, "no chain kernel for in_dtype %d", in);
@@ -358,9 +372,9 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     args.K = (int)d->K;
     args.L = (int)d->L;
     args.batch = (int)d->batch;
-    args.mblocks = (int)((d->M + 63) / 64);
+    args.mblocks = (int)((d->M + plan.tile.block_m - 1) / plan.tile.block_m);
     args.Lp = plan.tile.block_l;
-    hipError_t e = ditto::launch_gemm_chain_i8(args, st);
+    hipError_t e = ditto::launch_gemm_chain_i8(args, plan.d_pad, plan.qt, st);
     if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
     return DITTO_OK;
   }

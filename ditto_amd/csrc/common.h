@@ -134,6 +134,16 @@ __device__ __forceinline__ i32x4 make_rsrc(const void* base, unsigned bytes) {
   return r;
 }
 
+// Same, for a base/extent computed inside a loop: the compiler's divergence analysis can lose
+// track of their uniformity, and a descriptor must live in SGPRs.
+__device__ __forceinline__ i32x4 make_rsrc_uniform(const void* base, unsigned bytes) {
+  const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+  i32x4 r = {__builtin_amdgcn_readfirstlane((int)(unsigned)a),
+             __builtin_amdgcn_readfirstlane((int)(unsigned)((a >> 32) & 0xffff)),
+             __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
+  return r;
+}
+
 // Workgroups are dealt round-robin to the 8 XCDs (each with a private L2) by
 // linear id.  Remap so that ids that are neighbours in the logical order (and
 // share operands) land on the same XCD.

@@ -19,8 +19,9 @@ struct I8ChainArgs {
   int Lp;  // L rounded up to the weight-chunk width
 };
 
-// dynamic LDS bytes of the kernel for a given padded L
-int i8_chain_lds_bytes_host(int Lp);
-hipError_t launch_gemm_chain_i8(const I8ChainArgs& args, hipStream_t stream);
+// dynamic LDS bytes of the kernel for a padded L, mt = 1|2 row tiles of 32 per workgroup and a
+// ring of nst = 2..4 staged chunks
+int i8_chain_lds_bytes_host(int Lp, int mt, int nst);
+hipError_t launch_gemm_chain_i8(const I8ChainArgs& args, int mt, int nst, hipStream_t stream);
 
 }  // namespace ditto

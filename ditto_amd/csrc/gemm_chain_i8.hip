@@ -7,30 +7,46 @@
 // the requantise, which is one fp32 multiply and one round-to-nearest-even: results are
 // bit-identical to the CPU checker.
 //
-// A workgroup of 4 waves owns 64 rows of A.  Phase 1 computes the middle result TRANSPOSED
+// A workgroup owns 32*MT rows of A and has two kinds of waves: four compute waves (one per
+// SIMD) and four loader waves that do nothing but issue the global -> LDS loads and wait for
+// them.  A wave that issues a load while the CU's load queue is full stalls until there is
+// room, and the loads of a chunk take about as long as its MFMAs; kept in a wave of their own,
+// these stalls never hold up a compute wave.  Phase 1 computes the middle result TRANSPOSED
 // (mid^T = B^T.A^T) with v_mfma_i32_32x32x32_i8 so that each lane ends up with 4 consecutive
-// l for one row m, requantises in registers and writes the int8 row block mid[64][L] to LDS
+// l for one row m, requantises in registers and writes the int8 row block mid[rows][L] to LDS
 // (it never goes to HBM).  Phase 2 walks N in chunks of 256 and multiplies the LDS-resident
 // mid by D.  B and D are row-major with the contraction index as the ROW index, the opposite
 // of what an MFMA operand wants (16 consecutive k per lane); they are staged row-major in LDS
 // and read with the transposing LDS read ds_read_b64_tr_b8.
+//
+// The whole kernel is one stream of staged chunks: (128 rows of B x 256 columns, plus the
+// matching 128 columns of the A rows) for phase 1, then (128 rows of D x 256 columns) for
+// phase 2.  Every workgroup reads all of B and D, so the kernel is bound by how fast a CU
+// pulls them out of L2, not by the MFMA pipe: chunks go global -> LDS directly
+// (buffer_load ... lds, no staging registers) into a ring of NST stages, NST-1 chunks in
+// flight, one barrier per chunk (loader waves: wait for chunk c, barrier, issue chunk c+NST-1;
+// compute waves: barrier, consume chunk c).  Tiles are stored unpadded; 32-byte column groups (weights)
+// and 16-byte chunks (A) are XOR-swizzled by row on the global-address side so that the
+// transposing reads and the 16-byte row reads are bank-conflict free.
 #include "common.h"
 #include "gemm_chain_i8.h"
 
 namespace ditto {
 
 namespace i8 {
-constexpr int BM = 64;     // rows of A per workgroup
-constexpr int KC = 64;     // contraction chunk staged per step
-constexpr int WC = 256;    // width of a staged weight chunk (columns of B / D)
-constexpr int ASTR = 80;   // LDS row stride of the A tile: 64 + 16, conflict-free 16-byte row reads
-constexpr int WSTR = 288;  // LDS row stride of a weight tile: 8 rows x 32 B of a transpose read
-                           // fall into different banks when the stride is 32 mod 64 bytes
-constexpr int MIDPAD = 16;
+constexpr int KC = 128;          // contraction rows per staged chunk
+constexpr int NKS = KC / 32;     // MFMA contraction steps per chunk
+constexpr int NCW = 4;           // compute waves (one per SIMD), each owning 64 of a chunk's 256 columns
+constexpr int NLW = 4;           // loader waves
+constexpr int NW = NCW + NLW;
+constexpr int NWI = KC * 256 / 1024 / NLW;  // weight-chunk load instructions per loader wave
+constexpr int WC = 256;          // columns of a staged weight chunk (B / D)
+constexpr int WBYTES = KC * WC;  // weight chunk in LDS, row stride 256 bytes
+constexpr int MIDPAD = 16;       // row padding of the requantised block (conflict-free row reads)
 }  // namespace i8
 
-__host__ __device__ inline int i8_chain_lds_bytes(int Lp) {
-  return 2 * i8::BM * i8::ASTR + 2 * i8::KC * i8::WSTR + i8::BM * (Lp + i8::MIDPAD) + Lp * 4;
+__host__ __device__ inline int i8_chain_lds_bytes(int Lp, int mt, int nst) {
+  return nst * (i8::WBYTES + 32 * mt * i8::KC) + 32 * mt * (Lp + i8::MIDPAD) + Lp * 4;
 }
 
 // 8 k-rows x 16 columns of a row-major int8 LDS tile, transposed: lane i of each 16-lane
@@ -45,205 +61,293 @@ __device__ __forceinline__ int requant_i8(int acc, float s) {
   return (int)v;
 }
 
-__global__ __launch_bounds__(256) void gemm_chain_i8_kernel(I8ChainArgs p) {
+template <int MT, int NST>
+__global__ __launch_bounds__(512) void gemm_chain_i8_kernel(I8ChainArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
   using namespace i8;
-  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  int8_t* const As = reinterpret_cast<int8_t*>(smem_raw);  // [2][BM*ASTR]
-  int8_t* const Ws = As + 2 * BM * ASTR;                   // [2][KC*WSTR]
+  constexpr int BM = 32 * MT;
+  constexpr int ABYTES = BM * KC;
+  constexpr int STAGE = WBYTES + ABYTES;
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   const int MIDSTR = p.Lp + MIDPAD;
-  int8_t* const mid = Ws + 2 * KC * WSTR;                  // [BM][MIDSTR]
-  float* const sc = reinterpret_cast<float*>(mid + BM * MIDSTR);  // [Lp]
+  int8_t* const mid = reinterpret_cast<int8_t*>(smem_raw) + NST * STAGE;  // [BM][MIDSTR]
+  float* const sc = reinterpret_cast<float*>(mid + BM * MIDSTR);          // [Lp]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31, g = lane >> 5;
   const int i16 = lane & 15, h = (lane >> 4) & 1;
   const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
   const int mb = lid % p.mblocks, bz = lid / p.mblocks;
   const int m0 = mb * BM;
   const int M = p.M, N = p.N, K = p.K, L = p.L, Lp = p.Lp;
-  const int8_t* __restrict__ Ag = p.a + (long long)bz * p.a_bs;
-  const int8_t* __restrict__ Bg = p.b + (long long)bz * p.b_bs;
-  const int8_t* __restrict__ Dg = p.d + (long long)bz * p.d_bs;
+  const int8_t* Ag = p.a + (long long)bz * p.a_bs;
+  const int8_t* Bg = p.b + (long long)bz * p.b_bs;
+  const int8_t* Dg = p.d + (long long)bz * p.d_bs;
   int32_t* __restrict__ Eg = p.e + (long long)bz * p.e_bs;
+  const unsigned a_bytes = (unsigned)((long long)(M - 1) * p.a_rs + K);
+  const unsigned b_bytes = (unsigned)((long long)(K - 1) * p.b_rs + L);
+  const unsigned d_bytes = (unsigned)((long long)(L - 1) * p.d_rs + N);
+  const unsigned lds0 = (unsigned)(size_t)(DITTO_LDS char*)smem_raw;
 
-  for (int l = tid; l < Lp; l += 256) sc[l] = l < L ? (p.scale ? p.scale[l] : p.scale_uniform) : 0.f;
+  for (int l = tid; l < Lp; l += 64 * NW) sc[l] = l < L ? (p.scale ? p.scale[l] : p.scale_uniform) : 0.f;
 
-  // ---- staging helpers (global -> registers -> LDS), 16 bytes per access, zero filled
-  i32x4 areg, wreg[4];
-  auto load_a = [&](int k0) {
-    const int r = tid >> 2, c = (tid & 3) * 16;
-    i32x4 v = {0, 0, 0, 0};
-    if (m0 + r < M && k0 + c < K) v = *reinterpret_cast<const i32x4*>(Ag + (long long)(m0 + r) * p.a_rs + k0 + c);
-    areg = v;
-  };
-  auto store_a = [&](int buf) {
-    const int r = tid >> 2, c = (tid & 3) * 16;
-    *reinterpret_cast<i32x4*>(As + buf * BM * ASTR + r * ASTR + c) = areg;
-  };
-  // weight tile: rows r0..r0+63 (< rmax) and columns c0..c0+255 (< cmax) of W
-  auto load_w = [&](const int8_t* __restrict__ W, int rs, int r0, int rmax, int c0, int cmax) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int ch = tid + 256 * i;
-      const int r = ch >> 4, c = (ch & 15) * 16;
-      i32x4 v = {0, 0, 0, 0};
-      if (r0 + r < rmax && c0 + c < cmax) v = *reinterpret_cast<const i32x4*>(W + (long long)(r0 + r) * rs + c0 + c);
-      wreg[i] = v;
-    }
-  };
-  auto store_w = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int ch = tid + 256 * i;
-      const int r = ch >> 4, c = (ch & 15) * 16;
-      *reinterpret_cast<i32x4*>(Ws + buf * KC * WSTR + r * WSTR + c) = wreg[i];
-    }
-  };
-  // operand fragment of a weight tile for the 32-wide column tile `ct` of this wave and the
-  // 32-deep contraction step `ks`: lane (ln, g) receives W[32ks + 16g + 0..15][64*wave + 32ct + ln]
-  auto w_frag = [&](const int8_t* ws, int ks, int ct) -> i32x4 {
-    const int8_t* q = ws + (32 * ks + 16 * g + (i16 >> 1)) * WSTR + 64 * wave + 32 * ct + 16 * h + 8 * (i16 & 1);
-    const i32x2 lo = lds_read_tr8(q);
-    const i32x2 hi = lds_read_tr8(q + 8 * WSTR);
-    i32x4 r = {lo[0], lo[1], hi[0], hi[1]};
-    return r;
-  };
+  const int nk = (K + KC - 1) / KC;  // chunks per 256-column block of B
+  const int nl = Lp / KC;            // chunks per 256-column block of D
+  const int nlc = Lp / WC, nnc = (N + WC - 1) / WC;
+  const int NC1 = nlc * nk;
+  const int NC = NC1 + nnc * nl;
+  // All workgroups walk the same B and D.  Started together on the same chunk they would all hit
+  // the same few L2 channels at the same time, so each workgroup starts its walk at a different
+  // chunk: the contraction order and the column-block order are rotated by the workgroup index
+  // (integer accumulation is exact in any order).
+  const int rot_k = mb % nk, rot_lc = (mb / nk) % nlc;
+  const int rot_l = mb % nl, rot_nc = (mb / nl) % nnc;
+  auto rot = [](int i, int r, int n) __attribute__((always_inline)) { return i + r >= n ? i + r - n : i + r; };
 
-  // ================= phase 1: mid = requant(A.B), kept in LDS =================
-  for (int lc = 0; lc < Lp; lc += WC) {
-    i32x16 acc[2][2];
+  if (wave >= NCW) {
+    // ======================= loader waves =======================
+    // A weight chunk is 32 instructions of 1 KB (4 rows of 256 bytes each), eight per loader
+    // wave: lane l of instruction j fills LDS row R = 4j + l/16, physical 16-byte chunk l%16,
+    // which holds logical chunk 2*((l%16)/2 ^ (R&7)) + l%2 of that row.
+    // The per-lane byte offsets are relative to the chunk's first element; the chunk's position
+    // goes into the buffer descriptor (base advanced, range shortened by the same amount), so
+    // issuing a chunk costs scalar instructions only and rows past the end of the matrix still
+    // fall out of range and read as zero.  Columns past the end of a row are in range of the
+    // buffer (they alias the next row) and are masked per lane: only the last column block can
+    // have them, and it uses a second set of offsets whose masked lanes are out of range.
+    const int pw = wave - NCW;
+    constexpr unsigned kOut = 0x7fffffffu;
+    unsigned wv_b[NWI], wv_bm[NWI], wv_d[NWI], wv_dm[NWI];
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-      for (int b = 0; b < 2; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
-    const int nk = (K + KC - 1) / KC;
-    __syncthreads();  // previous users of the staging buffers are done
-    load_a(0);
-    load_w(Bg, p.b_rs, 0, K, lc, L);
-    store_a(0);
-    store_w(0);
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-      const int buf = kt & 1;
-      if (kt + 1 < nk) {
-        load_a((kt + 1) * KC);
-        load_w(Bg, p.b_rs, (kt + 1) * KC, K, lc, L);
-      }
-      const int8_t* as = As + buf * BM * ASTR;
-      const int8_t* ws = Ws + buf * KC * WSTR;
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        i32x4 af[2], bf[2];
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-          af[mt] = *reinterpret_cast<const i32x4*>(as + (32 * mt + ln) * ASTR + 32 * ks + 16 * g);
-#pragma unroll
-        for (int lt = 0; lt < 2; ++lt) bf[lt] = w_frag(ws, ks, lt);
-#pragma unroll
-        for (int lt = 0; lt < 2; ++lt)
-#pragma unroll
-          for (int mt = 0; mt < 2; ++mt)
-            acc[lt][mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[lt], af[mt], acc[lt][mt], 0, 0, 0);
-      }
-      if (kt + 1 < nk) {
-        store_a(buf ^ 1);
-        store_w(buf ^ 1);
-      }
-      __syncthreads();
+    for (int q = 0; q < NWI; ++q) {
+      const int R = 4 * (NWI * pw + q) + (lane >> 4), pc = lane & 15;
+      const int col = 16 * (2 * ((pc >> 1) ^ (R & 7)) + (pc & 1));
+      wv_b[q] = (unsigned)R * (unsigned)p.b_rs + col;
+      wv_d[q] = (unsigned)R * (unsigned)p.d_rs + col;
+      wv_bm[q] = col < L - (L - 1) / WC * WC ? wv_b[q] : kOut;
+      wv_dm[q] = col < N - (N - 1) / WC * WC ? wv_d[q] : kOut;
     }
-    // requantise: acc[lt][mt][r] = mid^T[l][m], l = lc + 64*wave + 32lt + 8(r/4) + 4g + r%4,
-    // m = 32mt + ln; 4 consecutive l pack into one dword of mid[m][l..l+3]
+    // A chunk: BM rows of 128 bytes, 8 rows per instruction, MT instructions per loader wave: lane
+    // l of instruction j fills row R = 8j + l/8, physical chunk l%8 = logical chunk (l%8) ^ ((R>>1)&7)
+    unsigned av[MT], av_m[MT];
 #pragma unroll
-    for (int lt = 0; lt < 2; ++lt)
+    for (int q = 0; q < MT; ++q) {
+      const int R = 8 * (MT * pw + q) + (lane >> 3);
+      const int col = 16 * ((lane & 7) ^ ((R >> 1) & 7));
+      av[q] = (unsigned)(m0 + R) * (unsigned)p.a_rs + col;  // rows >= M are out of range
+      av_m[q] = col < K - (K - 1) / KC * KC ? av[q] : kOut;
+    }
+    int i_n = 0, i_inner = 0, i_outer = 0, i_stage = 0;
+    auto issue = [&]() __attribute__((always_inline)) {
+      if (i_n >= NC) return;
+      const unsigned sbase = lds0 + i_stage * STAGE + 1024 * NWI * pw;
+      if (i_n < NC1) {
+        const int kb = rot(i_inner, rot_k, nk), cb = rot(i_outer, rot_lc, nlc);
+        const unsigned off = (unsigned)(kb * KC) * (unsigned)p.b_rs + cb * WC;
+        const i32x4 rs = make_rsrc_uniform(Bg + off, b_bytes - off);
+        const bool edge = cb * WC + WC > L;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int l = lc + 64 * wave + 32 * lt + 8 * q + 4 * g;
-        const f32x4 s4 = *reinterpret_cast<const f32x4*>(sc + l);
+        for (int q = 0; q < NWI; ++q) lds_dma_16(rs, edge ? wv_bm[q] : wv_b[q], sbase + 1024 * q);
+        const i32x4 ra = make_rsrc_uniform(Ag + kb * KC, a_bytes - kb * KC);
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-          const int b0 = requant_i8(acc[lt][mt][4 * q + 0], s4[0]);
-          const int b1 = requant_i8(acc[lt][mt][4 * q + 1], s4[1]);
-          const int b2 = requant_i8(acc[lt][mt][4 * q + 2], s4[2]);
-          const int b3 = requant_i8(acc[lt][mt][4 * q + 3], s4[3]);
-          const int packed = (b0 & 0xff) | ((b1 & 0xff) << 8) | ((b2 & 0xff) << 16) | ((unsigned)b3 << 24);
-          *reinterpret_cast<int*>(mid + (32 * mt + ln) * MIDSTR + l) = packed;
+        for (int q = 0; q < MT; ++q)
+          lds_dma_16(ra, kb * KC + KC > K ? av_m[q] : av[q], lds0 + i_stage * STAGE + WBYTES + 1024 * (MT * pw + q));
+      } else {
+        const int lb = rot(i_inner, rot_l, nl), cb = rot(i_outer, rot_nc, nnc);
+        const unsigned off = (unsigned)(lb * KC) * (unsigned)p.d_rs + cb * WC;
+        // row blocks past L (L is padded to a multiple of 256 here) lie entirely out of range
+        const i32x4 rs = make_rsrc_uniform(Dg + off, off < d_bytes ? d_bytes - off : 0u);
+        const bool edge = cb * WC + WC > N;
+#pragma unroll
+        for (int q = 0; q < NWI; ++q) lds_dma_16(rs, edge ? wv_dm[q] : wv_d[q], sbase + 1024 * q);
+      }
+      ++i_n;
+      i_stage = i_stage + 1 == NST ? 0 : i_stage + 1;
+      if (++i_inner == (i_n <= NC1 ? nk : nl)) {
+        i_inner = 0;
+        ++i_outer;
+      }
+      if (i_n == NC1) i_outer = 0, i_inner = 0;
+    };
+#pragma unroll
+    for (int i = 0; i < NST - 1; ++i) issue();
+    // Loads retire in issue order, so "at most n outstanding" means everything but the newest n
+    // is done; chunk c is followed by NST-2 newer chunks of at least NWI loads each.
+    constexpr int kNewer = NWI * (NST - 2);
+    for (int c = 0; c < NC; ++c) {
+      if (c + NST - 2 >= NC) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kNewer) : "memory");
+      }
+      __syncthreads();  // chunk c has landed; the compute waves are done with chunk c-1
+      issue();          // chunk c+NST-1 into the stage chunk c-1 occupied
+    }
+  } else {
+    // ======================= compute waves =======================
+    // weight fragment for the wave's 32-wide column tile ct and the 32-deep step ks: lane (ln, g)
+    // receives W[32ks + 16g + 0..15][64*wave + 32ct + ln]; two transposing reads of 8 rows each
+    int w_ad[2];
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+      w_ad[ct] = (16 * g + (i16 >> 1)) * WC + (((2 * wave + ct) ^ (i16 >> 1)) * 32) + 16 * h + 8 * (i16 & 1);
+    // A fragment: lane (ln, g) receives A[32mt + ln][32ks + 16g + 0..15]
+    int a_ad[NKS];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) a_ad[ks] = WBYTES + ln * KC + (((2 * ks + g) ^ ((ln >> 1) & 7)) * 16);
+    auto w_frag = [&](const char* st, int ks, int ct) __attribute__((always_inline)) -> i32x4 {
+      const int8_t* q = reinterpret_cast<const int8_t*>(st) + w_ad[ct] + 32 * ks * WC;
+      const i32x2 lo = lds_read_tr8(q);
+      const i32x2 hi = lds_read_tr8(q + 8 * WC);
+      i32x4 r = {lo[0], lo[1], hi[0], hi[1]};
+      return r;
+    };
+    i32x16 acc[2][MT];
+    auto zero_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < MT; ++b)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
+    };
+    zero_acc();
+
+    // ---------------- phase 1: mid = requant(A.B), kept in LDS ----------------
+    int c_stage = 0;
+    for (int ob = 0; ob < nlc; ++ob) {
+      for (int ib = 0; ib < nk; ++ib) {
+        __syncthreads();
+        const char* st = smem_raw + c_stage * STAGE;
+        c_stage = c_stage + 1 == NST ? 0 : c_stage + 1;
+        // all fragments of the chunk first (one LDS round trip), then the MFMAs
+        i32x4 af[NKS][MT], bf[NKS][2];
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) af[ks][mt] = *reinterpret_cast<const i32x4*>(st + a_ad[ks] + 32 * mt * KC);
+#pragma unroll
+          for (int lt = 0; lt < 2; ++lt) bf[ks][lt] = w_frag(st, ks, lt);
         }
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+          for (int lt = 0; lt < 2; ++lt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+              acc[lt][mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks][lt], af[ks][mt], acc[lt][mt], 0, 0, 0);
       }
-  }
-  __syncthreads();
+      // requantise: acc[lt][mt][r] = mid^T[l][m], l = lc + 64*wave + 32lt + 8(r/4) + 4g + r%4,
+      // m = 32mt + ln; 4 consecutive l pack into one dword of mid[m][l..l+3]
+      const int lc = rot(ob, rot_lc, nlc) * WC;
+#pragma unroll
+      for (int lt = 0; lt < 2; ++lt)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int l = lc + 64 * wave + 32 * lt + 8 * q + 4 * g;
+          const f32x4 s4 = *reinterpret_cast<const f32x4*>(sc + l);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const int b0 = requant_i8(acc[lt][mt][4 * q + 0], s4[0]);
+            const int b1 = requant_i8(acc[lt][mt][4 * q + 1], s4[1]);
+            const int b2 = requant_i8(acc[lt][mt][4 * q + 2], s4[2]);
+            const int b3 = requant_i8(acc[lt][mt][4 * q + 3], s4[3]);
+            const int packed = (b0 & 0xff) | ((b1 & 0xff) << 8) | ((b2 & 0xff) << 16) | ((unsigned)b3 << 24);
+            *reinterpret_cast<int*>(mid + (32 * mt + ln) * MIDSTR + l) = packed;
+          }
+        }
+      zero_acc();
+    }
 
-  // ================= phase 2: E = mid.D, N walked in chunks of 256 =================
-  const int nl = Lp / KC;
-  for (int nc = 0; nc < N; nc += WC) {
-    i32x16 acc[2][2];
+    // ---------------- phase 2: E = mid.D, N walked in chunks of 256 ----------------
+    // (the barrier of the first chunk below also publishes mid to all compute waves)
+    for (int ob = 0; ob < nnc; ++ob) {
+      for (int ib = 0; ib < nl; ++ib) {
+        __syncthreads();
+        const char* st = smem_raw + c_stage * STAGE;
+        c_stage = c_stage + 1 == NST ? 0 : c_stage + 1;
+        i32x4 af[NKS][MT], bf[NKS][2];
+        const int8_t* mrow = mid + ln * MIDSTR + rot(ib, rot_l, nl) * KC + 16 * g;
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+        for (int ks = 0; ks < NKS; ++ks) {
 #pragma unroll
-      for (int b = 0; b < 2; ++b)
+          for (int mt = 0; mt < MT; ++mt) af[ks][mt] = *reinterpret_cast<const i32x4*>(mrow + 32 * mt * MIDSTR + 32 * ks);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
-    load_w(Dg, p.d_rs, 0, L, nc, N);
-    store_w(0);
-    __syncthreads();
-    for (int lt = 0; lt < nl; ++lt) {
-      const int buf = lt & 1;
-      if (lt + 1 < nl) load_w(Dg, p.d_rs, (lt + 1) * KC, L, nc, N);
-      const int8_t* ws = Ws + buf * KC * WSTR;
+          for (int nt = 0; nt < 2; ++nt) bf[ks][nt] = w_frag(st, ks, nt);
+        }
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        i32x4 af[2], bf[2];
+        for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-          af[mt] = *reinterpret_cast<const i32x4*>(mid + (32 * mt + ln) * MIDSTR + lt * KC + 32 * ks + 16 * g);
+          for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) bf[nt] = w_frag(ws, ks, nt);
+            for (int mt = 0; mt < MT; ++mt)
+              acc[nt][mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks][mt], bf[ks][nt], acc[nt][mt], 0, 0, 0);
+      }
+      // acc[nt][mt][r] = E[m][n], m = m0 + 32mt + 8(r/4) + 4g + r%4, n = nc + 64*wave + 32nt + ln:
+      // the 32 lanes of a half-wave write 128 contiguous bytes of one output row
+      const int nc = rot(ob, rot_nc, nnc) * WC;
+      if (m0 + BM <= M && nc + WC <= N) {
+        // whole tile in range: the row of register r is a scalar offset, the lane part of the
+        // address is constant, so a store costs no address arithmetic
+        const int voff = (4 * g * p.e_rs + ln) * 4;
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-          for (int mt = 0; mt < 2; ++mt)
-            acc[nt][mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[mt], bf[nt], acc[nt][mt], 0, 0, 0);
-      }
-      if (lt + 1 < nl) store_w(buf ^ 1);
-      __syncthreads();
-    }
-    // acc[nt][mt][r] = E[m][n], m = m0 + 32mt + 8(r/4) + 4g + r%4, n = nc + 64*wave + 32nt + ln:
-    // the 32 lanes of a half-wave write 128 contiguous bytes of one output row
+          for (int mt = 0; mt < MT; ++mt) {
+            int32_t* tile = Eg + (long long)(m0 + 32 * mt) * p.e_rs + nc + 64 * wave + 32 * nt;
+            const __amdgpu_buffer_rsrc_t er = __builtin_amdgcn_make_buffer_rsrc(tile, 0, 0x7fffffff, 0x00020000);
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-      const int n = nc + 64 * wave + 32 * nt + ln;
-      if (n >= N) continue;
+            for (int r = 0; r < 16; ++r)
+              __builtin_amdgcn_raw_buffer_store_b32(acc[nt][mt][r], er, voff, (8 * (r >> 2) + (r & 3)) * p.e_rs * 4, 0);
+          }
+      } else {
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
+        for (int nt = 0; nt < 2; ++nt) {
+          const int n = nc + 64 * wave + 32 * nt + ln;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = m0 + 32 * mt + 8 * (r >> 2) + 4 * g + (r & 3);
-          if (m < M) Eg[(long long)m * p.e_rs + n] = acc[nt][mt][r];
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int m = m0 + 32 * mt + 8 * (r >> 2) + 4 * g + (r & 3);
+              if (n < N && m < M) Eg[(long long)m * p.e_rs + n] = acc[nt][mt][r];
+            }
         }
+      }
+      zero_acc();
     }
   }
+#else
+  (void)p;
+#endif
 }
 
-int i8_chain_lds_bytes_host(int Lp) { return i8_chain_lds_bytes(Lp); }
+int i8_chain_lds_bytes_host(int Lp, int mt, int nst) { return i8_chain_lds_bytes(Lp, mt, nst); }
 
-hipError_t launch_gemm_chain_i8(const I8ChainArgs& args, hipStream_t stream) {
-  const int lds = i8_chain_lds_bytes(args.Lp);
+template <int MT, int NST>
+static hipError_t launch_i8(const I8ChainArgs& args, hipStream_t stream) {
+  const int lds = i8_chain_lds_bytes(args.Lp, MT, NST);
+  auto kern = gemm_chain_i8_kernel<MT, NST>;
   static thread_local int configured_dev = -1;
-  static thread_local int configured_lds = 0;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
-  if (configured_dev != dev || configured_lds < lds) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_chain_i8_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (configured_dev != dev) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) return e;
     configured_dev = dev;
-    configured_lds = 160 * 1024;
   }
   const unsigned grid = (unsigned)args.mblocks * (unsigned)args.batch;
-  hipLaunchKernelGGL(gemm_chain_i8_kernel, dim3(grid), dim3(256), lds, stream, args);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * i8::NW), lds, stream, args);
   return hipGetLastError();
+}
+
+hipError_t launch_gemm_chain_i8(const I8ChainArgs& args, int mt, int nst, hipStream_t stream) {
+  if (mt == 1 && nst == 4) return launch_i8<1, 4>(args, stream);
+  if (mt == 1 && nst == 2) return launch_i8<1, 2>(args, stream);
+  if (mt == 2 && nst == 3) return launch_i8<2, 3>(args, stream);
+  if (mt == 2 && nst == 2) return launch_i8<2, 2>(args, stream);
+  return hipErrorInvalidValue;
 }
 
 }  // namespace ditto
