@@ -188,7 +188,7 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     plan->d_pad = mt;
     plan->qt = nst;
     ditto_tile_param& t = plan->tile;
-    t.block_threads = 512;
+    t.block_threads = ditto::i8_chain_threads();
     t.block_m = 32 * mt;
     t.block_l = (int)Lp;
     t.block_n = 256;

@@ -22,6 +22,8 @@ struct I8ChainArgs {
 // dynamic LDS bytes of the kernel for a padded L, mt = 1|2 row tiles of 32 per workgroup and a
 // ring of nst = 2..4 staged chunks
 int i8_chain_lds_bytes_host(int Lp, int mt, int nst);
+// threads per workgroup of the kernel
+int i8_chain_threads();
 hipError_t launch_gemm_chain_i8(const I8ChainArgs& args, int mt, int nst, hipStream_t stream);
 
 }  // namespace ditto

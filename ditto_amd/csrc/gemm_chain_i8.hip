@@ -7,7 +7,7 @@
 // the requantise, which is one fp32 multiply and one round-to-nearest-even: results are
 // bit-identical to the CPU checker.
 //
-// A workgroup owns 32*MT rows of A and has two kinds of waves: four compute waves (one per
+// A workgroup owns 32*MT rows of A and has two kinds of waves: eight compute waves (two per
 // SIMD) and four loader waves that do nothing but issue the global -> LDS loads and wait for
 // them.  A wave that issues a load while the CU's load queue is full stalls until there is
 // room, and the loads of a chunk take about as long as its MFMAs; kept in a wave of their own,
@@ -36,8 +36,12 @@ namespace ditto {
 namespace i8 {
 constexpr int KC = 128;          // contraction rows per staged chunk
 constexpr int NKS = KC / 32;     // MFMA contraction steps per chunk
-constexpr int NCW = 4;           // compute waves (one per SIMD), each owning 64 of a chunk's 256 columns
-constexpr int NLW = 4;           // loader waves
+constexpr int NCW = 8;             // compute waves, each owning 256/NCW of a chunk's 256 columns
+constexpr int CTW = 8 / NCW;       // 32-wide column tiles per compute wave
+constexpr int NLW = 4;             // loader waves
+// Output stores are write-through (sc0 sc1): the int32 result is most of the kernel's HBM
+// traffic, and left dirty in L2 it would all be written back after the last wave has finished.
+constexpr int kStoreAux = 17;
 constexpr int NW = NCW + NLW;
 constexpr int NWI = KC * 256 / 1024 / NLW;  // weight-chunk load instructions per loader wave
 constexpr int WC = 256;          // columns of a staged weight chunk (B / D)
@@ -62,7 +66,7 @@ __device__ __forceinline__ int requant_i8(int acc, float s) {
 }
 
 template <int MT, int NST>
-__global__ __launch_bounds__(512) void gemm_chain_i8_kernel(I8ChainArgs p) {
+__global__ __launch_bounds__(64 * i8::NW) void gemm_chain_i8_kernel(I8ChainArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   using namespace i8;
   constexpr int BM = 32 * MT;
@@ -89,8 +93,6 @@ __global__ __launch_bounds__(512) void gemm_chain_i8_kernel(I8ChainArgs p) {
   const unsigned b_bytes = (unsigned)((long long)(K - 1) * p.b_rs + L);
   const unsigned d_bytes = (unsigned)((long long)(L - 1) * p.d_rs + N);
   const unsigned lds0 = (unsigned)(size_t)(DITTO_LDS char*)smem_raw;
-
-  for (int l = tid; l < Lp; l += 64 * NW) sc[l] = l < L ? (p.scale ? p.scale[l] : p.scale_uniform) : 0.f;
 
   const int nk = (K + KC - 1) / KC;  // chunks per 256-column block of B
   const int nl = Lp / KC;            // chunks per 256-column block of D
@@ -128,12 +130,13 @@ __global__ __launch_bounds__(512) void gemm_chain_i8_kernel(I8ChainArgs p) {
       wv_bm[q] = col < L - (L - 1) / WC * WC ? wv_b[q] : kOut;
       wv_dm[q] = col < N - (N - 1) / WC * WC ? wv_d[q] : kOut;
     }
-    // A chunk: BM rows of 128 bytes, 8 rows per instruction, MT instructions per loader wave: lane
+    // A chunk: BM rows of 128 bytes, 8 rows per instruction, shared out over the loader waves: lane
     // l of instruction j fills row R = 8j + l/8, physical chunk l%8 = logical chunk (l%8) ^ ((R>>1)&7)
-    unsigned av[MT], av_m[MT];
+    constexpr int NAI = (4 * MT + NLW - 1) / NLW;  // A-chunk instructions per loader wave
+    unsigned av[NAI], av_m[NAI];
 #pragma unroll
-    for (int q = 0; q < MT; ++q) {
-      const int R = 8 * (MT * pw + q) + (lane >> 3);
+    for (int q = 0; q < NAI; ++q) {
+      const int R = 8 * (NAI * pw + q) + (lane >> 3);
       const int col = 16 * ((lane & 7) ^ ((R >> 1) & 7));
       av[q] = (unsigned)(m0 + R) * (unsigned)p.a_rs + col;  // rows >= M are out of range
       av_m[q] = col < K - (K - 1) / KC * KC ? av[q] : kOut;
@@ -151,8 +154,9 @@ __global__ __launch_bounds__(512) void gemm_chain_i8_kernel(I8ChainArgs p) {
         for (int q = 0; q < NWI; ++q) lds_dma_16(rs, edge ? wv_bm[q] : wv_b[q], sbase + 1024 * q);
         const i32x4 ra = make_rsrc_uniform(Ag + kb * KC, a_bytes - kb * KC);
 #pragma unroll
-        for (int q = 0; q < MT; ++q)
-          lds_dma_16(ra, kb * KC + KC > K ? av_m[q] : av[q], lds0 + i_stage * STAGE + WBYTES + 1024 * (MT * pw + q));
+        for (int q = 0; q < NAI; ++q)
+          if (NAI * pw + q < 4 * MT)
+            lds_dma_16(ra, kb * KC + KC > K ? av_m[q] : av[q], lds0 + i_stage * STAGE + WBYTES + 1024 * (NAI * pw + q));
       } else {
         const int lb = rot(i_inner, rot_l, nl), cb = rot(i_outer, rot_nc, nnc);
         const unsigned off = (unsigned)(lb * KC) * (unsigned)p.d_rs + cb * WC;
@@ -187,11 +191,11 @@ __global__ __launch_bounds__(512) void gemm_chain_i8_kernel(I8ChainArgs p) {
   } else {
     // ======================= compute waves =======================
     // weight fragment for the wave's 32-wide column tile ct and the 32-deep step ks: lane (ln, g)
-    // receives W[32ks + 16g + 0..15][64*wave + 32ct + ln]; two transposing reads of 8 rows each
-    int w_ad[2];
+    // receives W[32ks + 16g + 0..15][32(CTW*wave + ct) + ln]; two transposing reads of 8 rows each
+    int w_ad[CTW];
 #pragma unroll
-    for (int ct = 0; ct < 2; ++ct)
-      w_ad[ct] = (16 * g + (i16 >> 1)) * WC + (((2 * wave + ct) ^ (i16 >> 1)) * 32) + 16 * h + 8 * (i16 & 1);
+    for (int ct = 0; ct < CTW; ++ct)
+      w_ad[ct] = (16 * g + (i16 >> 1)) * WC + (((CTW * wave + ct) ^ (i16 >> 1)) * 32) + 16 * h + 8 * (i16 & 1);
     // A fragment: lane (ln, g) receives A[32mt + ln][32ks + 16g + 0..15]
     int a_ad[NKS];
 #pragma unroll
@@ -203,16 +207,18 @@ __global__ __launch_bounds__(512) void gemm_chain_i8_kernel(I8ChainArgs p) {
       i32x4 r = {lo[0], lo[1], hi[0], hi[1]};
       return r;
     };
-    i32x16 acc[2][MT];
+    i32x16 acc[CTW][MT];
     auto zero_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
-      for (int a = 0; a < 2; ++a)
+      for (int a = 0; a < CTW; ++a)
 #pragma unroll
         for (int b = 0; b < MT; ++b)
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
     };
     zero_acc();
+    // per-column scales (first needed after the first barriers)
+    for (int l = tid; l < Lp; l += 64 * NCW) sc[l] = l < L ? (p.scale ? p.scale[l] : p.scale_uniform) : 0.f;
 
     // ---------------- phase 1: mid = requant(A.B), kept in LDS ----------------
     int c_stage = 0;
@@ -222,30 +228,30 @@ __global__ __launch_bounds__(512) void gemm_chain_i8_kernel(I8ChainArgs p) {
         const char* st = smem_raw + c_stage * STAGE;
         c_stage = c_stage + 1 == NST ? 0 : c_stage + 1;
         // all fragments of the chunk first (one LDS round trip), then the MFMAs
-        i32x4 af[NKS][MT], bf[NKS][2];
+        i32x4 af[NKS][MT], bf[NKS][CTW];
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) af[ks][mt] = *reinterpret_cast<const i32x4*>(st + a_ad[ks] + 32 * mt * KC);
 #pragma unroll
-          for (int lt = 0; lt < 2; ++lt) bf[ks][lt] = w_frag(st, ks, lt);
+          for (int lt = 0; lt < CTW; ++lt) bf[ks][lt] = w_frag(st, ks, lt);
         }
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
-          for (int lt = 0; lt < 2; ++lt)
+          for (int lt = 0; lt < CTW; ++lt)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
               acc[lt][mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks][lt], af[ks][mt], acc[lt][mt], 0, 0, 0);
       }
-      // requantise: acc[lt][mt][r] = mid^T[l][m], l = lc + 64*wave + 32lt + 8(r/4) + 4g + r%4,
+      // requantise: acc[lt][mt][r] = mid^T[l][m], l = lc + 32(CTW*wave + lt) + 8(r/4) + 4g + r%4,
       // m = 32mt + ln; 4 consecutive l pack into one dword of mid[m][l..l+3]
       const int lc = rot(ob, rot_lc, nlc) * WC;
 #pragma unroll
-      for (int lt = 0; lt < 2; ++lt)
+      for (int lt = 0; lt < CTW; ++lt)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int l = lc + 64 * wave + 32 * lt + 8 * q + 4 * g;
+          const int l = lc + 32 * (CTW * wave + lt) + 8 * q + 4 * g;
           const f32x4 s4 = *reinterpret_cast<const f32x4*>(sc + l);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
@@ -267,24 +273,24 @@ __global__ __launch_bounds__(512) void gemm_chain_i8_kernel(I8ChainArgs p) {
         __syncthreads();
         const char* st = smem_raw + c_stage * STAGE;
         c_stage = c_stage + 1 == NST ? 0 : c_stage + 1;
-        i32x4 af[NKS][MT], bf[NKS][2];
+        i32x4 af[NKS][MT], bf[NKS][CTW];
         const int8_t* mrow = mid + ln * MIDSTR + rot(ib, rot_l, nl) * KC + 16 * g;
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) af[ks][mt] = *reinterpret_cast<const i32x4*>(mrow + 32 * mt * MIDSTR + 32 * ks);
 #pragma unroll
-          for (int nt = 0; nt < 2; ++nt) bf[ks][nt] = w_frag(st, ks, nt);
+          for (int nt = 0; nt < CTW; ++nt) bf[ks][nt] = w_frag(st, ks, nt);
         }
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
-          for (int nt = 0; nt < 2; ++nt)
+          for (int nt = 0; nt < CTW; ++nt)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
               acc[nt][mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks][mt], bf[ks][nt], acc[nt][mt], 0, 0, 0);
       }
-      // acc[nt][mt][r] = E[m][n], m = m0 + 32mt + 8(r/4) + 4g + r%4, n = nc + 64*wave + 32nt + ln:
+      // acc[nt][mt][r] = E[m][n], m = m0 + 32mt + 8(r/4) + 4g + r%4, n = nc + 32(CTW*wave + nt) + ln:
       // the 32 lanes of a half-wave write 128 contiguous bytes of one output row
       const int nc = rot(ob, rot_nc, nnc) * WC;
       if (m0 + BM <= M && nc + WC <= N) {
@@ -292,19 +298,19 @@ __global__ __launch_bounds__(512) void gemm_chain_i8_kernel(I8ChainArgs p) {
         // address is constant, so a store costs no address arithmetic
         const int voff = (4 * g * p.e_rs + ln) * 4;
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
+        for (int nt = 0; nt < CTW; ++nt)
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
-            int32_t* tile = Eg + (long long)(m0 + 32 * mt) * p.e_rs + nc + 64 * wave + 32 * nt;
+            int32_t* tile = Eg + (long long)(m0 + 32 * mt) * p.e_rs + nc + 32 * (CTW * wave + nt);
             const __amdgpu_buffer_rsrc_t er = __builtin_amdgcn_make_buffer_rsrc(tile, 0, 0x7fffffff, 0x00020000);
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-              __builtin_amdgcn_raw_buffer_store_b32(acc[nt][mt][r], er, voff, (8 * (r >> 2) + (r & 3)) * p.e_rs * 4, 0);
+              __builtin_amdgcn_raw_buffer_store_b32(acc[nt][mt][r], er, voff, (8 * (r >> 2) + (r & 3)) * p.e_rs * 4, kStoreAux);
           }
       } else {
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-          const int n = nc + 64 * wave + 32 * nt + ln;
+        for (int nt = 0; nt < CTW; ++nt) {
+          const int n = nc + 32 * (CTW * wave + nt) + ln;
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -322,6 +328,7 @@ __global__ __launch_bounds__(512) void gemm_chain_i8_kernel(I8ChainArgs p) {
 #endif
 }
 
+int i8_chain_threads() { return 64 * i8::NW; }
 int i8_chain_lds_bytes_host(int Lp, int mt, int nst) { return i8_chain_lds_bytes(Lp, mt, nst); }
 
 template <int MT, int NST>
