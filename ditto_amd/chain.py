@@ -163,16 +163,40 @@ def conv_chain_desc(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op
     return d
 
 
+_WORKSPACES = {}
+
+
+def _workspace(dev, nbytes):
+    """A per-device scratch buffer (uint8) of at least ``nbytes``; the library writes the repacked
+    first-convolution weights there on every call, so calls on one device must not overlap."""
+    buf = _WORKSPACES.get(dev)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        _WORKSPACES[dev] = buf
+    return buf
+
+
 def run_conv_chain(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op="cast", relu_out=False,
-                   desc=None):
-    """Y = conv2d(inter(conv2d(X, W1)), W2) as ONE kernel on the current stream."""
+                   desc=None, workspace=None):
+    """Y = conv2d(inter(conv2d(X, W1)), W2) on the current stream: one fused kernel, preceded by
+    a small kernel that repacks W1 into ``workspace`` (a uint8 tensor of
+    ``ditto_conv_chain_workspace_bytes``; None: a cached per-device buffer; False: no
+    workspace, the fused kernel re-lays W1 out itself, slower)."""
     lib = _lib.load()
     dev = _check_device(X, W1, W2, Y)
     if desc is None:
         desc = conv_chain_desc(X, W1, W2, Y, pad1, stride1, pad2, stride2, inter_op, relu_out)
+    ws_bytes = lib.ditto_conv_chain_workspace_bytes(ctypes.byref(desc))
+    if workspace is None:
+        ws = _workspace(dev, ws_bytes) if ws_bytes else None
+    elif workspace is False:
+        ws = None
+    else:
+        ws = workspace
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         rc = lib.ditto_conv_chain_run(ctypes.byref(desc), X.data_ptr(), W1.data_ptr(), W2.data_ptr(),
-                                      Y.data_ptr(), None, 0, stream)
+                                      Y.data_ptr(), ws.data_ptr() if ws is not None else None,
+                                      ws.numel() * ws.element_size() if ws is not None else 0, stream)
     _lib.check(rc)
     return Y

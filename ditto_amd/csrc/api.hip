@@ -204,6 +204,8 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
 
 struct ConvPlan {
   int c1_tiles;
+  int ch;              // input channels per staged chunk
+  size_t w1p_bytes;    // size of the repacked W1 (the workspace)
   ditto::ConvChainArgs args;
   ditto_tile_param tile;
 };
@@ -247,18 +249,33 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan) {
   a.TW = (int)(Q < slots ? Q : slots);
   a.TH = slots / a.TW;
   if (a.TH > P) a.TH = (int)P;
-  // shrink the tile until the halo tile and the weight chunk fit in LDS
+  // Shrink the tile until the halo tile and the weight chunk fit in LDS; prefer 32-channel
+  // chunks and a footprint that lets two workgroups share a CU (one stages while the other
+  // computes), then 32-channel chunks alone, then 16-channel chunks.
   const int RS = a.R * a.S;
-  int lds = 0;
-  for (;;) {
-    a.rows_in = (a.TH - 1) * a.stride + a.R;
-    a.cols_in = (a.TW - 1) * a.stride + a.S;
-    lds = ditto::conv_chain_lds_bytes(a.rows_in, a.cols_in, RS, 32 * c1t);
-    if (lds <= 150 * 1024) break;
-    if (a.TH > 1) a.TH = (a.TH + 1) / 2;
-    else if (a.TW > 16) a.TW = (a.TW + 1) / 2;
-    else return fail(DITTO_EUNSUPPORTED, "conv chain tile does not fit in LDS");
+  const int th0 = a.TH, tw0 = a.TW;
+  int lds = 0, ch = 32;
+  for (int attempt = 0;; ++attempt) {
+    ch = attempt < 2 ? 32 : 16;
+    const int limit = attempt == 0 ? 78 * 1024 : 150 * 1024;
+    a.TH = th0;
+    a.TW = tw0;
+    bool ok = false;
+    for (;;) {
+      a.rows_in = (a.TH - 1) * a.stride + a.R;
+      a.cols_in = (a.TW - 1) * a.stride + a.S;
+      lds = ditto::conv_chain_lds_bytes(a.rows_in, a.cols_in, RS, 32 * c1t, ch);
+      if (lds <= limit) { ok = true; break; }
+      // the first attempt only gives up rows down to half the slots
+      if (a.TH > (attempt == 0 ? (th0 + 1) / 2 : 1)) a.TH = a.TH - 1;
+      else if (attempt > 0 && a.TW > 16) a.TW = (a.TW + 1) / 2;
+      else break;
+    }
+    if (ok) break;
+    if (attempt == 2) return fail(DITTO_EUNSUPPORTED, "conv chain tile does not fit in LDS");
   }
+  plan->ch = ch;
+  plan->w1p_bytes = (size_t)ditto::conv_w1_chunk_bytes(RS, 32 * c1t, ch) * (size_t)((d->C0 + ch - 1) / ch);
   a.tiles_h = (int)((P + a.TH - 1) / a.TH);
   a.tiles_w = (int)((Q + a.TW - 1) / a.TW);
   a.relu_mid = d->inter_op == DITTO_INTER_RELU;
@@ -270,12 +287,12 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan) {
   t.block_m = a.TH * a.TW;   // output pixels per workgroup
   t.block_l = 32 * c1t;      // intermediate channels held in registers
   t.block_n = (int)d->C2;
-  t.head_pad = ditto::kConvCh;
+  t.head_pad = ch;
   t.lds_bytes = lds;
   t.grid_x = a.N * a.tiles_h * a.tiles_w;
   t.grid_y = a.TH;
   t.grid_z = a.TW;
-  t.variant = 3000 + c1t * 10 + pxw;
+  t.variant = 3000 + c1t * 10 + pxw + (ch == 16 ? 100 : 0);
   return DITTO_OK;
 }
 
@@ -391,28 +408,36 @@ int ditto_conv_chain_select_tile(const ditto_conv_chain_desc* desc, ditto_tile_p
 }
 
 size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
-  (void)desc;
-  return 0;
+  ConvPlan plan;
+  if (plan_conv(desc, &plan) != DITTO_OK) return 0;
+  return plan.w1p_bytes;
 }
 
 int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const void* w1, const void* w2,
                          void* y, void* workspace, size_t workspace_bytes, void* stream) {
-  (void)workspace;
-  (void)workspace_bytes;
   ConvPlan plan;
   int rc = plan_conv(d, &plan);
   if (rc != DITTO_OK) return rc;
   if (!x || !w1 || !w2 || !y) return fail(DITTO_EINVAL, "null data pointer");
   if (!aligned(x, 2) || !aligned(w1, 2) || !aligned(w2, 8) || !aligned(y, 4))
     return fail(DITTO_EINVAL, "misaligned data pointer");
+  if (workspace && workspace_bytes < plan.w1p_bytes)
+    return fail(DITTO_EWORKSPACE, "workspace of %zu bytes, need %zu", workspace_bytes, plan.w1p_bytes);
+  if (workspace && !aligned(workspace, 16)) return fail(DITTO_EINVAL, "workspace must be 16-byte aligned");
   ditto::ConvChainArgs a = plan.args;
   a.x = x;
   a.w1 = w1;
   a.w2 = w2;
+  a.w1p = workspace;
   a.y = y;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  hipError_t e = d->in_dtype == DITTO_F16 ? ditto::launch_conv_f16(plan.c1_tiles, a, st)
-                                          : ditto::launch_conv_bf16(plan.c1_tiles, a, st);
+  const bool f16 = d->in_dtype == DITTO_F16;
+  hipError_t e = hipSuccess;
+  if (workspace)  // W1 into the chunked layout the chain kernel copies straight into LDS
+    e = f16 ? ditto::pack_conv_w1_f16(plan.c1_tiles, plan.ch, a, workspace, st)
+            : ditto::pack_conv_w1_bf16(plan.c1_tiles, plan.ch, a, workspace, st);
+  if (e == hipSuccess)
+    e = f16 ? ditto::launch_conv_f16(plan.c1_tiles, plan.ch, a, st) : ditto::launch_conv_bf16(plan.c1_tiles, plan.ch, a, st);
   if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
   return DITTO_OK;
 }

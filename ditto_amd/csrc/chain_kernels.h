@@ -15,7 +15,11 @@ hipError_t launch_bf16_cast(int d_pad, int q, bool b_kl, const BmmChainArgs& arg
 hipError_t launch_bf16_softmax(int d_pad, int q, bool b_kl, const BmmChainArgs& args, hipStream_t stream);
 
 // conv_chain_inst.hip, one object per element type; c1_tiles in {1, 2, 4, 8}
-hipError_t launch_conv_f16(int c1_tiles, const ConvChainArgs& args, hipStream_t stream);
-hipError_t launch_conv_bf16(int c1_tiles, const ConvChainArgs& args, hipStream_t stream);
+// ch in {32, 16}: input channels per staged chunk
+hipError_t launch_conv_f16(int c1_tiles, int ch, const ConvChainArgs& args, hipStream_t stream);
+hipError_t launch_conv_bf16(int c1_tiles, int ch, const ConvChainArgs& args, hipStream_t stream);
+// W1 -> the chunked layout the chain kernel loads directly (conv_w1_chunk_bytes per chunk)
+hipError_t pack_conv_w1_f16(int c1_tiles, int ch, const ConvChainArgs& args, void* out, hipStream_t stream);
+hipError_t pack_conv_w1_bf16(int c1_tiles, int ch, const ConvChainArgs& args, void* out, hipStream_t stream);
 
 }  // namespace ditto

@@ -17,10 +17,11 @@
 //
 // A workgroup (4 waves) owns TH output rows x TW output columns of one image
 // (TH*TW <= 128*PXW pixel slots, 32*PXW per wave) and all C1 / C2 channels.  Input channels
-// are walked in chunks of 16: the halo tile X[16][rows_in][cols_in] is staged to LDS as
+// are walked in chunks of 32: the halo tile X[32][rows_in][cols_in] is staged to LDS as
 // [row][col][channel] and the weight chunk as [r*S+s][c1][channel], so that both MFMA
-// operands are 16-byte LDS reads.  W2 is read straight from global memory (it is small and
-// shared by every workgroup, so it stays in L2/L1).
+// operands are 16-byte LDS reads.  W2 is staged row by row through the same LDS once the first
+// convolution is done.  The tile is sized so that two workgroups fit in a CU's LDS: one
+// stages while the other feeds the MFMA pipe.
 #pragma once
 #include "common.h"
 
@@ -30,6 +31,7 @@ struct ConvChainArgs {
   const void* x;
   const void* w1;
   const void* w2;
+  const void* w1p;   // W1 repacked by pack_conv_w1 (null: the kernel re-lays W1 out itself, slower)
   void* y;
   int N, C0, H, W;
   int C1, R, S, pad, stride;
@@ -41,23 +43,55 @@ struct ConvChainArgs {
   int relu_mid, relu_out, out_f32;
 };
 
-constexpr int kConvCh = 16;       // input channels per chunk = one MFMA k step
-constexpr int kConvChStr = 24;    // LDS stride of a channel vector: 16 + 8 pad (48 B, conflict-free)
+// Input channels per staged chunk: 32 (two MFMA k steps per tap) or, where that does not fit in
+// LDS, 16.  A channel vector is padded by 8 elements in LDS (strides of 80 / 48 bytes put the
+// 16-byte reads of consecutive pixels / rows into different bank groups).
+__host__ __device__ constexpr int conv_ch_stride(int ch) { return ch + 8; }
 
-__host__ __device__ inline int conv_chain_lds_bytes(int rows_in, int cols_in, int RS, int C1p) {
-  return (rows_in * cols_in + RS * C1p) * kConvChStr * 2;
+// bytes of one repacked W1 chunk [R*S][C1p][ch + 8]
+__host__ __device__ inline int conv_w1_chunk_bytes(int RS, int C1p, int ch) { return RS * C1p * conv_ch_stride(ch) * 2; }
+
+__host__ __device__ inline int conv_chain_lds_bytes(int rows_in, int cols_in, int RS, int C1p, int ch) {
+  // halo tile, then the W1 chunk rounded up to whole 1 KB direct-load instructions
+  const int first = rows_in * cols_in * conv_ch_stride(ch) * 2 + (conv_w1_chunk_bytes(RS, C1p, ch) + 1023) / 1024 * 1024;
+  const int second = 32 * (C1p + 4) * 2;  // at least 32 rows of W2
+  return first > second ? first : second;
 }
 
-template <typename T, int C1T, int PXW>
+// W1[c1][c0][r][s] -> chunks [c0 / ch][r*S+s][C1p][ch + 8] (zero padded): the layout the chain
+// kernel keeps a chunk in, so that it can load one with direct global -> LDS copies.
+template <typename T>
+__global__ void pack_conv_w1_kernel(const T* __restrict__ w1, T* __restrict__ out, int C0, int C1, int RS, int C1p, int ch,
+                                    long long total) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int chs = conv_ch_stride(ch);
+  const int c = (int)(i % chs);
+  long long q = i / chs;
+  const int c1 = (int)(q % C1p);
+  q /= C1p;
+  const int rs = (int)(q % RS);
+  const int chunk = (int)(q / RS);
+  const int c0 = chunk * ch + c;
+  T v = (T)0.f;
+  if (c < ch && c1 < C1 && c0 < C0) v = w1[((long long)c1 * C0 + c0) * RS + rs];
+  out[i] = v;
+}
+
+template <typename T, int C1T, int PXW, int CH>
 __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
   typedef typename Elem<T>::v8 V8;
   typedef typename Elem<T>::v4 V4;
   constexpr int C1p = 32 * C1T;
-  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  T* const Xs = reinterpret_cast<T*>(smem_raw);                       // [rows_in][cols_in][24]
-  T* const Ws = Xs + p.rows_in * p.cols_in * kConvChStr;              // [R*S][C1p][24]
+  constexpr int CHS = conv_ch_stride(CH);
+  constexpr int W2S = C1p + 4;  // LDS row stride of the staged W2 block (8-byte reads, conflict-free)
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  T* const Xs = reinterpret_cast<T*>(smem_raw);                // [rows_in][cols_in][CHS]
+  T* const Ws = Xs + p.rows_in * p.cols_in * CHS;              // [R*S][C1p][CHS]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31, g = lane >> 5;
   const int RS = p.R * p.S;
 
@@ -83,7 +117,7 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
     const int ph = slot / p.TW, pw = slot % p.TW;
     valid[j] = ph < p.TH && (p0 + ph) < p.P && (q0 + pw) < p.Q;
     const int phc = valid[j] ? ph : 0, pwc = valid[j] ? pw : 0;
-    xoff[j] = ((phc * p.stride) * p.cols_in + pwc * p.stride) * kConvChStr + 8 * g;
+    xoff[j] = ((phc * p.stride) * p.cols_in + pwc * p.stride) * CHS + 8 * g;
     opix[j] = (p0 + phc) * p.Q + q0 + pwc;
   }
 
@@ -95,48 +129,93 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[c][j][r] = 0.f;
 
-  const int xelems = kConvCh * p.rows_in * p.cols_in;
-  const int welems = C1p * kConvCh * RS;
   const T zero = (T)0.f;
+  const long long hw = (long long)p.H * p.W;
+  // in-kernel W1 staging (no repacked copy given) walks, for one c1, the contiguous run of CH*RS
+  // source elements 64 at a time; a lane's element index advances by 64 per step, i.e. its
+  // (channel, tap) pair by (dq, dr)
+  const int dq = 64 / RS, dr = 64 % RS;
+  const int c_first = lane / RS, rs_first = lane % RS;
+  const int wrun = CH * RS;
+  // repacked W1: one chunk is w1_bytes contiguous bytes, copied by 1 KB direct loads
+  const int w1_bytes = conv_w1_chunk_bytes(RS, C1p, CH);
+  const int nchunks = (p.C0 + CH - 1) / CH;
+  const i32x4 w1_rsrc = make_rsrc(p.w1p, (unsigned)(w1_bytes * nchunks));
+  const unsigned ws_lds = (unsigned)(size_t)(DITTO_LDS char*)smem_raw + p.rows_in * p.cols_in * CHS * 2;
 
-  for (int c0 = 0; c0 < p.C0; c0 += kConvCh) {
+  for (int c0 = 0, chunk = 0; c0 < p.C0; c0 += CH, ++chunk) {
     __syncthreads();  // everyone is done reading the previous chunk
-    // ---- stage X[c0..c0+15][halo] as [row][col][channel]; consecutive threads read along w
-    for (int e = tid; e < xelems; e += 256) {
-      const int c = e / (p.rows_in * p.cols_in);
-      const int rem = e - c * (p.rows_in * p.cols_in);
-      const int ri = rem / p.cols_in, ci = rem - ri * p.cols_in;
-      const int h = h0 + ri, w = w0 + ci;
-      T v = zero;
-      if (c0 + c < p.C0 && h >= 0 && h < p.H && w >= 0 && w < p.W)
-        v = Xg[((long long)(c0 + c) * p.H + h) * p.W + w];
-      Xs[(ri * p.cols_in + ci) * kConvChStr + c] = v;
+    if (p.w1p) {
+      // the W1 chunk streams into LDS while the halo tile is staged through registers below
+      for (int j = wave; j * 1024 < w1_bytes; j += 4) {
+        const int off = j * 1024 + lane * 16;
+        lds_dma_16(w1_rsrc, off < w1_bytes ? (unsigned)(chunk * w1_bytes + off) : 0x7fffffffu, ws_lds + j * 1024);
+      }
     }
-    // ---- stage W1[c1][c0..c0+15][r][s] as [r*S+s][c1][channel]; for one c1 the 16*RS
-    //      source elements are contiguous
-    for (int e = tid; e < welems; e += 256) {
-      const int c1 = e / (kConvCh * RS);
-      const int rem = e - c1 * (kConvCh * RS);
-      const int c = rem / RS, rs = rem - c * RS;
-      T v = zero;
-      if (c1 < p.C1 && c0 + c < p.C0) v = W1g[((long long)c1 * p.C0 + c0 + c) * RS + rs];
-      Ws[(rs * C1p + c1) * kConvChStr + c] = v;
+    // ---- stage X[c0..c0+CH-1][halo] as [row][col][channel]: a lane owns one halo column, four
+    //      channels at a time (one 8-byte LDS write); consecutive lanes read along w.  Four
+    //      (row, channel group) tasks are in flight per lane so that the load latency overlaps.
+    constexpr int CG = CH / 4;  // channel groups of 4 (a power of two)
+    for (int rc0 = wave; rc0 < CG * p.rows_in; rc0 += 16) {
+      for (int ci = lane; ci < p.cols_in; ci += 64) {
+        const int w = w0 + ci;
+        const bool col_ok = w >= 0 && w < p.W;
+        V4 v[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int rc = rc0 + 4 * t;
+          const int cg = rc & (CG - 1), ri = rc / CG;
+          const int h = h0 + ri;
+          const bool ok = col_ok && rc < CG * p.rows_in && h >= 0 && h < p.H;
+          const T* src = Xg + (long long)(c0 + 4 * cg) * hw + (long long)h * p.W + w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[t][e] = (ok && c0 + 4 * cg + e < p.C0) ? src[e * hw] : zero;
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int rc = rc0 + 4 * t;
+          const int cg = rc & (CG - 1), ri = rc / CG;
+          if (rc < CG * p.rows_in) *reinterpret_cast<V4*>(Xs + (ri * p.cols_in + ci) * CHS + 4 * cg) = v[t];
+        }
+      }
     }
+    if (!p.w1p) {
+      // ---- stage W1[c1][c0..c0+CH-1][r][s] as [r*S+s][c1][channel]; for one c1 the CH*RS source
+      //      elements are contiguous and consecutive lanes read consecutive elements
+      for (int c1 = wave; c1 < C1p; c1 += 4) {
+        const T* src = W1g + ((long long)c1 * p.C0 + c0) * RS;
+        int c = c_first, rs = rs_first;
+        for (int e = lane; e < wrun; e += 64) {
+          T v = zero;
+          if (c1 < p.C1 && c0 + c < p.C0) v = src[e];
+          Ws[(rs * C1p + c1) * CHS + c] = v;
+          c += dq;
+          rs += dr;
+          if (rs >= RS) rs -= RS, ++c;
+        }
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    // ---- first convolution: one MFMA k step (16 channels) per filter tap
+    // ---- first convolution: CH/16 MFMA k steps per filter tap
     for (int r = 0; r < p.R; ++r)
       for (int s = 0; s < p.S; ++s) {
-        const int tap = (r * p.cols_in + s) * kConvChStr;
-        V8 xf[PXW];
+        const int tap = (r * p.cols_in + s) * CHS;
+        const T* wrow = Ws + ((r * p.S + s) * C1p + ln) * CHS + 8 * g;
+        V8 xf[CH / 16][PXW], wf[CH / 16][C1T];
 #pragma unroll
-        for (int j = 0; j < PXW; ++j) xf[j] = *reinterpret_cast<const V8*>(Xs + xoff[j] + tap);
-        const T* wrow = Ws + ((r * p.S + s) * C1p + ln) * kConvChStr + 8 * g;
+        for (int kk = 0; kk < CH / 16; ++kk) {
 #pragma unroll
-        for (int c = 0; c < C1T; ++c) {
-          const V8 wf = *reinterpret_cast<const V8*>(wrow + 32 * c * kConvChStr);
+          for (int j = 0; j < PXW; ++j) xf[kk][j] = *reinterpret_cast<const V8*>(Xs + xoff[j] + tap + 16 * kk);
 #pragma unroll
-          for (int j = 0; j < PXW; ++j) acc[c][j] = Elem<T>::mfma32(wf, xf[j], acc[c][j]);
+          for (int c = 0; c < C1T; ++c) wf[kk][c] = *reinterpret_cast<const V8*>(wrow + 32 * c * CHS + 16 * kk);
         }
+#pragma unroll
+        for (int kk = 0; kk < CH / 16; ++kk)
+#pragma unroll
+          for (int c = 0; c < C1T; ++c)
+#pragma unroll
+            for (int j = 0; j < PXW; ++j) acc[c][j] = Elem<T>::mfma32(wf[kk][c], xf[kk][j], acc[c][j]);
       }
   }
 
@@ -161,53 +240,72 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
         pf[2 * c + hh][j] = w;
       }
 
-  // ---- second convolution (1x1): 32 output channels at a time, W2 rows from global
+  // ---- second convolution (1x1).  W2 is staged through the LDS the first convolution has
+  // finished with, as many rows (output channels) at a time as fit, rows zero-padded to C1p.
   const long long plane = (long long)p.P * p.Q;
-  for (int ct = 0; ct * 32 < p.C2; ++ct) {
-    const int c2row = 32 * ct + ln;  // A operand row of this lane
-    f32x16 o[PXW];
-#pragma unroll
-    for (int j = 0; j < PXW; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o[j][r] = 0.f;
-#pragma unroll
-    for (int u = 0; u < 2 * C1T; ++u) {
-      V4 lo = {zero, zero, zero, zero}, hi = {zero, zero, zero, zero};
-      const int k0 = 16 * u + 4 * g;
-      if (c2row < p.C2) {
-        const T* wr = W2g + (long long)c2row * p.C1;
-        if (k0 + 3 < p.C1) lo = *reinterpret_cast<const V4*>(wr + k0);
-        if (k0 + 8 + 3 < p.C1) hi = *reinterpret_cast<const V4*>(wr + k0 + 8);
-      }
-      const V8 wf = concat4<V4, V8>(lo, hi);
-#pragma unroll
-      for (int j = 0; j < PXW; ++j) o[j] = Elem<T>::mfma32(wf, pf[u][j], o[j]);
+  T* const W2s = reinterpret_cast<T*>(smem_raw);
+  const int lds_elems = conv_chain_lds_bytes(p.rows_in, p.cols_in, RS, C1p, CH) / 2;
+  int c2blk = (lds_elems / W2S) & ~31;
+  if (c2blk > ((p.C2 + 31) & ~31)) c2blk = (p.C2 + 31) & ~31;
+  constexpr int VPR = C1p / 8;  // 16-byte vectors per staged row
+  for (int cb = 0; cb < p.C2; cb += c2blk) {
+    __syncthreads();  // the LDS region is free (first convolution / previous block done)
+    for (int e = tid; e < c2blk * VPR; e += 256) {
+      const int row = e / VPR, vc = e % VPR;
+      V8 v = {zero, zero, zero, zero, zero, zero, zero, zero};
+      if (cb + row < p.C2 && 8 * vc < p.C1) v = *reinterpret_cast<const V8*>(W2g + (long long)(cb + row) * p.C1 + 8 * vc);
+      V4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+      *reinterpret_cast<V4*>(W2s + row * W2S + 8 * vc) = lo;  // rows are only 8-byte aligned
+      *reinterpret_cast<V4*>(W2s + row * W2S + 8 * vc + 4) = hi;
     }
-    // o[j][r] = out^T[c2 = 32ct + 8(r/4) + 4g + r%4][pixel of lane]: for one r the 32 lanes of
-    // a half-wave write consecutive pixels of one channel plane
+    __syncthreads();
+    for (int ct = 0; ct * 32 < c2blk && cb + ct * 32 < p.C2; ++ct) {
+      const T* wr = W2s + (32 * ct + ln) * W2S + 4 * g;  // A operand row of this lane
+      f32x16 o[PXW];
 #pragma unroll
-    for (int j = 0; j < PXW; ++j) {
-      if (!valid[j]) continue;
+      for (int j = 0; j < PXW; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int c2 = 32 * ct + 8 * (r >> 2) + 4 * g + (r & 3);
-        if (c2 >= p.C2) continue;
-        float v = o[j][r];
-        if (p.relu_out) v = fmaxf(v, 0.f);
-        const long long off = ((long long)n * p.C2 + c2) * plane + opix[j];
-        if (p.out_f32)
-          reinterpret_cast<float*>(p.y)[off] = v;
-        else
-          reinterpret_cast<T*>(p.y)[off] = (T)v;
+        for (int r = 0; r < 16; ++r) o[j][r] = 0.f;
+      V8 wf[2 * C1T];
+#pragma unroll
+      for (int u = 0; u < 2 * C1T; ++u) {
+        const V4 lo = *reinterpret_cast<const V4*>(wr + 16 * u);
+        const V4 hi = *reinterpret_cast<const V4*>(wr + 16 * u + 8);
+        wf[u] = concat4<V4, V8>(lo, hi);
+      }
+#pragma unroll
+      for (int u = 0; u < 2 * C1T; ++u)
+#pragma unroll
+        for (int j = 0; j < PXW; ++j) o[j] = Elem<T>::mfma32(wf[u], pf[u][j], o[j]);
+      // o[j][r] = out^T[c2 = cb + 32ct + 8(r/4) + 4g + r%4][pixel of lane]: for one r the 32 lanes
+      // of a half-wave write consecutive pixels of one channel plane
+#pragma unroll
+      for (int j = 0; j < PXW; ++j) {
+        if (!valid[j]) continue;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int c2 = cb + 32 * ct + 8 * (r >> 2) + 4 * g + (r & 3);
+          if (c2 >= p.C2) continue;
+          float v = o[j][r];
+          if (p.relu_out) v = fmaxf(v, 0.f);
+          const long long off = ((long long)n * p.C2 + c2) * plane + opix[j];
+          if (p.out_f32)
+            reinterpret_cast<float*>(p.y)[off] = v;
+          else
+            reinterpret_cast<T*>(p.y)[off] = (T)v;
+        }
       }
     }
   }
+#else
+  (void)p;
+#endif
 }
 
-template <typename T, int C1T, int PXW>
+template <typename T, int C1T, int PXW, int CH>
 hipError_t launch_conv_chain(const ConvChainArgs& args, hipStream_t stream) {
-  const int lds = conv_chain_lds_bytes(args.rows_in, args.cols_in, args.R * args.S, 32 * C1T);
-  auto kern = conv_chain_kernel<T, C1T, PXW>;
+  const int lds = conv_chain_lds_bytes(args.rows_in, args.cols_in, args.R * args.S, 32 * C1T, CH);
+  auto kern = conv_chain_kernel<T, C1T, PXW, CH>;
   static thread_local int configured_dev = -1;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -220,6 +318,18 @@ hipError_t launch_conv_chain(const ConvChainArgs& args, hipStream_t stream) {
   }
   const unsigned grid = (unsigned)args.N * (unsigned)args.tiles_h * (unsigned)args.tiles_w;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, args);
+  return hipGetLastError();
+}
+
+// repack W1 into `out` (conv_w1_chunk_bytes * chunks bytes) on `stream`
+template <typename T>
+hipError_t launch_pack_conv_w1(const ConvChainArgs& args, int C1p, int ch, void* out, hipStream_t stream) {
+  const int RS = args.R * args.S;
+  const int nchunks = (args.C0 + ch - 1) / ch;
+  const long long total = (long long)nchunks * RS * C1p * conv_ch_stride(ch);
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  hipLaunchKernelGGL(pack_conv_w1_kernel<T>, dim3(grid), dim3(256), 0, stream, reinterpret_cast<const T*>(args.w1),
+                     reinterpret_cast<T*>(out), args.C0, args.C1, RS, C1p, ch, total);
   return hipGetLastError();
 }
 

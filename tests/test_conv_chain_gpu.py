@@ -11,14 +11,14 @@ pytestmark = pytest.mark.gpu
 MAX_ABS, REL_L2, REL_L2_BF16_QUANT = 1e-2, 1e-3, 3e-3
 
 
-def run_conv(X, W1, W2, dtype, pad1=1, stride1=1, inter="cast", relu_out=False, out_dtype=None):
+def run_conv(X, W1, W2, dtype, pad1=1, stride1=1, inter="cast", relu_out=False, out_dtype=None, workspace=None):
     x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
     N, _, H, W = X.shape
     R, S = W1.shape[2:]
     P = (H + 2 * pad1 - R) // stride1 + 1
     Q = (W + 2 * pad1 - S) // stride1 + 1
     y = torch.full((N, W2.shape[0], P, Q), float("nan"), device=x.device, dtype=TORCH_DTYPES[out_dtype or dtype])
-    chain.run_conv_chain(x, w1, w2, y, pad1, stride1, 0, 1, inter, relu_out)
+    chain.run_conv_chain(x, w1, w2, y, pad1, stride1, 0, 1, inter, relu_out, workspace=workspace)
     torch.cuda.synchronize()
     return y.float().cpu().numpy()
 
@@ -42,14 +42,16 @@ def test_conv_chain_vs_oracle(oracle, case, dtype):
     N, C0, H, W, C1, R, pad, stride, C2 = case
     X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, R, 1, dtype, seed=C0 + C1, w_std=0.05)
     want32 = oracle.conv_chain_f32(X, W1, W2, pad, stride, 0, 1, round_mid=dtype)
-    got32 = run_conv(X, W1, W2, dtype, pad, stride, out_dtype="float32")
-    assert np.isfinite(got32).all()
-    mx, rel = errors(got32, want32)
-    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
-    got = run_conv(X, W1, W2, dtype, pad, stride)
-    assert np.array_equal(got, oracle.np_round_to(got32, dtype))
-    mx, rel = errors(got, oracle.np_round_to(want32, dtype))
-    assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (mx, rel)
+    # with the repacked-weights workspace (None: the wrapper's cached buffer) and without (False)
+    for ws in (None, False):
+        got32 = run_conv(X, W1, W2, dtype, pad, stride, out_dtype="float32", workspace=ws)
+        assert np.isfinite(got32).all(), ws
+        mx, rel = errors(got32, want32)
+        assert mx <= MAX_ABS and rel <= REL_L2, (ws, mx, rel)
+        got = run_conv(X, W1, W2, dtype, pad, stride, workspace=ws)
+        assert np.array_equal(got, oracle.np_round_to(got32, dtype)), ws
+        mx, rel = errors(got, oracle.np_round_to(want32, dtype))
+        assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (ws, mx, rel)
 
 
 def test_conv_relu_conv_relu_vs_torch(oracle):
