@@ -245,8 +245,19 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
   const long long plane = (long long)p.P * p.Q;
   T* const W2s = reinterpret_cast<T*>(smem_raw);
   const int lds_elems = conv_chain_lds_bytes(p.rows_in, p.cols_in, RS, C1p, CH) / 2;
-  int c2blk = (lds_elems / W2S) & ~31;
+  // Output path.  A lane holds ONE pixel per register, so storing from registers means 2-byte
+  // stores.  When the tile is a run of whole image rows (its pixels are contiguous in a channel
+  // plane) and everything is 16-byte aligned, each wave instead turns its 32-channel x 32*PXW
+  // pixel result around in a private corner of LDS and stores 8 pixels (16 bytes) per lane.
+  constexpr int SLW = 32 * PXW;          // pixel slots of a wave
+  constexpr int OSS = SLW + 8;           // LDS row stride of the turn-around buffer (elements)
+  constexpr int OS_ELEMS = 4 * 32 * OSS; // four waves
+  const int nvalid = (p.P - p0 < p.TH ? p.P - p0 : p.TH) * p.Q;  // valid slots when TW == Q
+  const bool wide = p.TW == p.Q && !p.out_f32 && (nvalid & 7) == 0 && ((p0 * p.Q) & 7) == 0 && (plane & 7) == 0 &&
+              (reinterpret_cast<unsigned long long>(p.y) & 15) == 0 && lds_elems - OS_ELEMS >= 32 * W2S;
+  int c2blk = ((wide ? lds_elems - OS_ELEMS : lds_elems) / W2S) & ~31;
   if (c2blk > ((p.C2 + 31) & ~31)) c2blk = (p.C2 + 31) & ~31;
+  T* const Os = W2s + (lds_elems - OS_ELEMS) + wave * 32 * OSS;  // this wave's turn-around buffer
   constexpr int VPR = C1p / 8;  // 16-byte vectors per staged row
   for (int cb = 0; cb < p.C2; cb += c2blk) {
     __syncthreads();  // the LDS region is free (first convolution / previous block done)
@@ -277,22 +288,44 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
       for (int u = 0; u < 2 * C1T; ++u)
 #pragma unroll
         for (int j = 0; j < PXW; ++j) o[j] = Elem<T>::mfma32(wf[u], pf[u][j], o[j]);
-      // o[j][r] = out^T[c2 = cb + 32ct + 8(r/4) + 4g + r%4][pixel of lane]: for one r the 32 lanes
-      // of a half-wave write consecutive pixels of one channel plane
+      // o[j][r] = out^T[c2 = cb + 32ct + 8(r/4) + 4g + r%4][pixel of lane]
+      if (wide) {
 #pragma unroll
-      for (int j = 0; j < PXW; ++j) {
-        if (!valid[j]) continue;
+        for (int j = 0; j < PXW; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int c2 = cb + 32 * ct + 8 * (r >> 2) + 4 * g + (r & 3);
-          if (c2 >= p.C2) continue;
-          float v = o[j][r];
-          if (p.relu_out) v = fmaxf(v, 0.f);
-          const long long off = ((long long)n * p.C2 + c2) * plane + opix[j];
-          if (p.out_f32)
-            reinterpret_cast<float*>(p.y)[off] = v;
-          else
-            reinterpret_cast<T*>(p.y)[off] = (T)v;
+          for (int r = 0; r < 16; ++r) {
+            float v = o[j][r];
+            if (p.relu_out) v = fmaxf(v, 0.f);
+            Os[(8 * (r >> 2) + 4 * g + (r & 3)) * OSS + 32 * j + ln] = (T)v;
+          }
+        // 32 rows x SLW/8 vectors of 8 pixels, 64 per pass
+#pragma unroll
+        for (int v0 = 0; v0 < 32 * (SLW / 8); v0 += 64) {
+          const int v = v0 + lane;
+          const int ch = v / (SLW / 8), sv = v % (SLW / 8);
+          const int c2 = cb + 32 * ct + ch;
+          const int slot = SLW * wave + 8 * sv;
+          const V8 px = *reinterpret_cast<const V8*>(Os + ch * OSS + 8 * sv);
+          if (c2 < p.C2 && slot < nvalid)
+            *reinterpret_cast<V8*>(reinterpret_cast<T*>(p.y) + ((long long)n * p.C2 + c2) * plane + p0 * p.Q + slot) = px;
+        }
+      } else {
+        // for one r the 32 lanes of a half-wave write consecutive pixels of one channel plane
+#pragma unroll
+        for (int j = 0; j < PXW; ++j) {
+          if (!valid[j]) continue;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int c2 = cb + 32 * ct + 8 * (r >> 2) + 4 * g + (r & 3);
+            if (c2 >= p.C2) continue;
+            float v = o[j][r];
+            if (p.relu_out) v = fmaxf(v, 0.f);
+            const long long off = ((long long)n * p.C2 + c2) * plane + opix[j];
+            if (p.out_f32)
+              reinterpret_cast<float*>(p.y)[off] = v;
+            else
+              reinterpret_cast<T*>(p.y)[off] = (T)v;
+          }
         }
       }
     }
