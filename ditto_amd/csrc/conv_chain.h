@@ -143,6 +143,46 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
   const i32x4 w1_rsrc = make_rsrc(p.w1p, (unsigned)(w1_bytes * nchunks));
   const unsigned ws_lds = (unsigned)(size_t)(DITTO_LDS char*)smem_raw + p.rows_in * p.cols_in * CHS * 2;
 
+  // ---- halo tile staging: X[c0..c0+CH-1][halo] goes to LDS as [row][col][channel].
+  // Two-byte global loads issue very slowly, so when the image rows are 16-byte multiples a task
+  // is an aligned group of 8 pixels x 8 channels of one halo row: eight 16-byte loads (one per
+  // channel), an 8x8 transposition in registers (one byte-permute per output dword) and eight
+  // 16-byte LDS writes (one per pixel).  If every thread has at most one task per chunk, the
+  // loads of chunk i+1 are issued before the MFMAs of chunk i and written to LDS after them.
+  const bool x_vec = (p.W & 7) == 0 && (reinterpret_cast<unsigned long long>(p.x) & 15) == 0;
+  const int wg0 = (w0 >= 0 ? w0 : w0 - 7) / 8 * 8;              // first aligned group (floor)
+  const int ngc = (w0 + p.cols_in - wg0 + 7) / 8;               // groups per halo row
+  const int xtasks = p.rows_in * ngc * (CH / 8);
+  const bool x_prefetch = x_vec && xtasks <= 256;
+  // task of this thread: channel group fastest, then column group, then row
+  const int t_chg = tid % (CH / 8), t_gi = (tid / (CH / 8)) % ngc, t_ri = tid / (CH / 8) / ngc;
+  i32x4 xr[8];
+  auto xv_load = [&](int c0, int chg, int gi, int ri, bool live) __attribute__((always_inline)) {
+    const int h = h0 + ri, wg = wg0 + 8 * gi;
+    const bool ok = live && h >= 0 && h < p.H && wg >= 0 && wg < p.W;
+    const T* src = Xg + (long long)(c0 + 8 * chg) * hw + (long long)h * p.W + wg;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      i32x4 v = {0, 0, 0, 0};
+      if (ok && c0 + 8 * chg + c < p.C0) v = *reinterpret_cast<const i32x4*>(src + c * hw);
+      xr[c] = v;
+    }
+  };
+  auto xv_store = [&](int chg, int gi, int ri, bool live) __attribute__((always_inline)) {
+    const int ci0 = wg0 + 8 * gi - w0;  // halo column of the group's first pixel
+#pragma unroll
+    for (int px = 0; px < 8; ++px) {
+      i32x4 o;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        o[d] = __builtin_amdgcn_perm(xr[2 * d + 1][px >> 1], xr[2 * d][px >> 1], (px & 1) ? 0x07060302 : 0x05040100);
+      const int ci = ci0 + px;
+      if (live && ci >= 0 && ci < p.cols_in)
+        *reinterpret_cast<i32x4*>(Xs + (ri * p.cols_in + ci) * CHS + 8 * chg) = o;
+    }
+  };
+  if (x_prefetch) xv_load(0, t_chg, t_gi, t_ri, tid < xtasks);
+
   for (int c0 = 0, chunk = 0; c0 < p.C0; c0 += CH, ++chunk) {
     __syncthreads();  // everyone is done reading the previous chunk
     if (p.w1p) {
@@ -152,30 +192,39 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
         lds_dma_16(w1_rsrc, off < w1_bytes ? (unsigned)(chunk * w1_bytes + off) : 0x7fffffffu, ws_lds + j * 1024);
       }
     }
-    // ---- stage X[c0..c0+CH-1][halo] as [row][col][channel]: a lane owns one halo column, four
-    //      channels at a time (one 8-byte LDS write); consecutive lanes read along w.  Four
-    //      (row, channel group) tasks are in flight per lane so that the load latency overlaps.
-    constexpr int CG = CH / 4;  // channel groups of 4 (a power of two)
-    for (int rc0 = wave; rc0 < CG * p.rows_in; rc0 += 16) {
-      for (int ci = lane; ci < p.cols_in; ci += 64) {
-        const int w = w0 + ci;
-        const bool col_ok = w >= 0 && w < p.W;
-        V4 v[4];
+    if (x_prefetch) {
+      xv_store(t_chg, t_gi, t_ri, tid < xtasks);
+    } else if (x_vec) {
+      for (int t = tid; t < xtasks; t += 256) {
+        const int chg = t % (CH / 8), gi = (t / (CH / 8)) % ngc, ri = t / (CH / 8) / ngc;
+        xv_load(c0, chg, gi, ri, true);
+        xv_store(chg, gi, ri, true);
+      }
+    } else {
+      // rows that are not 16-byte multiples: a lane owns one halo column and, per task, one
+      // (row, group of 4 channels): four 2-byte loads, one 8-byte LDS write; four tasks in flight
+      constexpr int CG = CH / 4;
+      for (int rc0 = wave; rc0 < CG * p.rows_in; rc0 += 16) {
+        for (int ci = lane; ci < p.cols_in; ci += 64) {
+          const int w = w0 + ci;
+          const bool col_ok = w >= 0 && w < p.W;
+          V4 v[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int rc = rc0 + 4 * t;
-          const int cg = rc & (CG - 1), ri = rc / CG;
-          const int h = h0 + ri;
-          const bool ok = col_ok && rc < CG * p.rows_in && h >= 0 && h < p.H;
-          const T* src = Xg + (long long)(c0 + 4 * cg) * hw + (long long)h * p.W + w;
+          for (int t = 0; t < 4; ++t) {
+            const int rc = rc0 + 4 * t;
+            const int cg = rc & (CG - 1), ri = rc / CG;
+            const int h = h0 + ri;
+            const bool ok = col_ok && rc < CG * p.rows_in && h >= 0 && h < p.H;
+            const T* src = Xg + (long long)(c0 + 4 * cg) * hw + (long long)h * p.W + w;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[t][e] = (ok && c0 + 4 * cg + e < p.C0) ? src[e * hw] : zero;
-        }
+            for (int e = 0; e < 4; ++e) v[t][e] = (ok && c0 + 4 * cg + e < p.C0) ? src[e * hw] : zero;
+          }
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int rc = rc0 + 4 * t;
-          const int cg = rc & (CG - 1), ri = rc / CG;
-          if (rc < CG * p.rows_in) *reinterpret_cast<V4*>(Xs + (ri * p.cols_in + ci) * CHS + 4 * cg) = v[t];
+          for (int t = 0; t < 4; ++t) {
+            const int rc = rc0 + 4 * t;
+            const int cg = rc & (CG - 1), ri = rc / CG;
+            if (rc < CG * p.rows_in) *reinterpret_cast<V4*>(Xs + (ri * p.cols_in + ci) * CHS + 4 * cg) = v[t];
+          }
         }
       }
     }
@@ -197,6 +246,7 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    if (x_prefetch && c0 + CH < p.C0) xv_load(c0 + CH, t_chg, t_gi, t_ri, tid < xtasks);  // in flight during the MFMAs
     // ---- first convolution: CH/16 MFMA k steps per filter tap
     for (int r = 0; r < p.R; ++r)
       for (int s = 0; s < p.S; ++s) {
@@ -284,19 +334,26 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
         const V4 hi = *reinterpret_cast<const V4*>(wr + 16 * u + 8);
         wf[u] = concat4<V4, V8>(lo, hi);
       }
-#pragma unroll
-      for (int u = 0; u < 2 * C1T; ++u)
-#pragma unroll
-        for (int j = 0; j < PXW; ++j) o[j] = Elem<T>::mfma32(wf[u], pf[u][j], o[j]);
-      // o[j][r] = out^T[c2 = cb + 32ct + 8(r/4) + 4g + r%4][pixel of lane]
       if (wide) {
+#pragma unroll
+        for (int u = 0; u < 2 * C1T; ++u)
+#pragma unroll
+          for (int j = 0; j < PXW; ++j) o[j] = Elem<T>::mfma32(pf[u][j], wf[u], o[j]);
+        // operands swapped: o[j][r] = out[pixel 32j + 8(r/4) + 4g + r%4][c2 = cb + 32ct + ln], four
+        // consecutive pixels of one channel per register quad -> one 8-byte LDS write
 #pragma unroll
         for (int j = 0; j < PXW; ++j)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            float v = o[j][r];
-            if (p.relu_out) v = fmaxf(v, 0.f);
-            Os[(8 * (r >> 2) + 4 * g + (r & 3)) * OSS + 32 * j + ln] = (T)v;
+          for (int q = 0; q < 4; ++q) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              v[e] = o[j][4 * q + e];
+              if (p.relu_out) v[e] = fmaxf(v[e], 0.f);
+            }
+            const typename Elem<T>::v2 a0 = cvt2<T>(v[0], v[1]), a1 = cvt2<T>(v[2], v[3]);
+            const V4 w = {a0[0], a0[1], a1[0], a1[1]};
+            *reinterpret_cast<V4*>(Os + ln * OSS + 32 * j + 8 * q + 4 * g) = w;
           }
         // 32 rows x SLW/8 vectors of 8 pixels, 64 per pass
 #pragma unroll
@@ -307,10 +364,15 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
           const int slot = SLW * wave + 8 * sv;
           const V8 px = *reinterpret_cast<const V8*>(Os + ch * OSS + 8 * sv);
           if (c2 < p.C2 && slot < nvalid)
-            *reinterpret_cast<V8*>(reinterpret_cast<T*>(p.y) + ((long long)n * p.C2 + c2) * plane + p0 * p.Q + slot) = px;
+            __builtin_nontemporal_store(px, reinterpret_cast<V8*>(reinterpret_cast<T*>(p.y) + ((long long)n * p.C2 + c2) * plane + p0 * p.Q + slot));
         }
       } else {
-        // for one r the 32 lanes of a half-wave write consecutive pixels of one channel plane
+#pragma unroll
+        for (int u = 0; u < 2 * C1T; ++u)
+#pragma unroll
+          for (int j = 0; j < PXW; ++j) o[j] = Elem<T>::mfma32(wf[u], pf[u][j], o[j]);
+        // o[j][r] = out^T[c2 = cb + 32ct + 8(r/4) + 4g + r%4][pixel of lane]: for one r the 32 lanes
+        // of a half-wave write consecutive pixels of one channel plane
 #pragma unroll
         for (int j = 0; j < PXW; ++j) {
           if (!valid[j]) continue;
