@@ -143,6 +143,43 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
   const i32x4 w1_rsrc = make_rsrc(p.w1p, (unsigned)(w1_bytes * nchunks));
   const unsigned ws_lds = (unsigned)(size_t)(DITTO_LDS char*)smem_raw + p.rows_in * p.cols_in * CHS * 2;
 
+  // ---- set-up of the second convolution (1x1).  W2 is staged through the LDS the first
+  // convolution has finished with, as many rows (output channels) at a time as fit, rows zero-padded to C1p.
+  const long long plane = (long long)p.P * p.Q;
+  T* const W2s = reinterpret_cast<T*>(smem_raw);
+  const int lds_elems = conv_chain_lds_bytes(p.rows_in, p.cols_in, RS, C1p, CH) / 2;
+  // Output path.  A lane holds ONE pixel per register, so storing from registers means 2-byte
+  // stores.  When the tile is a run of whole image rows (its pixels are contiguous in a channel
+  // plane) and everything is 16-byte aligned, each wave instead turns its 32-channel x 32*PXW
+  // pixel result around in a private corner of LDS and stores 8 pixels (16 bytes) per lane.
+  constexpr int SLW = 32 * PXW;          // pixel slots of a wave
+  constexpr int OSS = SLW + 8;           // LDS row stride of the turn-around buffer (elements)
+  constexpr int OS_ELEMS = 4 * 32 * OSS; // four waves
+  const int nvalid = (p.P - p0 < p.TH ? p.P - p0 : p.TH) * p.Q;  // valid slots when TW == Q
+  const bool wide = p.TW == p.Q && !p.out_f32 && (nvalid & 7) == 0 && ((p0 * p.Q) & 7) == 0 && (plane & 7) == 0 &&
+              (reinterpret_cast<unsigned long long>(p.y) & 15) == 0 && lds_elems - OS_ELEMS >= 32 * W2S;
+  int c2blk = ((wide ? lds_elems - OS_ELEMS : lds_elems) / W2S) & ~31;
+  if (c2blk > ((p.C2 + 31) & ~31)) c2blk = (p.C2 + 31) & ~31;
+  T* const Os = W2s + (lds_elems - OS_ELEMS) + wave * 32 * OSS;  // this wave's turn-around buffer
+  constexpr int VPR = C1p / 8;  // 16-byte vectors per staged row
+  // The first W2 block is fetched into the halo-tile staging registers during the MFMAs of the
+  // last chunk (they are free by then) when it is at most 8 vectors per thread.
+  const bool w2_prefetch = c2blk * VPR <= 8 * 256;
+  auto w2_load = [&](int cb, int e) __attribute__((always_inline)) -> i32x4 {
+    const int row = e / VPR, vc = e % VPR;
+    i32x4 v = {0, 0, 0, 0};
+    if (e < c2blk * VPR && cb + row < p.C2 && 8 * vc < p.C1)
+      v = *reinterpret_cast<const i32x4*>(W2g + (long long)(cb + row) * p.C1 + 8 * vc);
+    return v;
+  };
+  auto w2_store = [&](int e, i32x4 v) __attribute__((always_inline)) {
+    const int row = e / VPR, vc = e % VPR;
+    if (e < c2blk * VPR) {  // rows are only 8-byte aligned
+      *reinterpret_cast<i32x2*>(W2s + row * W2S + 8 * vc) = i32x2{v[0], v[1]};
+      *reinterpret_cast<i32x2*>(W2s + row * W2S + 8 * vc + 4) = i32x2{v[2], v[3]};
+    }
+  };
+
   // ---- halo tile staging: X[c0..c0+CH-1][halo] goes to LDS as [row][col][channel].
   // Two-byte global loads issue very slowly, so when the image rows are 16-byte multiples a task
   // is an aligned group of 8 pixels x 8 channels of one halo row: eight 16-byte loads (one per
@@ -247,6 +284,10 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (x_prefetch && c0 + CH < p.C0) xv_load(c0 + CH, t_chg, t_gi, t_ri, tid < xtasks);  // in flight during the MFMAs
+    if (w2_prefetch && c0 + CH >= p.C0) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) xr[k] = w2_load(0, tid + 256 * k);
+    }
     // ---- first convolution: CH/16 MFMA k steps per filter tap
     for (int r = 0; r < p.R; ++r)
       for (int s = 0; s < p.S; ++s) {
@@ -269,7 +310,8 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
       }
   }
 
-  // ---- inter op on the accumulators, cast: mid^T tile (c, j) regs 8(u%2)..+7 are the
+  // ---- second convolution (1x1): W2 blocks go through the LDS the first convolution has finished
+  // with.  Inter op on the accumulators, cast: mid^T tile (c, j) regs 8(u%2)..+7 are the
   // B operand of k step u (channels 16u + 4g + {0..3} and 16u + 8 + 4g + {0..3})
   V8 pf[2 * C1T][PXW];
 #pragma unroll
@@ -290,34 +332,13 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
         pf[2 * c + hh][j] = w;
       }
 
-  // ---- second convolution (1x1).  W2 is staged through the LDS the first convolution has
-  // finished with, as many rows (output channels) at a time as fit, rows zero-padded to C1p.
-  const long long plane = (long long)p.P * p.Q;
-  T* const W2s = reinterpret_cast<T*>(smem_raw);
-  const int lds_elems = conv_chain_lds_bytes(p.rows_in, p.cols_in, RS, C1p, CH) / 2;
-  // Output path.  A lane holds ONE pixel per register, so storing from registers means 2-byte
-  // stores.  When the tile is a run of whole image rows (its pixels are contiguous in a channel
-  // plane) and everything is 16-byte aligned, each wave instead turns its 32-channel x 32*PXW
-  // pixel result around in a private corner of LDS and stores 8 pixels (16 bytes) per lane.
-  constexpr int SLW = 32 * PXW;          // pixel slots of a wave
-  constexpr int OSS = SLW + 8;           // LDS row stride of the turn-around buffer (elements)
-  constexpr int OS_ELEMS = 4 * 32 * OSS; // four waves
-  const int nvalid = (p.P - p0 < p.TH ? p.P - p0 : p.TH) * p.Q;  // valid slots when TW == Q
-  const bool wide = p.TW == p.Q && !p.out_f32 && (nvalid & 7) == 0 && ((p0 * p.Q) & 7) == 0 && (plane & 7) == 0 &&
-              (reinterpret_cast<unsigned long long>(p.y) & 15) == 0 && lds_elems - OS_ELEMS >= 32 * W2S;
-  int c2blk = ((wide ? lds_elems - OS_ELEMS : lds_elems) / W2S) & ~31;
-  if (c2blk > ((p.C2 + 31) & ~31)) c2blk = (p.C2 + 31) & ~31;
-  T* const Os = W2s + (lds_elems - OS_ELEMS) + wave * 32 * OSS;  // this wave's turn-around buffer
-  constexpr int VPR = C1p / 8;  // 16-byte vectors per staged row
   for (int cb = 0; cb < p.C2; cb += c2blk) {
     __syncthreads();  // the LDS region is free (first convolution / previous block done)
-    for (int e = tid; e < c2blk * VPR; e += 256) {
-      const int row = e / VPR, vc = e % VPR;
-      V8 v = {zero, zero, zero, zero, zero, zero, zero, zero};
-      if (cb + row < p.C2 && 8 * vc < p.C1) v = *reinterpret_cast<const V8*>(W2g + (long long)(cb + row) * p.C1 + 8 * vc);
-      V4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
-      *reinterpret_cast<V4*>(W2s + row * W2S + 8 * vc) = lo;  // rows are only 8-byte aligned
-      *reinterpret_cast<V4*>(W2s + row * W2S + 8 * vc + 4) = hi;
+    if (w2_prefetch && cb == 0) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) w2_store(tid + 256 * k, xr[k]);
+    } else {
+      for (int e = tid; e < c2blk * VPR; e += 256) w2_store(e, w2_load(cb, e));
     }
     __syncthreads();
     for (int ct = 0; ct * 32 < c2blk && cb + ct * 32 < p.C2; ++ct) {
