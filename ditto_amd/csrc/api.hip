@@ -151,6 +151,33 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     t.variant = plan->d_pad * 10 + plan->qt;
     return DITTO_OK;
   }
+  if (in == DITTO_F32) {
+    if (d->acc_dtype != DITTO_F32 || d->out_dtype != DITTO_F32)
+      return fail(DITTO_EINVAL, "the fp32 chain accumulates and outputs fp32");
+    if (d->inter_op != DITTO_INTER_CAST && d->inter_op != DITTO_INTER_RELU)
+      return fail(DITTO_EUNSUPPORTED, "the fp32 chain takes inter_op cast or relu");
+    if (d->tile_variant != 0) return fail(DITTO_EINVAL, "the fp32 chain has a single variant (tile_variant must be 0)");
+    if (d->K > ditto::f32_chain_max_dim() || d->N > ditto::f32_chain_max_dim())
+      return fail(DITTO_EUNSUPPORTED, "the fp32 chain supports K, N up to %d", ditto::f32_chain_max_dim());
+    if (d->a_row_stride < d->K || d->c_row_stride < d->N || d->f_row_stride < d->N ||
+        d->b_row_stride < (d->b_layout == DITTO_B_KL ? d->L : d->K))
+      return fail(DITTO_EINVAL, "row stride smaller than row extent");
+    if (d->a_row_stride > 0x7fffffff || d->b_row_stride > 0x7fffffff || d->c_row_stride > 0x7fffffff ||
+        d->f_row_stride > 0x7fffffff)
+      return fail(DITTO_EINVAL, "row stride too large");
+    plan->family = 1;
+    ditto_tile_param& t = plan->tile;
+    t.block_threads = 256;
+    t.block_m = 32;
+    t.block_l = 64;
+    t.block_n = (int)d->N;
+    t.head_pad = 0;
+    t.lds_bytes = ditto::f32_chain_lds_bytes_host((int)d->K, (int)d->N);
+    t.grid_x = (int)(((d->M + 31) / 32) * d->batch);
+    t.grid_y = t.grid_z = 1;
+    t.variant = 1000;  // fp32 FMA chain
+    return DITTO_OK;
+  }
   if (in == DITTO_I8) {
     if (d->acc_dtype != DITTO_I32 || d->out_dtype != DITTO_I32)
       return fail(DITTO_EINVAL, "the int8 chain accumulates and outputs int32");
@@ -364,6 +391,32 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     else
       e = sm ? ditto::launch_bf16_softmax(plan.d_pad, plan.qt, kl, args, st)
              : ditto::launch_bf16_cast(plan.d_pad, plan.qt, kl, args, st);
+    if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
+    return DITTO_OK;
+  }
+  if (plan.family == 1) {
+    ditto::F32ChainArgs args;
+    args.a = static_cast<const float*>(a);
+    args.b = static_cast<const float*>(b);
+    args.c = static_cast<const float*>(c);
+    args.f = static_cast<float*>(f);
+    args.a_bs = d->a_batch_stride;
+    args.b_bs = d->b_batch_stride;
+    args.c_bs = d->c_batch_stride;
+    args.f_bs = d->f_batch_stride;
+    args.a_rs = (int)d->a_row_stride;
+    args.b_rs = (int)d->b_row_stride;
+    args.c_rs = (int)d->c_row_stride;
+    args.f_rs = (int)d->f_row_stride;
+    args.M = (int)d->M;
+    args.N = (int)d->N;
+    args.K = (int)d->K;
+    args.L = (int)d->L;
+    args.batch = (int)d->batch;
+    args.mblocks = (int)((d->M + 31) / 32);
+    args.b_lk = d->b_layout == DITTO_B_LK;
+    args.relu = d->inter_op == DITTO_INTER_RELU;
+    hipError_t e = ditto::launch_gemm_chain_f32(args, st);
     if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
     return DITTO_OK;
   }

@@ -4,6 +4,7 @@
 
 #include "bmm_chain_fp.h"
 #include "conv_chain.h"
+#include "gemm_chain_f32.h"
 #include "gemm_chain_i8.h"
 
 namespace ditto {

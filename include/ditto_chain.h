@@ -137,9 +137,12 @@ const char* ditto_last_error(void);
 int ditto_bmm_chain_select_tile(const ditto_bmm_chain_desc* desc, ditto_tile_param* out);
 int ditto_conv_chain_select_tile(const ditto_conv_chain_desc* desc, ditto_tile_param* out);
 
-/* Bytes of device workspace the run call needs (0 for every chain today; the
- * reference's generated code allocates an fp32 E_frag[B,M,ext_N] internally,
- * evaluation/asplos/ncu_summary_chimera_bmm_softmax_bmm.txt:8). */
+/* Bytes of device workspace the run call can use.  BMM chains: 0 (the reference's
+ * generated code allocates an fp32 E_frag[B,M,ext_N] internally,
+ * evaluation/asplos/ncu_summary_chimera_bmm_softmax_bmm.txt:8).  conv chain: room for
+ * the first convolution's weights repacked in channel blocks -- the reference's
+ * placeholders are already packed that way by the host
+ * (conv3x3_conv1x1_cuda.py:99-103); 0 if the descriptor is invalid. */
 size_t ditto_bmm_chain_workspace_bytes(const ditto_bmm_chain_desc* desc);
 size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc);
 
@@ -151,13 +154,22 @@ size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc);
  *             mid = saturate_to_[-128,127](round_to_nearest_even((float)acc * scale[l]));
  *             NULL to use desc->requant_scale for every column.  Other chains: NULL
  *   f       : output (device), must not alias an input
+ * in_dtype DITTO_F16 / DITTO_BF16: the MFMA chains (cast, relu, softmax);
+ * DITTO_F32: the reference's fp32 configuration
+ * (python_test/auto_tensorize/test_hyper_fusion.py:16-21), cast / relu, K, N <= 128;
+ * DITTO_I8: the requantised chain.
  */
 int ditto_bmm_chain_run(const ditto_bmm_chain_desc* desc, const void* a, const void* b,
                         const void* c, const void* aux, void* f, void* workspace,
                         size_t workspace_bytes, void* stream);
 
 /* Run one fused conv->conv chain: replaces `func(Img, W1, W2, Out)`
- * (conv3x3_conv1x1_cuda.py:296-305). */
+ * (conv3x3_conv1x1_cuda.py:296-305).
+ *   workspace : NULL, or ditto_conv_chain_workspace_bytes() bytes of device memory,
+ *               16-byte aligned.  Given, a small kernel repacks w1 into it ahead of the
+ *               fused kernel on `stream` (every call; calls that share a workspace must
+ *               not overlap).  NULL: the fused kernel re-lays w1 out itself, slower.
+ *               DITTO_EWORKSPACE if non-NULL and too small. */
 int ditto_conv_chain_run(const ditto_conv_chain_desc* desc, const void* x, const void* w1,
                          const void* w2, void* y, void* workspace, size_t workspace_bytes,
                          void* stream);
