@@ -48,6 +48,11 @@ class BmmChainDesc(ctypes.Structure):
         ("requant_scale", ctypes.c_float),
         ("tile_variant", ctypes.c_int32),
         ("reserved", ctypes.c_int32),
+        ("batch_inner", ctypes.c_int64),
+        ("a_batch_stride_outer", ctypes.c_int64),
+        ("b_batch_stride_outer", ctypes.c_int64),
+        ("c_batch_stride_outer", ctypes.c_int64),
+        ("f_batch_stride_outer", ctypes.c_int64),
     ]
 
 

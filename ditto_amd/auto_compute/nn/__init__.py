@@ -1,1 +1,3 @@
 from . import functional
+from . import module
+from .module import MultiHeadAttentionMMA

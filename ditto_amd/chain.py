@@ -49,14 +49,28 @@ def _as3d(t, name):
     return t
 
 
+def _split_levels(t, name):
+    """[outer, inner, rows, cols] (any strides) -> (3-D view of the first outer entry with the inner
+    level as its batch, outer extent, outer stride); 2-D / 3-D tensors have a single level."""
+    if t.dim() == 4:
+        return t[0], t.shape[0], t.stride(0)
+    return _as3d(t, name), 1, 0
+
+
 def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=1.0, tile_variant=0):
     """Fill a ``ditto_bmm_chain_desc`` from tensors A[b,M,K], B[b,K,L], C[b,L,N], F[b,M,N].
 
     B may be a transposed view of a ``[b, L, K]`` tensor (stride 1 along K); it is then
-    consumed in place (``DITTO_B_LK``).  ``tile_variant`` forces a kernel variant (an id that
+    consumed in place (``DITTO_B_LK``).  All four may instead be 4-D ``[outer, inner, rows, cols]``
+    views with arbitrary outer / inner strides (e.g. the per-head views of a packed
+    ``[batch, seq, 3 * hidden]`` projection): the two batch levels are walked by stride, nothing
+    is copied.  ``tile_variant`` forces a kernel variant (an id that
     ``select_tile`` reports); 0 leaves the choice to the library's per-shape table.
     """
-    A, B, C, F = _as3d(A, "A"), _as3d(B, "B"), _as3d(C, "C"), _as3d(F, "F")
+    (A, ao, a_so), (B, bo, b_so), (C, co, c_so), (F, fo, f_so) = (
+        _split_levels(A, "A"), _split_levels(B, "B"), _split_levels(C, "C"), _split_levels(F, "F"))
+    if not (ao == bo == co == fo):
+        raise ValueError("A, B, C, F must agree in their outer batch extent")
     batch, M, K = A.shape
     if B.shape[0] != batch or B.shape[1] != K:
         raise ValueError("B must be [batch, K, L] = [%d, %d, L], got %s" % (batch, K, tuple(B.shape)))
@@ -85,7 +99,10 @@ def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale
         d.b_row_stride = B.stride(2)
     else:
         raise ValueError("B must be contiguous along L or along K")
-    d.batch, d.M, d.N, d.K, d.L = batch, M, N, K, L
+    d.batch, d.M, d.N, d.K, d.L = batch * ao, M, N, K, L
+    d.batch_inner = batch if ao > 1 else 0
+    d.a_batch_stride_outer, d.b_batch_stride_outer = a_so, b_so
+    d.c_batch_stride_outer, d.f_batch_stride_outer = c_so, f_so
     d.a_batch_stride, d.a_row_stride = A.stride(0), A.stride(1)
     d.b_batch_stride = B.stride(0)
     d.c_batch_stride, d.c_row_stride = C.stride(0), C.stride(1)

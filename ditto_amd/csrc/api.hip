@@ -66,6 +66,11 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
                 DITTO_CHAIN_ABI_VERSION);
   if (d->reserved != 0) return fail(DITTO_EINVAL, "descriptor field `reserved` must be 0");
   if (d->tile_variant < 0) return fail(DITTO_EINVAL, "tile_variant must be 0 or a variant id");
+  if (d->batch_inner < 0 || (d->batch_inner > 0 && d->batch > 0 && d->batch % d->batch_inner != 0))
+    return fail(DITTO_EINVAL, "batch_inner must be 0 or divide batch");
+  const bool two_level = d->batch_inner > 0 && d->batch_inner != d->batch;
+  if (two_level && d->in_dtype != DITTO_F16 && d->in_dtype != DITTO_BF16)
+    return fail(DITTO_EUNSUPPORTED, "two-level batch strides are implemented for the fp16/bf16 chains");
   if (d->batch <= 0 || d->M <= 0 || d->N <= 0 || d->K <= 0 || d->L <= 0)
     return fail(DITTO_EINVAL, "batch, M, N, K, L must be positive (got %lld %lld %lld %lld %lld)",
                 (long long)d->batch, (long long)d->M, (long long)d->N, (long long)d->K,
@@ -95,6 +100,9 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     if (d->a_row_stride % 8 || d->b_row_stride % 8 || d->c_row_stride % 8 || d->a_batch_stride % 8 ||
         d->b_batch_stride % 8 || d->c_batch_stride % 8)
       return fail(DITTO_EINVAL, "input strides must be multiples of 8 elements");
+    if (two_level && (d->a_batch_stride_outer % 8 || d->b_batch_stride_outer % 8 || d->c_batch_stride_outer % 8 ||
+                      d->f_batch_stride_outer % 4))
+      return fail(DITTO_EINVAL, "outer batch strides must be multiples of 8 (inputs) / 4 (output) elements");
     const int out_vec = 4;
     if (d->f_row_stride % out_vec || d->f_batch_stride % out_vec)
       return fail(DITTO_EINVAL, "output strides must be multiples of 4 elements");
@@ -369,6 +377,14 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     args.b_bs = d->b_batch_stride;
     args.c_bs = d->c_batch_stride;
     args.f_bs = d->f_batch_stride;
+    {
+      const bool two = d->batch_inner > 0 && d->batch_inner != d->batch;
+      args.batch_inner = two ? (int)d->batch_inner : (int)d->batch;
+      args.a_bs2 = two ? d->a_batch_stride_outer : 0;
+      args.b_bs2 = two ? d->b_batch_stride_outer : 0;
+      args.c_bs2 = two ? d->c_batch_stride_outer : 0;
+      args.f_bs2 = two ? d->f_batch_stride_outer : 0;
+    }
     args.a_rs = (int)d->a_row_stride;
     args.b_rs = (int)d->b_row_stride;
     args.c_rs = (int)d->c_row_stride;

@@ -34,7 +34,9 @@ struct BmmChainArgs {
   const void* b;
   const void* c;
   void* f;
-  long long a_bs, b_bs, c_bs, f_bs;  // batch strides, elements
+  long long a_bs, b_bs, c_bs, f_bs;  // batch strides, elements (inner level)
+  long long a_bs2, b_bs2, c_bs2, f_bs2;  // outer-level batch strides
+  int batch_inner;                   // entries of the inner batch level (= batch: single level)
   int a_rs, b_rs, c_rs, f_rs;        // row strides, elements
   int M, N, K, L, batch;
   int mblocks;       // workgroups per batch entry
@@ -104,9 +106,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
   const int mb = lid % p.mblocks;
   const int bz = lid / p.mblocks;
-  const T* __restrict__ Ag = reinterpret_cast<const T*>(p.a) + (long long)bz * p.a_bs;
-  const T* Bg = reinterpret_cast<const T*>(p.b) + (long long)bz * p.b_bs;
-  const T* Cg = reinterpret_cast<const T*>(p.c) + (long long)bz * p.c_bs;
+  // batch entry bz = zo * batch_inner + zi
+  const int zo = bz / p.batch_inner, zi = bz - zo * p.batch_inner;
+  const T* __restrict__ Ag = reinterpret_cast<const T*>(p.a) + zo * p.a_bs2 + zi * p.a_bs;
+  const T* Bg = reinterpret_cast<const T*>(p.b) + zo * p.b_bs2 + zi * p.b_bs;
+  const T* Cg = reinterpret_cast<const T*>(p.c) + zo * p.c_bs2 + zi * p.c_bs;
   const int m_wave = mb * BM + wave * 32 * QT;
   const int M = p.M, N = p.N, K = p.K, L = p.L;
 
@@ -442,7 +446,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         if (n >= N) continue;
         const float v0 = o[t][j][4 * q4 + 0] * inv, v1 = o[t][j][4 * q4 + 1] * inv;
         const float v2 = o[t][j][4 * q4 + 2] * inv, v3 = o[t][j][4 * q4 + 3] * inv;
-        const long long off = (long long)bz * p.f_bs + (long long)row * p.f_rs + n;
+        const long long off = zo * p.f_bs2 + zi * p.f_bs + (long long)row * p.f_rs + n;
         if (p.out_f32) {
           f32x4 w = {v0, v1, v2, v3};
           *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.f) + off) = w;

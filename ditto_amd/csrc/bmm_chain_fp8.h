@@ -69,9 +69,11 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
   const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
   const int mb = lid % p.mblocks;
   const int bz = lid / p.mblocks;
-  const T* __restrict__ Ag = reinterpret_cast<const T*>(p.a) + (long long)bz * p.a_bs;
-  const T* Bg = reinterpret_cast<const T*>(p.b) + (long long)bz * p.b_bs;
-  const T* Cg = reinterpret_cast<const T*>(p.c) + (long long)bz * p.c_bs;
+  // batch entry bz = zo * batch_inner + zi
+  const int zo = bz / p.batch_inner, zi = bz - zo * p.batch_inner;
+  const T* __restrict__ Ag = reinterpret_cast<const T*>(p.a) + zo * p.a_bs2 + zi * p.a_bs;
+  const T* Bg = reinterpret_cast<const T*>(p.b) + zo * p.b_bs2 + zi * p.b_bs;
+  const T* Cg = reinterpret_cast<const T*>(p.c) + zo * p.c_bs2 + zi * p.c_bs;
   const int m_wave = mb * BM + wave * 32;
   const int M = p.M, N = p.N, K = p.K, L = p.L;
 
@@ -367,7 +369,7 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
         if (n >= N) continue;
         const float v0 = o[t][4 * q4 + 0] * inv, v1 = o[t][4 * q4 + 1] * inv;
         const float v2 = o[t][4 * q4 + 2] * inv, v3 = o[t][4 * q4 + 3] * inv;
-        const long long off = (long long)bz * p.f_bs + (long long)row * p.f_rs + n;
+        const long long off = zo * p.f_bs2 + zi * p.f_bs + (long long)row * p.f_rs + n;
         if (p.out_f32) {
           f32x4 w = {v0, v1, v2, v3};
           *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.f) + off) = w;

@@ -89,6 +89,14 @@ typedef struct ditto_bmm_chain_desc {
                             an explicit CUDATensorizeParam, hyper_fusion.cc:586-607);
                             DITTO_EINVAL if that variant cannot run the shape              */
   int32_t reserved;      /* must be 0 */
+  /* Two-level batch (fp16/bf16 chains): batch entry z = zo * batch_inner + zi lives at
+   * zo * x_batch_stride_outer + zi * x_batch_stride.  This is how an attention caller hands
+   * over [batch, heads] without the reshape/transpose copies of
+   * nn/module/self_attention.py:47-57,71-73: heads are the inner level with stride head_dim,
+   * the outer stride is one sequence of the packed projection.  batch_inner = 0 (or = batch):
+   * single level, the outer strides are ignored. */
+  int64_t batch_inner;
+  int64_t a_batch_stride_outer, b_batch_stride_outer, c_batch_stride_outer, f_batch_stride_outer;
 } ditto_bmm_chain_desc;
 
 /*

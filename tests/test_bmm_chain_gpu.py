@@ -242,6 +242,38 @@ def test_attention_full_size_bf16_long_sequence(oracle, variant):
     assert bool(((a - b).abs() <= 2.0 ** -7 * b.abs() + 1e-6).all())
 
 
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("cfg", [(2, 3, 200, 64), (1, 16, 256, 128), (8, 12, 512, 64)])
+def test_multi_head_attention_module(oracle, dtype, cfg):
+    # packed [batch, M, 3*hidden] projection in, [batch, M, hidden] out, heads walked by stride;
+    # checked against the reference's own formulation (split, reshape, transpose, chain, merge:
+    # nn/module/self_attention.py:46-73) evaluated in fp64 on the CPU
+    from ditto_amd import auto_compute as ac
+
+    batch, heads, M, d = cfg
+    hidden = heads * d
+    rng = np.random.default_rng(heads + M)
+    qkv = oracle.np_round_to(rng.standard_normal((batch, M, 3 * hidden)).astype(np.float32), dtype)
+    mha = ac.nn.module.MultiHeadAttentionMMA(heads, hidden, in_dtype=dtype, scale=None)
+    x = to_dev(qkv, dtype)
+    out = mha(x)
+    torch.cuda.synchronize()
+    assert out.shape == (batch, M, hidden) and out.is_contiguous()
+    q, k, v = (qkv[:, :, i * hidden:(i + 1) * hidden].reshape(batch, M, heads, d).transpose(0, 2, 1, 3)
+               .reshape(batch * heads, M, d) for i in range(3))
+    want = oracle.bmm_chain_f64(q, np.ascontiguousarray(k.transpose(0, 2, 1)), v, inter="softmax", scale=d ** -0.5)
+    want = want.reshape(batch, heads, M, d).transpose(0, 2, 1, 3).reshape(batch, M, hidden)
+    mx, rel = errors(out.float().cpu().numpy(), want)
+    assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (mx, rel)
+    # same numbers as the chain on materialised per-head tensors (bit for bit: same kernel, same order)
+    qd, kd, vd = (to_dev(np.ascontiguousarray(t), dtype) for t in (q, k, v))
+    ref = torch.empty(batch * heads, M, d, device=x.device, dtype=x.dtype)
+    chain.run_bmm_chain(qd, kd.transpose(1, 2), vd, ref, "softmax", d ** -0.5,
+                        tile_variant=chain.select_tile(chain.bmm_chain_desc(*mha.head_views(x), out.view(batch, M, heads, d).permute(0, 2, 1, 3), "softmax", d ** -0.5)).variant)
+    torch.cuda.synchronize()
+    assert torch.equal(ref.view(batch, heads, M, d).permute(0, 2, 1, 3).reshape(batch, M, hidden), out)
+
+
 def test_strided_views_and_errors():
     dev = "cuda:0"
     torch.manual_seed(0)

@@ -158,3 +158,29 @@ def test_conv_chain_recognition():
     assert sch.dims["C1"] == 128 and sch.dims["pad1"] == 1 and sch.dims["R2"] == 1
     func = ditto.build(sch, layer.schedule_tensors, "hip")
     assert func.entry_name == "default_function" and len(func.tensors) == 4
+
+
+def test_multi_head_attention_views_map_onto_two_level_strides():
+    # the head split / merge of nn/module/self_attention.py:46-73 as strides of the chain descriptor
+    import torch
+    from ditto_amd import auto_compute as ac, chain
+
+    batch, heads, M, d = 4, 16, 128, 64
+    hidden = heads * d
+    mha = ac.nn.module.MultiHeadAttentionMMA(heads, hidden, in_dtype="float16")
+    assert mha.name == "multi_head_attention_mma_layer" and ac.nn.module.is_self_attention_layer(mha)
+    qkv = torch.zeros(batch, M, 3 * hidden, dtype=torch.float16)
+    out = torch.zeros(batch, M, hidden, dtype=torch.float16)
+    q, k, v = mha.head_views(qkv)
+    assert q.shape == (batch, heads, M, d) and k.shape == (batch, heads, d, M) and v.shape == q.shape
+    assert q.data_ptr() == qkv.data_ptr() and k.data_ptr() == qkv.data_ptr() + 2 * hidden
+    desc = chain.bmm_chain_desc(q, k, v, out.view(batch, M, heads, d).permute(0, 2, 1, 3), "softmax", 0.125)
+    assert (desc.batch, desc.batch_inner, desc.M, desc.K, desc.L, desc.N) == (batch * heads, heads, M, d, M, d)
+    assert desc.b_layout == 1  # keys stay [L][K]
+    assert (desc.a_batch_stride, desc.a_batch_stride_outer, desc.a_row_stride) == (d, M * 3 * hidden, 3 * hidden)
+    assert (desc.f_batch_stride, desc.f_batch_stride_outer, desc.f_row_stride) == (d, M * hidden, hidden)
+    tile = chain.select_tile(desc)  # valid for the library
+    assert tile.head_pad == 64
+    import pytest
+    with pytest.raises(RuntimeError):
+        mha.head_views(torch.zeros(batch, M, 3 * hidden + 8, dtype=torch.float16))
