@@ -73,3 +73,12 @@ def Conv3x3Conv1x1(batch, in_channel, H, W, out_channel1, out_channel2, stride1=
     assert stride2 == 1
     return conv_chain(batch, in_channel, H, W, out_channel1, 3, 3, out_channel2, 1, 1, 1, 0, stride1, stride2,
                       in_dtype, acc_dtype)
+
+
+def Conv1x1Conv3x3(batch, in_channel, H, W, out_channel1, out_channel2, stride1=1, stride2=1,
+                   in_dtype="float16", acc_dtype="float32"):
+    """conv1x1 -> cast -> conv3x3 (pad 1, zero padding of the intermediate); argument list of
+    benchmark/chimera/cuda/conv1x1_conv3x3_cuda.py:77-88."""
+    assert stride2 == 1
+    return conv_chain(batch, in_channel, H, W, out_channel1, 1, 1, out_channel2, 3, 3, 0, 1, stride1, stride2,
+                      in_dtype, acc_dtype)

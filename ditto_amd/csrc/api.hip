@@ -238,6 +238,8 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
 }
 
 struct ConvPlan {
+  int px2;             // 0: 1x1 second convolution; 1 | 2: larger one, output-pixel tiles per wave
+  size_t w2p_bytes;    // size of the repacked W2 (second part of the workspace, px2 > 0)
   int c1_tiles;
   int ch;              // input channels per staged chunk
   size_t w1p_bytes;    // size of the repacked W1 (the workspace)
@@ -259,10 +261,11 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan) {
   if (d->N <= 0 || d->C0 <= 0 || d->H <= 0 || d->W <= 0 || d->C1 <= 0 || d->C2 <= 0 || d->R1 <= 0 ||
       d->S1 <= 0 || d->R2 <= 0 || d->S2 <= 0 || d->stride1 <= 0 || d->stride2 <= 0 || d->pad1 < 0 || d->pad2 < 0)
     return fail(DITTO_EINVAL, "conv extents must be positive and paddings non-negative");
-  if (d->R2 != 1 || d->S2 != 1 || d->pad2 != 0 || d->stride2 != 1)
+  const bool second_1x1 = d->R2 == 1 && d->S2 == 1 && d->pad2 == 0;
+  if (d->stride2 != 1) return fail(DITTO_EUNSUPPORTED, "the second convolution must have stride 1");
+  if (!second_1x1 && (d->R2 > 3 || d->S2 > 3 || d->C1 > 64))
     return fail(DITTO_EUNSUPPORTED,
-                "the fused conv chain needs a 1x1, stride 1, unpadded second convolution (got %lldx%lld)",
-                (long long)d->R2, (long long)d->S2);
+                "a second convolution larger than 1x1 takes filters up to 3x3 and at most 64 intermediate channels");
   if (d->C1 % 8) return fail(DITTO_EINVAL, "C1 must be a multiple of 8");
   if (d->C1 > 256) return fail(DITTO_EUNSUPPORTED, "C1=%lld: at most 256 intermediate channels", (long long)d->C1);
   if (d->R1 > 7 || d->S1 > 7) return fail(DITTO_EUNSUPPORTED, "first filter larger than 7x7");
@@ -281,6 +284,49 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan) {
   a.N = (int)d->N; a.C0 = (int)d->C0; a.H = (int)d->H; a.W = (int)d->W;
   a.C1 = (int)d->C1; a.R = (int)d->R1; a.S = (int)d->S1; a.pad = (int)d->pad1; a.stride = (int)d->stride1;
   a.C2 = (int)d->C2; a.P = (int)P; a.Q = (int)Q;
+  if (!second_1x1) {
+    // The first convolution produces the output tile grown by the second filter's halo (recomputed
+    // per workgroup) into at most `slots` pixel slots; the second reads it from LDS.
+    const long long P2 = P + 2 * d->pad2 - d->R2 + 1, Q2 = Q + 2 * d->pad2 - d->S2 + 1;
+    if (P2 <= 0 || Q2 <= 0) return fail(DITTO_EINVAL, "empty convolution output");
+    if (d->N * d->C2 * P2 * Q2 > 0x7fffffffLL * 4) return fail(DITTO_EINVAL, "tensor too large");
+    a.R2 = (int)d->R2; a.S2 = (int)d->S2; a.pad2 = (int)d->pad2; a.P2 = (int)P2; a.Q2 = (int)Q2;
+    a.TW2 = (int)Q2;
+    while ((a.TW2 + a.S2 - 1) * a.R2 > slots) a.TW2 = (a.TW2 + 1) / 2;
+    a.TW = a.TW2 + a.S2 - 1;
+    a.TH = slots / a.TW;
+    if (a.TH > P2 + a.R2 - 1) a.TH = (int)P2 + a.R2 - 1;
+    a.TH2 = a.TH - (a.R2 - 1);
+    a.rows_in = (a.TH - 1) * a.stride + a.R;
+    a.cols_in = (a.TW - 1) * a.stride + a.S;
+    const int RS1 = a.R * a.S;
+    int lds = ditto::conv_chain_lds_bytes(a.rows_in, a.cols_in, RS1, 32 * c1t, 32);
+    const int lds2 = ditto::conv_chain2_lds_bytes(slots, 32 * c1t, a.R2 * a.S2);
+    if (lds2 > lds) lds = lds2;
+    if (lds > 160 * 1024) return fail(DITTO_EUNSUPPORTED, "conv chain tile does not fit in LDS");
+    a.tiles_h = (int)((P2 + a.TH2 - 1) / a.TH2);
+    a.tiles_w = (int)((Q2 + a.TW2 - 1) / a.TW2);
+    a.relu_mid = d->inter_op == DITTO_INTER_RELU;
+    a.relu_out = d->relu_out != 0;
+    a.out_f32 = d->out_dtype == DITTO_F32;
+    plan->c1_tiles = c1t;
+    plan->ch = 32;
+    plan->px2 = a.TH2 * a.TW2 <= 128 ? 1 : 2;
+    plan->w1p_bytes = ((size_t)ditto::conv_w1_chunk_bytes(RS1, 32 * c1t, 32) * (size_t)((d->C0 + 31) / 32) + 255) / 256 * 256;
+    plan->w2p_bytes = (size_t)ditto::conv_w2_chunk_bytes(a.R2 * a.S2) * (size_t)((d->C2 + 63) / 64) * (size_t)c1t;
+    ditto_tile_param& t = plan->tile;
+    t.block_threads = 256;
+    t.block_m = a.TH2 * a.TW2;
+    t.block_l = 32 * c1t;
+    t.block_n = (int)d->C2;
+    t.head_pad = 32;
+    t.lds_bytes = lds;
+    t.grid_x = a.N * a.tiles_h * a.tiles_w;
+    t.grid_y = a.TH2;
+    t.grid_z = a.TW2;
+    t.variant = 3500 + c1t * 10 + plan->px2;  // second convolution through LDS
+    return DITTO_OK;
+  }
   a.TW = (int)(Q < slots ? Q : slots);
   a.TH = slots / a.TW;
   if (a.TH > P) a.TH = (int)P;
@@ -479,7 +525,7 @@ int ditto_conv_chain_select_tile(const ditto_conv_chain_desc* desc, ditto_tile_p
 size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
   ConvPlan plan;
   if (plan_conv(desc, &plan) != DITTO_OK) return 0;
-  return plan.w1p_bytes;
+  return plan.w1p_bytes + plan.w2p_bytes;
 }
 
 int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const void* w1, const void* w2,
@@ -490,8 +536,11 @@ int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const vo
   if (!x || !w1 || !w2 || !y) return fail(DITTO_EINVAL, "null data pointer");
   if (!aligned(x, 2) || !aligned(w1, 2) || !aligned(w2, 8) || !aligned(y, 4))
     return fail(DITTO_EINVAL, "misaligned data pointer");
-  if (workspace && workspace_bytes < plan.w1p_bytes)
-    return fail(DITTO_EWORKSPACE, "workspace of %zu bytes, need %zu", workspace_bytes, plan.w1p_bytes);
+  const size_t need = plan.w1p_bytes + plan.w2p_bytes;
+  if (plan.px2 > 0 && !workspace)
+    return fail(DITTO_EWORKSPACE, "a second convolution larger than 1x1 needs the workspace (%zu bytes)", need);
+  if (workspace && workspace_bytes < need)
+    return fail(DITTO_EWORKSPACE, "workspace of %zu bytes, need %zu", workspace_bytes, need);
   if (workspace && !aligned(workspace, 16)) return fail(DITTO_EINVAL, "workspace must be 16-byte aligned");
   ditto::ConvChainArgs a = plan.args;
   a.x = x;
@@ -505,8 +554,16 @@ int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const vo
   if (workspace)  // W1 into the chunked layout the chain kernel copies straight into LDS
     e = f16 ? ditto::pack_conv_w1_f16(plan.c1_tiles, plan.ch, a, workspace, st)
             : ditto::pack_conv_w1_bf16(plan.c1_tiles, plan.ch, a, workspace, st);
-  if (e == hipSuccess)
+  if (plan.px2 > 0) {
+    void* w2p = static_cast<char*>(workspace) + plan.w1p_bytes;
+    a.w2p = w2p;
+    if (e == hipSuccess)
+      e = f16 ? ditto::pack_conv_w2_f16(plan.c1_tiles, a, w2p, st) : ditto::pack_conv_w2_bf16(plan.c1_tiles, a, w2p, st);
+    if (e == hipSuccess)
+      e = f16 ? ditto::launch_conv2_f16(plan.c1_tiles, plan.px2, a, st) : ditto::launch_conv2_bf16(plan.c1_tiles, plan.px2, a, st);
+  } else if (e == hipSuccess) {
     e = f16 ? ditto::launch_conv_f16(plan.c1_tiles, plan.ch, a, st) : ditto::launch_conv_bf16(plan.c1_tiles, plan.ch, a, st);
+  }
   if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
   return DITTO_OK;
 }

@@ -41,6 +41,12 @@ struct ConvChainArgs {
   int tiles_h, tiles_w;
   int rows_in, cols_in;  // halo tile extent
   int relu_mid, relu_out, out_f32;
+  // second convolution larger than 1x1 (stride 1): then P, Q, TH, TW above describe the
+  // INTERMEDIATE tile (the output tile grown by the second filter's halo) and these the output
+  const void* w2p;   // W2 repacked by pack_conv_w2
+  int R2, S2, pad2;
+  int P2, Q2;        // output extent
+  int TH2, TW2;      // output tile per workgroup
 };
 
 // Input channels per staged chunk: 32 (two MFMA k steps per tap) or, where that does not fit in
@@ -56,6 +62,34 @@ __host__ __device__ inline int conv_chain_lds_bytes(int rows_in, int cols_in, in
   const int first = rows_in * cols_in * conv_ch_stride(ch) * 2 + (conv_w1_chunk_bytes(RS, C1p, ch) + 1023) / 1024 * 1024;
   const int second = 32 * (C1p + 4) * 2;  // at least 32 rows of W2
   return first > second ? first : second;
+}
+
+// Second convolution larger than 1x1: the intermediate tile lives in LDS as [slot][C1p + 8] and W2
+// streams through two buffers of [R2*S2][64 output channels][32 + 8] (chunks of 32 intermediate
+// channels for blocks of 64 output channels).
+__host__ __device__ inline int conv_w2_chunk_bytes(int RS2) { return RS2 * 64 * conv_ch_stride(32) * 2; }
+__host__ __device__ inline int conv_chain2_lds_bytes(int slots, int C1p, int RS2) {
+  return slots * (C1p + 8) * 2 + 2 * ((conv_w2_chunk_bytes(RS2) + 1023) / 1024 * 1024);
+}
+
+// W2[c2][c1][r][s] -> [c2 / 64][c1 / 32][r*S+s][64][32 + 8] (zero padded)
+template <typename T>
+__global__ void pack_conv_w2_kernel(const T* __restrict__ w2, T* __restrict__ out, int C1, int C2, int RS2, int C1p,
+                                    long long total) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int c = (int)(i % 40);
+  long long q = i / 40;
+  const int c2l = (int)(q % 64);
+  q /= 64;
+  const int tap = (int)(q % RS2);
+  q /= RS2;
+  const int chunk = (int)(q % (C1p / 32));
+  const int c2b = (int)(q / (C1p / 32));
+  const int c1 = chunk * 32 + c, c2 = c2b * 64 + c2l;
+  T v = (T)0.f;
+  if (c < 32 && c1 < C1 && c2 < C2) v = w2[((long long)c2 * C1 + c1) * RS2 + tap];
+  out[i] = v;
 }
 
 // W1[c1][c0][r][s] -> chunks [c0 / ch][r*S+s][C1p][ch + 8] (zero padded): the layout the chain
@@ -78,7 +112,10 @@ __global__ void pack_conv_w1_kernel(const T* __restrict__ w1, T* __restrict__ ou
   out[i] = v;
 }
 
-template <typename T, int C1T, int PXW, int CH>
+// PX2 = 0: the second convolution is 1x1 and consumes the first one's accumulators from registers;
+// PX2 = 1 | 2: it is R2 x S2 (stride 1) and reads the intermediate tile from LDS, PX2 tiles of 32
+// output pixels per wave.
+template <typename T, int C1T, int PXW, int CH, int PX2 = 0>
 __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef typename Elem<T>::v8 V8;
@@ -100,7 +137,8 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
   const int tiles = p.tiles_h * p.tiles_w;
   const int n = lid / tiles;
   const int th = (lid % tiles) / p.tiles_w, tw = (lid % tiles) % p.tiles_w;
-  const int p0 = th * p.TH, q0 = tw * p.TW;
+  // origin of the tile the FIRST convolution produces (the intermediate tile when PX2 > 0)
+  const int p0 = PX2 ? th * p.TH2 - p.pad2 : th * p.TH, q0 = PX2 ? tw * p.TW2 - p.pad2 : tw * p.TW;
   const int h0 = p0 * p.stride - p.pad, w0 = q0 * p.stride - p.pad;  // input coords of the halo origin
 
   const T* __restrict__ Xg = reinterpret_cast<const T*>(p.x) + (long long)n * p.C0 * p.H * p.W;
@@ -115,7 +153,7 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
   for (int j = 0; j < PXW; ++j) {
     const int slot = 32 * (PXW * wave + j) + ln;
     const int ph = slot / p.TW, pw = slot % p.TW;
-    valid[j] = ph < p.TH && (p0 + ph) < p.P && (q0 + pw) < p.Q;
+    valid[j] = ph < p.TH && (p0 + ph) >= 0 && (p0 + ph) < p.P && (q0 + pw) >= 0 && (q0 + pw) < p.Q;
     const int phc = valid[j] ? ph : 0, pwc = valid[j] ? pw : 0;
     xoff[j] = ((phc * p.stride) * p.cols_in + pwc * p.stride) * CHS + 8 * g;
     opix[j] = (p0 + phc) * p.Q + q0 + pwc;
@@ -284,7 +322,7 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (x_prefetch && c0 + CH < p.C0) xv_load(c0 + CH, t_chg, t_gi, t_ri, tid < xtasks);  // in flight during the MFMAs
-    if (w2_prefetch && c0 + CH >= p.C0) {
+    if (PX2 == 0 && w2_prefetch && c0 + CH >= p.C0) {
 #pragma unroll
       for (int k = 0; k < 8; ++k) xr[k] = w2_load(0, tid + 256 * k);
     }
@@ -308,6 +346,120 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
 #pragma unroll
             for (int j = 0; j < PXW; ++j) acc[c][j] = Elem<T>::mfma32(wf[kk][c], xf[kk][j], acc[c][j]);
       }
+  }
+
+  if constexpr (PX2 > 0) {
+    // ================= second convolution R2 x S2, intermediate tile through LDS =================
+    constexpr int MS = C1p + 8;  // element stride of an intermediate pixel's channel vector
+    T* const Ms = reinterpret_cast<T*>(smem_raw);  // [128*PXW][MS]
+    T* const W2b = Ms + 128 * PXW * MS;            // two chunk buffers
+    const int RS2 = p.R2 * p.S2;
+    const int w2_bytes = conv_w2_chunk_bytes(RS2);
+    const int w2_buf = (w2_bytes + 1023) / 1024 * 1024;
+    constexpr int nch2 = C1p / 32;
+    const int nc2b = (p.C2 + 63) / 64;
+    const int nstage = nc2b * nch2;
+    const i32x4 w2_rsrc = make_rsrc(p.w2p, (unsigned)(w2_bytes * nstage));
+    const unsigned w2_lds = (unsigned)(size_t)(DITTO_LDS char*)smem_raw + 128 * PXW * MS * 2;
+    auto w2_issue = [&](int stage) __attribute__((always_inline)) {
+      for (int j = wave; j * 1024 < w2_bytes; j += 4) {
+        const int off = j * 1024 + lane * 16;
+        lds_dma_16(w2_rsrc, off < w2_bytes ? (unsigned)(stage * w2_bytes + off) : 0x7fffffffu,
+                   w2_lds + (stage & 1) * w2_buf + j * 1024);
+      }
+    };
+    __syncthreads();  // the first convolution's LDS is no longer read
+    w2_issue(0);
+    // intermediate -> LDS: inter op, cast, zero outside the first convolution's output (that is the
+    // second one's padding); 4 consecutive channels per register quad
+#pragma unroll
+    for (int c = 0; c < C1T; ++c)
+#pragma unroll
+      for (int j = 0; j < PXW; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] = valid[j] ? acc[c][j][4 * q + e] : 0.f;
+            if (p.relu_mid) v[e] = fmaxf(v[e], 0.f);
+          }
+          const typename Elem<T>::v2 a0 = cvt2<T>(v[0], v[1]), a1 = cvt2<T>(v[2], v[3]);
+          const V4 w = {a0[0], a0[1], a1[0], a1[1]};
+          *reinterpret_cast<V4*>(Ms + (32 * (PXW * wave + j) + ln) * MS + 32 * c + 8 * q + 4 * g) = w;
+        }
+    // output pixel slots of this lane
+    int moff[PX2];
+    bool valid2[PX2];
+    long long opix2[PX2];
+    const int op0 = th * p.TH2, oq0 = tw * p.TW2;
+#pragma unroll
+    for (int j = 0; j < PX2; ++j) {
+      const int slot = 32 * (PX2 * wave + j) + ln;
+      const int oh = slot / p.TW2, ow = slot % p.TW2;
+      valid2[j] = oh < p.TH2 && op0 + oh < p.P2 && oq0 + ow < p.Q2;
+      const int ohc = valid2[j] ? oh : 0, owc = valid2[j] ? ow : 0;
+      moff[j] = (ohc * p.TW + owc) * MS + 8 * g;
+      opix2[j] = (long long)(op0 + ohc) * p.Q2 + oq0 + owc;
+    }
+    const long long plane2 = (long long)p.P2 * p.Q2;
+    f32x16 o[2][PX2];
+    for (int stage = 0; stage < nstage; ++stage) {
+      const int c2b = stage / nch2, ch = stage % nch2;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();  // this stage's chunk has landed; everyone is done with the previous one
+      if (stage + 1 < nstage) w2_issue(stage + 1);
+      if (ch == 0) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < PX2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[t][j][r] = 0.f;
+      }
+      const T* wbuf = reinterpret_cast<const T*>(reinterpret_cast<const char*>(W2b) + (stage & 1) * w2_buf);
+      for (int r = 0; r < p.R2; ++r)
+        for (int s2 = 0; s2 < p.S2; ++s2) {
+          const int tap = (r * p.TW + s2) * MS + 32 * ch;
+          const T* wrow = wbuf + ((r * p.S2 + s2) * 64 + ln) * 40 + 8 * g;
+          V8 mf[2][PX2], wf[2][2];
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+            for (int j = 0; j < PX2; ++j) mf[kk][j] = *reinterpret_cast<const V8*>(Ms + moff[j] + tap + 16 * kk);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) wf[kk][t] = *reinterpret_cast<const V8*>(wrow + 32 * t * 40 + 16 * kk);
+          }
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+              for (int j = 0; j < PX2; ++j) o[t][j] = Elem<T>::mfma32(wf[kk][t], mf[kk][j], o[t][j]);
+        }
+      if (ch == nch2 - 1) {
+        // o[t][j][r] = out^T[c2 = 64 c2b + 32t + 8(r/4) + 4g + r%4][pixel of lane]
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < PX2; ++j) {
+            if (!valid2[j]) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int c2 = 64 * c2b + 32 * t + 8 * (r >> 2) + 4 * g + (r & 3);
+              if (c2 >= p.C2) continue;
+              float v = o[t][j][r];
+              if (p.relu_out) v = fmaxf(v, 0.f);
+              const long long off = ((long long)n * p.C2 + c2) * plane2 + opix2[j];
+              if (p.out_f32)
+                reinterpret_cast<float*>(p.y)[off] = v;
+              else
+                reinterpret_cast<T*>(p.y)[off] = (T)v;
+            }
+          }
+      }
+    }
+    return;
   }
 
   // ---- second convolution (1x1): W2 blocks go through the LDS the first convolution has finished
@@ -418,10 +570,14 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
 #endif
 }
 
-template <typename T, int C1T, int PXW, int CH>
+template <typename T, int C1T, int PXW, int CH, int PX2 = 0>
 hipError_t launch_conv_chain(const ConvChainArgs& args, hipStream_t stream) {
-  const int lds = conv_chain_lds_bytes(args.rows_in, args.cols_in, args.R * args.S, 32 * C1T, CH);
-  auto kern = conv_chain_kernel<T, C1T, PXW, CH>;
+  int lds = conv_chain_lds_bytes(args.rows_in, args.cols_in, args.R * args.S, 32 * C1T, CH);
+  if (PX2 > 0) {
+    const int lds2 = conv_chain2_lds_bytes(128 * PXW, 32 * C1T, args.R2 * args.S2);
+    if (lds2 > lds) lds = lds2;
+  }
+  auto kern = conv_chain_kernel<T, C1T, PXW, CH, PX2>;
   static thread_local int configured_dev = -1;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -446,6 +602,17 @@ hipError_t launch_pack_conv_w1(const ConvChainArgs& args, int C1p, int ch, void*
   const unsigned grid = (unsigned)((total + 255) / 256);
   hipLaunchKernelGGL(pack_conv_w1_kernel<T>, dim3(grid), dim3(256), 0, stream, reinterpret_cast<const T*>(args.w1),
                      reinterpret_cast<T*>(out), args.C0, args.C1, RS, C1p, ch, total);
+  return hipGetLastError();
+}
+
+// repack W2 for a second convolution larger than 1x1 (conv_w2_chunk_bytes * blocks * chunks bytes)
+template <typename T>
+hipError_t launch_pack_conv_w2(const ConvChainArgs& args, int C1p, void* out, hipStream_t stream) {
+  const int RS2 = args.R2 * args.S2;
+  const long long total = (long long)((args.C2 + 63) / 64) * (C1p / 32) * RS2 * 64 * 40;
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  hipLaunchKernelGGL(pack_conv_w2_kernel<T>, dim3(grid), dim3(256), 0, stream, reinterpret_cast<const T*>(args.w2),
+                     reinterpret_cast<T*>(out), args.C1, args.C2, RS2, C1p, total);
   return hipGetLastError();
 }
 

@@ -51,6 +51,10 @@ CONV3X3_CONV1X1_SHAPES = [
     (128, 28, 28, 256, 128, 1, 1),  # Darknet-19
     (16, 227, 227, 64, 16, 4, 1),  # Squeezenet-V1.1
 ]
+# (C, H, W, K1, K2, stride1, stride2): conv1x1_conv3x3_cuda.py:348-350
+CONV1X1_CONV3X3_SHAPES = [
+    (64, 56, 56, 64, 64, 1, 1),  # ResNet-50
+]
 
 
 def cal_ai(B, M, N, K, L):

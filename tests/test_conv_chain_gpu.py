@@ -11,14 +11,15 @@ pytestmark = pytest.mark.gpu
 MAX_ABS, REL_L2, REL_L2_BF16_QUANT = 1e-2, 1e-3, 3e-3
 
 
-def run_conv(X, W1, W2, dtype, pad1=1, stride1=1, inter="cast", relu_out=False, out_dtype=None, workspace=None):
+def run_conv(X, W1, W2, dtype, pad1=1, stride1=1, inter="cast", relu_out=False, out_dtype=None, workspace=None,
+             pad2=0):
     x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
     N, _, H, W = X.shape
     R, S = W1.shape[2:]
-    P = (H + 2 * pad1 - R) // stride1 + 1
-    Q = (W + 2 * pad1 - S) // stride1 + 1
+    P = (H + 2 * pad1 - R) // stride1 + 1 + 2 * pad2 - W2.shape[2] + 1
+    Q = (W + 2 * pad1 - S) // stride1 + 1 + 2 * pad2 - W2.shape[3] + 1
     y = torch.full((N, W2.shape[0], P, Q), float("nan"), device=x.device, dtype=TORCH_DTYPES[out_dtype or dtype])
-    chain.run_conv_chain(x, w1, w2, y, pad1, stride1, 0, 1, inter, relu_out, workspace=workspace)
+    chain.run_conv_chain(x, w1, w2, y, pad1, stride1, pad2, 1, inter, relu_out, workspace=workspace)
     torch.cuda.synchronize()
     return y.float().cpu().numpy()
 
@@ -52,6 +53,47 @@ def test_conv_chain_vs_oracle(oracle, case, dtype):
         assert np.array_equal(got, oracle.np_round_to(got32, dtype)), ws
         mx, rel = errors(got, oracle.np_round_to(want32, dtype))
         assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (ws, mx, rel)
+
+
+CASES_3X3_SECOND = [
+    # N, C0, H, W, C1, R1, pad1, stride1, C2, R2, pad2
+    (2, 64, 56, 56, 64, 1, 0, 1, 64, 3, 1),    # conv1x1 -> conv3x3 (conv1x1_conv3x3_cuda.py:77-189)
+    (1, 32, 20, 28, 32, 1, 0, 1, 72, 3, 1),    # C2 not a multiple of 64
+    (1, 16, 33, 45, 64, 1, 0, 2, 32, 3, 1),    # strided 1x1 first, odd extents
+    (1, 32, 18, 18, 32, 3, 1, 1, 48, 3, 1),    # conv3x3 -> conv3x3
+    (1, 16, 12, 150, 16, 1, 0, 1, 16, 3, 1),   # wider than one tile
+    (1, 16, 16, 16, 32, 3, 1, 1, 32, 3, 0),    # unpadded second convolution
+    (2, 24, 30, 30, 64, 3, 1, 1, 128, 3, 1),   # conv3x3 -> conv3x3, 64 intermediate channels, C0 % 32 != 0
+]
+
+
+@pytest.mark.parametrize("case", CASES_3X3_SECOND)
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_conv_chain_with_wide_second_filter(oracle, case, dtype):
+    N, C0, H, W, C1, R1, pad1, stride1, C2, R2, pad2 = case
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, R1, R2, dtype, seed=C0 + C2, w_std=0.05)
+    for relu in (False, True):
+        want32 = oracle.conv_chain_f32(X, W1, W2, pad1, stride1, pad2, 1, relu_mid=relu, relu_out=relu, round_mid=dtype)
+        got32 = run_conv(X, W1, W2, dtype, pad1, stride1, "relu" if relu else "cast", relu, "float32", None, pad2)
+        assert got32.shape == want32.shape and np.isfinite(got32).all()
+        mx, rel = errors(got32, want32)
+        assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
+    got = run_conv(X, W1, W2, dtype, pad1, stride1, "relu", True, None, None, pad2)
+    assert np.array_equal(got, oracle.np_round_to(got32, dtype))
+    with pytest.raises(ValueError):  # this variant cannot run without its workspace
+        run_conv(X, W1, W2, dtype, pad1, stride1, workspace=False, pad2=pad2)
+
+
+def test_conv_chain_rejects_what_it_cannot_fuse():
+    x = torch.zeros(1, 16, 14, 14, device="cuda:0", dtype=torch.float16)
+    w1 = torch.zeros(32, 16, 1, 1, device="cuda:0", dtype=torch.float16)
+    with pytest.raises(NotImplementedError):  # 5x5 second filter
+        chain.run_conv_chain(x, w1, torch.zeros(32, 32, 5, 5, device="cuda:0", dtype=torch.float16),
+                             torch.zeros(1, 32, 14, 14, device="cuda:0", dtype=torch.float16), 0, 1, 2, 1)
+    w1b = torch.zeros(128, 16, 1, 1, device="cuda:0", dtype=torch.float16)
+    with pytest.raises(NotImplementedError):  # 3x3 second filter over more than 64 intermediate channels
+        chain.run_conv_chain(x, w1b, torch.zeros(32, 128, 3, 3, device="cuda:0", dtype=torch.float16),
+                             torch.zeros(1, 32, 14, 14, device="cuda:0", dtype=torch.float16), 0, 1, 1, 1)
 
 
 def test_conv_relu_conv_relu_vs_torch(oracle):
@@ -114,7 +156,7 @@ def test_conv_chain_rejects_unsupported():
     w1 = torch.zeros(16, 16, 3, 3, device=dev, dtype=torch.float16)
     w2 = torch.zeros(16, 16, 3, 3, device=dev, dtype=torch.float16)
     y = torch.zeros(1, 16, 8, 8, device=dev, dtype=torch.float16)
-    with pytest.raises(NotImplementedError, match="1x1"):
-        chain.run_conv_chain(x, w1, w2, y, 1, 1, 1, 1)
+    with pytest.raises(NotImplementedError, match="stride 1"):  # strided second convolution
+        chain.run_conv_chain(x, w1, w2, y[:, :, :4, :4].contiguous(), 1, 1, 1, 2)
     with pytest.raises(ValueError):
         chain.run_conv_chain(x, w1, w2[:, :, :1, :1].contiguous(), y[:, :8].contiguous(), 1, 1, 0, 1)

@@ -5,7 +5,7 @@ import sys
 
 import pytest
 
-from ditto_amd.drivers import bmm_bmm, bmm_softmax_bmm, common, conv3x3_conv1x1
+from ditto_amd.drivers import bmm_bmm, bmm_softmax_bmm, common, conv1x1_conv3x3, conv3x3_conv1x1
 
 
 def test_shape_tables_match_reference():
@@ -39,6 +39,9 @@ def test_drivers_run_one_row_each(capsys):
     assert 0 < cost < 5.0  # milliseconds
     C, H, W, K1, K2, s1, s2 = common.CONV3X3_CONV1X1_SHAPES[2]
     cost = conv3x3_conv1x1.main(1, C, H, W, K1, K2, s1, s2)
+    assert 0 < cost < 5.0
+    C, H, W, K1, K2, s1, s2 = common.CONV1X1_CONV3X3_SHAPES[0]
+    cost = conv1x1_conv3x3.main(1, C, H, W, K1, K2, s1, s2)
     assert 0 < cost < 5.0
 
 
