@@ -1,0 +1,152 @@
+"""Choice of the kernel variant of a BMM chain: analytic filter, measurement, tuning log.
+
+Counterpart of python/ditto/auto_schedule/schedulers/chimera_integrate.py.  The reference
+searches a 10-dimensional CUDATensorizeParam space (:99-123) with an analytic
+capacity / traffic filter (:229-295: over-capacity -> 1e10, else waves x staged kilobytes /
+shared-memory bandwidth), measures the survivors and appends one JSON line per measurement to
+``chimera_<log_file>`` (:326-333); ``auto_schedule_build_tasks`` later keeps, per workload key,
+the entry with the smallest ``value`` (:527-537).
+
+Here the space is the library's handful of kernel variants for the shape
+(``ditto_bmm_chain_select_tile`` with ``tile_variant`` forced), the filter has the same two
+parts, and the log keeps the reference's line format
+``{"wkl_key": ..., "entry": {"record": {...}, "value": <ms>}}`` with the tile description
+as the record, so a log written here can be re-read by ``load_best_records`` / ``best_variant``
+and fed back through ``run_bmm_chain(..., tile_variant=...)``.
+"""
+import copy
+import ctypes
+import json
+import os
+
+from ... import _lib, chain
+from ...hardware import query_hw_param
+
+FP_VARIANT_CODES = (1, 2, 8)  # rows-per-wave code of the fp16/bf16 chain kernels
+
+
+class TuneEntry:
+    """One measurement: ``record`` (the tile description, JSON-able) and ``value`` (ms)."""
+
+    def __init__(self, record, value):
+        self.record = record
+        self.value = value
+
+    def to_json(self):
+        return {"record": self.record, "value": self.value}
+
+
+def make_tile_variant_space(desc):
+    """Variants of the library that can run ``desc`` (capacity filter: the library rejects the
+    ones whose tile does not fit), as a list of tile descriptions."""
+    lib = _lib.load()
+    tile = _lib.TileParam()
+    auto = copy.copy(desc)
+    auto.tile_variant = 0
+    _lib.check(lib.ditto_bmm_chain_select_tile(ctypes.byref(auto), ctypes.byref(tile)))
+    space = []
+    if desc.in_dtype in (_lib.F16, _lib.BF16):
+        for q in FP_VARIANT_CODES:
+            d = copy.copy(desc)
+            d.tile_variant = tile.head_pad * 10 + q
+            t = _lib.TileParam()
+            if lib.ditto_bmm_chain_select_tile(ctypes.byref(d), ctypes.byref(t)) == _lib.OK:
+                space.append(t.to_json())
+    else:
+        space.append(tile.to_json())
+    return space
+
+
+def evaluate_param_hip(desc, tile, hw_param=None):
+    """Analytic score of a tile (lower is better; 1e10 = over capacity), the shape of the
+    reference's filter: rounds of workgroups over the CUs x bytes each workgroup stages through
+    LDS / LDS bandwidth, plus the MFMA time of a round.  It ranks variants; it is not a time."""
+    hw = hw_param or query_hw_param("gpu.hip.MI355X")
+    if tile["lds_bytes"] > hw.shared_memory_per_group_kb * 1024:
+        return 1e10
+    groups = hw.num_groups
+    per_cu = max(1, int(hw.shared_memory_per_group_kb * 1024 // max(tile["lds_bytes"], 1)))
+    per_cu = min(per_cu, 2 if tile["block_threads"] <= 256 else 1)
+    rounds = -(-tile["grid_x"] // (groups * per_cu))
+    elem = 1 if desc.in_dtype == _lib.I8 else (4 if desc.in_dtype == _lib.F32 else 2)
+    staged = desc.L * (desc.K + desc.N) * elem                     # B and C tiles of one workgroup
+    flops = 2.0 * tile["block_m"] * desc.L * (desc.K + desc.N)     # of one workgroup
+    lds_s = staged / (hw.shared_memory_bandwidth_gbs * 1e9 / groups)
+    mfma_s = flops * per_cu / (2.5e15 / groups)
+    return rounds * max(lds_s, mfma_s)
+
+
+def _log(log_file, wkl_key, entry):
+    with open(log_file, "a") as flog:
+        print(json.dumps({"wkl_key": wkl_key, "entry": entry.to_json()}), file=flog, flush=True)
+
+
+def select_tile_variant(wkl_key, log_file, A, B, C, F, inter_op="softmax", softmax_scale=1.0, top=3,
+                        min_repeat_ms=50):
+    """Measure the ``top`` analytically best variants for these operands, append every measurement
+    to ``log_file`` and return the best ``TuneEntry``."""
+    import torch
+
+    desc = chain.bmm_chain_desc(A, B, C, F, inter_op, softmax_scale)
+    space = sorted(make_tile_variant_space(desc), key=lambda t: evaluate_param_hip(desc, t))[:max(1, top)]
+    best = None
+    for tile in space:
+        d = copy.copy(desc)
+        d.tile_variant = tile["variant"]
+        call = lambda: chain.run_bmm_chain(A, B, C, F, desc=d)
+        call()
+        torch.cuda.synchronize()
+        n = 1
+        while True:
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                call()
+            e1.record()
+            e1.synchronize()
+            ms = e0.elapsed_time(e1)
+            if ms >= min_repeat_ms or n >= 1 << 20:
+                break
+            n = max(n + 1, int(n * max(1.5, min_repeat_ms / max(ms, 1e-3) * 1.05)))
+        entry = TuneEntry(tile, ms / n)
+        _log(log_file, wkl_key, entry)
+        if best is None or entry.value < best.value:
+            best = entry
+    return best
+
+
+def load_best_records(log_file):
+    """{wkl_key: entry} keeping the smallest ``value`` per key (chimera_integrate.py:527-537)."""
+    params = {}
+    if not os.path.exists(log_file):
+        return params
+    with open(log_file, "r") as fin:
+        for line in fin:
+            line = line.strip()
+            if not line:
+                continue
+            obj = json.loads(line)
+            if obj["wkl_key"] not in params or obj["entry"]["value"] < params[obj["wkl_key"]]["value"]:
+                params[obj["wkl_key"]] = obj["entry"]
+    return params
+
+
+def best_variant(log_file, wkl_key, default=0):
+    """Variant id recorded as best for ``wkl_key`` (``default`` = the library's table if unseen)."""
+    entry = load_best_records(log_file).get(wkl_key)
+    return entry["record"]["variant"] if entry else default
+
+
+def workload_key(desc):
+    """A stable key for a chain shape (the reference keys on the layer fingerprint)."""
+    return "bmm_chain/dt%d/i%d/l%d/b%d/m%d/n%d/k%d/l%d" % (desc.in_dtype, desc.inter_op, desc.b_layout, desc.batch,
+                                                         desc.M, desc.N, desc.K, desc.L)
+
+
+def auto_schedule_bmm_chain_hip(key, log_file, A, B, C, F, inter_op="softmax", softmax_scale=1.0):
+    """Tune once per key, then reuse the log: returns the variant id to pass as ``tile_variant``."""
+    known = best_variant(log_file, key, default=None)
+    if known is not None:
+        return known
+    return select_tile_variant(key, log_file, A, B, C, F, inter_op, softmax_scale).record["variant"]

@@ -274,6 +274,26 @@ def test_multi_head_attention_module(oracle, dtype, cfg):
     assert torch.equal(ref.view(batch, heads, M, d).permute(0, 2, 1, 3).reshape(batch, M, hidden), out)
 
 
+def test_tile_variant_tuning_round_trip(tmp_path, oracle):
+    # measure the variants for one shape, log them in the reference's format, reuse the log
+    from ditto_amd.auto_schedule.schedulers import chimera_integrate as ci
+
+    dev = "cuda:0"
+    torch.manual_seed(1)
+    q, k, v = (torch.randn(16, 1024, 64, device=dev).half() for _ in range(3))
+    f = torch.empty_like(q)
+    log = str(tmp_path / "chimera_tune.log")
+    key = ci.workload_key(chain.bmm_chain_desc(q, k.transpose(1, 2), v, f, "softmax", 0.125))
+    best = ci.select_tile_variant(key, log, q, k.transpose(1, 2), v, f, "softmax", 0.125, top=3, min_repeat_ms=5)
+    records = ci.load_best_records(log)
+    assert len(open(log).read().strip().splitlines()) == 3
+    assert records[key]["record"]["variant"] == best.record["variant"] and 0 < best.value < 5.0
+    assert ci.auto_schedule_bmm_chain_hip(key, log, q, k.transpose(1, 2), v, f, "softmax", 0.125) == best.record["variant"]
+    chain.run_bmm_chain(q, k.transpose(1, 2), v, f, "softmax", 0.125, tile_variant=best.record["variant"])
+    ref = torch.softmax(q.float() @ k.float().transpose(1, 2) * 0.125, -1) @ v.float()
+    assert (f.float() - ref).abs().max().item() <= MAX_ABS
+
+
 def test_strided_views_and_errors():
     dev = "cuda:0"
     torch.manual_seed(0)

@@ -184,3 +184,44 @@ def test_multi_head_attention_views_map_onto_two_level_strides():
     import pytest
     with pytest.raises(RuntimeError):
         mha.head_views(torch.zeros(batch, M, 3 * hidden + 8, dtype=torch.float16))
+
+
+def test_tuning_log_format_and_best_record(tmp_path):
+    # line format and "smallest value per key wins" of chimera_integrate.py:326-333, 527-537
+    import json
+    from ditto_amd.auto_schedule.schedulers import chimera_integrate as ci
+
+    log = str(tmp_path / "chimera_log.txt")
+    for key, variant, value in (("a", 641, 0.5), ("a", 648, 0.3), ("b", 1282, 2.0), ("a", 642, 0.4)):
+        ci._log(log, key, ci.TuneEntry({"variant": variant}, value))
+    lines = [json.loads(l) for l in open(log)]
+    assert set(lines[0]) == {"wkl_key", "entry"} and set(lines[0]["entry"]) == {"record", "value"}
+    best = ci.load_best_records(log)
+    assert best["a"]["record"]["variant"] == 648 and best["b"]["value"] == 2.0
+    assert ci.best_variant(log, "a") == 648 and ci.best_variant(log, "zzz") == 0
+    assert ci.load_best_records(str(tmp_path / "missing")) == {}
+
+
+def test_tile_variant_space_and_analytic_filter():
+    import torch
+    from ditto_amd import chain
+    from ditto_amd.auto_schedule.schedulers import chimera_integrate as ci
+
+    def desc(b, s, d):
+        q = torch.zeros(b, s, d, dtype=torch.bfloat16)
+        return chain.bmm_chain_desc(q, q.transpose(1, 2), q, torch.zeros_like(q), "softmax", 0.1)
+
+    big = desc(64, 4096, 128)
+    space = ci.make_tile_variant_space(big)
+    assert sorted(t["variant"] for t in space) == [1281, 1282, 1288]
+    assert all(t["lds_bytes"] <= 160 * 1024 for t in space)
+    scores = {t["variant"]: ci.evaluate_param_hip(big, t) for t in space}
+    assert all(0 < v < 1e10 for v in scores.values())
+    assert scores[1282] <= scores[1281]          # 256-row workgroups stage half as much per row
+    over = dict(space[0], lds_bytes=200 * 1024)
+    assert ci.evaluate_param_hip(big, over) == 1e10
+    # few row blocks: the 128-row variant needs fewer rounds than the 256-row ones leave idle CUs
+    small = desc(8, 2048, 128)
+    sc = {t["variant"]: ci.evaluate_param_hip(small, t) for t in ci.make_tile_variant_space(small)}
+    assert min(sc, key=sc.get) in (1281, 1282, 1288)
+    assert ci.workload_key(big) != ci.workload_key(small)
