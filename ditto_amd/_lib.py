@@ -78,6 +78,7 @@ class ConvChainDesc(ctypes.Structure):
         ("S2", ctypes.c_int64),
         ("pad2", ctypes.c_int64),
         ("stride2", ctypes.c_int64),
+        ("groups1", ctypes.c_int64),
     ]
 
 

@@ -227,7 +227,7 @@ def _recognise(layer, state):
         C2, _, R2, S2 = w2.shape
         dims = dict(N=N, C0=C0, H=H, W=W, C1=C1, R1=R1, S1=S1, pad1=first.attrs["padding"],
                     stride1=first.attrs["stride"], C2=C2, R2=R2, S2=S2, pad2=second.attrs["padding"],
-                    stride2=second.attrs["stride"])
+                    stride2=second.attrs["stride"], groups1=first.attrs.get("groups", 1))
         return dict(kind="conv_chain", inter_op=inter[0], dims=dims, relu_out=epi == ["relu_cast"],
                     in_dtype=img.dtype, acc_dtype=first.output(0).dtype, out_dtype=out_t.dtype, softmax_scale=1.0)
     # batched GEMM chain: dims from the layer's input placeholders

@@ -149,8 +149,11 @@ def run_bmm_chain(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=
     return F
 
 
-def conv_chain_desc(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op="cast", relu_out=False):
-    """Fill a ``ditto_conv_chain_desc`` for X[N,C0,H,W], W1[C1,C0,R1,S1], W2[C2,C1,R2,S2] -> Y."""
+def conv_chain_desc(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op="cast", relu_out=False,
+                    groups1=1):
+    """Fill a ``ditto_conv_chain_desc`` for X[N,C0,H,W], W1[C1,C0/groups1,R1,S1], W2[C2,C1,R2,S2] -> Y.
+
+    ``groups1``: 1 (dense first convolution) or C0 (depthwise, C1 / C0 outputs per input channel)."""
     for t, name in ((X, "X"), (W1, "W1"), (W2, "W2"), (Y, "Y")):
         if t.dim() != 4 or not t.is_contiguous():
             raise ValueError("%s must be a contiguous 4-D NCHW/KCRS tensor" % name)
@@ -159,7 +162,9 @@ def conv_chain_desc(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op
     N, C0, H, W = X.shape
     C1, c0, R1, S1 = W1.shape
     C2, c1, R2, S2 = W2.shape
-    if c0 != C0 or c1 != C1:
+    if groups1 not in (1, C0):
+        raise ValueError("groups1 must be 1 or C0 = %d (depthwise), got %d" % (C0, groups1))
+    if c0 * groups1 != C0 or c1 != C1 or C1 % groups1:
         raise ValueError("channel mismatch: X %s, W1 %s, W2 %s" % (tuple(X.shape), tuple(W1.shape), tuple(W2.shape)))
     P1 = (H + 2 * pad1 - R1) // stride1 + 1
     Q1 = (W + 2 * pad1 - S1) // stride1 + 1
@@ -177,6 +182,7 @@ def conv_chain_desc(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op
     d.N, d.C0, d.H, d.W = N, C0, H, W
     d.C1, d.R1, d.S1, d.pad1, d.stride1 = C1, R1, S1, pad1, stride1
     d.C2, d.R2, d.S2, d.pad2, d.stride2 = C2, R2, S2, pad2, stride2
+    d.groups1 = groups1
     return d
 
 
@@ -194,15 +200,16 @@ def _workspace(dev, nbytes):
 
 
 def run_conv_chain(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op="cast", relu_out=False,
-                   desc=None, workspace=None):
+                   desc=None, workspace=None, groups1=1):
     """Y = conv2d(inter(conv2d(X, W1)), W2) on the current stream: one fused kernel, preceded by
     a small kernel that repacks W1 into ``workspace`` (a uint8 tensor of
     ``ditto_conv_chain_workspace_bytes``; None: a cached per-device buffer; False: no
-    workspace, the fused kernel re-lays W1 out itself, slower)."""
+    workspace, the fused kernel re-lays W1 out itself, slower).  A depthwise first convolution
+    (``groups1 = C0``) is a single kernel and uses no workspace."""
     lib = _lib.load()
     dev = _check_device(X, W1, W2, Y)
     if desc is None:
-        desc = conv_chain_desc(X, W1, W2, Y, pad1, stride1, pad2, stride2, inter_op, relu_out)
+        desc = conv_chain_desc(X, W1, W2, Y, pad1, stride1, pad2, stride2, inter_op, relu_out, groups1)
     ws_bytes = lib.ditto_conv_chain_workspace_bytes(ctypes.byref(desc))
     if workspace is None:
         ws = _workspace(dev, ws_bytes) if ws_bytes else None

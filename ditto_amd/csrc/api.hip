@@ -244,8 +244,85 @@ struct ConvPlan {
   int ch;              // input channels per staged chunk
   size_t w1p_bytes;    // size of the repacked W1 (the workspace)
   ditto::ConvChainArgs args;
+  bool dw;             // depthwise first convolution: dwargs / c2_tiles / dw_shared describe the launch
+  int c2_tiles;
+  bool dw_shared;
+  ditto::DwConvArgs dwargs;
   ditto_tile_param tile;
 };
+
+// Depthwise first convolution + 1x1 second (dw_conv_chain.h): everything in one kernel, no workspace.
+int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvPlan* plan) {
+  if (d->C1 % d->C0) return fail(DITTO_EINVAL, "depthwise: C1 must be a multiple of C0");
+  const long long mult = d->C1 / d->C0;
+  if (!(d->R2 == 1 && d->S2 == 1 && d->pad2 == 0 && d->stride2 == 1))
+    return fail(DITTO_EUNSUPPORTED, "depthwise chain: the second convolution must be 1x1, stride 1, no padding");
+  if (d->R1 * d->S1 > 2 * ditto::kDwPairs - 1)
+    return fail(DITTO_EUNSUPPORTED, "depthwise chain: filters of at most 9 taps");
+  if (!(mult == 1 || mult == 2 || mult == 4 || mult % 8 == 0))
+    return fail(DITTO_EUNSUPPORTED, "depthwise chain: channel multiplier must be 1, 2, 4 or a multiple of 8");
+  if (d->C2 > 256) return fail(DITTO_EUNSUPPORTED, "depthwise chain: at most 256 output channels");
+  if (d->C1 > 32768) return fail(DITTO_EUNSUPPORTED, "depthwise chain: at most 32768 intermediate channels");
+  memset(plan, 0, sizeof(*plan));
+  plan->dw = true;
+  const int c2t = d->C2 <= 32 ? 1 : d->C2 <= 64 ? 2 : d->C2 <= 128 ? 4 : 8;
+  const int pxw = c2t == 8 ? 1 : 2;
+  const int slots = 128 * pxw;
+  ditto::DwConvArgs& a = plan->dwargs;
+  a.N = (int)d->N; a.C0 = (int)d->C0; a.H = (int)d->H; a.W = (int)d->W;
+  a.mult = (int)mult; a.C1 = (int)d->C1; a.R = (int)d->R1; a.S = (int)d->S1;
+  a.pad = (int)d->pad1; a.stride = (int)d->stride1; a.C2 = (int)d->C2; a.P = (int)P; a.Q = (int)Q;
+  a.TW = (int)(Q < slots ? Q : slots);
+  a.TH = slots / a.TW;
+  if (a.TH > P) a.TH = (int)P;
+  // input channels per chunk: chx * mult a multiple of 16 (one MFMA k step); as many channels as
+  // keep two workgroups on a CU, else as many as fit at all, else a smaller pixel tile
+  int step = 16;
+  for (int m = (int)(mult > 16 ? 16 : mult); m > 1 && step > 1; m >>= 1) step >>= 1;
+  const int chx_max = (int)((d->C0 + step - 1) / step) * step;
+  int lds = 0;
+  for (;;) {
+    a.rows_in = (a.TH - 1) * a.stride + a.R;
+    a.cols_in = (a.TW - 1) * a.stride + a.S;
+    a.chx = 0;
+    for (int limit : {64 * 1024, 150 * 1024}) {
+      for (int chx = chx_max; chx >= step; chx -= step) {
+        lds = ditto::dw_conv_lds_bytes(chx, a.mult, a.rows_in, a.cols_in, 32 * c2t) + 16;
+        if (lds <= limit) { a.chx = chx; break; }
+      }
+      if (a.chx) break;
+    }
+    if (a.chx) break;
+    if (a.TH > 1) a.TH = (a.TH + 1) / 2;
+    else if (a.TW > 16) a.TW = (a.TW + 1) / 2;
+    else return fail(DITTO_EUNSUPPORTED, "depthwise chain tile does not fit in LDS");
+  }
+  {  // same number of chunks, evenly sized
+    const int chunks = (int)((d->C0 + a.chx - 1) / a.chx);
+    const int even = (int)((d->C0 + chunks - 1) / chunks);
+    a.chx = (even + step - 1) / step * step;
+    lds = ditto::dw_conv_lds_bytes(a.chx, a.mult, a.rows_in, a.cols_in, 32 * c2t) + 16;
+  }
+  a.tiles_h = (int)((P + a.TH - 1) / a.TH);
+  a.tiles_w = (int)((Q + a.TW - 1) / a.TW);
+  a.relu_mid = d->inter_op == DITTO_INTER_RELU;
+  a.relu_out = d->relu_out != 0;
+  a.out_f32 = d->out_dtype == DITTO_F32;
+  plan->c2_tiles = c2t;
+  plan->dw_shared = mult % 8 == 0;
+  ditto_tile_param& t = plan->tile;
+  t.block_threads = 256;
+  t.block_m = a.TH * a.TW;
+  t.block_l = a.chx * a.mult;
+  t.block_n = 32 * c2t;
+  t.head_pad = 0;
+  t.lds_bytes = lds;
+  t.grid_x = a.N * a.tiles_h * a.tiles_w;
+  t.grid_y = a.TH;
+  t.grid_z = a.TW;
+  t.variant = 4000 + c2t * 10 + (plan->dw_shared ? 1 : 0);
+  return DITTO_OK;
+}
 
 int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan) {
   if (!d) return fail(DITTO_EINVAL, "null descriptor");
@@ -261,13 +338,17 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan) {
   if (d->N <= 0 || d->C0 <= 0 || d->H <= 0 || d->W <= 0 || d->C1 <= 0 || d->C2 <= 0 || d->R1 <= 0 ||
       d->S1 <= 0 || d->R2 <= 0 || d->S2 <= 0 || d->stride1 <= 0 || d->stride2 <= 0 || d->pad1 < 0 || d->pad2 < 0)
     return fail(DITTO_EINVAL, "conv extents must be positive and paddings non-negative");
+  const bool dw = d->groups1 != 0 && d->groups1 != 1;
+  if (dw && d->groups1 != d->C0) return fail(DITTO_EUNSUPPORTED, "groups1 must be 1 (dense) or C0 (depthwise)");
   const bool second_1x1 = d->R2 == 1 && d->S2 == 1 && d->pad2 == 0;
   if (d->stride2 != 1) return fail(DITTO_EUNSUPPORTED, "the second convolution must have stride 1");
-  if (!second_1x1 && (d->R2 > 3 || d->S2 > 3 || d->C1 > 64))
-    return fail(DITTO_EUNSUPPORTED,
-                "a second convolution larger than 1x1 takes filters up to 3x3 and at most 64 intermediate channels");
-  if (d->C1 % 8) return fail(DITTO_EINVAL, "C1 must be a multiple of 8");
-  if (d->C1 > 256) return fail(DITTO_EUNSUPPORTED, "C1=%lld: at most 256 intermediate channels", (long long)d->C1);
+  if (!dw) {
+    if (!second_1x1 && (d->R2 > 3 || d->S2 > 3 || d->C1 > 64))
+      return fail(DITTO_EUNSUPPORTED,
+                  "a second convolution larger than 1x1 takes filters up to 3x3 and at most 64 intermediate channels");
+    if (d->C1 % 8) return fail(DITTO_EINVAL, "C1 must be a multiple of 8");
+    if (d->C1 > 256) return fail(DITTO_EUNSUPPORTED, "C1=%lld: at most 256 intermediate channels", (long long)d->C1);
+  }
   if (d->R1 > 7 || d->S1 > 7) return fail(DITTO_EUNSUPPORTED, "first filter larger than 7x7");
   const long long P = (d->H + 2 * d->pad1 - d->R1) / d->stride1 + 1;
   const long long Q = (d->W + 2 * d->pad1 - d->S1) / d->stride1 + 1;
@@ -276,6 +357,7 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan) {
   if (d->N * d->C0 * d->H * d->W > 0x7fffffffLL * 4 || d->N * d->C2 * P * Q > 0x7fffffffLL * 4 ||
       d->H > 65535 || d->W > 65535 || d->N > 65535 || d->C0 > 65535 || d->C2 > 65535)
     return fail(DITTO_EINVAL, "tensor too large");
+  if (dw) return plan_dw_conv(d, P, Q, plan);
   memset(plan, 0, sizeof(*plan));
   const int c1t = d->C1 <= 32 ? 1 : d->C1 <= 64 ? 2 : d->C1 <= 128 ? 4 : 8;
   const int pxw = c1t == 8 ? 1 : 2;
@@ -536,6 +618,19 @@ int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const vo
   if (!x || !w1 || !w2 || !y) return fail(DITTO_EINVAL, "null data pointer");
   if (!aligned(x, 2) || !aligned(w1, 2) || !aligned(w2, 8) || !aligned(y, 4))
     return fail(DITTO_EINVAL, "misaligned data pointer");
+  if (plan.dw) {
+    if (!aligned(w2, 16)) return fail(DITTO_EINVAL, "misaligned data pointer");
+    ditto::DwConvArgs a = plan.dwargs;
+    a.x = x;
+    a.w1 = w1;
+    a.w2 = w2;
+    a.y = y;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    hipError_t e = d->in_dtype == DITTO_F16 ? ditto::launch_dw_conv_f16(plan.c2_tiles, plan.dw_shared, a, st)
+                                            : ditto::launch_dw_conv_bf16(plan.c2_tiles, plan.dw_shared, a, st);
+    if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
+    return DITTO_OK;
+  }
   const size_t need = plan.w1p_bytes + plan.w2p_bytes;
   if (plan.px2 > 0 && !workspace)
     return fail(DITTO_EWORKSPACE, "a second convolution larger than 1x1 needs the workspace (%zu bytes)", need);

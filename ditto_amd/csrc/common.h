@@ -48,6 +48,8 @@ struct Elem<f16> {
     const v2 ones = {(f16)1.0f, (f16)1.0f};
     return __builtin_amdgcn_fdot2(p, ones, acc, false);
   }
+  // acc + a[0]*b[0] + a[1]*b[1] in fp32 (v_dot2_f32_f16)
+  static __device__ __forceinline__ float dot2(v2 a, v2 b, float acc) { return __builtin_amdgcn_fdot2(a, b, acc, false); }
 };
 
 template <>
@@ -64,6 +66,9 @@ struct Elem<bf16> {
   static __device__ __forceinline__ float add_pair(v2 p, float acc) {
     const v2 ones = {(bf16)1.0f, (bf16)1.0f};
     return __builtin_amdgcn_fdot2_f32_bf16(p, ones, acc, false);
+  }
+  static __device__ __forceinline__ float dot2(v2 a, v2 b, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(a, b, acc, false);
   }
 };
 

@@ -1,6 +1,7 @@
 // Instantiates the conv chain kernels for one element type.
 // Compiled with -DDITTO_INST_T=<f16|bf16> and -DDITTO_{INST,PACK,INST2,PACK2}_NAME=<symbol>.
 #include "conv_chain.h"
+#include "dw_conv_chain.h"
 
 namespace ditto {
 
@@ -32,6 +33,21 @@ hipError_t DITTO_INST2_NAME(int c1_tiles, int px2, const ConvChainArgs& args, hi
 
 hipError_t DITTO_PACK2_NAME(int c1_tiles, const ConvChainArgs& args, void* out, hipStream_t stream) {
   return launch_pack_conv_w2<DITTO_INST_T>(args, 32 * c1_tiles, out, stream);
+}
+
+// depthwise first convolution: c2_tiles in {1, 2, 4, 8} (32 output channels each); shared: the
+// multiplier is a multiple of 8
+hipError_t DITTO_DW_NAME(int c2_tiles, bool shared, const DwConvArgs& args, hipStream_t stream) {
+  typedef DITTO_INST_T T;
+#define DITTO_CASE(C2T, PXW)                                                              \
+  if (c2_tiles == C2T)                                                                    \
+    return shared ? launch_dw_conv_chain<T, C2T, PXW, true>(args, stream) : launch_dw_conv_chain<T, C2T, PXW, false>(args, stream);
+  DITTO_CASE(1, 2)
+  DITTO_CASE(2, 2)
+  DITTO_CASE(4, 2)
+  DITTO_CASE(8, 1)
+#undef DITTO_CASE
+  return hipErrorInvalidValue;
 }
 
 }  // namespace ditto

@@ -55,6 +55,13 @@ CONV3X3_CONV1X1_SHAPES = [
 CONV1X1_CONV3X3_SHAPES = [
     (64, 56, 56, 64, 64, 1, 1),  # ResNet-50
 ]
+# (C, H, W, K, stride1, stride2): depthwise3x3_conv1x1_small_channel_cuda.py:340-346
+DEPTHWISE3X3_CONV1X1_SHAPES = [
+    (32, 112, 112, 64, 1, 1),  # mobilenet-v1
+    (32, 56, 56, 64, 1, 1),
+    (64, 112, 112, 64, 1, 1),
+    (16, 224, 224, 32, 2, 1),
+]
 
 
 def cal_ai(B, M, N, K, L):

@@ -50,7 +50,7 @@ class ChainFunction:
             X, W1, W2, Y = args
             d = s.dims
             chain.run_conv_chain(X, W1, W2, Y, d["pad1"], d["stride1"], d["pad2"], d["stride2"], s.inter_op,
-                                 s.relu_out)
+                                 s.relu_out, groups1=d.get("groups1", 1))
         else:
             raise NotImplementedError("no kernel family for chain kind %r" % s.kind)
 

@@ -104,7 +104,7 @@ typedef struct ditto_bmm_chain_desc {
  * testing/hyper_fusion/conv_relu_conv_relu_fuse_hw_cuda.py:17-262 for NCHW,
  * benchmark/chimera/cuda/conv3x3_conv1x1_cuda.py:77-172 for the chain; shape
  * tuple as python_test/auto_tensorize/test_hyper_fusion.py:51-192).
- *   X[N][C0][H][W], W1[C1][C0][R1][S1], W2[C2][C1][R2][S2] -> Y[N][C2][P2][Q2]
+ *   X[N][C0][H][W], W1[C1][C0 / groups1][R1][S1], W2[C2][C1][R2][S2] -> Y[N][C2][P2][Q2]
  */
 typedef struct ditto_conv_chain_desc {
   int32_t abi_version;
@@ -114,6 +114,11 @@ typedef struct ditto_conv_chain_desc {
   int64_t N, C0, H, W;
   int64_t C1, R1, S1, pad1, stride1;
   int64_t C2, R2, S2, pad2, stride2;
+  int64_t groups1;       /* groups of the first convolution: 1 (or 0) dense; C0: depthwise with
+                            C1 / C0 outputs per input channel, W1[C1][1][R1][S1]
+                            (benchmark/chimera/cuda/depthwise3x3_conv1x1_small_channel_cuda.py:77-169,
+                            `factor` = C1 / C0); then R1 * S1 <= 9, the second convolution is 1x1
+                            and C1 / C0 is 1, 2, 4 or a multiple of 8 */
 } ditto_conv_chain_desc;
 
 /* Tile choice reported back to the host; the static per-shape table replaces

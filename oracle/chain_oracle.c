@@ -30,6 +30,7 @@
  *                             requantise step is NOT in the reference (its int8 chain does a
  *                             wrapping astype("int8"), bmm_bmm_cuda.py:116): it is specified
  *                             by this build's workload definition.
+ *   oracle_conv_chain_grouped_f32  the same with a grouped (depthwise) first convolution
  *   oracle_conv_chain_f32     conv -> inter -> conv on NCHW tensors, the chain of
  *                             benchmark/chimera/cuda/conv3x3_conv1x1_cuda.py:77-172 in the
  *                             plain layout of testing/hyper_fusion/
@@ -424,8 +425,12 @@ ORACLE_API void oracle_gemm_chain_i8(int batch, int M, int N, int K, int L, cons
  * is rounded to out dtype after an optional ReLU.  `mid` is caller-provided scratch of
  * N*C1*P1*Q1 floats.
  * ---------------------------------------------------------------------------------- */
-static void conv2d_nchw(int N, int C, int H, int W, int Kc, int R, int S, int pad, int stride,
+/* groups: input channels and output channels are split into `groups` equal parts and output
+ * channel k only sees the inputs of its part (groups = C: depthwise, Kc / C outputs per input
+ * channel; weights [Kc][C / groups][R][S]) */
+static void conv2d_nchw(int N, int C, int H, int W, int Kc, int R, int S, int pad, int stride, int groups,
                         const float* x, const float* w, float* y, int relu, int round_mode) {
+  const int cg = C / groups, kg = Kc / groups;
   const int P = (H + 2 * pad - R) / stride + 1;
   const int Q = (W + 2 * pad - S) / stride + 1;
 #pragma omp parallel for collapse(2) schedule(static)
@@ -433,9 +438,10 @@ static void conv2d_nchw(int N, int C, int H, int W, int Kc, int R, int S, int pa
     for (int k = 0; k < Kc; ++k) {
       float* yp = y + ((size_t)n * Kc + k) * P * Q;
       for (int i = 0; i < P * Q; ++i) yp[i] = 0.f;
-      for (int c = 0; c < C; ++c) {
+      for (int ci = 0; ci < cg; ++ci) {
+        const int c = (k / kg) * cg + ci;
         const float* xp = x + ((size_t)n * C + c) * H * W;
-        const float* wp = w + ((size_t)k * C + c) * R * S;
+        const float* wp = w + ((size_t)k * cg + ci) * R * S;
         for (int r = 0; r < R; ++r)
           for (int s = 0; s < S; ++s) {
             const float wv = wp[r * S + s];
@@ -469,8 +475,22 @@ ORACLE_API void oracle_conv_chain_f32(int N, int C0, int H, int W, int C1, int R
                                       int round_out) {
   const int P1 = (H + 2 * pad1 - R1) / stride1 + 1;
   const int Q1 = (W + 2 * pad1 - S1) / stride1 + 1;
-  conv2d_nchw(N, C0, H, W, C1, R1, S1, pad1, stride1, X, W1, mid, relu_mid, round_mid);
-  conv2d_nchw(N, C1, P1, Q1, C2, R2, S2, pad2, stride2, mid, W2, Y, relu_out, round_out);
+  conv2d_nchw(N, C0, H, W, C1, R1, S1, pad1, stride1, 1, X, W1, mid, relu_mid, round_mid);
+  conv2d_nchw(N, C1, P1, Q1, C2, R2, S2, pad2, stride2, 1, mid, W2, Y, relu_out, round_out);
+}
+
+/* the same chain with a grouped first convolution (groups1 = C0: the depthwise -> 1x1 chain of
+ * benchmark/chimera/cuda/depthwise3x3_conv1x1_small_channel_cuda.py:77-169, whose `factor` is
+ * C1 / C0) */
+ORACLE_API void oracle_conv_chain_grouped_f32(int N, int C0, int H, int W, int C1, int R1, int S1, int pad1,
+                                              int stride1, int groups1, int C2, int R2, int S2, int pad2,
+                                              int stride2, const float* X, const float* W1, const float* W2,
+                                              float* mid, float* Y, int relu_mid, int relu_out, int round_mid,
+                                              int round_out) {
+  const int P1 = (H + 2 * pad1 - R1) / stride1 + 1;
+  const int Q1 = (W + 2 * pad1 - S1) / stride1 + 1;
+  conv2d_nchw(N, C0, H, W, C1, R1, S1, pad1, stride1, groups1, X, W1, mid, relu_mid, round_mid);
+  conv2d_nchw(N, C1, P1, Q1, C2, R2, S2, pad2, stride2, 1, mid, W2, Y, relu_out, round_out);
 }
 
 ORACLE_API int oracle_num_threads(void) {

@@ -63,6 +63,8 @@ def lib():
         L.oracle_gemm_chain_i8.argtypes = [ci] * 5 + [i8p] * 3 + [fp, i32p, i8p]
         L.oracle_conv_chain_f32.restype = None
         L.oracle_conv_chain_f32.argtypes = [ci] * 14 + [fp] * 5 + [ci] * 4
+        L.oracle_conv_chain_grouped_f32.restype = None
+        L.oracle_conv_chain_grouped_f32.argtypes = [ci] * 15 + [fp] * 5 + [ci] * 4
         L.oracle_num_threads.restype = ci
         L.oracle_num_threads.argtypes = []
         _lib = L
@@ -169,14 +171,16 @@ def gemm_chain_i8(A, B, D, scale, return_mid=False):
 
 
 def conv_chain_f32(X, W1, W2, pad1=1, stride1=1, pad2=0, stride2=1, relu_mid=False, relu_out=False,
-                   round_mid=None, round_out=None, return_mid=False):
-    """conv -> (relu) -> round -> conv -> (relu) -> round on NCHW fp32 arrays."""
+                   round_mid=None, round_out=None, return_mid=False, groups1=1):
+    """conv -> (relu) -> round -> conv -> (relu) -> round on NCHW fp32 arrays; ``groups1`` groups the
+    first convolution (``groups1 = C0``: depthwise, W1 is [C1, 1, R1, S1])."""
     X, px = _f(X)
     W1, p1 = _f(W1)
     W2, p2 = _f(W2)
     N, C0, H, W = X.shape
-    C1, _, R1, S1 = W1.shape
+    C1, cg, R1, S1 = W1.shape
     C2, _, R2, S2 = W2.shape
+    assert C0 % groups1 == 0 and C1 % groups1 == 0 and cg == C0 // groups1
     P1 = (H + 2 * pad1 - R1) // stride1 + 1
     Q1 = (W + 2 * pad1 - S1) // stride1 + 1
     P2 = (P1 + 2 * pad2 - R2) // stride2 + 1
@@ -184,9 +188,9 @@ def conv_chain_f32(X, W1, W2, pad1=1, stride1=1, pad2=0, stride2=1, relu_mid=Fal
     mid = np.empty((N, C1, P1, Q1), dtype=np.float32)
     Y = np.empty((N, C2, P2, Q2), dtype=np.float32)
     fp = ctypes.POINTER(ctypes.c_float)
-    lib().oracle_conv_chain_f32(N, C0, H, W, C1, R1, S1, pad1, stride1, C2, R2, S2, pad2, stride2, px, p1, p2,
-                                mid.ctypes.data_as(fp), Y.ctypes.data_as(fp), int(relu_mid), int(relu_out),
-                                ROUND_CODES[round_mid], ROUND_CODES[round_out])
+    lib().oracle_conv_chain_grouped_f32(N, C0, H, W, C1, R1, S1, pad1, stride1, groups1, C2, R2, S2, pad2, stride2,
+                                        px, p1, p2, mid.ctypes.data_as(fp), Y.ctypes.data_as(fp), int(relu_mid),
+                                        int(relu_out), ROUND_CODES[round_mid], ROUND_CODES[round_out])
     return (Y, mid) if return_mid else Y
 
 

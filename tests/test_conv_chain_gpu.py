@@ -12,14 +12,15 @@ MAX_ABS, REL_L2, REL_L2_BF16_QUANT = 1e-2, 1e-3, 3e-3
 
 
 def run_conv(X, W1, W2, dtype, pad1=1, stride1=1, inter="cast", relu_out=False, out_dtype=None, workspace=None,
-             pad2=0):
+             pad2=0, groups1=1):
     x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
     N, _, H, W = X.shape
     R, S = W1.shape[2:]
     P = (H + 2 * pad1 - R) // stride1 + 1 + 2 * pad2 - W2.shape[2] + 1
     Q = (W + 2 * pad1 - S) // stride1 + 1 + 2 * pad2 - W2.shape[3] + 1
     y = torch.full((N, W2.shape[0], P, Q), float("nan"), device=x.device, dtype=TORCH_DTYPES[out_dtype or dtype])
-    chain.run_conv_chain(x, w1, w2, y, pad1, stride1, pad2, 1, inter, relu_out, workspace=workspace)
+    chain.run_conv_chain(x, w1, w2, y, pad1, stride1, pad2, 1, inter, relu_out, workspace=workspace,
+                         groups1=groups1)
     torch.cuda.synchronize()
     return y.float().cpu().numpy()
 
@@ -82,6 +83,53 @@ def test_conv_chain_with_wide_second_filter(oracle, case, dtype):
     assert np.array_equal(got, oracle.np_round_to(got32, dtype))
     with pytest.raises(ValueError):  # this variant cannot run without its workspace
         run_conv(X, W1, W2, dtype, pad1, stride1, workspace=False, pad2=pad2)
+
+
+CASES_DEPTHWISE = [
+    # N, C0, H, W, factor, R, pad, stride, C2
+    (1, 32, 56, 56, 16, 3, 1, 1, 64),    # depthwise3x3_conv1x1_small_channel_cuda.py:340-346, row 2
+    (2, 16, 40, 40, 16, 3, 1, 2, 32),    # stride 2 (row 4, scaled down)
+    (1, 24, 17, 23, 8, 3, 1, 1, 40),     # odd extents, C2 not a multiple of 32, factor 8
+    (1, 40, 14, 14, 1, 3, 1, 1, 96),     # plain depthwise (factor 1), MobileNet block
+    (1, 12, 9, 300, 2, 3, 1, 1, 16),     # factor 2, wider than one tile, C1 = 24
+    (1, 6, 20, 20, 4, 3, 0, 1, 160),     # factor 4, no padding, 256-wide output tile set
+    (1, 64, 28, 28, 16, 3, 1, 1, 128),   # 1024 intermediate channels in several chunks
+    (1, 8, 12, 12, 24, 2, 0, 1, 32),     # 2x2 filter, factor 24
+]
+
+
+@pytest.mark.parametrize("case", CASES_DEPTHWISE)
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_depthwise_conv_chain_vs_oracle(oracle, case, dtype):
+    N, C0, H, W, factor, R, pad, stride, C2 = case
+    C1 = C0 * factor
+    rng = np.random.default_rng(C0 + C2)
+    X = oracle.np_round_to(rng.standard_normal((N, C0, H, W)).astype(np.float32), dtype)
+    W1 = oracle.np_round_to(rng.standard_normal((C1, 1, R, R)).astype(np.float32) * 0.3, dtype)
+    W2 = oracle.np_round_to(rng.standard_normal((C2, C1, 1, 1)).astype(np.float32) * 0.05, dtype)
+    for relu in (False, True):
+        want32 = oracle.conv_chain_f32(X, W1, W2, pad, stride, 0, 1, relu_mid=relu, relu_out=relu, round_mid=dtype,
+                                       groups1=C0)
+        got32 = run_conv(X, W1, W2, dtype, pad, stride, "relu" if relu else "cast", relu, "float32", groups1=C0)
+        assert got32.shape == want32.shape and np.isfinite(got32).all()
+        mx, rel = errors(got32, want32)
+        assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
+    got = run_conv(X, W1, W2, dtype, pad, stride, "relu", True, groups1=C0)
+    assert np.array_equal(got, oracle.np_round_to(got32, dtype))
+
+
+def test_depthwise_chain_rejects():
+    x = torch.zeros(1, 16, 14, 14, device="cuda:0", dtype=torch.float16)
+    y = torch.zeros(1, 32, 14, 14, device="cuda:0", dtype=torch.float16)
+    with pytest.raises(NotImplementedError):  # factor 3
+        chain.run_conv_chain(x, torch.zeros(48, 1, 3, 3, device="cuda:0", dtype=torch.float16),
+                             torch.zeros(32, 48, 1, 1, device="cuda:0", dtype=torch.float16), y, groups1=16)
+    with pytest.raises(NotImplementedError):  # 5x5 depthwise filter
+        chain.run_conv_chain(x, torch.zeros(16, 1, 5, 5, device="cuda:0", dtype=torch.float16),
+                             torch.zeros(32, 16, 1, 1, device="cuda:0", dtype=torch.float16), y, 2, groups1=16)
+    with pytest.raises(ValueError):  # groups that are neither 1 nor C0
+        chain.run_conv_chain(x, torch.zeros(16, 4, 3, 3, device="cuda:0", dtype=torch.float16),
+                             torch.zeros(32, 16, 1, 1, device="cuda:0", dtype=torch.float16), y, groups1=4)
 
 
 def test_conv_chain_rejects_what_it_cannot_fuse():

@@ -244,6 +244,27 @@ def test_conv_chain_vs_torch(oracle, cfg):
     assert np.allclose(got, want, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("cfg", [(2, 8, 9, 11, 1, 1, 12), (1, 4, 10, 10, 16, 2, 8), (1, 6, 7, 9, 2, 1, 5)])
+def test_depthwise_conv_chain_vs_torch(oracle, cfg):
+    # grouped (depthwise, `factor` outputs per input channel) first convolution against torch conv2d
+    N, C0, H, W, factor, s1, C2 = cfg
+    rng = np.random.default_rng(21)
+    X = rng.standard_normal((N, C0, H, W)).astype(np.float32)
+    W1 = (rng.standard_normal((C0 * factor, 1, 3, 3)) * 0.3).astype(np.float32)
+    W2 = (rng.standard_normal((C2, C0 * factor, 1, 1)) * 0.3).astype(np.float32)
+    got = oracle.conv_chain_f32(X, W1, W2, 1, s1, 0, 1, relu_mid=True, groups1=C0)
+    t = torch.nn.functional
+    mid = t.conv2d(torch.from_numpy(X).double(), torch.from_numpy(W1).double(), padding=1, stride=s1, groups=C0)
+    want = t.conv2d(mid.clamp_min(0), torch.from_numpy(W2).double()).numpy()
+    assert np.abs(got - want).max() <= 1e-4
+    # one output per input channel and a centre-tap delta filter: the depthwise stage is the identity
+    Wd = np.zeros((C0, 1, 3, 3), np.float32)
+    Wd[:, 0, 1, 1] = 1.0
+    W2i = (rng.standard_normal((C2, C0, 1, 1))).astype(np.float32)
+    got = oracle.conv_chain_f32(X, Wd, W2i, 1, 1, 0, 1, groups1=C0)
+    assert np.abs(got - np.einsum("kc,nchw->nkhw", W2i[:, :, 0, 0], X)).max() <= 1e-4
+
+
 def test_conv_chain_delta_kernels(oracle):
     # 3x3 kernel with a single one at (r, s) shifts the image; a 1x1 conv is a channel GEMM
     rng = np.random.default_rng(13)
