@@ -60,6 +60,11 @@ WORKLOADS.update({
         kind="conv", dtype="float16", N=32, C0=64, H=56, W=56, C1=64, R=1, pad=0, stride=1, C2=64, R2=3, pad2=1,
         bound="mfma",
         desc="conv1x1(64->64) -> conv3x3(64->64, s1 p1) on 32x56x56, NCHW fp16 (the reference's ResNet-50 row)"),
+    "dw3x3_conv1x1_f16_n32_c32_112x112_f16_k64": dict(
+        kind="conv", dtype="float16", N=32, C0=32, H=112, W=112, C1=512, R=3, pad=1, stride=1, C2=64, groups=32,
+        bound="hbm",
+        desc="depthwise conv3x3(32 channels x16, s1 p1) -> conv1x1(512->64) on 32x112x112, NCHW fp16 "
+             "(the reference's MobileNet-V1 row)"),
     "gemm_chain_i8_8192x1024x256x1024": dict(
         kind="requant", dtype="int8", batch=1, M=8192, K=1024, L=256, N=1024, scale=2.0 ** -10, bound="hbm",
         desc="int8 A[8192,1024].B[1024,256] -> requantise(2^-10, RNE, saturate) -> .D[256,1024], int32 out"),
@@ -74,7 +79,8 @@ def flops_of(w):
         Q = (w["W"] + 2 * w["pad"] - w["R"]) // w["stride"] + 1
         R2 = w.get("R2", 1)
         P2, Q2 = P + 2 * w.get("pad2", 0) - R2 + 1, Q + 2 * w.get("pad2", 0) - R2 + 1
-        return 2.0 * w["N"] * (P * Q * w["C0"] * w["C1"] * w["R"] * w["R"] + P2 * Q2 * w["C1"] * w["C2"] * R2 * R2)
+        c0g = w["C0"] // w.get("groups", 1)
+        return 2.0 * w["N"] * (P * Q * c0g * w["C1"] * w["R"] * w["R"] + P2 * Q2 * w["C1"] * w["C2"] * R2 * R2)
     return 2.0 * w["batch"] * w["M"] * w["L"] * (w["K"] + w["N"])
 
 
@@ -85,7 +91,7 @@ def bytes_of(w):
         Q = (w["W"] + 2 * w["pad"] - w["R"]) // w["stride"] + 1
         R2 = w.get("R2", 1)
         P2, Q2 = P + 2 * w.get("pad2", 0) - R2 + 1, Q + 2 * w.get("pad2", 0) - R2 + 1
-        return 2 * (w["N"] * w["C0"] * w["H"] * w["W"] + w["C1"] * w["C0"] * w["R"] * w["R"]
+        return 2 * (w["N"] * w["C0"] * w["H"] * w["W"] + w["C1"] * (w["C0"] // w.get("groups", 1)) * w["R"] * w["R"]
                     + w["C2"] * w["C1"] * R2 * R2 + w["N"] * w["C2"] * P2 * Q2)
     if w["kind"] == "requant":
         return w["batch"] * (w["M"] * w["K"] + w["K"] * w["L"] + w["L"] * w["N"] + 4 * w["M"] * w["N"])
@@ -102,13 +108,15 @@ def make_call(w, dev):
     g = torch.Generator().manual_seed(0)
     if w["kind"] == "conv":
         x = torch.randn(w["N"], w["C0"], w["H"], w["W"], generator=g).half().to(dev)
-        w1 = (torch.randn(w["C1"], w["C0"], w["R"], w["R"], generator=g) * 0.05).half().to(dev)
+        groups = w.get("groups", 1)
+        w1 = (torch.randn(w["C1"], w["C0"] // groups, w["R"], w["R"], generator=g) * (0.3 if groups > 1 else 0.05)
+              ).half().to(dev)
         R2, pad2 = w.get("R2", 1), w.get("pad2", 0)
         w2 = (torch.randn(w["C2"], w["C1"], R2, R2, generator=g) * 0.05).half().to(dev)
         P = (w["H"] + 2 * w["pad"] - w["R"]) // w["stride"] + 1 + 2 * pad2 - R2 + 1
         Q = (w["W"] + 2 * w["pad"] - w["R"]) // w["stride"] + 1 + 2 * pad2 - R2 + 1
         y = torch.empty(w["N"], w["C2"], P, Q, dtype=torch.float16, device=dev)
-        desc = chain.conv_chain_desc(x, w1, w2, y, w["pad"], w["stride"], pad2, 1, "cast", False)
+        desc = chain.conv_chain_desc(x, w1, w2, y, w["pad"], w["stride"], pad2, 1, "cast", False, groups)
         return (lambda: chain.run_conv_chain(x, w1, w2, y, desc=desc)), desc
     if w["kind"] == "requant":
         a = torch.randint(-127, 128, (w["M"], w["K"]), generator=g, dtype=torch.int8).to(dev)

@@ -246,62 +246,122 @@ struct ConvPlan {
   ditto::ConvChainArgs args;
   bool dw;             // depthwise first convolution: dwargs / c2_tiles / dw_shared describe the launch
   int c2_tiles;
-  bool dw_shared;
+  int dw_mode;         // 0 | 1: vector-ALU depthwise stage (1: multiplier a multiple of 8); 2: MFMA
   ditto::DwConvArgs dwargs;
   ditto_tile_param tile;
 };
 
 // Depthwise first convolution + 1x1 second (dw_conv_chain.h): everything in one kernel, no workspace.
-int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvPlan* plan) {
+// Channel multipliers that are multiples of 16 run the depthwise stage on the matrix cores
+// (dw_mode 2), the others on the vector ALU (dw_mode 1: multiples of 8, 0: 1, 2, 4).
+int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvPlan* plan, bool need_device) {
   if (d->C1 % d->C0) return fail(DITTO_EINVAL, "depthwise: C1 must be a multiple of C0");
   const long long mult = d->C1 / d->C0;
+  const long long RS = d->R1 * d->S1;
   if (!(d->R2 == 1 && d->S2 == 1 && d->pad2 == 0 && d->stride2 == 1))
     return fail(DITTO_EUNSUPPORTED, "depthwise chain: the second convolution must be 1x1, stride 1, no padding");
-  if (d->R1 * d->S1 > 2 * ditto::kDwPairs - 1)
-    return fail(DITTO_EUNSUPPORTED, "depthwise chain: filters of at most 9 taps");
+  const bool mfma = mult % 16 == 0 && RS <= ditto::kDwMfmaTaps;
+  if (!mfma && RS > 2 * ditto::kDwPairs - 1)
+    return fail(DITTO_EUNSUPPORTED,
+                "depthwise chain: filters of at most 9 taps (16 when the channel multiplier is a multiple of 16)");
   if (!(mult == 1 || mult == 2 || mult == 4 || mult % 8 == 0))
     return fail(DITTO_EUNSUPPORTED, "depthwise chain: channel multiplier must be 1, 2, 4 or a multiple of 8");
   if (d->C2 > 256) return fail(DITTO_EUNSUPPORTED, "depthwise chain: at most 256 output channels");
   if (d->C1 > 32768) return fail(DITTO_EUNSUPPORTED, "depthwise chain: at most 32768 intermediate channels");
   memset(plan, 0, sizeof(*plan));
   plan->dw = true;
+  plan->dw_mode = mfma ? 2 : mult % 8 == 0 ? 1 : 0;
   const int c2t = d->C2 <= 32 ? 1 : d->C2 <= 64 ? 2 : d->C2 <= 128 ? 4 : 8;
-  const int pxw = c2t == 8 ? 1 : 2;
-  const int slots = 128 * pxw;
+  const int pxw = mfma ? ditto::dw_mfma_pxw(c2t) : c2t == 8 ? 1 : 2;
+  const int groups = mfma ? ditto::dw_mfma_groups(c2t) : 1;
+  const int slots = 128 * groups * pxw;  // pixels of a workgroup's tile
   ditto::DwConvArgs& a = plan->dwargs;
   a.N = (int)d->N; a.C0 = (int)d->C0; a.H = (int)d->H; a.W = (int)d->W;
   a.mult = (int)mult; a.C1 = (int)d->C1; a.R = (int)d->R1; a.S = (int)d->S1;
   a.pad = (int)d->pad1; a.stride = (int)d->stride1; a.C2 = (int)d->C2; a.P = (int)P; a.Q = (int)Q;
-  a.TW = (int)(Q < slots ? Q : slots);
-  a.TH = slots / a.TW;
-  if (a.TH > P) a.TH = (int)P;
-  // input channels per chunk: chx * mult a multiple of 16 (one MFMA k step); as many channels as
-  // keep two workgroups on a CU, else as many as fit at all, else a smaller pixel tile
-  int step = 16;
-  for (int m = (int)(mult > 16 ? 16 : mult); m > 1 && step > 1; m >>= 1) step >>= 1;
+  // Pixel tile: the split of the output plane into TH x TW pieces of at most `slots` pixels that
+  // costs the fewest 32-pixel tile rounds (a round = one tile on each of the four waves; the
+  // vector-ALU kernel always runs all its rounds); ties go to the wider tile.
+  {
+    long long best = -1;
+    for (int k = 1; k <= (int)Q; ++k) {
+      const int tw = (int)((Q + k - 1) / k);
+      if (tw > slots) continue;
+      if (tw < 8 && k > 1) break;
+      int th = slots / tw;
+      if (th > P) th = (int)P;
+      const long long th_n = (P + th - 1) / th;
+      th = (int)((P + th_n - 1) / th_n);
+      const long long tw_n = (Q + tw - 1) / tw;
+      const long long rounds = mfma ? ((th * tw + 31) / 32 + 4 * groups - 1) / (4 * groups) : pxw;
+      const long long cost = th_n * tw_n * rounds;
+      if (best < 0 || cost < best) { best = cost; a.TH = th; a.TW = tw; }
+    }
+  }
+  // input channels per chunk: chx * mult a multiple of the MFMA block (32 intermediate channels
+  // on the matrix-core path, 16 on the vector path); as many channels as keep two workgroups on a
+  // CU, else as many as fit at all, else a smaller pixel tile
+  const int cm_unit = mfma ? 32 : 16;
+  int step = 1;
+  while ((step * mult) % cm_unit) ++step;
+  // halo loads: vectors of up to 4 elements that divide W (the run call narrows them if x is less
+  // aligned); output through 16-byte stores when rows allow
+  const int vec_max = mfma ? (d->W % 4 == 0 ? 4 : d->W % 2 == 0 ? 2 : 1) : 1;
+  a.vec = vec_max;
+  a.wide = mfma && d->out_dtype != DITTO_F32 && Q % 8 == 0 && a.TW % 8 == 0;
+  auto lds_of = [&](int chx) {
+    return mfma ? ditto::dw_conv_mfma_lds_bytes(chx, a.mult, a.rows_in, a.cols_al, 32 * c2t, groups, a.wide != 0)
+                : ditto::dw_conv_lds_bytes(chx, a.mult, a.rows_in, a.cols_in, 32 * c2t) + 16;
+  };
+  // the MFMA kernel keeps a chunk's halo tile in flight in registers (kDwXpf vectors per thread)
+  // and addresses it with packed 32-bit offsets
+  auto fits_regs = [&](int chx) {
+    if (!mfma) return true;
+    // a thread owns one (row, vector) position of the halo tile and walks the channels, `cphases`
+    // at a time: kDwXpf passes must cover the chunk
+    const int nvr = a.cols_al / a.vec;
+    const int cphases = (256 * groups / nvr) / a.rows_in;
+    return cphases >= 1 && (chx + cphases - 1) / cphases <= ditto::kDwXpf &&
+           (long long)(chx + 1) * d->H * d->W < 0x7fffffffLL;
+  };
   const int chx_max = (int)((d->C0 + step - 1) / step) * step;
   int lds = 0;
   for (;;) {
     a.rows_in = (a.TH - 1) * a.stride + a.R;
     a.cols_in = (a.TW - 1) * a.stride + a.S;
     a.chx = 0;
-    for (int limit : {64 * 1024, 150 * 1024}) {
-      for (int chx = chx_max; chx >= step; chx -= step) {
-        lds = ditto::dw_conv_lds_bytes(chx, a.mult, a.rows_in, a.cols_in, 32 * c2t) + 16;
-        if (lds <= limit) { a.chx = chx; break; }
+    // everything resident (one chunk, filters staged once per workgroup) with the widest loads
+    // that leave room for it ...
+    for (int vec = vec_max; mfma && vec >= 1 && !a.chx; vec >>= 1) {
+      a.vec = vec;
+      a.cols_al = (a.cols_in + 2 * vec - 2) / vec * vec;
+      a.cols_al += a.cols_al & 1;
+      lds = lds_of(chx_max);
+      if (lds <= 160 * 1024 && fits_regs(chx_max)) a.chx = chx_max;
+    }
+    // ... else chunks: small enough for two workgroups per CU, else whatever fits
+    if (!a.chx) {
+      a.vec = vec_max;
+      a.cols_al = (a.cols_in + 2 * a.vec - 2) / a.vec * a.vec;
+      a.cols_al += a.cols_al & 1;
+      for (int limit : {78 * 1024, 150 * 1024}) {
+        for (int chx = chx_max; chx >= step; chx -= step) {
+          lds = lds_of(chx);
+          if (lds <= limit && fits_regs(chx)) { a.chx = chx; break; }
+        }
+        if (a.chx) break;
       }
-      if (a.chx) break;
     }
     if (a.chx) break;
     if (a.TH > 1) a.TH = (a.TH + 1) / 2;
-    else if (a.TW > 16) a.TW = (a.TW + 1) / 2;
+    else if (a.TW > 16) { a.TW = (a.TW + 1) / 2; a.wide = a.wide && a.TW % 8 == 0; }
     else return fail(DITTO_EUNSUPPORTED, "depthwise chain tile does not fit in LDS");
   }
   {  // same number of chunks, evenly sized
     const int chunks = (int)((d->C0 + a.chx - 1) / a.chx);
     const int even = (int)((d->C0 + chunks - 1) / chunks);
     a.chx = (even + step - 1) / step * step;
-    lds = ditto::dw_conv_lds_bytes(a.chx, a.mult, a.rows_in, a.cols_in, 32 * c2t) + 16;
+    lds = lds_of(a.chx);
   }
   a.tiles_h = (int)((P + a.TH - 1) / a.TH);
   a.tiles_w = (int)((Q + a.TW - 1) / a.TW);
@@ -309,22 +369,28 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   a.relu_out = d->relu_out != 0;
   a.out_f32 = d->out_dtype == DITTO_F32;
   plan->c2_tiles = c2t;
-  plan->dw_shared = mult % 8 == 0;
   ditto_tile_param& t = plan->tile;
-  t.block_threads = 256;
+  t.block_threads = 256 * groups;
   t.block_m = a.TH * a.TW;
   t.block_l = a.chx * a.mult;
   t.block_n = 32 * c2t;
   t.head_pad = 0;
   t.lds_bytes = lds;
   t.grid_x = a.N * a.tiles_h * a.tiles_w;
+  if (mfma) {  // persistent workgroups, as many as the CUs hold at this LDS footprint
+    const int per_cu = 160 * 1024 / lds < 2 ? 1 : 2;
+    const int cap = (need_device ? device_cus() : 256) * per_cu;
+    if (t.grid_x > cap) t.grid_x = cap;
+    a.grid = t.grid_x;
+    a.nt_store = (a.TW * 2) % 128 == 0;
+  }
   t.grid_y = a.TH;
   t.grid_z = a.TW;
-  t.variant = 4000 + c2t * 10 + (plan->dw_shared ? 1 : 0);
+  t.variant = 4000 + c2t * 10 + plan->dw_mode;
   return DITTO_OK;
 }
 
-int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan) {
+int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device = false) {
   if (!d) return fail(DITTO_EINVAL, "null descriptor");
   if (d->abi_version != DITTO_CHAIN_ABI_VERSION)
     return fail(DITTO_EINVAL, "descriptor abi_version %d, library %d", d->abi_version, DITTO_CHAIN_ABI_VERSION);
@@ -357,7 +423,7 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan) {
   if (d->N * d->C0 * d->H * d->W > 0x7fffffffLL * 4 || d->N * d->C2 * P * Q > 0x7fffffffLL * 4 ||
       d->H > 65535 || d->W > 65535 || d->N > 65535 || d->C0 > 65535 || d->C2 > 65535)
     return fail(DITTO_EINVAL, "tensor too large");
-  if (dw) return plan_dw_conv(d, P, Q, plan);
+  if (dw) return plan_dw_conv(d, P, Q, plan, need_device);
   memset(plan, 0, sizeof(*plan));
   const int c1t = d->C1 <= 32 ? 1 : d->C1 <= 64 ? 2 : d->C1 <= 128 ? 4 : 8;
   const int pxw = c1t == 8 ? 1 : 2;
@@ -613,7 +679,7 @@ size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
 int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const void* w1, const void* w2,
                          void* y, void* workspace, size_t workspace_bytes, void* stream) {
   ConvPlan plan;
-  int rc = plan_conv(d, &plan);
+  int rc = plan_conv(d, &plan, true);
   if (rc != DITTO_OK) return rc;
   if (!x || !w1 || !w2 || !y) return fail(DITTO_EINVAL, "null data pointer");
   if (!aligned(x, 2) || !aligned(w1, 2) || !aligned(w2, 8) || !aligned(y, 4))
@@ -621,13 +687,25 @@ int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const vo
   if (plan.dw) {
     if (!aligned(w2, 16)) return fail(DITTO_EINVAL, "misaligned data pointer");
     ditto::DwConvArgs a = plan.dwargs;
+    // less aligned pointers: narrower halo loads (the LDS layout stays valid) while the chunk still
+    // fits the registers that keep it in flight; plain 2-byte output stores
+    while (a.vec > 1 && !aligned(x, 2 * (size_t)a.vec)) a.vec >>= 1;
+    if (plan.dw_mode == 2) {
+      const int nvr = a.cols_al / a.vec;
+      const int cphases = (256 * ditto::dw_mfma_groups(plan.c2_tiles) / nvr) / a.rows_in;
+      if (cphases < 1 || (a.chx + cphases - 1) / cphases > ditto::kDwXpf)
+        return fail(DITTO_EINVAL, "misaligned data pointer: x must be aligned to %d bytes for this shape",
+                    2 * plan.dwargs.vec);
+      if (!aligned(w1, 16)) return fail(DITTO_EINVAL, "misaligned data pointer");
+    }
+    if (a.wide && !aligned(y, 16)) a.wide = 0;
     a.x = x;
     a.w1 = w1;
     a.w2 = w2;
     a.y = y;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    hipError_t e = d->in_dtype == DITTO_F16 ? ditto::launch_dw_conv_f16(plan.c2_tiles, plan.dw_shared, a, st)
-                                            : ditto::launch_dw_conv_bf16(plan.c2_tiles, plan.dw_shared, a, st);
+    hipError_t e = d->in_dtype == DITTO_F16 ? ditto::launch_dw_conv_f16(plan.c2_tiles, plan.dw_mode, a, st)
+                                            : ditto::launch_dw_conv_bf16(plan.c2_tiles, plan.dw_mode, a, st);
     if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
     return DITTO_OK;
   }

@@ -35,13 +35,17 @@ hipError_t DITTO_PACK2_NAME(int c1_tiles, const ConvChainArgs& args, void* out, 
   return launch_pack_conv_w2<DITTO_INST_T>(args, 32 * c1_tiles, out, stream);
 }
 
-// depthwise first convolution: c2_tiles in {1, 2, 4, 8} (32 output channels each); shared: the
-// multiplier is a multiple of 8
-hipError_t DITTO_DW_NAME(int c2_tiles, bool shared, const DwConvArgs& args, hipStream_t stream) {
+// depthwise first convolution: c2_tiles in {1, 2, 4, 8} (32 output channels each); mode 0 | 1:
+// vector-ALU depthwise stage (1: the multiplier is a multiple of 8), 2: MFMA depthwise stage
+hipError_t DITTO_DW_NAME(int c2_tiles, int mode, const DwConvArgs& args, hipStream_t stream) {
   typedef DITTO_INST_T T;
-#define DITTO_CASE(C2T, PXW)                                                              \
-  if (c2_tiles == C2T)                                                                    \
-    return shared ? launch_dw_conv_chain<T, C2T, PXW, true>(args, stream) : launch_dw_conv_chain<T, C2T, PXW, false>(args, stream);
+#define DITTO_CASE(C2T, PXW)                                                                    \
+  if (c2_tiles == C2T) {                                                                        \
+    if (mode == 2)                                                                              \
+      return launch_dw_conv_mfma<T, C2T, dw_mfma_pxw(C2T), dw_mfma_groups(C2T)>(args, args.grid, stream); \
+    return mode == 1 ? launch_dw_conv_chain<T, C2T, PXW, true>(args, stream)                    \
+                     : launch_dw_conv_chain<T, C2T, PXW, false>(args, stream);                  \
+  }
   DITTO_CASE(1, 2)
   DITTO_CASE(2, 2)
   DITTO_CASE(4, 2)

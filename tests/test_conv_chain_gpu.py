@@ -95,6 +95,8 @@ CASES_DEPTHWISE = [
     (1, 6, 20, 20, 4, 3, 0, 1, 160),     # factor 4, no padding, 256-wide output tile set
     (1, 64, 28, 28, 16, 3, 1, 1, 128),   # 1024 intermediate channels in several chunks
     (1, 8, 12, 12, 24, 2, 0, 1, 32),     # 2x2 filter, factor 24
+    (1, 8, 12, 12, 48, 4, 1, 1, 32),     # 4x4 filter (16 taps), factor 48
+    (2, 6, 13, 21, 32, 2, 1, 1, 72),     # 2x2 filter (no second tap group), factor 32
 ]
 
 
