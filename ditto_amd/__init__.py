@@ -8,7 +8,8 @@ The sub-packages keep the reference's names (``auto_compute``, ``auto_tensorize`
 chain.  The compute runs in ``csrc/libditto_chain.so`` (hand-written gfx950 kernels behind the
 C ABI of ``include/ditto_chain.h``); there is no CPU or PyTorch fallback.
 """
-from . import auto_compute, auto_schedule, auto_tensorize, hardware, runtime, te  # noqa: F401
+from . import auto_compute, auto_schedule, auto_tensorize, chimera, hardware, runtime, te  # noqa: F401
 from .module import ChainFunction, build  # noqa: F401
 
-__all__ = ["auto_compute", "auto_schedule", "auto_tensorize", "hardware", "runtime", "te", "build", "ChainFunction"]
+__all__ = ["auto_compute", "auto_schedule", "auto_tensorize", "chimera", "hardware", "runtime", "te", "build",
+           "ChainFunction"]

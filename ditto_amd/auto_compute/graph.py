@@ -68,7 +68,9 @@ class Layer:
         parts = []
         for op in self.all_ops:
             kind = getattr(op, "kind", "placeholder")
-            parts.append("%s:%s:%s:%s" % (op.name, kind, list(op.output(0).shape), op.output(0).dtype))
+            attrs = getattr(op, "attrs", None)
+            tail = (":" + ",".join("%s=%s" % kv for kv in sorted(attrs.items()))) if attrs else ""
+            parts.append("%s:%s:%s:%s%s" % (op.name, kind, list(op.output(0).shape), op.output(0).dtype, tail))
         return "|".join(parts)
 
     def __str__(self):

@@ -10,7 +10,8 @@ every head straight into its columns of the ``[batch, M, hidden]`` output.
 """
 import torch
 
-from .... import chain
+from .... import chain, te
+from ...graph import Layer
 
 MUTI_HEAD_ATTENTION_LAYER = "multi_head_attention_mma_layer"  # the reference's dispatch key (:7)
 SELF_ATTENTION_MODULE_REG = set([MUTI_HEAD_ATTENTION_LAYER])
@@ -48,7 +49,25 @@ class MultiHeadAttentionMMA:
         return (query.view(shape).permute(0, 2, 1, 3), key.view(shape).permute(0, 2, 3, 1),
                 value.view(shape).permute(0, 2, 1, 3))
 
-    def forward(self, query_key_value, out=None):
+    def layer(self, batch, M):
+        """The attention block as a ``Layer`` named ``multi_head_attention_mma_layer`` (the name
+        ``is_self_attention_layer`` / ``chimera.task_binding`` dispatch on, :7-12): one input, the
+        packed ``[batch, M, 3 * hidden]`` projection, one output ``[batch, M, hidden]``.  The head
+        split / merge of :47-57, :71-73 is part of the op (``kind = "mha"``) rather than separate
+        layout ops, because the kernel does it by addressing."""
+        qkv = te.placeholder([batch, M, 3 * self.hidden_size], name="query_key_value", dtype=self.in_dtype)
+        out = te.compute(
+            [batch, M, self.hidden_size], "multi_head_attention", self.in_dtype, "mha",
+            lambda b, m, c: [(qkv, [b, m, c])], axis_names=["b", "m", "c"],
+            attrs={"num_heads": self.num_heads, "head_dim": self.model_k, "scale": self.scale,
+                   "acc_dtype": self.acc_dtype, "mma": (self.MI, self.NI, self.KI)},
+        )
+        return Layer(self.name, [out.op], [qkv], [], [], [])
+
+    def __call__(self, query_key_value, out=None):
+        return self.forward(query_key_value, out)
+
+    def forward(self, query_key_value, out=None, tile_variant=0):
         """query_key_value: [batch, M, 3 * hidden] (query | key | value along the last axis).
         Returns [batch, M, hidden]; ``out`` may be given (destination passing)."""
         q, k, v = self.head_views(query_key_value)
@@ -56,7 +75,7 @@ class MultiHeadAttentionMMA:
         if out is None:
             out = torch.empty(batch, M, self.hidden_size, dtype=query_key_value.dtype, device=query_key_value.device)
         o = out.view(batch, M, self.num_heads, self.model_k).permute(0, 2, 1, 3)
-        chain.run_bmm_chain(q, k, v, o, "softmax", self.scale)
+        chain.run_bmm_chain(q, k, v, o, "softmax", self.scale, tile_variant=tile_variant)
         return out
 
     __call__ = forward

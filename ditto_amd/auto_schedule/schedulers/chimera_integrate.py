@@ -150,3 +150,75 @@ def auto_schedule_bmm_chain_hip(key, log_file, A, B, C, F, inter_op="softmax", s
     if known is not None:
         return known
     return select_tile_variant(key, log_file, A, B, C, F, inter_op, softmax_scale).record["variant"]
+
+
+# ---- layer-level entry points (chimera_integrate.py:452-556 of the reference) -------------------
+class AttentionSchedule:
+    """What scheduling a ``multi_head_attention_mma_layer`` yields: the layer, the module that runs
+    it and the kernel variant chosen for its shape (0: the library's table)."""
+
+    def __init__(self, layer, module, tile_variant=0):
+        self.layer = layer
+        self.module = module
+        self.tile_variant = int(tile_variant)
+
+
+def _attention_module(layer, schedule_option=None):
+    from ...auto_compute.nn.module import MultiHeadAttentionMMA
+
+    op = layer.ops[0]
+    if getattr(op, "kind", None) != "mha":
+        raise ValueError("layer %s is not a multi-head attention layer" % layer.name)
+    a = op.attrs
+    mi, ni, ki = a.get("mma", (16, 16, 16))
+    return MultiHeadAttentionMMA(a["num_heads"], a["num_heads"] * a["head_dim"], op.output(0).dtype,
+                                 a.get("acc_dtype", "float32"), mi, ni, ki, scale=a["scale"])
+
+
+def _attention_operands(layer, module, dev="cuda:0"):
+    """Synthetic operands of the layer's shape for measurement: the packed projection and the
+    output, and the per-head views the kernel is called with."""
+    import torch
+
+    dt = {"float16": torch.float16, "bfloat16": torch.bfloat16}[layer.inputs[0].dtype]
+    qkv = torch.randn(tuple(layer.inputs[0].shape), device=dev).to(dt)
+    out = torch.empty(tuple(layer.ops[0].output(0).shape), dtype=dt, device=dev)
+    q, k, v = module.head_views(qkv)
+    batch, M = qkv.shape[0], qkv.shape[1]
+    o = out.view(batch, M, module.num_heads, module.model_k).permute(0, 2, 1, 3)
+    return q, k, v, o
+
+
+def chimera_log_file(schedule_option):
+    """The reference writes its measurements to ``chimera_<log_file>`` (:326-333, :530)."""
+    head, tail = os.path.split(schedule_option.log_file)
+    return os.path.join(head, "chimera_" + tail)
+
+
+def auto_schedule(wkl_key, layer, schedule_option):
+    """Measure the kernel variants for the layer's shape and log them (:452-512)."""
+    module = _attention_module(layer, schedule_option)
+    q, k, v, o = _attention_operands(layer, module)
+    return select_tile_variant(wkl_key, chimera_log_file(schedule_option), q, k, v, o, "softmax", module.scale)
+
+
+def auto_schedule_tasks(tasks, schedule_option):
+    """``tasks``: OrderedDict[workload key, [layers]]; tunes the first layer of every key (:515-519)."""
+    params = []
+    for wkl_key, layers in tasks.items():
+        entry = auto_schedule(wkl_key, layers[0], schedule_option)
+        params.append({"wkl_key": wkl_key, "entry": entry.to_json()})
+    return params
+
+
+def auto_schedule_build_tasks(tasks, schedule_option):
+    """{workload key: (schedule, schedule_tensors)} from the best logged record of every task
+    (:527-556); a task without a record gets the library's own choice."""
+    best = load_best_records(chimera_log_file(schedule_option))
+    schedules = {}
+    for k, layers in tasks.items():
+        layer = layers[0]
+        variant = best[k]["record"]["variant"] if k in best else 0
+        schedules[k] = (AttentionSchedule(layer, _attention_module(layer, schedule_option), variant),
+                        layer.schedule_tensors)
+    return schedules

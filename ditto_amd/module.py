@@ -84,5 +84,28 @@ class ChainFunction:
         return evaluator
 
 
+class AttentionFunction:
+    """The built ``multi_head_attention_mma_layer``: ``f(query_key_value, out)`` runs the fused
+    BMM -> softmax -> BMM chain over the per-head views of the packed projection."""
+
+    entry_name = "default_function"
+
+    def __init__(self, sch, tensors=None, target="hip"):
+        if target not in ("hip", "rocm", "cuda"):
+            raise ValueError("the fused chains are built for HIP devices only (target %r)" % target)
+        self.sch = sch
+        self.tensors = list(tensors) if tensors is not None else sch.layer.schedule_tensors
+
+    def __call__(self, query_key_value, out):
+        for a, t in zip((query_key_value, out), self.tensors):
+            if tuple(a.shape) != tuple(t.shape):
+                raise ValueError("argument for %s has shape %s, expected %s" % (t.name, tuple(a.shape), t.shape))
+        self.sch.module.forward(query_key_value, out, tile_variant=self.sch.tile_variant)
+
+
 def build(sch, tensors=None, target="hip", name="default_function"):
+    from .auto_schedule.schedulers.chimera_integrate import AttentionSchedule
+
+    if isinstance(sch, AttentionSchedule):
+        return AttentionFunction(sch, tensors, target)
     return ChainFunction(sch, tensors, target)

@@ -225,3 +225,53 @@ def test_tile_variant_space_and_analytic_filter():
     sc = {t["variant"]: ci.evaluate_param_hip(small, t) for t in ci.make_tile_variant_space(small)}
     assert min(sc, key=sc.get) in (1281, 1282, 1288)
     assert ci.workload_key(big) != ci.workload_key(small)
+
+
+def test_attention_layer_task_extraction_and_binding():
+    """bert_inference.py:88-92 -- tasks keyed by layer fingerprint, attention layers bound to the
+    chimera scheduler (chimera/task_binding.py:6-20), everything else to ansor."""
+    from ditto_amd import auto_schedule, chimera, runtime
+
+    mha = ac.nn.module.MultiHeadAttentionMMA(12, 768, "float16", "float32", scale=None)
+    other = ac.nn.module.MultiHeadAttentionMMA(6, 768, "float16", "float32", scale=None)
+    layer = mha.layer(2, 512)
+    assert layer.name == "multi_head_attention_mma_layer" and ac.nn.module.is_self_attention_layer(layer)
+    assert [tuple(t.shape) for t in layer.schedule_tensors] == [(2, 512, 2304), (2, 512, 768)]
+    # same shapes, different head count: a different workload
+    assert layer.fingerprint != other.layer(2, 512).fingerprint
+    assert layer.fingerprint == mha.layer(2, 512).fingerprint
+    ins, outs = ac.nn.functional.BatchGemmGemm(4, 64, 64, 64, 64, "float16", "float32")
+    gemm = ac.layer([outs[0].op], inputs=ins, name="gemm_chain_layer")
+    graph = chimera.graph_fusion(runtime.Graph([mha.layer(2, 512), gemm, mha.layer(2, 512)], outputs=[(2, 0)]))
+    tasks = auto_schedule.extract_tasks_from_graph(graph)
+    assert list(tasks) == [layer.fingerprint, gemm.fingerprint] and [len(v) for v in tasks.values()] == [2, 1]
+    bound = chimera.task_binding(tasks)
+    assert list(bound) == ["chimera", "ansor"]
+    assert list(bound["chimera"]) == [layer.fingerprint] and list(bound["ansor"]) == [gemm.fingerprint]
+    opt = auto_schedule.ScheduleOption("hip", log_file="x.log", device_name="gpu.hip.MI355X", mma_MI=32)
+    assert opt.trials == 100 and opt.mma_in_dtype == "float16" and opt.mma_MI == 32 and opt.device is not None
+    with pytest.raises(NotImplementedError):  # the generic scheduler is outside this package
+        auto_schedule.retrieve_schedule_bound_tasks(bound, opt)
+    with pytest.raises(ValueError):
+        auto_schedule.get_tasks_scheduler_builder("tvm")
+
+
+def test_retrieve_attention_schedule_from_log(tmp_path):
+    """auto_schedule_build_tasks keeps the record with the smallest value per workload key
+    (chimera_integrate.py:527-556) and falls back to the library's choice for an unseen key."""
+    import json
+
+    from ditto_amd import auto_schedule, chimera, runtime
+
+    mha = ac.nn.module.MultiHeadAttentionMMA(12, 768, "float16", "float32", scale=None)
+    graph = runtime.Graph([mha.layer(1, 512)])
+    bound = chimera.task_binding(auto_schedule.extract_tasks_from_graph(graph))
+    opt = auto_schedule.ScheduleOption("hip", log_file=str(tmp_path / "bert.log"))
+    (key,) = bound["chimera"]
+    sch, args = auto_schedule.retrieve_schedule_bound_tasks(bound, opt)[key]
+    assert sch.tile_variant == 0 and [tuple(t.shape) for t in args] == [(1, 512, 2304), (1, 512, 768)]
+    with open(tmp_path / "chimera_bert.log", "w") as f:
+        for variant, value in ((641, 0.03), (648, 0.02), (642, 0.05)):
+            print(json.dumps({"wkl_key": key, "entry": {"record": {"variant": variant}, "value": value}}), file=f)
+    sch, _ = auto_schedule.retrieve_schedule_bound_tasks(bound, opt)[key]
+    assert sch.tile_variant == 648 and sch.module.num_heads == 12 and sch.module.scale == 64 ** -0.5

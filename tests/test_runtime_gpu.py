@@ -75,3 +75,55 @@ def test_hip_graph_engine_replays_match_eager():
         eager.run()
         torch.cuda.synchronize()
     assert 0 < replay.timeit(20) < 5.0
+
+
+def test_attention_blocks_through_task_binding_and_graph_engine(tmp_path, oracle):
+    """The flow of benchmark/chimera/cuda/bert_inference.py:59-129 for the attention layers: extract
+    tasks, bind to the chimera scheduler, tune (log written), build, run through the graph engine;
+    then ``test`` mode rebuilds from the log alone and must give the same numbers."""
+    import json
+
+    import numpy as np
+
+    from ditto_amd.drivers import bert_inference
+
+    kw = dict(dtype="float16", batch=2, seq_len=256, hidden=256, n_layers=3, attn_heads=4, number=5,
+              log_dir=str(tmp_path))
+    cost, outs, schedules = bert_inference.inference(test=False, **kw)
+    assert 0 < cost < 50 and len(outs) == 3 and len(schedules) == 1
+    logs = list(tmp_path.glob("chimera_*.log"))
+    assert len(logs) == 1
+    lines = [json.loads(l) for l in logs[0].read_text().splitlines()]
+    assert lines and all(set(l) == {"wkl_key", "entry"} and l["entry"]["value"] > 0 for l in lines)
+    (key,) = schedules
+    best = min(lines, key=lambda l: l["entry"]["value"])["entry"]["record"]["variant"]
+    assert schedules[key][0].tile_variant == best
+    # test mode: nothing is measured, the schedule comes from the log
+    before = logs[0].read_text()
+    cost2, outs2, schedules2 = bert_inference.inference(test=True, hip_graph=False, **kw)
+    assert logs[0].read_text() == before and schedules2[key][0].tile_variant == best
+
+    # numbers: feed one known projection to every layer and compare with the CPU checker
+    from ditto_amd import auto_schedule, chimera
+
+    mha = ac.nn.module.MultiHeadAttentionMMA(4, 256, "float16", "float32", scale=None)
+    graph = runtime.Graph([mha.layer(2, 256) for _ in range(2)], outputs=[(0, 0), (1, 0)])
+    bound = chimera.task_binding(auto_schedule.extract_tasks_from_graph(graph))
+    opt = auto_schedule.ScheduleOption("hip", log_file=str(tmp_path / logs[0].name[len("chimera_"):]))
+    mods = {k: ditto.build(s, a, "hip") for k, (s, a) in auto_schedule.retrieve_schedule_bound_tasks(bound, opt).items()}
+    rng = np.random.default_rng(7)
+    qkv = oracle.np_round_to(rng.standard_normal((2, 256, 768)).astype(np.float32), "float16")
+    x = torch.from_numpy(qkv).half().cuda()
+    for make in (runtime.create_graph_engine, runtime.create_hip_graph_engine):
+        eng = make(graph, mods, "cuda:0")
+        eng.set_inputs([x, x])
+        eng.compile()
+        eng.run()
+        torch.cuda.synchronize()
+        q, k, v = (qkv[:, :, i * 256:(i + 1) * 256].reshape(2, 256, 4, 64).transpose(0, 2, 1, 3).reshape(8, 256, 64)
+                   for i in range(3))
+        want = oracle.bmm_chain_f64(q, np.ascontiguousarray(k.transpose(0, 2, 1)), v, inter="softmax", scale=0.125)
+        want = want.reshape(2, 4, 256, 64).transpose(0, 2, 1, 3).reshape(2, 256, 256)
+        for got in eng.get_outputs():
+            err = np.abs(got.float().cpu().numpy() - want)
+            assert err.max() <= 1e-2 and np.linalg.norm(err) / np.linalg.norm(want) <= 1e-3
