@@ -449,7 +449,8 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
     a.cols_in = (a.TW - 1) * a.stride + a.S;
     const int RS1 = a.R * a.S;
     int lds = ditto::conv_chain_lds_bytes(a.rows_in, a.cols_in, RS1, 32 * c1t, 32);
-    const int lds2 = ditto::conv_chain2_lds_bytes(slots, 32 * c1t, a.R2 * a.S2);
+    a.wide2 = d->out_dtype != DITTO_F32 && Q2 % 8 == 0 && a.TW2 % 8 == 0;
+    const int lds2 = ditto::conv_chain2_lds_bytes(slots, 32 * c1t, a.S2, a.wide2 != 0);
     if (lds2 > lds) lds = lds2;
     if (lds > 160 * 1024) return fail(DITTO_EUNSUPPORTED, "conv chain tile does not fit in LDS");
     a.tiles_h = (int)((P2 + a.TH2 - 1) / a.TH2);
@@ -724,14 +725,16 @@ int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const vo
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool f16 = d->in_dtype == DITTO_F16;
   hipError_t e = hipSuccess;
-  if (workspace)  // W1 into the chunked layout the chain kernel copies straight into LDS
+  if (workspace && plan.px2 == 0)  // W1 into the chunked layout the chain kernel copies straight into LDS
     e = f16 ? ditto::pack_conv_w1_f16(plan.c1_tiles, plan.ch, a, workspace, st)
             : ditto::pack_conv_w1_bf16(plan.c1_tiles, plan.ch, a, workspace, st);
   if (plan.px2 > 0) {
     void* w2p = static_cast<char*>(workspace) + plan.w1p_bytes;
     a.w2p = w2p;
-    if (e == hipSuccess)
-      e = f16 ? ditto::pack_conv_w2_f16(plan.c1_tiles, a, w2p, st) : ditto::pack_conv_w2_bf16(plan.c1_tiles, a, w2p, st);
+    if (a.wide2 && !aligned(y, 16)) a.wide2 = 0;  // plain 2-byte stores (the LDS size follows the flag)
+    // both weight tensors into their chunked layouts, one launch
+    e = f16 ? ditto::pack_conv_w2_f16(plan.c1_tiles, a, workspace, w2p, st)
+            : ditto::pack_conv_w2_bf16(plan.c1_tiles, a, workspace, w2p, st);
     if (e == hipSuccess)
       e = f16 ? ditto::launch_conv2_f16(plan.c1_tiles, plan.px2, a, st) : ditto::launch_conv2_bf16(plan.c1_tiles, plan.px2, a, st);
   } else if (e == hipSuccess) {

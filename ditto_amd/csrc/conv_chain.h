@@ -23,6 +23,8 @@
 // convolution is done.  The tile is sized so that two workgroups fit in a CU's LDS: one
 // stages while the other feeds the MFMA pipe.
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 
 namespace ditto {
@@ -47,6 +49,7 @@ struct ConvChainArgs {
   int R2, S2, pad2;
   int P2, Q2;        // output extent
   int TH2, TW2;      // output tile per workgroup
+  int wide2;         // 16-byte output stores through LDS: Q2 and TW2 multiples of 8, y 16-byte aligned, not fp32
 };
 
 // Input channels per staged chunk: 32 (two MFMA k steps per tap) or, where that does not fit in
@@ -65,32 +68,18 @@ __host__ __device__ inline int conv_chain_lds_bytes(int rows_in, int cols_in, in
 }
 
 // Second convolution larger than 1x1: the intermediate tile lives in LDS as [slot][C1p + 8] and W2
-// streams through two buffers of [R2*S2][64 output channels][32 + 8] (chunks of 32 intermediate
-// channels for blocks of 64 output channels).
+// streams through two buffers of [S2][64 output channels][32 + 8]: one filter row of a chunk of 32
+// intermediate channels for a block of 64 output channels per stage (small enough for two
+// workgroups per CU).  The packed W2 holds the R2 rows of a (block, chunk) back to back.  `wide`
+// adds the per-wave turn-around buffers of the 16-byte output stores.
+constexpr int kConv2Oss = 40;  // row stride (elements) of a wave's output turn-around buffer: 32 pixels + 8
 __host__ __device__ inline int conv_w2_chunk_bytes(int RS2) { return RS2 * 64 * conv_ch_stride(32) * 2; }
-__host__ __device__ inline int conv_chain2_lds_bytes(int slots, int C1p, int RS2) {
-  return slots * (C1p + 8) * 2 + 2 * ((conv_w2_chunk_bytes(RS2) + 1023) / 1024 * 1024);
+__host__ __device__ inline int conv_w2_row_bytes(int S2) { return S2 * 64 * conv_ch_stride(32) * 2; }
+__host__ __device__ inline int conv_chain2_lds_bytes(int slots, int C1p, int S2, bool wide) {
+  return slots * (C1p + 8) * 2 + 2 * ((conv_w2_row_bytes(S2) + 1023) / 1024 * 1024) + (wide ? 4 * 32 * kConv2Oss * 2 : 0);
 }
 
-// W2[c2][c1][r][s] -> [c2 / 64][c1 / 32][r*S+s][64][32 + 8] (zero padded)
-template <typename T>
-__global__ void pack_conv_w2_kernel(const T* __restrict__ w2, T* __restrict__ out, int C1, int C2, int RS2, int C1p,
-                                    long long total) {
-  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= total) return;
-  const int c = (int)(i % 40);
-  long long q = i / 40;
-  const int c2l = (int)(q % 64);
-  q /= 64;
-  const int tap = (int)(q % RS2);
-  q /= RS2;
-  const int chunk = (int)(q % (C1p / 32));
-  const int c2b = (int)(q / (C1p / 32));
-  const int c1 = chunk * 32 + c, c2 = c2b * 64 + c2l;
-  T v = (T)0.f;
-  if (c < 32 && c1 < C1 && c2 < C2) v = w2[((long long)c2 * C1 + c1) * RS2 + tap];
-  out[i] = v;
-}
+// The packed W2 is [c2 / 64][c1 / 32][r*S2+s][64][32 + 8] (zero padded); see pack_conv_w12_kernel.
 
 // W1[c1][c0][r][s] -> chunks [c0 / ch][r*S+s][C1p][ch + 8] (zero padded): the layout the chain
 // kernel keeps a chunk in, so that it can load one with direct global -> LDS copies.
@@ -352,15 +341,16 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
     // ================= second convolution R2 x S2, intermediate tile through LDS =================
     constexpr int MS = C1p + 8;  // element stride of an intermediate pixel's channel vector
     T* const Ms = reinterpret_cast<T*>(smem_raw);  // [128*PXW][MS]
-    T* const W2b = Ms + 128 * PXW * MS;            // two chunk buffers
+    T* const W2b = Ms + 128 * PXW * MS;            // two row-chunk buffers
     const int RS2 = p.R2 * p.S2;
-    const int w2_bytes = conv_w2_chunk_bytes(RS2);
+    const int w2_bytes = conv_w2_row_bytes(p.S2);
     const int w2_buf = (w2_bytes + 1023) / 1024 * 1024;
     constexpr int nch2 = C1p / 32;
     const int nc2b = (p.C2 + 63) / 64;
-    const int nstage = nc2b * nch2;
+    const int nstage = nc2b * nch2 * p.R2;  // stage = (output block, intermediate chunk, filter row)
     const i32x4 w2_rsrc = make_rsrc(p.w2p, (unsigned)(w2_bytes * nstage));
     const unsigned w2_lds = (unsigned)(size_t)(DITTO_LDS char*)smem_raw + 128 * PXW * MS * 2;
+    T* const Ow = reinterpret_cast<T*>(reinterpret_cast<char*>(W2b) + 2 * w2_buf) + wave * 32 * kConv2Oss;
     auto w2_issue = [&](int stage) __attribute__((always_inline)) {
       for (int j = wave; j * 1024 < w2_bytes; j += 4) {
         const int off = j * 1024 + lane * 16;
@@ -404,24 +394,27 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
     }
     const long long plane2 = (long long)p.P2 * p.Q2;
     f32x16 o[2][PX2];
-    for (int stage = 0; stage < nstage; ++stage) {
-      const int c2b = stage / nch2, ch = stage % nch2;
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();  // this stage's chunk has landed; everyone is done with the previous one
-      if (stage + 1 < nstage) w2_issue(stage + 1);
-      if (ch == 0) {
+    // WIDE: operands swapped, pixel-major result o[t][j][r] = out[pixel 8(r/4) + 4g + r%4][c2 = 32t + ln]
+    auto run_stages = [&](auto wide_tag) __attribute__((always_inline)) {
+      constexpr bool WIDE = decltype(wide_tag)::value;
+      for (int stage = 0; stage < nstage; ++stage) {
+        const int r = stage % p.R2, sc = stage / p.R2;
+        const int c2b = sc / nch2, ch = sc % nch2;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();  // this stage's rows have landed; everyone is done with the previous ones
+        if (stage + 1 < nstage) w2_issue(stage + 1);
+        if (ch == 0 && r == 0) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+          for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int j = 0; j < PX2; ++j)
+            for (int j = 0; j < PX2; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o[t][j][r] = 0.f;
-      }
-      const T* wbuf = reinterpret_cast<const T*>(reinterpret_cast<const char*>(W2b) + (stage & 1) * w2_buf);
-      for (int r = 0; r < p.R2; ++r)
+              for (int q = 0; q < 16; ++q) o[t][j][q] = 0.f;
+        }
+        const T* wbuf = reinterpret_cast<const T*>(reinterpret_cast<const char*>(W2b) + (stage & 1) * w2_buf);
         for (int s2 = 0; s2 < p.S2; ++s2) {
           const int tap = (r * p.TW + s2) * MS + 32 * ch;
-          const T* wrow = wbuf + ((r * p.S2 + s2) * 64 + ln) * 40 + 8 * g;
+          const T* wrow = wbuf + (s2 * 64 + ln) * 40 + 8 * g;
           V8 mf[2][PX2], wf[2][2];
 #pragma unroll
           for (int kk = 0; kk < 2; ++kk) {
@@ -435,30 +428,67 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-              for (int j = 0; j < PX2; ++j) o[t][j] = Elem<T>::mfma32(wf[kk][t], mf[kk][j], o[t][j]);
+              for (int j = 0; j < PX2; ++j)
+                o[t][j] = WIDE ? Elem<T>::mfma32(mf[kk][j], wf[kk][t], o[t][j]) : Elem<T>::mfma32(wf[kk][t], mf[kk][j], o[t][j]);
         }
-      if (ch == nch2 - 1) {
-        // o[t][j][r] = out^T[c2 = 64 c2b + 32t + 8(r/4) + 4g + r%4][pixel of lane]
+        if (ch == nch2 - 1 && r == p.R2 - 1) {
+          if constexpr (WIDE) {
+            // four consecutive pixels of one channel per register quad -> 8-byte LDS writes into this
+            // wave's corner, then 16-byte stores (8 pixels of one output row)
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int j = 0; j < PX2; ++j) {
-            if (!valid2[j]) continue;
+              for (int j = 0; j < PX2; ++j) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int c2 = 64 * c2b + 32 * t + 8 * (r >> 2) + 4 * g + (r & 3);
-              if (c2 >= p.C2) continue;
-              float v = o[t][j][r];
-              if (p.relu_out) v = fmaxf(v, 0.f);
-              const long long off = ((long long)n * p.C2 + c2) * plane2 + opix2[j];
-              if (p.out_f32)
-                reinterpret_cast<float*>(p.y)[off] = v;
-              else
-                reinterpret_cast<T*>(p.y)[off] = (T)v;
-            }
+                for (int q = 0; q < 4; ++q) {
+                  float v[4];
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) {
+                    v[e] = o[t][j][4 * q + e];
+                    if (p.relu_out) v[e] = fmaxf(v[e], 0.f);
+                  }
+                  const typename Elem<T>::v2 a0 = cvt2<T>(v[0], v[1]), a1 = cvt2<T>(v[2], v[3]);
+                  *reinterpret_cast<V4*>(Ow + ln * kConv2Oss + 8 * q + 4 * g) = V4{a0[0], a0[1], a1[0], a1[1]};
+                }
+#pragma unroll
+                for (int v0 = 0; v0 < 128; v0 += 64) {
+                  const int v = v0 + lane;
+                  const int chn = v >> 2, sv = v & 3;
+                  const int c2 = 64 * c2b + 32 * t + chn;
+                  const int slot = 32 * (PX2 * wave + j) + 8 * sv;
+                  const int oh = slot / p.TW2, ow = slot - oh * p.TW2;
+                  const V8 px = *reinterpret_cast<const V8*>(Ow + chn * kConv2Oss + 8 * sv);
+                  if (c2 < p.C2 && oh < p.TH2 && op0 + oh < p.P2 && oq0 + ow < p.Q2)
+                    *reinterpret_cast<V8*>(reinterpret_cast<T*>(p.y) + ((long long)n * p.C2 + c2) * plane2 +
+                                           (long long)(op0 + oh) * p.Q2 + oq0 + ow) = px;
+                }
+              }
+          } else {
+            // o[t][j][q] = out^T[c2 = 64 c2b + 32t + 8(q/4) + 4g + q%4][pixel of lane]
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+              for (int j = 0; j < PX2; ++j) {
+                if (!valid2[j]) continue;
+#pragma unroll
+                for (int q = 0; q < 16; ++q) {
+                  const int c2 = 64 * c2b + 32 * t + 8 * (q >> 2) + 4 * g + (q & 3);
+                  if (c2 >= p.C2) continue;
+                  float v = o[t][j][q];
+                  if (p.relu_out) v = fmaxf(v, 0.f);
+                  const long long off = ((long long)n * p.C2 + c2) * plane2 + opix2[j];
+                  if (p.out_f32)
+                    reinterpret_cast<float*>(p.y)[off] = v;
+                  else
+                    reinterpret_cast<T*>(p.y)[off] = (T)v;
+                }
+              }
           }
+        }
       }
-    }
+    };
+    if (p.wide2) run_stages(std::true_type());
+    else run_stages(std::false_type());
     return;
   }
 
@@ -574,7 +604,7 @@ template <typename T, int C1T, int PXW, int CH, int PX2 = 0>
 hipError_t launch_conv_chain(const ConvChainArgs& args, hipStream_t stream) {
   int lds = conv_chain_lds_bytes(args.rows_in, args.cols_in, args.R * args.S, 32 * C1T, CH);
   if (PX2 > 0) {
-    const int lds2 = conv_chain2_lds_bytes(128 * PXW, 32 * C1T, args.R2 * args.S2);
+    const int lds2 = conv_chain2_lds_bytes(128 * PXW, 32 * C1T, args.S2, args.wide2 != 0);
     if (lds2 > lds) lds = lds2;
   }
   auto kern = conv_chain_kernel<T, C1T, PXW, CH, PX2>;
@@ -605,14 +635,55 @@ hipError_t launch_pack_conv_w1(const ConvChainArgs& args, int C1p, int ch, void*
   return hipGetLastError();
 }
 
-// repack W2 for a second convolution larger than 1x1 (conv_w2_chunk_bytes * blocks * chunks bytes)
+// repack W1 (as launch_pack_conv_w1) and, for a second convolution larger than 1x1, W2
+// (conv_w2_chunk_bytes * blocks * chunks bytes) in ONE launch: the first blocks do W1, the rest W2
 template <typename T>
-hipError_t launch_pack_conv_w2(const ConvChainArgs& args, int C1p, void* out, hipStream_t stream) {
-  const int RS2 = args.R2 * args.S2;
-  const long long total = (long long)((args.C2 + 63) / 64) * (C1p / 32) * RS2 * 64 * 40;
-  const unsigned grid = (unsigned)((total + 255) / 256);
-  hipLaunchKernelGGL(pack_conv_w2_kernel<T>, dim3(grid), dim3(256), 0, stream, reinterpret_cast<const T*>(args.w2),
-                     reinterpret_cast<T*>(out), args.C1, args.C2, RS2, C1p, total);
+__global__ void pack_conv_w12_kernel(const T* __restrict__ w1, T* __restrict__ out1, int C0, int C1, int RS, int C1p,
+                                     int ch, long long total1, unsigned blocks1, const T* __restrict__ w2,
+                                     T* __restrict__ out2, int C2, int RS2, long long total2) {
+  if (blockIdx.x < blocks1) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total1) return;
+    const int chs = conv_ch_stride(ch);
+    const int c = (int)(i % chs);
+    long long q = i / chs;
+    const int c1 = (int)(q % C1p);
+    q /= C1p;
+    const int rs = (int)(q % RS);
+    const int chunk = (int)(q / RS);
+    const int c0 = chunk * ch + c;
+    T v = (T)0.f;
+    if (c < ch && c1 < C1 && c0 < C0) v = w1[((long long)c1 * C0 + c0) * RS + rs];
+    out1[i] = v;
+  } else {
+    const long long i = (long long)(blockIdx.x - blocks1) * blockDim.x + threadIdx.x;
+    if (i >= total2) return;
+    const int c = (int)(i % 40);
+    long long q = i / 40;
+    const int c2l = (int)(q % 64);
+    q /= 64;
+    const int tap = (int)(q % RS2);
+    q /= RS2;
+    const int chunk = (int)(q % (C1p / 32));
+    const int c2b = (int)(q / (C1p / 32));
+    const int c1 = chunk * 32 + c, c2 = c2b * 64 + c2l;
+    T v = (T)0.f;
+    if (c < 32 && c1 < C1 && c2 < C2) v = w2[((long long)c2 * C1 + c1) * RS2 + tap];
+    out2[i] = v;
+  }
+}
+
+template <typename T>
+hipError_t launch_pack_conv_w12(const ConvChainArgs& args, int C1p, int ch, void* out1, void* out2, hipStream_t stream) {
+  const int RS = args.R * args.S, RS2 = args.R2 * args.S2;
+  const int nchunks = (args.C0 + ch - 1) / ch;
+  const long long total1 = (long long)nchunks * RS * C1p * conv_ch_stride(ch);
+  const long long total2 = (long long)((args.C2 + 63) / 64) * (C1p / 32) * RS2 * 64 * 40;
+  const unsigned blocks1 = (unsigned)((total1 + 255) / 256), blocks2 = (unsigned)((total2 + 255) / 256);
+  hipLaunchKernelGGL(pack_conv_w12_kernel<T>, dim3(blocks1 + blocks2), dim3(256), 0, stream,
+                     reinterpret_cast<const T*>(args.w1), reinterpret_cast<T*>(out1), args.C0, args.C1, RS, C1p, ch,
+                     total1, blocks1, reinterpret_cast<const T*>(args.w2), reinterpret_cast<T*>(out2), args.C2, RS2,
+                     total2);
   return hipGetLastError();
 }
 

@@ -31,8 +31,8 @@ hipError_t DITTO_INST2_NAME(int c1_tiles, int px2, const ConvChainArgs& args, hi
   return hipErrorInvalidValue;
 }
 
-hipError_t DITTO_PACK2_NAME(int c1_tiles, const ConvChainArgs& args, void* out, hipStream_t stream) {
-  return launch_pack_conv_w2<DITTO_INST_T>(args, 32 * c1_tiles, out, stream);
+hipError_t DITTO_PACK2_NAME(int c1_tiles, const ConvChainArgs& args, void* out1, void* out2, hipStream_t stream) {
+  return launch_pack_conv_w12<DITTO_INST_T>(args, 32 * c1_tiles, 32, out1, out2, stream);
 }
 
 // depthwise first convolution: c2_tiles in {1, 2, 4, 8} (32 output channels each); mode 0 | 1:
