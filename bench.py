@@ -99,8 +99,10 @@ def bytes_of(w):
     return eb * w["batch"] * (w["M"] * w["K"] + w["K"] * w["L"] + w["L"] * w["N"] + w["M"] * w["N"])
 
 
-def make_call(w, dev):
-    """Synthetic inputs resident on the device and a zero-argument callable that runs one step."""
+def make_call(w, dev, prepared=False):
+    """Synthetic inputs resident on the device and a zero-argument callable that runs one step.
+    ``prepared`` (conv chains that take a workspace): the weights are repacked once, outside the
+    step, as the reference's drivers are handed host-packed weights; the step is the fused kernel alone."""
     import torch
 
     from ditto_amd import chain
@@ -117,6 +119,9 @@ def make_call(w, dev):
         Q = (w["W"] + 2 * w["pad"] - w["R"]) // w["stride"] + 1 + 2 * pad2 - R2 + 1
         y = torch.empty(w["N"], w["C2"], P, Q, dtype=torch.float16, device=dev)
         desc = chain.conv_chain_desc(x, w1, w2, y, w["pad"], w["stride"], pad2, 1, "cast", False, groups)
+        if prepared:
+            ws = chain.prepare_conv_chain(desc, w1, w2)
+            return (lambda: chain.run_conv_chain(x, w1, w2, y, desc=desc, workspace=ws, prepared=True)), desc
         return (lambda: chain.run_conv_chain(x, w1, w2, y, desc=desc)), desc
     if w["kind"] == "requant":
         a = torch.randint(-127, 128, (w["M"], w["K"]), generator=g, dtype=torch.int8).to(dev)
@@ -140,14 +145,14 @@ def make_call(w, dev):
     return (lambda: chain.run_bmm_chain(a, b, c, f, desc=desc)), desc
 
 
-def time_gpu(w, steps, warmup, dev):
+def time_gpu(w, steps, warmup, dev, prepared=False):
     """(ms per step over the synchronised wall clock, ms per launch from HIP events around the eager
     loop, ms per launch from a graph replay of the same loop)."""
     import torch
 
     from ditto_amd import chain
 
-    call, desc = make_call(w, dev)
+    call, desc = make_call(w, dev, prepared)
     for _ in range(max(warmup, 1)):
         call()
     torch.cuda.synchronize()
@@ -250,6 +255,12 @@ def run_one(name, steps, warmup, dev):
     roof["algorithmic_bytes"] = by
     roof["kernel_ms"] = k_ms
     roof["graph_replay_ms"] = gr_ms
+    if w["kind"] == "conv" and w.get("groups", 1) == 1:
+        # the same step with the weight repacking done once beforehand (ditto_conv_chain_prepare +
+        # ditto_conv_chain_run_prepared): what a caller with fixed weights pays per call
+        _, pev_ms, pgr_ms, _ = time_gpu(w, steps, warmup, dev, prepared=True)
+        roof["weights_prepared_ms"] = pev_ms
+        roof["weights_prepared_graph_replay_ms"] = pgr_ms
     return w, wall_ms, ev_ms, tile, roof
 
 

@@ -113,6 +113,10 @@ EXPORTS = [
      [ctypes.POINTER(BmmChainDesc), _P, _P, _P, _P, _P, _P, ctypes.c_size_t, _P]),
     ("ditto_conv_chain_run", ctypes.c_int,
      [ctypes.POINTER(ConvChainDesc), _P, _P, _P, _P, _P, ctypes.c_size_t, _P]),
+    ("ditto_conv_chain_prepare", ctypes.c_int,
+     [ctypes.POINTER(ConvChainDesc), _P, _P, _P, ctypes.c_size_t, _P]),
+    ("ditto_conv_chain_run_prepared", ctypes.c_int,
+     [ctypes.POINTER(ConvChainDesc), _P, _P, _P, _P, _P, ctypes.c_size_t, _P]),
 ]
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libditto_chain.so")

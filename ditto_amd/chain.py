@@ -199,13 +199,38 @@ def _workspace(dev, nbytes):
     return buf
 
 
+def conv_chain_workspace_bytes(desc):
+    return _lib.load().ditto_conv_chain_workspace_bytes(ctypes.byref(desc))
+
+
+def prepare_conv_chain(desc, W1, W2, workspace=None):
+    """Repack the weights of a conv chain once (``ditto_conv_chain_prepare``); returns the workspace
+    tensor to hand to ``run_conv_chain(..., workspace=ws, prepared=True)`` for as long as W1 / W2 keep
+    their values.  ``workspace``: a uint8 tensor of ``conv_chain_workspace_bytes(desc)`` or None to
+    allocate one."""
+    lib = _lib.load()
+    dev = _check_device(W1, W2)
+    nbytes = conv_chain_workspace_bytes(desc)
+    if workspace is None:
+        workspace = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        rc = lib.ditto_conv_chain_prepare(ctypes.byref(desc), W1.data_ptr(), W2.data_ptr(), workspace.data_ptr(),
+                                          workspace.numel(), stream)
+    _lib.check(rc)
+    return workspace
+
+
 def run_conv_chain(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op="cast", relu_out=False,
-                   desc=None, workspace=None, groups1=1):
+                   desc=None, workspace=None, groups1=1, prepared=False):
     """Y = conv2d(inter(conv2d(X, W1)), W2) on the current stream: one fused kernel, preceded by
     a small kernel that repacks W1 into ``workspace`` (a uint8 tensor of
     ``ditto_conv_chain_workspace_bytes``; None: a cached per-device buffer; False: no
     workspace, the fused kernel re-lays W1 out itself, slower).  A depthwise first convolution
-    (``groups1 = C0``) is a single kernel and uses no workspace."""
+    (``groups1 = C0``) is a single kernel and uses no workspace.  ``prepared=True``: ``workspace`` was
+    filled by ``prepare_conv_chain`` for these weights; only the fused kernel runs."""
+    if prepared and (workspace is None or workspace is False):
+        raise ValueError("prepared=True needs the workspace that prepare_conv_chain returned")
     lib = _lib.load()
     dev = _check_device(X, W1, W2, Y)
     if desc is None:
@@ -219,8 +244,9 @@ def run_conv_chain(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op=
         ws = workspace
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        rc = lib.ditto_conv_chain_run(ctypes.byref(desc), X.data_ptr(), W1.data_ptr(), W2.data_ptr(),
-                                      Y.data_ptr(), ws.data_ptr() if ws is not None else None,
-                                      ws.numel() * ws.element_size() if ws is not None else 0, stream)
+        fn = lib.ditto_conv_chain_run_prepared if prepared else lib.ditto_conv_chain_run
+        rc = fn(ctypes.byref(desc), X.data_ptr(), W1.data_ptr(), W2.data_ptr(),
+                Y.data_ptr(), ws.data_ptr() if ws is not None else None,
+                ws.numel() * ws.element_size() if ws is not None else 0, stream)
     _lib.check(rc)
     return Y

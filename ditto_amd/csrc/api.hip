@@ -677,15 +677,24 @@ size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
   return plan.w1p_bytes + plan.w2p_bytes;
 }
 
-int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const void* w1, const void* w2,
-                         void* y, void* workspace, size_t workspace_bytes, void* stream) {
+}  // extern "C"
+
+namespace {
+// what a conv chain call does: repack the weights into the workspace, run the fused kernel, or both
+enum ConvPhase { kConvPrepare = 1, kConvCompute = 2, kConvBoth = 3 };
+
+int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, const void* w1, const void* w2,
+                    void* y, void* workspace, size_t workspace_bytes, void* stream) {
   ConvPlan plan;
   int rc = plan_conv(d, &plan, true);
   if (rc != DITTO_OK) return rc;
-  if (!x || !w1 || !w2 || !y) return fail(DITTO_EINVAL, "null data pointer");
+  if (((phase & kConvCompute) && (!x || !y)) || !w1 || !w2) return fail(DITTO_EINVAL, "null data pointer");
   if (!aligned(x, 2) || !aligned(w1, 2) || !aligned(w2, 8) || !aligned(y, 4))
     return fail(DITTO_EINVAL, "misaligned data pointer");
+  if (phase != kConvBoth && !plan.dw && !workspace)
+    return fail(DITTO_EWORKSPACE, "prepared weights live in the workspace: none given");
   if (plan.dw) {
+    if (!(phase & kConvCompute)) return DITTO_OK;  // nothing to prepare: the kernel stages the filters itself
     if (!aligned(w2, 16)) return fail(DITTO_EINVAL, "misaligned data pointer");
     ditto::DwConvArgs a = plan.dwargs;
     // less aligned pointers: narrower halo loads (the LDS layout stays valid) while the chunk still
@@ -711,6 +720,8 @@ int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const vo
     return DITTO_OK;
   }
   const size_t need = plan.w1p_bytes + plan.w2p_bytes;
+  if (plan.w1p_bytes >= (1ull << 31) || plan.w2p_bytes >= (1ull << 31))  // the repack kernels index with 32 bits
+    return fail(DITTO_EUNSUPPORTED, "conv chain weights too large to repack");
   if (plan.px2 > 0 && !workspace)
     return fail(DITTO_EWORKSPACE, "a second convolution larger than 1x1 needs the workspace (%zu bytes)", need);
   if (workspace && workspace_bytes < need)
@@ -725,7 +736,8 @@ int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const vo
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool f16 = d->in_dtype == DITTO_F16;
   hipError_t e = hipSuccess;
-  if (workspace && plan.px2 == 0)  // W1 into the chunked layout the chain kernel copies straight into LDS
+  const bool prepare = (phase & kConvPrepare) != 0, compute = (phase & kConvCompute) != 0;
+  if (workspace && plan.px2 == 0 && prepare)  // W1 into the chunked layout the chain kernel copies straight into LDS
     e = f16 ? ditto::pack_conv_w1_f16(plan.c1_tiles, plan.ch, a, workspace, st)
             : ditto::pack_conv_w1_bf16(plan.c1_tiles, plan.ch, a, workspace, st);
   if (plan.px2 > 0) {
@@ -733,15 +745,35 @@ int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const vo
     a.w2p = w2p;
     if (a.wide2 && !aligned(y, 16)) a.wide2 = 0;  // plain 2-byte stores (the LDS size follows the flag)
     // both weight tensors into their chunked layouts, one launch
-    e = f16 ? ditto::pack_conv_w2_f16(plan.c1_tiles, a, workspace, w2p, st)
-            : ditto::pack_conv_w2_bf16(plan.c1_tiles, a, workspace, w2p, st);
-    if (e == hipSuccess)
+    if (prepare)
+      e = f16 ? ditto::pack_conv_w2_f16(plan.c1_tiles, a, workspace, w2p, st)
+              : ditto::pack_conv_w2_bf16(plan.c1_tiles, a, workspace, w2p, st);
+    if (e == hipSuccess && compute)
       e = f16 ? ditto::launch_conv2_f16(plan.c1_tiles, plan.px2, a, st) : ditto::launch_conv2_bf16(plan.c1_tiles, plan.px2, a, st);
-  } else if (e == hipSuccess) {
+  } else if (e == hipSuccess && compute) {
     e = f16 ? ditto::launch_conv_f16(plan.c1_tiles, plan.ch, a, st) : ditto::launch_conv_bf16(plan.c1_tiles, plan.ch, a, st);
   }
   if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
   return DITTO_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ditto_conv_chain_run(const ditto_conv_chain_desc* d, const void* x, const void* w1, const void* w2,
+                         void* y, void* workspace, size_t workspace_bytes, void* stream) {
+  return conv_chain_call(kConvBoth, d, x, w1, w2, y, workspace, workspace_bytes, stream);
+}
+
+int ditto_conv_chain_prepare(const ditto_conv_chain_desc* d, const void* w1, const void* w2, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+  return conv_chain_call(kConvPrepare, d, nullptr, w1, w2, nullptr, workspace, workspace_bytes, stream);
+}
+
+int ditto_conv_chain_run_prepared(const ditto_conv_chain_desc* d, const void* x, const void* w1, const void* w2,
+                                  void* y, void* workspace, size_t workspace_bytes, void* stream) {
+  return conv_chain_call(kConvCompute, d, x, w1, w2, y, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

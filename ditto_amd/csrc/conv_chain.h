@@ -86,15 +86,15 @@ __host__ __device__ inline int conv_chain2_lds_bytes(int slots, int C1p, int S2,
 template <typename T>
 __global__ void pack_conv_w1_kernel(const T* __restrict__ w1, T* __restrict__ out, int C0, int C1, int RS, int C1p, int ch,
                                     long long total) {
-  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;  // the packed tensors are far below 2^31 elements
   if (i >= total) return;
-  const int chs = conv_ch_stride(ch);
+  const unsigned chs = conv_ch_stride(ch);
   const int c = (int)(i % chs);
-  long long q = i / chs;
-  const int c1 = (int)(q % C1p);
-  q /= C1p;
-  const int rs = (int)(q % RS);
-  const int chunk = (int)(q / RS);
+  unsigned q = i / chs;
+  const int c1 = (int)(q % (unsigned)C1p);
+  q /= (unsigned)C1p;
+  const int rs = (int)(q % (unsigned)RS);
+  const int chunk = (int)(q / (unsigned)RS);
   const int c0 = chunk * ch + c;
   T v = (T)0.f;
   if (c < ch && c1 < C1 && c0 < C0) v = w1[((long long)c1 * C0 + c0) * RS + rs];
@@ -642,30 +642,30 @@ __global__ void pack_conv_w12_kernel(const T* __restrict__ w1, T* __restrict__ o
                                      int ch, long long total1, unsigned blocks1, const T* __restrict__ w2,
                                      T* __restrict__ out2, int C2, int RS2, long long total2) {
   if (blockIdx.x < blocks1) {
-    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;  // the packed tensors are far below 2^31 elements
     if (i >= total1) return;
-    const int chs = conv_ch_stride(ch);
+    const unsigned chs = conv_ch_stride(ch);
     const int c = (int)(i % chs);
-    long long q = i / chs;
-    const int c1 = (int)(q % C1p);
-    q /= C1p;
-    const int rs = (int)(q % RS);
-    const int chunk = (int)(q / RS);
+    unsigned q = i / chs;
+    const int c1 = (int)(q % (unsigned)C1p);
+    q /= (unsigned)C1p;
+    const int rs = (int)(q % (unsigned)RS);
+    const int chunk = (int)(q / (unsigned)RS);
     const int c0 = chunk * ch + c;
     T v = (T)0.f;
     if (c < ch && c1 < C1 && c0 < C0) v = w1[((long long)c1 * C0 + c0) * RS + rs];
     out1[i] = v;
   } else {
-    const long long i = (long long)(blockIdx.x - blocks1) * blockDim.x + threadIdx.x;
+    const unsigned i = (blockIdx.x - blocks1) * blockDim.x + threadIdx.x;
     if (i >= total2) return;
-    const int c = (int)(i % 40);
-    long long q = i / 40;
-    const int c2l = (int)(q % 64);
-    q /= 64;
-    const int tap = (int)(q % RS2);
-    q /= RS2;
-    const int chunk = (int)(q % (C1p / 32));
-    const int c2b = (int)(q / (C1p / 32));
+    const int c = (int)(i % 40u);
+    unsigned q = i / 40u;
+    const int c2l = (int)(q % 64u);
+    q /= 64u;
+    const int tap = (int)(q % (unsigned)RS2);
+    q /= (unsigned)RS2;
+    const int chunk = (int)(q % (unsigned)(C1p / 32));
+    const int c2b = (int)(q / (unsigned)(C1p / 32));
     const int c1 = chunk * 32 + c, c2 = c2b * 64 + c2l;
     T v = (T)0.f;
     if (c < 32 && c1 < C1 && c2 < C2) v = w2[((long long)c2 * C1 + c1) * RS2 + tap];

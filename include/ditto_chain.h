@@ -187,6 +187,22 @@ int ditto_conv_chain_run(const ditto_conv_chain_desc* desc, const void* x, const
                          const void* w2, void* y, void* workspace, size_t workspace_bytes,
                          void* stream);
 
+/* The same call in two steps, for weights that stay fixed over many calls (inference): the
+ * reference's drivers are handed weights the host has already packed
+ * (conv3x3_conv1x1_cuda.py:99-103, :289-292), outside the timed function.
+ *   ditto_conv_chain_prepare      : only the weight repacking kernel, into `workspace`
+ *                                   (a no-op for depthwise chains, which use no workspace);
+ *   ditto_conv_chain_run_prepared : only the fused kernel, reading the workspace a prepare call
+ *                                   (same descriptor, same w1 / w2) has filled; the workspace is
+ *                                   read-only here, so such calls may overlap.  w1 / w2 must still
+ *                                   be passed (a 1x1 second convolution reads w2 directly).
+ * DITTO_EWORKSPACE if the chain takes a workspace and none (or too small a one) is given. */
+int ditto_conv_chain_prepare(const ditto_conv_chain_desc* desc, const void* w1, const void* w2,
+                             void* workspace, size_t workspace_bytes, void* stream);
+int ditto_conv_chain_run_prepared(const ditto_conv_chain_desc* desc, const void* x, const void* w1,
+                                  const void* w2, void* y, void* workspace, size_t workspace_bytes,
+                                  void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -210,3 +210,33 @@ def test_conv_chain_rejects_unsupported():
         chain.run_conv_chain(x, w1, w2, y[:, :, :4, :4].contiguous(), 1, 1, 1, 2)
     with pytest.raises(ValueError):
         chain.run_conv_chain(x, w1, w2[:, :, :1, :1].contiguous(), y[:, :8].contiguous(), 1, 1, 0, 1)
+
+
+@pytest.mark.parametrize("case", [CASES[0], CASES[2], CASES_3X3_SECOND[0], CASES_3X3_SECOND[3]])
+def test_prepared_weights_give_the_same_bits(oracle, case):
+    """ditto_conv_chain_prepare + ditto_conv_chain_run_prepared == ditto_conv_chain_run."""
+    if len(case) == 9:
+        N, C0, H, W, C1, R1, pad1, stride1, C2 = case
+        R2, pad2 = 1, 0
+    else:
+        N, C0, H, W, C1, R1, pad1, stride1, C2, R2, pad2 = case
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, R1, R2, "float16", seed=3, w_std=0.05)
+    x, w1, w2 = to_dev(X, "float16"), to_dev(W1, "float16"), to_dev(W2, "float16")
+    P = (H + 2 * pad1 - R1) // stride1 + 1 + 2 * pad2 - R2 + 1
+    Q = (W + 2 * pad1 - R1) // stride1 + 1 + 2 * pad2 - R2 + 1
+    want = torch.full((N, C2, P, Q), float("nan"), device=x.device, dtype=torch.float16)
+    got = want.clone()
+    desc = chain.conv_chain_desc(x, w1, w2, want, pad1, stride1, pad2, 1, "relu", True)
+    chain.run_conv_chain(x, w1, w2, want, desc=desc)
+    ws = chain.prepare_conv_chain(desc, w1, w2)
+    assert ws.numel() >= chain.conv_chain_workspace_bytes(desc) > 0
+    for _ in range(2):  # the workspace is read-only for the prepared call
+        got.fill_(float("nan"))
+        chain.run_conv_chain(x, w1, w2, got, desc=desc, workspace=ws, prepared=True)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+    with pytest.raises(ValueError):  # no workspace, nothing prepared
+        chain.run_conv_chain(x, w1, w2, got, desc=desc, prepared=True)
+    small = torch.empty(16, dtype=torch.uint8, device=x.device)
+    with pytest.raises(ValueError):
+        chain.prepare_conv_chain(desc, w1, w2, workspace=small)
