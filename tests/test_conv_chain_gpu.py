@@ -97,6 +97,10 @@ CASES_DEPTHWISE = [
     (1, 8, 12, 12, 24, 2, 0, 1, 32),     # 2x2 filter, factor 24
     (1, 8, 12, 12, 48, 4, 1, 1, 32),     # 4x4 filter (16 taps), factor 48
     (2, 6, 13, 21, 32, 2, 1, 1, 72),     # 2x2 filter (no second tap group), factor 32
+    (6, 16, 112, 112, 16, 3, 1, 1, 32),  # more pixel tiles than persistent workgroups: several rounds
+    (1, 16, 30, 30, 16, 3, 1, 1, 256),   # 256 output channels; image rows of 30: 4-byte halo loads
+    (1, 16, 21, 23, 32, 3, 1, 1, 64),    # odd image rows: 2-byte halo loads, 2-byte output stores
+    (1, 48, 24, 24, 16, 3, 1, 2, 64),    # stride 2, 768 intermediate channels
 ]
 
 
@@ -118,6 +122,33 @@ def test_depthwise_conv_chain_vs_oracle(oracle, case, dtype):
         assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
     got = run_conv(X, W1, W2, dtype, pad, stride, "relu", True, groups1=C0)
     assert np.array_equal(got, oracle.np_round_to(got32, dtype))
+
+
+def test_depthwise_chain_with_less_aligned_pointers(oracle):
+    """x only 2-byte aligned (narrower halo loads) and y only 4-byte aligned (2-byte stores instead
+    of the 16-byte path) must give the same bits as the aligned call."""
+    N, C0, H, W, factor, C2 = 1, 8, 16, 16, 16, 64
+    C1 = C0 * factor
+    rng = np.random.default_rng(11)
+    X = oracle.np_round_to(rng.standard_normal((N, C0, H, W)).astype(np.float32), "float16")
+    W1 = oracle.np_round_to(rng.standard_normal((C1, 1, 3, 3)).astype(np.float32) * 0.3, "float16")
+    W2 = oracle.np_round_to(rng.standard_normal((C2, C1, 1, 1)).astype(np.float32) * 0.05, "float16")
+    x, w1, w2 = to_dev(X, "float16"), to_dev(W1, "float16"), to_dev(W2, "float16")
+    want = torch.empty(N, C2, H, W, device=x.device, dtype=torch.float16)
+    chain.run_conv_chain(x, w1, w2, want, groups1=C0)
+    xbuf = torch.zeros(x.numel() + 8, device=x.device, dtype=torch.float16)
+    ybuf = torch.zeros(want.numel() + 8, device=x.device, dtype=torch.float16)
+    for xo, yo in ((1, 0), (0, 2), (3, 6)):
+        xs = xbuf[xo:xo + x.numel()].view_as(x)
+        xs.copy_(x)
+        ys = ybuf[yo:yo + want.numel()].view_as(want)
+        ys.fill_(float("nan"))
+        chain.run_conv_chain(xs, w1, w2, ys, groups1=C0)
+        torch.cuda.synchronize()
+        assert torch.equal(ys, want), (xo, yo)
+    mx, rel = errors(want.float().cpu().numpy(),
+                     oracle.conv_chain_f32(X, W1, W2, 1, 1, 0, 1, round_mid="float16", groups1=C0))
+    assert mx <= MAX_ABS and rel <= REL_L2
 
 
 def test_depthwise_chain_rejects():
