@@ -26,9 +26,17 @@
 
 namespace ditto {
 
+// Raw C tiles kept in LDS: two (a tile is loaded two steps before its use) or, where LDS allows
+// (head_pad 64 with B consumed as loaded), four, so that loads run three steps ahead -- one step
+// of a short tile does not cover the memory latency.
+template <int D, bool B_KL>
+__host__ __device__ constexpr int bmm_chain8_raw_c_tiles() {
+  return (D == 64 && !B_KL) ? 4 : 2;
+}
+
 template <int D, bool B_KL>
 __host__ __device__ constexpr int bmm_chain8_lds_bytes() {
-  return ((B_KL ? 6 : 4) + 4) * kBN * D * 2;
+  return ((B_KL ? 6 : 4) + bmm_chain8_raw_c_tiles<D, B_KL>() + 2) * kBN * D * 2;
 }
 
 template <typename T, int D, int INTER, bool B_KL>
@@ -52,8 +60,12 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
   // LDS map (bytes): B tiles, then raw C tiles, then fragment-major C tiles
   constexpr int B_LOAD = 0;                             // as loaded: [4] row-read layout, or [2] raw
   constexpr int B_FRAG = 2 * TB;                        // [4] fragment major (B_KL only)
-  constexpr int C_RAW = (B_KL ? 6 : 4) * TB;            // [2]
-  constexpr int C_FRAG = C_RAW + 2 * TB;                // [2]
+  constexpr int NCR = bmm_chain8_raw_c_tiles<D, B_KL>();
+  constexpr int C_RAW = (B_KL ? 6 : 4) * TB;            // [NCR]
+  constexpr int C_FRAG = C_RAW + NCR * TB;              // [2]
+  // loads run this many steps ahead of the step that consumes them
+  constexpr int B_AHEAD = 3;                            // (B_KL: into the raw pair, transposed a step later)
+  constexpr int C_AHEAD = NCR == 4 ? 3 : 2;
   constexpr int B_USE = B_KL ? B_FRAG : B_LOAD;         // the four buffers the first contraction reads
 
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -238,14 +250,11 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
     constexpr int CF = C_FRAG + PAR * TB;
     // loads ahead (tiles past the end are out of range and load zeros); transposition reads
     V8 xb[NTR], xc[NTR];
-    if (B_KL) {
-      load_b(it + 3, PAR ^ 1);
-    } else {
-      load_b(it + 2, (J + 2) % 4);
-    }
-    load_c(it + 2, PAR);
+    // C first: the wait at the end of the step can then leave the (younger) B loads in flight
+    load_c(it + C_AHEAD, NCR == 4 ? (J + 3) % 4 : PAR);
+    load_b(it + B_AHEAD, B_KL ? (PAR ^ 1) : (J + 3) % 4);  // not B_KL: the buffer tile it - 1 used
     if (B_KL) tr_read_b(B_LOAD + PAR * TB, xb);
-    tr_read_c(C_RAW + (PAR ^ 1) * TB, xc);
+    tr_read_c(C_RAW + (NCR == 4 ? (J + 1) % 4 : (PAR ^ 1)) * TB, xc);
 
     if (!late) scores(IntC<B_USE + J * TB>{});
 
@@ -321,7 +330,12 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
       __builtin_amdgcn_sched_barrier(0);
     }
     if (late && it + 1 < ntiles) scores(IntC<B_USE + ((J + 1) % 4) * TB>{});
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // everything the next step reads has landed; what this step issued may stay in flight: its B
+    // loads always (B as loaded is consumed two steps on at the earliest), its C loads when there
+    // are four raw C tiles
+    if (B_KL) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if (NCR == 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLD) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
     __syncthreads();
   };
 
@@ -330,6 +344,8 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
   load_b(1, 1);
   load_c(0, 0);
   load_c(1, 1);
+  if (!B_KL) load_b(2, 2);
+  if (NCR == 4) load_c(2, 2);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   {
