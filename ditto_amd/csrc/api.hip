@@ -246,21 +246,29 @@ struct ConvPlan {
   ditto::ConvChainArgs args;
   bool dw;             // depthwise first convolution: dwargs / c2_tiles / dw_shared describe the launch
   int c2_tiles;
-  int dw_mode;         // 0 | 1: vector-ALU depthwise stage (1: multiplier a multiple of 8); 2: MFMA
+  int dw_mode;         // 0 | 1: plain kernel (1: multiplier a multiple of 8); 2 | 3: persistent kernel,
+                       // depthwise stage on the matrix cores (2) or the vector ALU (3)
   ditto::DwConvArgs dwargs;
   ditto_tile_param tile;
 };
 
 // Depthwise first convolution + 1x1 second (dw_conv_chain.h): everything in one kernel, no workspace.
-// Channel multipliers that are multiples of 16 run the depthwise stage on the matrix cores
-// (dw_mode 2), the others on the vector ALU (dw_mode 1: multiples of 8, 0: 1, 2, 4).
-int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvPlan* plan, bool need_device) {
+// dw_mode 2 | 3: the persistent kernel, depthwise stage on the matrix cores (multipliers that are
+// multiples of 16) or on the vector ALU (3x3, multiplier 1, 2, 4, 8); dw_mode 0 | 1: the plain
+// kernel for what is left (1: multiples of 8, 0: 1, 2, 4).
+int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvPlan* plan, bool need_device,
+                 bool allow_dwv = true) {
   if (d->C1 % d->C0) return fail(DITTO_EINVAL, "depthwise: C1 must be a multiple of C0");
   const long long mult = d->C1 / d->C0;
   const long long RS = d->R1 * d->S1;
   if (!(d->R2 == 1 && d->S2 == 1 && d->pad2 == 0 && d->stride2 == 1))
     return fail(DITTO_EUNSUPPORTED, "depthwise chain: the second convolution must be 1x1, stride 1, no padding");
-  const bool mfma = mult % 16 == 0 && RS <= ditto::kDwMfmaTaps;
+  // the persistent kernel: depthwise stage on the matrix cores (multipliers that are multiples of 16)
+  // or, for 3x3 filters with multiplier 1, 2, 4, 8 (and whole 16-byte vectors of W1, W2), on the vector ALU
+  // (that variant is built with the 16-byte output stores only: output rows of a multiple of 8, not fp32)
+  const bool dwv = allow_dwv && d->R1 == 3 && d->S1 == 3 && (mult == 1 || mult == 2 || mult == 4 || mult == 8) &&
+                   d->C1 % 8 == 0 && Q % 8 == 0 && d->out_dtype != DITTO_F32;
+  const bool mfma = (mult % 16 == 0 && RS <= ditto::kDwMfmaTaps) || dwv;
   if (!mfma && RS > 2 * ditto::kDwPairs - 1)
     return fail(DITTO_EUNSUPPORTED,
                 "depthwise chain: filters of at most 9 taps (16 when the channel multiplier is a multiple of 16)");
@@ -270,7 +278,7 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   if (d->C1 > 32768) return fail(DITTO_EUNSUPPORTED, "depthwise chain: at most 32768 intermediate channels");
   memset(plan, 0, sizeof(*plan));
   plan->dw = true;
-  plan->dw_mode = mfma ? 2 : mult % 8 == 0 ? 1 : 0;
+  plan->dw_mode = dwv ? 3 : mfma ? 2 : mult % 8 == 0 ? 1 : 0;
   const int c2t = d->C2 <= 32 ? 1 : d->C2 <= 64 ? 2 : d->C2 <= 128 ? 4 : 8;
   const int pxw = mfma ? ditto::dw_mfma_pxw(c2t) : c2t == 8 ? 1 : 2;
   const int groups = mfma ? ditto::dw_mfma_groups(c2t) : 1;
@@ -280,14 +288,17 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   a.mult = (int)mult; a.C1 = (int)d->C1; a.R = (int)d->R1; a.S = (int)d->S1;
   a.pad = (int)d->pad1; a.stride = (int)d->stride1; a.C2 = (int)d->C2; a.P = (int)P; a.Q = (int)Q;
   // Pixel tile: the split of the output plane into TH x TW pieces of at most `slots` pixels that
-  // costs the fewest 32-pixel tile rounds (a round = one tile on each of the four waves; the
-  // vector-ALU kernel always runs all its rounds); ties go to the wider tile.
-  {
+  // costs the fewest 32-pixel tile rounds (a round = one tile on each wave; the plain kernel always
+  // runs all its rounds); ties go to the wider tile.  Where 16-byte output stores are possible only
+  // tile widths that keep them (multiples of 8) are considered.
+  const bool want_wide = mfma && d->out_dtype != DITTO_F32 && Q % 8 == 0;
+  for (int pass = want_wide ? 0 : 1; pass < 2; ++pass) {  // pass 0: only widths that are multiples of 8
     long long best = -1;
     for (int k = 1; k <= (int)Q; ++k) {
       const int tw = (int)((Q + k - 1) / k);
       if (tw > slots) continue;
       if (tw < 8 && k > 1) break;
+      if (pass == 0 && tw % 8) continue;
       int th = slots / tw;
       if (th > P) th = (int)P;
       const long long th_n = (P + th - 1) / th;
@@ -297,6 +308,7 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
       const long long cost = th_n * tw_n * rounds;
       if (best < 0 || cost < best) { best = cost; a.TH = th; a.TW = tw; }
     }
+    if (best >= 0) break;
   }
   // input channels per chunk: chx * mult a multiple of the MFMA block (32 intermediate channels
   // on the matrix-core path, 16 on the vector path); as many channels as keep two workgroups on a
@@ -368,6 +380,7 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   a.relu_mid = d->inter_op == DITTO_INTER_RELU;
   a.relu_out = d->relu_out != 0;
   a.out_f32 = d->out_dtype == DITTO_F32;
+  if (dwv && !a.wide) return plan_dw_conv(d, P, Q, plan, need_device, false);  // that variant needs the wide stores
   plan->c2_tiles = c2t;
   ditto_tile_param& t = plan->tile;
   t.block_threads = 256 * groups;
@@ -378,7 +391,9 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   t.lds_bytes = lds;
   t.grid_x = a.N * a.tiles_h * a.tiles_w;
   if (mfma) {  // persistent workgroups, as many as the CUs hold at this LDS footprint
-    const int per_cu = 160 * 1024 / lds < 2 ? 1 : 2;
+    // two workgroups per CU where LDS and registers allow: the eight-wave variants use more than
+    // 128 registers per lane, so only one of them fits
+    const int per_cu = (groups == 1 && 160 * 1024 / lds >= 2) ? 2 : 1;
     const int cap = (need_device ? device_cus() : 256) * per_cu;
     if (t.grid_x > cap) t.grid_x = cap;
     a.grid = t.grid_x;
@@ -700,7 +715,7 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
     // less aligned pointers: narrower halo loads (the LDS layout stays valid) while the chunk still
     // fits the registers that keep it in flight; plain 2-byte output stores
     while (a.vec > 1 && !aligned(x, 2 * (size_t)a.vec)) a.vec >>= 1;
-    if (plan.dw_mode == 2) {
+    if (plan.dw_mode >= 2) {
       const int nvr = a.cols_al / a.vec;
       const int cphases = (256 * ditto::dw_mfma_groups(plan.c2_tiles) / nvr) / a.rows_in;
       if (cphases < 1 || (a.chx + cphases - 1) / cphases > ditto::kDwXpf)
@@ -708,7 +723,10 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
                     2 * plan.dwargs.vec);
       if (!aligned(w1, 16)) return fail(DITTO_EINVAL, "misaligned data pointer");
     }
-    if (a.wide && !aligned(y, 16)) a.wide = 0;
+    if (a.wide && !aligned(y, 16)) {
+      if (plan.dw_mode == 3) return fail(DITTO_EINVAL, "misaligned data pointer: y must be 16-byte aligned for this shape");
+      a.wide = 0;
+    }
     a.x = x;
     a.w1 = w1;
     a.w2 = w2;

@@ -28,8 +28,9 @@ hipError_t launch_conv2_f16(int c1_tiles, int px2, const ConvChainArgs& args, hi
 hipError_t launch_conv2_bf16(int c1_tiles, int px2, const ConvChainArgs& args, hipStream_t stream);
 hipError_t pack_conv_w2_f16(int c1_tiles, const ConvChainArgs& args, void* out1, void* out2, hipStream_t stream);
 hipError_t pack_conv_w2_bf16(int c1_tiles, const ConvChainArgs& args, void* out1, void* out2, hipStream_t stream);
-// depthwise first convolution (dw_conv_chain.h); c2_tiles in {1, 2, 4, 8}; mode 0 | 1: vector-ALU
-// depthwise stage (1: multiplier a multiple of 8), 2: MFMA depthwise stage (multiple of 16)
+// depthwise first convolution (dw_conv_chain.h); c2_tiles in {1, 2, 4, 8}; mode 0 | 1: plain kernel,
+// vector-ALU depthwise stage (1: multiplier a multiple of 8); 2: persistent kernel, MFMA depthwise
+// stage (multiplier a multiple of 16); 3: persistent kernel, vector-ALU stage (3x3, multiplier 1, 2, 4, 8)
 hipError_t launch_dw_conv_f16(int c2_tiles, int mode, const DwConvArgs& args, hipStream_t stream);
 hipError_t launch_dw_conv_bf16(int c2_tiles, int mode, const DwConvArgs& args, hipStream_t stream);
 

@@ -35,14 +35,15 @@ hipError_t DITTO_PACK2_NAME(int c1_tiles, const ConvChainArgs& args, void* out1,
   return launch_pack_conv_w12<DITTO_INST_T>(args, 32 * c1_tiles, 32, out1, out2, stream);
 }
 
-// depthwise first convolution: c2_tiles in {1, 2, 4, 8} (32 output channels each); mode 0 | 1:
-// vector-ALU depthwise stage (1: the multiplier is a multiple of 8), 2: MFMA depthwise stage
+// depthwise first convolution: c2_tiles in {1, 2, 4, 8} (32 output channels each); mode 0 | 1: plain
+// kernel with a vector-ALU depthwise stage (1: the multiplier is a multiple of 8); 2 | 3: persistent
+// kernel with the depthwise stage on the matrix cores (2) or the vector ALU (3)
 hipError_t DITTO_DW_NAME(int c2_tiles, int mode, const DwConvArgs& args, hipStream_t stream) {
   typedef DITTO_INST_T T;
 #define DITTO_CASE(C2T, PXW)                                                                    \
   if (c2_tiles == C2T) {                                                                        \
-    if (mode == 2)                                                                              \
-      return launch_dw_conv_mfma<T, C2T, dw_mfma_pxw(C2T), dw_mfma_groups(C2T)>(args, args.grid, stream); \
+    if (mode >= 2)                                                                              \
+      return launch_dw_conv_mfma<T, C2T, dw_mfma_pxw(C2T), dw_mfma_groups(C2T)>(args, args.grid, mode == 3, stream); \
     return mode == 1 ? launch_dw_conv_chain<T, C2T, PXW, true>(args, stream)                    \
                      : launch_dw_conv_chain<T, C2T, PXW, false>(args, stream);                  \
   }

@@ -310,8 +310,18 @@ __host__ __device__ constexpr int dw_tap_of_k(bool f33, int k) {
   return !f33 ? k : k == 0 ? 0 : k == 1 ? 1 : k == 2 ? 3 : k == 3 ? 4 : k == 4 ? 6 : k == 5 ? 7 : k == 6 ? 2 : k == 7 ? 5 : k;
 }
 
-template <typename T, int C2T, int PXW, int NG, bool WIDE, bool F33>
+//
+// DWV (3x3 filters, channel multiplier 1, 2, 4 or 8): the same persistent kernel with the depthwise
+// stage on the vector ALU -- a block-diagonal MFMA would use mult of every 16 rows.  A lane gathers
+// the taps of its pixel as above (once per input channel it needs) and takes five
+// v_dot2_f32_f16/bf16 per intermediate value against the filter's tap pairs, kept in LDS in the
+// same order: entry 2 * cm holds pairs 0..3, entry 2 * cm + 1 the ninth tap.
+// MSH = log2(multiplier) there (a compile-time constant keeps the gather-sharing pattern static);
+// -1: the matrix-core depthwise stage.
+template <typename T, int C2T, int PXW, int NG, bool WIDE, bool F33, int MSH = -1>
 __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
+  constexpr bool DWV = MSH >= 0;
+  static_assert(!DWV || (F33 && WIDE), "the vector-ALU depthwise stage is built for 3x3 filters and 16-byte stores");
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef typename Elem<T>::v8 V8;
   typedef typename Elem<T>::v4 V4;
@@ -369,10 +379,15 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
         reinterpret_cast<const T*>(p.x) + ((long long)n * p.C0 + c0 + st_cph) * hw + (long long)h * p.W + w;
     auto body = [&](auto vec_tag) __attribute__((always_inline)) {
       constexpr int VEC = decltype(vec_tag)::value;
+      const T* q = src;  // a running pointer: per-pass offsets would be hoisted out of the tile loop and spilled
+      int left = nch;
 #pragma unroll
       for (int u = 0; u < kDwXpf; ++u) {
         xr[u] = zero4;
-        if (ok && u * cphases < nch) dw_ld_vec<T, VEC>(xr[u], src + u * cphases * hw32);
+        if (ok && left > 0) dw_ld_vec<T, VEC>(xr[u], q);
+        q += cphases * hw32;
+        left -= cphases;
+        asm volatile("" : "+v"(q), "+v"(left));
       }
     };
     if (p.vec == 4) body(std::integral_constant<int, 4>());
@@ -382,9 +397,15 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
   auto xstore = [&]() __attribute__((always_inline)) {
     auto body = [&](auto vec_tag) __attribute__((always_inline)) {
       constexpr int VEC = decltype(vec_tag)::value;
+      T* q = Xs + st_dst;  // running, as in xload
+      int left = st_on ? p.chx - st_cph : 0;
 #pragma unroll
-      for (int u = 0; u < kDwXpf; ++u)
-        if (st_on && st_cph + u * cphases < p.chx) dw_st_vec<T, VEC>(Xs + st_dst + u * cphases * xplane, xr[u]);
+      for (int u = 0; u < kDwXpf; ++u) {
+        if (left > 0) dw_st_vec<T, VEC>(q, xr[u]);
+        q += cphases * xplane;
+        left -= cphases;
+        asm volatile("" : "+v"(q), "+v"(left));
+      }
     };
     if (p.vec == 4) body(std::integral_constant<int, 4>());
     else if (p.vec == 2) body(std::integral_constant<int, 2>());
@@ -457,12 +478,13 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
         }
         __syncthreads();
         // ... and are regrouped into A-operand entries: row m = 16 * hgrp + 8a + 4gg + b of a block is
-        // its intermediate channel 16 * hgrp + 8gg + 4a + b
+        // its intermediate channel 16 * hgrp + 8gg + 4a + b (DWV: two entries per intermediate channel)
         for (int e = tid; e < nblk * 64; e += NT) {
-          const int m = e & 31, half = (e >> 5) & 1, blk = e >> 6;
+          const int m = e & 31, half = DWV ? (e & 1) : ((e >> 5) & 1), blk = e >> 6;
           if (half && !second_half) continue;
           const int mm = m & 15;
-          const int cml = 32 * blk + 16 * (m >> 4) + 8 * ((mm >> 2) & 1) + 4 * (mm >> 3) + (mm & 3);
+          const int cml = DWV ? (e >> 1)
+                              : 32 * blk + 16 * (m >> 4) + 8 * ((mm >> 2) & 1) + 4 * (mm >> 3) + (mm & 3);
           unsigned raw[8];
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
@@ -583,6 +605,52 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
         }
       };
       const int last = nblk - 1;
+      if constexpr (DWV) {
+        constexpr int msh = DWV ? MSH : 0;  // log2 of the channel multiplier
+        const int row_dw = p.cols_al >> 1;  // dwords per halo row (cols_al is even here)
+        for (int blk = 0; blk < nblk; ++blk) {
+          load_w2(blk);
+#pragma unroll
+          for (int j = 0; j < PXW; ++j) {
+            const int xc = xoff[j] + lead;
+            const unsigned sh = (xc & 1) * 16;
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+              const int cm0 = 32 * blk + 16 * s + 8 * g;  // first of the lane's 8 intermediate channels
+              unsigned tp[5] = {0, 0, 0, 0, 0};           // tap pairs of the current input channel
+              float mid[8];
+#pragma unroll
+              for (int e = 0; e < 8; ++e) {
+                if ((e & ((1 << msh) - 1)) == 0) {  // a new input channel starts
+                  const unsigned* xw =
+                      reinterpret_cast<const unsigned*>(Xs + ((cm0 + e) >> msh) * xplane + (xc & ~1));
+                  unsigned t2[3];
+#pragma unroll
+                  for (int r = 0; r < 3; ++r) {
+                    const unsigned d0 = xw[r * row_dw], d1 = xw[r * row_dw + 1];
+                    tp[r] = __builtin_amdgcn_alignbit(d1, d0, sh);
+                    t2[r] = __builtin_amdgcn_alignbit(0u, d1, sh);
+                  }
+                  tp[3] = __builtin_amdgcn_perm(t2[1], t2[0], 0x05040100u);
+                  tp[4] = t2[2] & 0xffffu;
+                }
+                const uint4 w = W1h[2 * (cm0 + e)];
+                const unsigned w8 = W1h[2 * (cm0 + e) + 1].x;
+                float a = Elem<T>::dot2(__builtin_bit_cast(V2, w.x), __builtin_bit_cast(V2, tp[0]), 0.f);
+                a = Elem<T>::dot2(__builtin_bit_cast(V2, w.y), __builtin_bit_cast(V2, tp[1]), a);
+                a = Elem<T>::dot2(__builtin_bit_cast(V2, w.z), __builtin_bit_cast(V2, tp[2]), a);
+                a = Elem<T>::dot2(__builtin_bit_cast(V2, w.w), __builtin_bit_cast(V2, tp[3]), a);
+                a = Elem<T>::dot2(__builtin_bit_cast(V2, w8), __builtin_bit_cast(V2, tp[4]), a);
+                mid[e] = p.relu_mid ? fmaxf(a, 0.f) : a;
+              }
+              const V2 c0v = cvt2<T>(mid[0], mid[1]), c1v = cvt2<T>(mid[2], mid[3]);
+              const V2 c2v = cvt2<T>(mid[4], mid[5]), c3v = cvt2<T>(mid[6], mid[7]);
+              pf[j][s] = V8{c0v[0], c0v[1], c1v[0], c1v[1], c2v[0], c2v[1], c3v[0], c3v[1]};
+            }
+            pointwise(j);
+          }
+        }
+      } else {
       load_a(0);
       load_w2(0);
       load_b(0, 0);
@@ -625,6 +693,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
           depthwise();  // unit nx2
           __builtin_amdgcn_sched_barrier(0);
         }
+      }
       }
     }
     if (WIDE) {
@@ -692,21 +761,34 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
 #endif
 }
 
+// dwv: depthwise stage on the vector ALU (multipliers 1, 2, 4, 8; 3x3 filters; even cols_al; 16-byte stores)
 template <typename T, int C2T, int PXW, int NG>
-hipError_t launch_dw_conv_mfma(const DwConvArgs& args, int grid, hipStream_t stream) {
+hipError_t launch_dw_conv_mfma(const DwConvArgs& args, int grid, bool dwv, hipStream_t stream) {
   const bool wide = args.wide != 0;
   const bool f33 = args.R == 3 && args.S == 3 && args.cols_al % 2 == 0;
+  if (dwv && !(f33 && wide)) return hipErrorInvalidValue;
   const int lds = dw_conv_mfma_lds_bytes(args.chx, args.mult, args.rows_in, args.cols_al, 32 * C2T, NG, wide);
-  auto kern = wide ? (f33 ? dw_conv_mfma_kernel<T, C2T, PXW, NG, true, true> : dw_conv_mfma_kernel<T, C2T, PXW, NG, true, false>)
-                   : (f33 ? dw_conv_mfma_kernel<T, C2T, PXW, NG, false, true> : dw_conv_mfma_kernel<T, C2T, PXW, NG, false, false>);
-  static thread_local int configured_dev[4] = {-1, -1, -1, -1};
+  void (*kern)(DwConvArgs) = nullptr;
+  int slot = 0;
+  if (dwv) {
+    slot = 4 + (args.mult == 1 ? 0 : args.mult == 2 ? 1 : args.mult == 4 ? 2 : 3);
+    kern = args.mult == 1   ? dw_conv_mfma_kernel<T, C2T, PXW, NG, true, true, 0>
+           : args.mult == 2 ? dw_conv_mfma_kernel<T, C2T, PXW, NG, true, true, 1>
+           : args.mult == 4 ? dw_conv_mfma_kernel<T, C2T, PXW, NG, true, true, 2>
+                            : dw_conv_mfma_kernel<T, C2T, PXW, NG, true, true, 3>;
+  } else {
+    slot = 2 * wide + f33;
+    kern = wide ? (f33 ? dw_conv_mfma_kernel<T, C2T, PXW, NG, true, true> : dw_conv_mfma_kernel<T, C2T, PXW, NG, true, false>)
+                : (f33 ? dw_conv_mfma_kernel<T, C2T, PXW, NG, false, true> : dw_conv_mfma_kernel<T, C2T, PXW, NG, false, false>);
+  }
+  static thread_local int configured_dev[8] = {-1, -1, -1, -1, -1, -1, -1, -1};
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
-  if (configured_dev[2 * wide + f33] != dev) {
+  if (configured_dev[slot] != dev) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) return e;
-    configured_dev[2 * wide + f33] = dev;
+    configured_dev[slot] = dev;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256 * NG), lds, stream, args);
   return hipGetLastError();

@@ -101,7 +101,17 @@ CASES_DEPTHWISE = [
     (1, 16, 30, 30, 16, 3, 1, 1, 256),   # 256 output channels; image rows of 30: 4-byte halo loads
     (1, 16, 21, 23, 32, 3, 1, 1, 64),    # odd image rows: 2-byte halo loads, 2-byte output stores
     (1, 48, 24, 24, 16, 3, 1, 2, 64),    # stride 2, 768 intermediate channels
+    # output rows that are multiples of 8 with factor 1, 2, 4, 8: the persistent kernel with the
+    # depthwise stage on the vector ALU
+    (2, 32, 24, 24, 1, 3, 1, 1, 64),     # plain depthwise, MobileNet v1 block
+    (1, 40, 16, 16, 1, 3, 1, 1, 96),     # 40 channels: the last block of 32 is partly padding
+    (1, 16, 16, 40, 2, 3, 1, 1, 48),     # factor 2
+    (1, 8, 32, 32, 4, 3, 1, 2, 32),      # factor 4, stride 2
+    (1, 12, 16, 16, 8, 3, 1, 1, 128),    # factor 8, 96 intermediate channels
+    (8, 16, 96, 96, 1, 3, 1, 1, 32),     # more tiles than persistent workgroups
+    (1, 128, 8, 8, 2, 3, 1, 1, 256),     # 256 output channels
 ]
+DW_VECTOR_ALU_CASES = [c for c in CASES_DEPTHWISE if c[4] in (1, 2, 4, 8) and ((c[3] + 2 * c[6] - 3) // c[7] + 1) % 8 == 0]
 
 
 @pytest.mark.parametrize("case", CASES_DEPTHWISE)
@@ -121,7 +131,28 @@ def test_depthwise_conv_chain_vs_oracle(oracle, case, dtype):
         mx, rel = errors(got32, want32)
         assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
     got = run_conv(X, W1, W2, dtype, pad, stride, "relu", True, groups1=C0)
-    assert np.array_equal(got, oracle.np_round_to(got32, dtype))
+    if case in DW_VECTOR_ALU_CASES:
+        # fp32 output runs the plain kernel there and 16-bit output the persistent one: their
+        # summation orders differ, so the 16-bit result is held to the oracle, not to the fp32 bits
+        mx, rel = errors(got, oracle.np_round_to(want32, dtype))
+        assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (mx, rel)
+    else:
+        assert np.array_equal(got, oracle.np_round_to(got32, dtype))
+
+
+@pytest.mark.parametrize("case", DW_VECTOR_ALU_CASES)
+def test_small_factor_cases_run_the_persistent_kernel(case):
+    """The cases meant for it do select the persistent kernel with the vector-ALU depthwise stage
+    (variant 4000 + 10 * output-channel tiles + 3), so the parity cases above cover it."""
+    N, C0, H, W, factor, R, pad, stride, C2 = case
+    dev = "cuda:0"
+    x = torch.empty(N, C0, H, W, device=dev, dtype=torch.float16)
+    w1 = torch.empty(C0 * factor, 1, R, R, device=dev, dtype=torch.float16)
+    w2 = torch.empty(C2, C0 * factor, 1, 1, device=dev, dtype=torch.float16)
+    P, Q = (H + 2 * pad - R) // stride + 1, (W + 2 * pad - R) // stride + 1
+    y = torch.empty(N, C2, P, Q, device=dev, dtype=torch.float16)
+    desc = chain.conv_chain_desc(x, w1, w2, y, pad, stride, 0, 1, "cast", False, C0)
+    assert chain.select_tile(desc).variant % 10 == 3
 
 
 def test_depthwise_chain_with_less_aligned_pointers(oracle):
