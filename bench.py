@@ -53,6 +53,10 @@ WORKLOADS = {
     "gemm_chain_f16_b1_512x64x64x64": dict(kind="cast", dtype="float16", batch=1, M=512, N=64, K=64, L=64,
                                            scale=1.0, bound="hbm",
                                            desc="GEMM chain (A.B).D at the shape of the CPU plumbing case, fp16"),
+    "gemm_chain_bf16_b64_4096x128x4096x128": dict(kind="cast", dtype="bfloat16", batch=64, M=4096, N=128, K=128,
+                                                  L=4096, scale=1.0, bound="mfma",
+                                                  desc="batched GEMM chain (A.B).D with the cast between, at the "
+                                                       "long-sequence attention shape: the large GEMM-chain point"),
 }
 WORKLOADS.update({
     "conv_chain_f16_n32_c64_56x56_k64_k256": dict(

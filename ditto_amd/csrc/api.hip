@@ -129,8 +129,12 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     // below that the four-wave kernel with 128-row workgroups spreads over more CUs.  For
     // head_pad 128 and n8 >= 2 CUs the two are within noise and the four-wave, 256-row kernel
     // (half the LDS fragment traffic) is kept.
+    // Without a softmax between the contractions (nothing for a second wave to overlap) the
+    // four-wave, 256-row kernel also wins at head_pad 64 once n8 >= 2 CUs (249 vs 274 us at
+    // 64 x 4096 x 64 x 4096 x 64, bf16).
     const long long n8 = ((d->M + 255) / 256) * d->batch;
-    if (n8 * 4 >= 3LL * cus && !(plan->d_pad == 128 && n8 >= 2LL * cus))
+    const bool many = n8 >= 2LL * cus && (plan->d_pad == 128 || d->inter_op != DITTO_INTER_SOFTMAX);
+    if (n8 * 4 >= 3LL * cus && !many)
       plan->qt = 8;
     else
       plan->qt = (n8 >= 2LL * cus) ? 2 : 1;

@@ -242,6 +242,48 @@ def test_attention_full_size_bf16_long_sequence(oracle, variant):
     assert bool(((a - b).abs() <= 2.0 ** -7 * b.abs() + 1e-6).all())
 
 
+@pytest.mark.parametrize("variant", [0, 1281, 1288])
+def test_gemm_chain_full_size_bf16(oracle, variant):
+    # the large GEMM-chain point of the benchmark, (A.B).D with the cast between, 64 x (4096 x 128 x
+    # 4096 x 128) bf16, B as [K][L] like the reference's operand.  The checker over all of it would take
+    # minutes: whole entries across the batch, one row block of every entry, and properties.
+    batch, M, K, L, N = 64, 4096, 128, 4096, 128
+    dev = "cuda:0"
+    g = torch.Generator(device="cpu").manual_seed(35)
+    a = (torch.randn(batch, M, K, generator=g) * 0.25).to(torch.bfloat16)
+    b = (torch.randn(batch, K, L, generator=g) * 0.25).to(torch.bfloat16)
+    c = (torch.randn(batch, L, N, generator=g) / 64).to(torch.bfloat16)  # keeps the outputs O(1)
+    ad, bd, cd = a.to(dev), b.to(dev), c.to(dev)
+    out = torch.full((batch, M, N), float("nan"), device=dev, dtype=torch.bfloat16)
+    chain.run_bmm_chain(ad, bd, cd, out, "cast", 1.0, tile_variant=variant)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    an, bn, cn = a.float().numpy(), b.float().numpy(), c.float().numpy()
+    for h in (0, 40, 63):
+        want = oracle.bmm_chain_f64(an[h:h + 1], bn[h:h + 1], cn[h:h + 1], inter="cast", round_mid="bfloat16")
+        mx, rel = errors(got[h:h + 1], oracle.np_round_to(want.astype(np.float32), "bfloat16"))
+        assert rel <= REL_L2_BF16_QUANT and mx <= 4e-2, (h, mx, rel)  # one bf16 ulp at |x| ~ 4 is 3e-2
+    rows = slice(3000, 3040)
+    want = oracle.bmm_chain_f64(np.ascontiguousarray(an[:, rows]), bn, cn, inter="cast", round_mid="bfloat16")
+    mx, rel = errors(got[:, rows], oracle.np_round_to(want.astype(np.float32), "bfloat16"))
+    assert rel <= REL_L2_BF16_QUANT and mx <= 4e-2, (mx, rel)
+    # B = [I | 0]: the middle result is A itself (exact in bf16), so F = A . C[:K] -- one GEMM
+    eye = torch.zeros(batch, K, L, dtype=torch.bfloat16, device=dev)
+    eye[:, torch.arange(K), torch.arange(K)] = 1
+    chain.run_bmm_chain(ad, eye, cd, out, "cast", 1.0, tile_variant=variant)
+    torch.cuda.synchronize()
+    want_d = torch.bmm(ad.float(), cd[:, :K].float())
+    assert float((out.float() - want_d).norm() / want_d.norm()) <= REL_L2_BF16_QUANT
+    # rows of A permuted -> rows of F permuted, bit for bit (no cross-row state in this chain)
+    perm = torch.randperm(M, generator=g).to(dev)
+    chain.run_bmm_chain(ad, bd, cd, out, "cast", 1.0, tile_variant=variant)
+    out2 = torch.empty_like(out)
+    chain.run_bmm_chain(ad[:, perm].contiguous(), bd, cd, out2, "cast", 1.0, tile_variant=variant)
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out[:, perm])
+
+
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
 @pytest.mark.parametrize("cfg", [(2, 3, 200, 64), (1, 16, 256, 128), (8, 12, 512, 64)])
 def test_multi_head_attention_module(oracle, dtype, cfg):
