@@ -56,6 +56,46 @@ def test_conv_chain_vs_oracle(oracle, case, dtype):
         assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (ws, mx, rel)
 
 
+# Enough tiles of whole output rows for two rounds of persistent workgroups (at least 512), 16-bit
+# output, at most 64 input / intermediate channels: the opt-in kernel with both weight tensors resident
+# on the CU (DITTO_CONV_PERSIST=1).
+CASES_PERSISTENT = [
+    # N, C0, H, W, C1, R, pad, stride, C2
+    (520, 8, 8, 8, 16, 3, 1, 1, 32),      # one tile per image, 32-channel variants
+    (130, 40, 26, 16, 48, 3, 1, 1, 200),  # padded channels in every tensor; last tile of an image partial
+    (64, 64, 32, 32, 64, 3, 1, 1, 256),   # the largest weights: 64 -> 64 (3x3) -> 256
+    (128, 64, 33, 32, 64, 3, 1, 2, 128),  # stride 2, 17 x 16 output: two staging tasks per thread
+    (96, 16, 24, 48, 32, 1, 0, 1, 96),    # conv1x1 -> conv1x1, two rows of 48 per tile
+    (260, 24, 19, 32, 64, 3, 1, 2, 64),   # stride 2, 10 x 16 output, 8-row tiles
+]
+
+
+@pytest.mark.parametrize("case", CASES_PERSISTENT)
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_persistent_conv_chain_vs_oracle(oracle, case, dtype, monkeypatch):
+    monkeypatch.setenv("DITTO_CONV_PERSIST", "1")
+    N, C0, H, W, C1, R, pad, stride, C2 = case
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, R, 1, dtype, seed=C0 + C2, w_std=0.05)
+    x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
+    P, Q = (H + 2 * pad - R) // stride + 1, (W + 2 * pad - R) // stride + 1
+    y = torch.empty((N, C2, P, Q), device=x.device, dtype=TORCH_DTYPES[dtype])
+    desc = chain.conv_chain_desc(x, w1, w2, y, pad, stride, 0, 1, "cast", False)
+    assert chain.select_tile(desc).variant // 100 == 39  # the persistent kernel
+    for relu in (False, True):
+        want32 = oracle.conv_chain_f32(X, W1, W2, pad, stride, 0, 1, relu_mid=relu, relu_out=relu, round_mid=dtype)
+        got = run_conv(X, W1, W2, dtype, pad, stride, "relu" if relu else "cast", relu)
+        assert got.shape == want32.shape and np.isfinite(got).all()
+        mx, rel = errors(got, oracle.np_round_to(want32, dtype))
+        assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (relu, mx, rel)
+        # against the one-tile-per-workgroup kernel (taken when there is no workspace); their summation
+        # orders differ (here two waves each sum half of the taps x channel groups)
+        other = run_conv(X, W1, W2, dtype, pad, stride, "relu" if relu else "cast", relu, workspace=False)
+        assert errors(got, other)[1] <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), relu
+    # a second call right away (the halo prefetch and the stores of the first are independent of it)
+    again = run_conv(X, W1, W2, dtype, pad, stride, "relu", True)
+    assert np.array_equal(again, got)
+
+
 CASES_3X3_SECOND = [
     # N, C0, H, W, C1, R1, pad1, stride1, C2, R2, pad2
     (2, 64, 56, 56, 64, 1, 0, 1, 64, 3, 1),    # conv1x1 -> conv3x3 (conv1x1_conv3x3_cuda.py:77-189)
