@@ -285,7 +285,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the chains shard over batch entries with no "
-                 "exchange step; see DESIGN.md); --gpus %d is not supported" % args.gpus)
+                 "exchange step, each GPU would run this same kernel on its share); --gpus %d is not supported" % args.gpus)
 
     import torch
 

@@ -1,7 +1,7 @@
 """Host-side mirror of the reference's descriptor API (no GPU): pattern classification,
 DAG partition, chain recognition, error behaviour.  Expected values restate what the
 reference's own tests / drivers show (python_test/auto_tensorize/test_pattern.py:9-66,
-benchmark/chimera/cuda/bmm_softmax_bmm_cuda.py:158-236, SURVEY of hyper_fusion.cc:51-216)."""
+benchmark/chimera/cuda/bmm_softmax_bmm_cuda.py:158-236, src/auto_tensorize/hyper_fusion.cc:51-216)."""
 import pytest
 
 import ditto_amd as ditto
