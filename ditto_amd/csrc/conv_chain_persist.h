@@ -61,8 +61,11 @@ __host__ __device__ inline int conv_persist_x_elems(int rows_in, int cols_in, in
 }
 // bytes of the exchange buffer: per pixel tile the upper wave's partial sums, C1T x 16 floats per lane
 __host__ __device__ inline int conv_persist_xchg_bytes(int C1p) { return 4 * (C1p / 32) * 16 * 64 * 4; }
+// halo tile + exchange buffer, or (in the prologue) all 256 rows of W2 at a stride of C1p + 4 elements
 __host__ __device__ inline int conv_persist_lds_bytes(int rows_in, int cols_in, int RS, int C1p, int ch) {
-  return conv_persist_w1_lds_bytes(RS, C1p, ch) + conv_persist_x_elems(rows_in, cols_in, ch) * 2 + conv_persist_xchg_bytes(C1p);
+  const int work = conv_persist_x_elems(rows_in, cols_in, ch) * 2 + conv_persist_xchg_bytes(C1p);
+  const int w2 = 256 * (C1p + 4) * 2;
+  return conv_persist_w1_lds_bytes(RS, C1p, ch) + (work > w2 ? work : w2);
 }
 
 // Requirements (checked by the host): TW == Q (tiles are runs of whole output rows), TH * TW <= 128,
@@ -107,20 +110,33 @@ __global__ __launch_bounds__(512) void conv_chain_persist_kernel(ConvChainArgs p
   }
   // This wave's half of W2 as operand fragments, in registers for the whole kernel: for k step u of its
   // output-channel block b (channels 32 (NB kh + b) ..) the lane holds W2[c2 = .. + ln][16u + 4g + {0..3}]
-  // and [16u + 8 + 4g + {0..3}] (zero past C2 / C1)
-  static_assert(C2T % 2 == 0, "the output channel blocks are split between two waves");
+  // and [16u + 8 + 4g + {0..3}] (zero past C2 / C1).  W2 passes through LDS (the halo tile and exchange
+  // areas, not yet in use) with 16-byte loads: fetched straight from memory the fragments are 8-byte
+  // pieces of 32 different rows per load, an L2 request each (5.7 us of a 9 us prologue measured).
+  static_assert(C2T % 2 == 0 && 32 * C2T <= 256, "the output channel blocks are split between two waves; the LDS size allows for 256 rows of W2");
   constexpr int NB = C2T / 2;
+  constexpr int W2S = C1p + 4;  // row stride (elements): conflict-free 8-byte reads
   V8 w2r[NB][2 * C1T];
-#pragma unroll
-  for (int b = 0; b < NB; ++b)
-#pragma unroll
-    for (int u = 0; u < 2 * C1T; ++u) {
-      const int c2 = 32 * (NB * kh + b) + ln, k0 = 16 * u + 4 * g;
-      V4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
-      if (c2 < p.C2 && k0 < p.C1) lo = *reinterpret_cast<const V4*>(W2g + (long long)c2 * p.C1 + k0);
-      if (c2 < p.C2 && k0 + 8 < p.C1) hi = *reinterpret_cast<const V4*>(W2g + (long long)c2 * p.C1 + k0 + 8);
-      w2r[b][u] = concat4<V4, V8>(lo, hi);
+  {
+    T* const W2s = Xs;
+    constexpr int VPR = C1p / 8;  // 16-byte vectors per row
+    for (int e = tid; e < 32 * C2T * VPR; e += NTH) {
+      const int row = e / VPR, vc = e % VPR;
+      i32x4 v = {0, 0, 0, 0};
+      if (row < p.C2 && 8 * vc < p.C1) v = *reinterpret_cast<const i32x4*>(W2g + (long long)row * p.C1 + 8 * vc);
+      *reinterpret_cast<i32x2*>(W2s + row * W2S + 8 * vc) = i32x2{v[0], v[1]};  // rows are only 8-byte aligned
+      *reinterpret_cast<i32x2*>(W2s + row * W2S + 8 * vc + 4) = i32x2{v[2], v[3]};
     }
+    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int u = 0; u < 2 * C1T; ++u) {
+        const T* wr = W2s + (32 * (NB * kh + b) + ln) * W2S + 16 * u + 4 * g;
+        w2r[b][u] = concat4<V4, V8>(*reinterpret_cast<const V4*>(wr), *reinterpret_cast<const V4*>(wr + 8));
+      }
+    __syncthreads();  // before the area is zeroed below
+  }
   // the halo tile's padding columns are never written again: zero the whole tile once
   for (int e = tid; e * 8 < xs_elems; e += NTH) *reinterpret_cast<i32x4*>(Xs + 8 * e) = i32x4{0, 0, 0, 0};
 
