@@ -302,6 +302,23 @@ def test_conv_chain_full_size_linearity(oracle):
     assert errors(s, got)[1] <= 1e-5
 
 
+def test_persistent_conv_chain_full_size(oracle, monkeypatch):
+    # the full configuration through the opt-in persistent kernel: two images against the checker, all
+    # of them against the default kernel (two summation orders, both rounded to fp16 at the end)
+    N, C0, H, W, C1, C2 = 32, 64, 56, 56, 64, 256
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, 3, 1, "float16", seed=1)
+    default = run_conv(X, W1, W2, "float16", inter="relu", relu_out=True)
+    monkeypatch.setenv("DITTO_CONV_PERSIST", "1")
+    got = run_conv(X, W1, W2, "float16", inter="relu", relu_out=True)
+    sel = [0, 31]
+    want = oracle.np_round_to(oracle.conv_chain_f32(X[sel], W1, W2, relu_mid=True, relu_out=True, round_mid="float16"),
+                              "float16")
+    mx, rel = errors(got[sel], want)
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
+    assert np.isfinite(got).all() and errors(got, default)[1] <= REL_L2
+    assert (got >= 0).all() and (got == 0).mean() > 0.2  # the output ReLU took effect
+
+
 def test_conv_chain_rejects_unsupported():
     dev = "cuda:0"
     x = torch.zeros(1, 16, 8, 8, device=dev, dtype=torch.float16)
