@@ -156,6 +156,9 @@ __global__ __launch_bounds__(512) void conv_chain_persist_kernel(ConvChainArgs p
   // the tensor, so the number of loads per tile is fixed.  They are issued as inline asm, which keeps
   // them out of the compiler's own wait-count bookkeeping (it would wait for everything outstanding,
   // the previous tile's stores included, before the first use): xv_wait() below is the wait.
+  // INVARIANT: until that wait nothing may read, copy or spill the destination registers (a copy
+  // made by the register allocator would take stale values and free a register that the returning
+  // load then overwrites); tests/test_async_registers.py checks the generated code for it.
   const i32x4 x_rsrc = make_rsrc(p.x, (unsigned)(p.N * p.C0 * p.H * p.W * 2));
   const int hw2 = p.H * p.W * 2;  // bytes of one channel plane
   auto xv_load = [&](int tile) __attribute__((always_inline)) {
