@@ -105,6 +105,41 @@ def test_select_tile_and_validation_without_gpu():
         _lib.check(rc_msg(_desc(K=512, a_row_stride=512, b_row_stride=512))[0])
 
 
+def _conv_desc(**kw):
+    d = dict(abi_version=_lib.ABI_VERSION, in_dtype=_lib.F16, acc_dtype=_lib.F32, out_dtype=_lib.F16, inter_op=_lib.INTER_CAST,
+             relu_out=0, N=32, C0=64, H=56, W=56, C1=64, R1=3, S1=3, pad1=1, stride1=1, C2=256, R2=1, S2=1, pad2=0,
+             stride2=1, groups1=1)
+    d.update(kw)
+    return _lib.ConvChainDesc(**d)
+
+
+def test_conv_tile_choice_without_gpu(monkeypatch):
+    lib = _lib.load()
+    tile = _lib.TileParam()
+    monkeypatch.delenv("DITTO_CONV_PERSIST", raising=False)
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc()), ctypes.byref(tile)) == _lib.OK
+    assert tile.variant == 3022 and tile.grid_x == 32 * 14 and tile.lds_bytes <= 80 * 1024  # two workgroups per CU
+    default_ws = lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc()))
+    assert default_ws == 2 * 9 * 64 * 40 * 2  # two chunks of 32 input channels, [tap][c1][32 + 8]
+    # the opt-in persistent kernel: one workgroup per CU, tiles of two output rows, everything resident
+    monkeypatch.setenv("DITTO_CONV_PERSIST", "1")
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc()), ctypes.byref(tile)) == _lib.OK
+    assert tile.variant == 3928 and tile.block_threads == 256 and tile.grid_x == 256 and tile.grid_y == 2
+    assert tile.lds_bytes <= 160 * 1024
+    # its workspace request also covers the kernel that less aligned pointers fall back to
+    assert lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc())) == default_ws
+    # too few tiles for two rounds, fp32 output, or more than 64 channels: the default kernel
+    for kw in (dict(N=2), dict(out_dtype=_lib.F32), dict(C1=128)):
+        assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(**kw)), ctypes.byref(tile)) == _lib.OK
+        assert tile.variant // 100 != 39, kw
+    # depthwise first convolution: persistent kernel with the matrix-core or the vector-ALU depthwise stage
+    dw = dict(C0=32, H=112, W=112, C2=64, groups1=32)
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=512, **dw)), ctypes.byref(tile)) == _lib.OK
+    assert tile.variant == 4022 and tile.grid_x == 256
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=32, **dw)), ctypes.byref(tile)) == _lib.OK
+    assert tile.variant == 4023
+
+
 def test_run_rejects_bad_arguments_before_touching_the_device():
     lib = _lib.load()
     # null pointers are refused by validation, no launch happens
