@@ -72,6 +72,11 @@ WORKLOADS.update({
         bound="hbm",
         desc="depthwise conv3x3(32 channels x16, s1 p1) -> conv1x1(512->64) on 32x112x112, NCHW fp16 "
              "(the reference's MobileNet-V1 row)"),
+    "dw3x3_conv1x1_f16_n32_c32_112x112_x1_k64": dict(
+        kind="conv", dtype="float16", N=32, C0=32, H=112, W=112, C1=32, R=3, pad=1, stride=1, C2=64, groups=32,
+        bound="hbm",
+        desc="depthwise conv3x3(32 channels, multiplier 1, s1 p1) -> conv1x1(32->64) on 32x112x112, NCHW fp16 "
+             "(MobileNet-V1's first depthwise-separable block)"),
     "gemm_chain_i8_8192x1024x256x1024": dict(
         kind="requant", dtype="int8", batch=1, M=8192, K=1024, L=256, N=1024, scale=2.0 ** -10, bound="hbm",
         desc="int8 A[8192,1024].B[1024,256] -> requantise(2^-10, RNE, saturate) -> .D[256,1024], int32 out"),
