@@ -149,18 +149,6 @@ __device__ __forceinline__ i32x4 make_rsrc_uniform(const void* base, unsigned by
   return r;
 }
 
-// Workgroup barrier for data exchanged through LDS only.  __syncthreads() carries a workgroup-scope
-// release fence, which on this target also waits for every outstanding global store and load of the
-// wave (s_waitcnt vmcnt(0)): a persistent kernel that keeps the previous tile's output stores in
-// flight would wait for their whole round trip at every barrier (4.8 us per tile measured in the
-// depthwise chain).  This one waits for the wave's LDS operations only.  Not for data exchanged
-// through global memory.
-__device__ __forceinline__ void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
-
 // Workgroups are dealt round-robin to the 8 XCDs (each with a private L2) by
 // linear id.  Remap so that ids that are neighbours in the logical order (and
 // share operands) land on the same XCD.

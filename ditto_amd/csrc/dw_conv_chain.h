@@ -255,7 +255,7 @@ __global__ __launch_bounds__(256) void dw_conv_chain_kernel(DwConvArgs p) {
 // are staged once per workgroup and stay in LDS; the halo tile of the next (tile, chunk) is
 // loaded into registers while the current one is computed.
 //
-// LDS:  Xs  2 x [chx][rows_in][cols_al]        halo tiles (two buffers); columns start at the tile's first column
+// LDS:  Xs  [chx][rows_in][cols_al]            halo tile; columns start at the tile's first column
 //                                            rounded down to the load width, so rows are stored
 //                                            with the vectors they were loaded with
 //       W1h [CM / 32][2][32] x 16 bytes      taps 0..7 | 8..15 of the 32 rows of each block, then
@@ -275,7 +275,7 @@ __host__ __device__ constexpr int dw_mfma_groups(int c2_tiles) { return c2_tiles
 __host__ __device__ inline int dw_conv_mfma_lds_bytes(int chx, int mult, int rows_in, int cols_al, int C2p,
                                                       int groups, bool wide) {
   const int cm = chx * mult;
-  return 2 * ((chx * rows_in * cols_al + 7) & ~7) * 2 + ((cm / 32) * 64 + 1) * 16 + C2p * (cm + 8) * 2 +
+  return ((chx * rows_in * cols_al + 7) & ~7) * 2 + ((cm / 32) * 64 + 1) * 16 + C2p * (cm + 8) * 2 +
          (wide ? 4 * groups * 32 * kDwOss * 2 : 0);
 }
 
@@ -335,11 +335,8 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   constexpr int NT = 256 * NG, NW = 4 * NG;  // threads, waves of the workgroup
   const int ln = lane & 31, g = lane >> 5;
-  // two halo buffers: a stage (tile, chunk) reads one while the next stage's halo tile is written to the other
-  T* const Xs0 = reinterpret_cast<T*>(smem_raw);
-  const T* Xrd = Xs0;  // the buffer the current stage reads
-  T* Xwr = Xs0;        // the buffer the next halo tile is written to
-  uint4* const W1h = reinterpret_cast<uint4*>(Xs0 + 2 * xs_elems);
+  T* const Xs = reinterpret_cast<T*>(smem_raw);
+  uint4* const W1h = reinterpret_cast<uint4*>(Xs + xs_elems);
   T* const W2s = reinterpret_cast<T*>(W1h + nblk * 64 + 1);
   T* const Ow = W2s + C2p * W2S + wave * 32 * kDwOss;  // this wave's turn-around buffer
 
@@ -407,7 +404,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
       int left = st_on ? p.chx - st_cph : 0;
 #pragma unroll
       for (int u = 0; u < kDwXpf; ++u) {
-        if (left > 0) dw_st_vec<T, VEC>(Xwr + q, xr[u]);
+        if (left > 0) dw_st_vec<T, VEC>(Xs + q, xr[u]);
         q += cphases * xplane;
         left -= cphases;
         asm volatile("" : "+v"(q), "+v"(left));
@@ -447,17 +444,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
   const int zero_entry = nblk * 64;
   const float inv_m16 = 16.0f / (float)p.mult;
 
-  // Stages (tile, chunk) alternate between the two halo buffers.  The halo tile of stage s + 1 is
-  // loaded into registers before the arithmetic of stage s and written to the other buffer after it:
-  // the wait for those loads (the compiler's, a full vmcnt(0)) then sits BEFORE the output stores of
-  // the tile, so it never waits for them -- with a single buffer it sat after them, at the top of the
-  // next tile, and cost the whole round trip of the stores (5.6 us of a 14.6 us tile measured for
-  // multiplier 1).  One barrier per stage.
-  int stage = 0;
-  if ((int)lid < ntiles) {
-    xload((int)lid, 0);
-    xstore();
-  }
+  if ((int)lid < ntiles) xload((int)lid, 0);
   bool weights_staged = false;
   for (int tile = (int)lid; tile < ntiles; tile += (int)gridDim.x) {
     const int tile_next = tile + (int)gridDim.x < ntiles ? tile + (int)gridDim.x : -1;
@@ -478,11 +465,9 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
     for (int chunk = 0; chunk < nchunks; ++chunk) {
       const int c0 = chunk * p.chx;
       const int cm_base = c0 * p.mult;
-      Xrd = Xs0 + (stage & 1) * xs_elems;
-      Xwr = Xs0 + ((stage + 1) & 1) * xs_elems;
-      ++stage;
+      __syncthreads();  // every wave is done with the previous halo tiles (and filters, if restaged)
+      xstore();
       if (!weights_staged || nchunks > 1) {
-        if (weights_staged) lds_barrier();  // every wave is done with the previous chunk's filters
         weights_staged = true;
         // the chunk's depthwise filters, CM * RS contiguous elements, pass through the W2 area (16-byte
         // loads; C1 * RS is a multiple of 8 and the chunk starts on a 16-byte boundary) ...
@@ -494,7 +479,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
             *reinterpret_cast<V8*>(W2s + 8 * e) = v;
           }
         }
-        lds_barrier();
+        __syncthreads();
         // ... and are regrouped into A-operand entries: row m = 16 * hgrp + 8a + 4gg + b of a block is
         // its intermediate channel 16 * hgrp + 8gg + 4a + b (DWV: two entries per intermediate channel)
         for (int e = tid; e < nblk * 64; e += NT) {
@@ -513,7 +498,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
                          raw[6] | (raw[7] << 16)};
         }
         if (tid == 0) W1h[zero_entry] = uint4{0, 0, 0, 0};
-        lds_barrier();
+        __syncthreads();
         const int nv = CM / 8;  // 16-byte vectors per row of the W2 chunk (C1 is a multiple of 16 here)
         const float inv_nv = 1.0f / (float)nv;
         for (int e0 = tid; e0 < C2p * nv; e0 += 4 * NT) {
@@ -534,11 +519,8 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
             if (dst[u] >= 0) *reinterpret_cast<V8*>(W2s + dst[u]) = v[u];
         }
       }
-      // this stage's halo tile (written at the end of the previous stage) and the filters are visible;
-      // every wave has finished the previous stage, whose buffer the next halo tile will overwrite
-      lds_barrier();
+      __syncthreads();
       // the next (tile, chunk) travels while this one is computed
-      const bool has_next = chunk + 1 < nchunks || tile_next >= 0;
       if (chunk + 1 < nchunks) xload(tile, c0 + p.chx);
       else if (tile_next >= 0) xload(tile_next, 0);
 
@@ -569,7 +551,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
         if constexpr (F33) {
           // dword pair (4 elements) from the even column at or below the pixel's first tap column
           const int xc = xoff[j] + lead;
-          const unsigned* xw = reinterpret_cast<const unsigned*>(Xrd + c * xplane + (xc & ~1));
+          const unsigned* xw = reinterpret_cast<const unsigned*>(Xs + c * xplane + (xc & ~1));
           const unsigned sh = (xc & 1) * 16;
           unsigned p01[3], t2[3];
 #pragma unroll
@@ -583,7 +565,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
           b1n = __builtin_bit_cast(V8, b1r);
           b2n = __builtin_bit_cast(V8, b2r);
         } else {
-          const T* xs = Xrd + c * xplane + xoff[j] + lead;
+          const T* xs = Xs + c * xplane + xoff[j] + lead;
           b1n = V8{xs[tap_off[0]], xs[tap_off[1]], xs[tap_off[2]], xs[tap_off[3]],
                    xs[tap_off[4]], xs[tap_off[5]], xs[tap_off[6]], xs[tap_off[7]]};
           b2n = V8{xs[tap_off[8]], zero, zero, zero, zero, zero, zero, zero};
@@ -640,7 +622,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
             // stays in scalar registers.  Left to itself the compiler keeps one vector register
             // per address for the whole kernel plus one per address and tile; that does not fit,
             // and every reload from scratch waits for all outstanding output stores.
-            int xlane = (int)(Xrd - Xs0) + ((8 * g) >> msh) * xplane + (xc & ~1);
+            int xlane = ((8 * g) >> msh) * xplane + (xc & ~1);
             asm volatile("" : "+v"(xlane));
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
@@ -653,7 +635,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
                 if ((e & ((1 << msh) - 1)) == 0) {  // a new input channel starts
                   // (cm0 + e) >> msh = ((cu0 + e) >> msh) + ((8 * g) >> msh): cu0 is a multiple of 16
                   const unsigned* xw =
-                      reinterpret_cast<const unsigned*>(Xs0 + (xlane + ((cu0 + e) >> msh) * xplane));
+                      reinterpret_cast<const unsigned*>(Xs + (xlane + ((cu0 + e) >> msh) * xplane));
                   unsigned t2[3];
 #pragma unroll
                   for (int r = 0; r < 3; ++r) {
@@ -725,7 +707,6 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
         }
       }
       }
-      if (has_next) xstore();  // into the other buffer; the barrier of the next stage publishes it
     }
     if (WIDE) {
       // o[t][j][r] = out[pixel 8(r/4) + 4g + r%4 of tile j][c2 = 32t + ln]: four consecutive pixels of
