@@ -262,8 +262,9 @@ struct ConvPlan {
 // dw_mode 2 | 3: the persistent kernel, depthwise stage on the matrix cores (multipliers that are
 // multiples of 16) or on the vector ALU (3x3, multiplier 1, 2, 4, 8); dw_mode 0 | 1: the plain
 // kernel for what is left (1: multiples of 8, 0: 1, 2, 4).
+// vec_cap: the widest halo vector (elements) the pointer of this call allows; 8 when planning without one.
 int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvPlan* plan, bool need_device,
-                 bool allow_dwv = true) {
+                 bool allow_dwv = true, int vec_cap = 8) {
   if (d->C1 % d->C0) return fail(DITTO_EINVAL, "depthwise: C1 must be a multiple of C0");
   const long long mult = d->C1 / d->C0;
   const long long RS = d->R1 * d->S1;
@@ -322,9 +323,9 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   const int cm_unit = mfma ? 32 : 16;
   int step = 1;
   while ((step * mult) % cm_unit) ++step;
-  // halo loads: vectors of up to 4 elements that divide W (the run call narrows them if x is less
+  // halo loads: vectors of up to 8 elements that divide W (the run call narrows them if x is less
   // aligned); output through 16-byte stores when rows allow
-  const int vec_max = mfma ? (d->W % 4 == 0 ? 4 : d->W % 2 == 0 ? 2 : 1) : 1;
+  const int vec_max = mfma ? (d->W % 8 == 0 && vec_cap >= 8 ? 8 : d->W % 4 == 0 ? 4 : d->W % 2 == 0 ? 2 : 1) : 1;
   a.vec = vec_max;
   a.wide = mfma && d->out_dtype != DITTO_F32 && Q % 8 == 0 && a.TW % 8 == 0;
   auto lds_of = [&](int chx) {
@@ -339,7 +340,8 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
     // at a time: kDwXpf passes must cover the chunk
     const int nvr = a.cols_al / a.vec;
     const int cphases = (256 * groups / nvr) / a.rows_in;
-    return cphases >= 1 && (chx + cphases - 1) / cphases <= ditto::kDwXpf &&
+    const int passes_max = a.vec == 8 ? ditto::kDwXpf / 2 : ditto::kDwXpf;  // a 16-byte vector takes two entries
+    return cphases >= 1 && (chx + cphases - 1) / cphases <= passes_max &&
            (long long)(chx + 1) * d->H * d->W < 0x7fffffffLL;
   };
   const int chx_max = (int)((d->C0 + step - 1) / step) * step;
@@ -354,12 +356,15 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
       a.vec = vec;
       a.cols_al = (a.cols_in + 2 * vec - 2) / vec * vec;
       a.cols_al += a.cols_al & 1;
+      // 16-byte vectors halve the load and LDS-write instructions of the halo staging (5-6 % of the
+      // kernel on 16-wide tiles) but pad the halo rows more: not where that is over a third
+      if (vec == 8 && 3 * a.cols_al > 4 * ((a.cols_in + 6) / 4 * 4)) continue;
       lds = lds_of(chx_max);
       if (lds <= 160 * 1024 && fits_regs(chx_max)) a.chx = chx_max;
     }
     // ... else chunks: small enough for two workgroups per CU, else whatever fits
     if (!a.chx) {
-      a.vec = vec_max;
+      a.vec = vec_max > 4 ? 4 : vec_max;  // chunks: the narrower halo rows leave room for more channels
       a.cols_al = (a.cols_in + 2 * a.vec - 2) / a.vec * a.vec;
       a.cols_al += a.cols_al & 1;
       for (int limit : {78 * 1024, 150 * 1024}) {
@@ -386,7 +391,7 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   a.relu_mid = d->inter_op == DITTO_INTER_RELU;
   a.relu_out = d->relu_out != 0;
   a.out_f32 = d->out_dtype == DITTO_F32;
-  if (dwv && !a.wide) return plan_dw_conv(d, P, Q, plan, need_device, false);  // that variant needs the wide stores
+  if (dwv && !a.wide) return plan_dw_conv(d, P, Q, plan, need_device, false, vec_cap);  // that variant needs the wide stores
   plan->c2_tiles = c2t;
   ditto_tile_param& t = plan->tile;
   t.block_threads = 256 * groups;
@@ -416,7 +421,8 @@ bool persist_requested() {
   return v && v[0] == '1';
 }
 
-int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device = false, bool allow_persist = true) {
+int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device = false, bool allow_persist = true,
+              int dw_vec_cap = 8) {
   if (!d) return fail(DITTO_EINVAL, "null descriptor");
   if (d->abi_version != DITTO_CHAIN_ABI_VERSION)
     return fail(DITTO_EINVAL, "descriptor abi_version %d, library %d", d->abi_version, DITTO_CHAIN_ABI_VERSION);
@@ -449,7 +455,7 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
   if (d->N * d->C0 * d->H * d->W > 0x7fffffffLL * 4 || d->N * d->C2 * P * Q > 0x7fffffffLL * 4 ||
       d->H > 65535 || d->W > 65535 || d->N > 65535 || d->C0 > 65535 || d->C2 > 65535)
     return fail(DITTO_EINVAL, "tensor too large");
-  if (dw) return plan_dw_conv(d, P, Q, plan, need_device);
+  if (dw) return plan_dw_conv(d, P, Q, plan, need_device, true, dw_vec_cap);
   memset(plan, 0, sizeof(*plan));
   const int c1t = d->C1 <= 32 ? 1 : d->C1 <= 64 ? 2 : d->C1 <= 128 ? 4 : 8;
   const int pxw = c1t == 8 ? 1 : 2;
@@ -773,7 +779,8 @@ enum ConvPhase { kConvPrepare = 1, kConvCompute = 2, kConvBoth = 3 };
 int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, const void* w1, const void* w2,
                     void* y, void* workspace, size_t workspace_bytes, void* stream) {
   ConvPlan plan;
-  int rc = plan_conv(d, &plan, true);
+  // (depthwise chains: 16-byte halo vectors only for a 16-byte aligned x; the tile query assumes one)
+  int rc = plan_conv(d, &plan, true, true, x && aligned(x, 16) ? 8 : 4);
   if (rc != DITTO_OK) return rc;
   if (((phase & kConvCompute) && (!x || !y)) || !w1 || !w2) return fail(DITTO_EINVAL, "null data pointer");
   if (!aligned(x, 2) || !aligned(w1, 2) || !aligned(w2, 8) || !aligned(y, 4))
@@ -790,7 +797,7 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
     if (plan.dw_mode >= 2) {
       const int nvr = a.cols_al / a.vec;
       const int cphases = (256 * ditto::dw_mfma_groups(plan.c2_tiles) / nvr) / a.rows_in;
-      if (cphases < 1 || (a.chx + cphases - 1) / cphases > ditto::kDwXpf)
+      if (cphases < 1 || (a.chx + cphases - 1) / cphases > (a.vec == 8 ? ditto::kDwXpf / 2 : ditto::kDwXpf))
         return fail(DITTO_EINVAL, "misaligned data pointer: x must be aligned to %d bytes for this shape",
                     2 * plan.dwargs.vec);
       if (!aligned(w1, 16)) return fail(DITTO_EINVAL, "misaligned data pointer");

@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void dw_conv_chain_kernel(DwConvArgs p) {
 //       W2s [32 * C2T][CM + 8]               the chunk's columns of W2
 //       Os  [waves][32][40]                  WIDE: per-wave turn-around for 16-byte stores
 constexpr int kDwMfmaTaps = 16;  // R * S <= 16 on the MFMA path
-constexpr int kDwXpf = 12;      // halo vectors (of up to 4 elements) a thread keeps in flight
+constexpr int kDwXpf = 12;      // halo vectors of up to 4 elements (or half as many of 8) a thread keeps in flight
 
 constexpr int kDwOss = 40;  // row stride (elements) of a wave's turn-around buffer: 32 pixels + 8
 
@@ -289,6 +289,18 @@ __device__ __forceinline__ void dw_ld_vec(typename Elem<T>::v4& r, const T* src)
   } else {
     r[0] = *src;
   }
+}
+
+// 8-element (16-byte) halo vectors occupy two consecutive entries of the register array
+template <typename T>
+__device__ __forceinline__ void dw_ld_vec8(typename Elem<T>::v4& lo, typename Elem<T>::v4& hi, const T* src) {
+  const typename Elem<T>::v8 t = *reinterpret_cast<const typename Elem<T>::v8*>(src);
+  lo = typename Elem<T>::v4{t[0], t[1], t[2], t[3]};
+  hi = typename Elem<T>::v4{t[4], t[5], t[6], t[7]};
+}
+template <typename T>
+__device__ __forceinline__ void dw_st_vec8(T* dst, const typename Elem<T>::v4& lo, const typename Elem<T>::v4& hi) {
+  *reinterpret_cast<typename Elem<T>::v8*>(dst) = typename Elem<T>::v8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 }
 
 template <typename T, int VEC>
@@ -384,6 +396,18 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
       // known to point to global memory)
       long long q = src;
       int left = nch;
+      if constexpr (VEC == 8) {
+#pragma unroll
+        for (int u = 0; u < kDwXpf / 2; ++u) {
+          xr[2 * u] = zero4;
+          xr[2 * u + 1] = zero4;
+          if (ok && left > 0) dw_ld_vec8<T>(xr[2 * u], xr[2 * u + 1], Xg + q);
+          q += cphases * hw32;
+          left -= cphases;
+          asm volatile("" : "+v"(q), "+v"(left));
+        }
+        return;
+      }
 #pragma unroll
       for (int u = 0; u < kDwXpf; ++u) {
         xr[u] = zero4;
@@ -393,7 +417,8 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
         asm volatile("" : "+v"(q), "+v"(left));
       }
     };
-    if (p.vec == 4) body(std::integral_constant<int, 4>());
+    if (p.vec == 8) body(std::integral_constant<int, 8>());
+    else if (p.vec == 4) body(std::integral_constant<int, 4>());
     else if (p.vec == 2) body(std::integral_constant<int, 2>());
     else body(std::integral_constant<int, 1>());
   };
@@ -402,6 +427,16 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
       constexpr int VEC = decltype(vec_tag)::value;
       int q = st_dst;  // a running offset, as in xload (a pointer would no longer be known to point to LDS)
       int left = st_on ? p.chx - st_cph : 0;
+      if constexpr (VEC == 8) {
+#pragma unroll
+        for (int u = 0; u < kDwXpf / 2; ++u) {
+          if (left > 0) dw_st_vec8<T>(Xs + q, xr[2 * u], xr[2 * u + 1]);
+          q += cphases * xplane;
+          left -= cphases;
+          asm volatile("" : "+v"(q), "+v"(left));
+        }
+        return;
+      }
 #pragma unroll
       for (int u = 0; u < kDwXpf; ++u) {
         if (left > 0) dw_st_vec<T, VEC>(Xs + q, xr[u]);
@@ -410,7 +445,8 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
         asm volatile("" : "+v"(q), "+v"(left));
       }
     };
-    if (p.vec == 4) body(std::integral_constant<int, 4>());
+    if (p.vec == 8) body(std::integral_constant<int, 8>());
+    else if (p.vec == 4) body(std::integral_constant<int, 4>());
     else if (p.vec == 2) body(std::integral_constant<int, 2>());
     else body(std::integral_constant<int, 1>());
   };
