@@ -40,8 +40,8 @@ MEASURED_TRAFFIC_BYTES = {
     "conv_chain_f16_n32_c64_56x56_k64_k256": int((13.44 + 54.50) * 2 ** 20),
     "gemm_chain_i8_8192x1024x256x1024": int((12.15 + 32.00) * 2 ** 20),
     "conv1x1_conv3x3_f16_n32_c64_56x56_k64_k64": int((13.25 + 12.25) * 2 ** 20),
-    "dw3x3_conv1x1_f16_n32_c32_112x112_f16_k64": int((29.77 + 49.00) * 2 ** 20),
-    "dw3x3_conv1x1_f16_n32_c32_112x112_x1_k64": int((29.29 + 49.00) * 2 ** 20),
+    "dw3x3_conv1x1_f16_n32_c32_112x112_f16_k64": int((29.79 + 49.00) * 2 ** 20),
+    "dw3x3_conv1x1_f16_n32_c32_112x112_x1_k64": int((29.30 + 49.00) * 2 ** 20),
 }
 
 WORKLOADS = {
