@@ -209,7 +209,7 @@ def test_depthwise_chain_with_less_aligned_pointers(oracle):
     chain.run_conv_chain(x, w1, w2, want, groups1=C0)
     xbuf = torch.zeros(x.numel() + 8, device=x.device, dtype=torch.float16)
     ybuf = torch.zeros(want.numel() + 8, device=x.device, dtype=torch.float16)
-    for xo, yo in ((1, 0), (0, 2), (3, 6)):
+    for xo, yo in ((1, 0), (0, 2), (3, 6), (4, 0)):  # the last: x 8-byte aligned, 4-element halo vectors
         xs = xbuf[xo:xo + x.numel()].view_as(x)
         xs.copy_(x)
         ys = ybuf[yo:yo + want.numel()].view_as(want)
