@@ -364,7 +364,8 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
     }
     // ... else chunks: small enough for two workgroups per CU, else whatever fits
     if (!a.chx) {
-      a.vec = vec_max > 4 ? 4 : vec_max;  // chunks: the narrower halo rows leave room for more channels
+      a.vec = vec_max;  // 16-byte vectors under the same padding rule as above
+      if (a.vec == 8 && 3 * ((a.cols_in + 14) / 8 * 8) > 4 * ((a.cols_in + 6) / 4 * 4)) a.vec = 4;
       a.cols_al = (a.cols_in + 2 * a.vec - 2) / a.vec * a.vec;
       a.cols_al += a.cols_al & 1;
       for (int limit : {78 * 1024, 150 * 1024}) {
