@@ -50,7 +50,7 @@ def test_kernel_metadata_parser():
     assert md["_ZN5ditto1bEv"] == {"private_segment_fixed_size": 112, "vgpr_spill_count": 28}
 
 
-@pytest.mark.parametrize("dtype", ["f16"])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_depthwise_kernels_with_wide_stores_use_no_scratch_and_no_flat_accesses(tmp_path, dtype):
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
