@@ -37,8 +37,6 @@ UNITS = [
     ("api", "api.hip", []),
     ("gemm_chain_i8", "gemm_chain_i8.hip", []),
     ("gemm_chain_f32", "gemm_chain_f32.hip", []),
-    ("conv_persist_f16", "conv_chain_persist_inst.hip", ["-DDITTO_INST_T=f16", "-DDITTO_PERSIST_NAME=launch_conv_persist_f16"]),
-    ("conv_persist_bf16", "conv_chain_persist_inst.hip", ["-DDITTO_INST_T=bf16", "-DDITTO_PERSIST_NAME=launch_conv_persist_bf16"]),
     ("conv_f16", "conv_chain_inst.hip", ["-DDITTO_INST_T=f16", "-DDITTO_INST_NAME=launch_conv_f16", "-DDITTO_PACK_NAME=pack_conv_w1_f16",
                                           "-DDITTO_INST2_NAME=launch_conv2_f16", "-DDITTO_PACK2_NAME=pack_conv_w2_f16", "-DDITTO_DW_NAME=launch_dw_conv_f16"]),
     ("conv_bf16", "conv_chain_inst.hip", ["-DDITTO_INST_T=bf16", "-DDITTO_INST_NAME=launch_conv_bf16", "-DDITTO_PACK_NAME=pack_conv_w1_bf16",

@@ -248,8 +248,6 @@ struct ConvPlan {
   int ch;              // input channels per staged chunk
   size_t w1p_bytes;    // size of the repacked W1 (the workspace)
   ditto::ConvChainArgs args;
-  bool persist;        // 1x1 second convolution, weights resident in LDS: conv_chain_persist.h (c2_tiles, grid)
-  int grid;
   bool dw;             // depthwise first convolution: dwargs / c2_tiles / dw_shared describe the launch
   int c2_tiles;
   int dw_mode;         // 0 | 1: plain kernel (1: multiplier a multiple of 8); 2 | 3: persistent kernel,
@@ -422,8 +420,7 @@ bool persist_requested() {
   return v && v[0] == '1';
 }
 
-int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device = false, bool allow_persist = true,
-              int dw_vec_cap = 8) {
+int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device = false, int dw_vec_cap = 8) {
   if (!d) return fail(DITTO_EINVAL, "null descriptor");
   if (d->abi_version != DITTO_CHAIN_ABI_VERSION)
     return fail(DITTO_EINVAL, "descriptor abi_version %d, library %d", d->abi_version, DITTO_CHAIN_ABI_VERSION);
@@ -509,61 +506,14 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
     t.variant = 3500 + c1t * 10 + plan->px2;  // second convolution through LDS
     return DITTO_OK;
   }
-  // Persistent variant (conv_chain_persist.h): W1 resident in LDS and W2 in registers beside one halo
-  // tile of whole output rows (at most 128 pixels), one workgroup per CU walking over the tiles; needs
-  // tiles for at least two rounds.  Opt-in (environment variable DITTO_CONV_PERSIST=1, read at every
-  // call): correct, but on the 32 x 64 x 56 x 56 -> 64 -> 256 chain it runs 33-36 us against 28 us for
-  // the one-tile-per-workgroup kernel below.
-  if (allow_persist && persist_requested() && d->out_dtype != DITTO_F32 && d->C0 <= 64 && d->C1 <= 64 && d->C2 <= 256 && d->W % 8 == 0 &&
-      d->R1 == d->S1 && (d->R1 == 1 || d->R1 == 3) &&
-      Q % 8 == 0 && Q <= 128 && d->N * d->C0 * d->H * d->W * 2 < 0x7fffffffLL && d->N * d->C2 * P * Q * 2 < 0x7fffffffLL) {
-    const int pc1t = d->C1 <= 32 ? 1 : 2, pch = d->C0 <= 32 ? 32 : 64, pc2t = 8;  // the instantiated variants
-    const int RS = a.R * a.S;
-    const int cus = need_device ? device_cus() : 256;
-    // rows per tile: among those that fit and leave tiles for two rounds, the fewest rounds x
-    // (pixels + a fixed cost per tile)
-    int th = 0, lds = 0;
-    long long ntiles = 0, best = -1;
-    for (int t = (int)(128 / Q < P ? 128 / Q : P); t >= 1; --t) {
-      const int rows = (t - 1) * a.stride + a.R, cols = ((int)Q - 1) * a.stride + a.S;
-      const int l = ditto::conv_persist_lds_bytes(rows, cols, RS, 32 * pc1t, pch);
-      const long long nt = d->N * ((P + t - 1) / t);
-      if (l > 160 * 1024 || rows * (a.W / 8) * (pch / 8) > 512 || nt < 2LL * cus) continue;
-      const long long cost = ((nt + cus - 1) / cus) * (t * Q + 24);
-      if (best < 0 || cost < best) { best = cost; th = t; lds = l; ntiles = nt; }
-    }
-    if (th >= 1) {
-      a.rows_in = (th - 1) * a.stride + a.R;
-      a.cols_in = ((int)Q - 1) * a.stride + a.S;
-    }
-    if (ntiles >= 2LL * cus) {
-      a.TH = th;
-      a.TW = (int)Q;
-      a.tiles_h = (int)((P + th - 1) / th);
-      a.tiles_w = 1;
-      a.relu_mid = d->inter_op == DITTO_INTER_RELU;
-      a.relu_out = d->relu_out != 0;
-      a.out_f32 = 0;
-      plan->persist = true;
-      plan->c1_tiles = pc1t;
-      plan->ch = pch;
-      plan->c2_tiles = pc2t;
-      plan->grid = (int)(ntiles < cus ? ntiles : cus);
-      plan->w1p_bytes = (size_t)ditto::conv_w1_chunk_bytes(RS, 32 * pc1t, pch);
-      ditto_tile_param& t = plan->tile;
-      t.block_threads = 256;
-      t.block_m = a.TH * a.TW;
-      t.block_l = 32 * pc1t;
-      t.block_n = (int)d->C2;
-      t.head_pad = pch;
-      t.lds_bytes = lds;
-      t.grid_x = plan->grid;
-      t.grid_y = a.TH;
-      t.grid_z = a.TW;
-      t.variant = 3900 + pc1t * 10 + pc2t;  // persistent workgroups, weights resident
-      return DITTO_OK;
-    }
-  }
+  // The persistent variant (conv_chain_persist.h: W1 resident in LDS, W2 in registers, one workgroup per
+  // CU walking over the tiles) is switched off: it waits for its prefetched halo tile with a hand-counted
+  // `s_waitcnt vmcnt` over loads the compiler does not track, and it is slower than the kernel below
+  // (33.5 against 30.5 us on 32 x 64 x 56 x 56 -> 64 -> 256).  Asking for it is refused, not ignored.
+  if (persist_requested())
+    return fail(DITTO_EUNSUPPORTED,
+                "DITTO_CONV_PERSIST=1: the persistent conv chain kernel is switched off (untracked prefetch loads; "
+                "slower than the default kernel); unset the variable");
   a.TW = (int)(Q < slots ? Q : slots);
   a.TH = slots / a.TW;
   if (a.TH > P) a.TH = (int)P;
@@ -762,13 +712,7 @@ int ditto_conv_chain_select_tile(const ditto_conv_chain_desc* desc, ditto_tile_p
 size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
   ConvPlan plan;
   if (plan_conv(desc, &plan) != DITTO_OK) return 0;
-  size_t need = plan.w1p_bytes + plan.w2p_bytes;
-  if (plan.persist) {  // a call with less aligned pointers runs the one-tile-per-workgroup kernel instead
-    ConvPlan other;
-    if (plan_conv(desc, &other, false, false) == DITTO_OK && other.w1p_bytes + other.w2p_bytes > need)
-      need = other.w1p_bytes + other.w2p_bytes;
-  }
-  return need;
+  return plan.w1p_bytes + plan.w2p_bytes;
 }
 
 }  // extern "C"
@@ -781,7 +725,7 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
                     void* y, void* workspace, size_t workspace_bytes, void* stream) {
   ConvPlan plan;
   // (depthwise chains: 16-byte halo vectors only for a 16-byte aligned x; the tile query assumes one)
-  int rc = plan_conv(d, &plan, true, true, x && aligned(x, 16) ? 8 : 4);
+  int rc = plan_conv(d, &plan, true, x && aligned(x, 16) ? 8 : 4);
   if (rc != DITTO_OK) return rc;
   if (((phase & kConvCompute) && (!x || !y)) || !w1 || !w2) return fail(DITTO_EINVAL, "null data pointer");
   if (!aligned(x, 2) || !aligned(w1, 2) || !aligned(w2, 8) || !aligned(y, 4))
@@ -817,13 +761,6 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
     if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
     return DITTO_OK;
   }
-  if (plan.persist && !(workspace && aligned(x, 16) && aligned(y, 16) && aligned(w2, 16))) {
-    // the persistent kernel needs the repacked W1 and 16-byte aligned tensors
-    if (phase == kConvCompute)
-      return fail(DITTO_EINVAL, "misaligned data pointer: x, y and w2 must be 16-byte aligned to run these prepared weights");
-    rc = plan_conv(d, &plan, true, false);
-    if (rc != DITTO_OK) return rc;
-  }
   const size_t need = plan.w1p_bytes + plan.w2p_bytes;
   if (plan.w1p_bytes >= (1ull << 31) || plan.w2p_bytes >= (1ull << 31))  // the repack kernels index with 32 bits
     return fail(DITTO_EUNSUPPORTED, "conv chain weights too large to repack");
@@ -856,11 +793,7 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
     if (e == hipSuccess && compute)
       e = f16 ? ditto::launch_conv2_f16(plan.c1_tiles, plan.px2, a, st) : ditto::launch_conv2_bf16(plan.c1_tiles, plan.px2, a, st);
   } else if (e == hipSuccess && compute) {
-    if (plan.persist)
-      e = f16 ? ditto::launch_conv_persist_f16(plan.c1_tiles, plan.ch, plan.c2_tiles, a, plan.grid, st)
-              : ditto::launch_conv_persist_bf16(plan.c1_tiles, plan.ch, plan.c2_tiles, a, plan.grid, st);
-    else
-      e = f16 ? ditto::launch_conv_f16(plan.c1_tiles, plan.ch, a, st) : ditto::launch_conv_bf16(plan.c1_tiles, plan.ch, a, st);
+    e = f16 ? ditto::launch_conv_f16(plan.c1_tiles, plan.ch, a, st) : ditto::launch_conv_bf16(plan.c1_tiles, plan.ch, a, st);
   }
   if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
   return DITTO_OK;

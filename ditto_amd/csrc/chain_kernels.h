@@ -4,7 +4,6 @@
 
 #include "bmm_chain_fp.h"
 #include "conv_chain.h"
-#include "conv_chain_persist.h"
 #include "dw_conv_chain.h"
 #include "gemm_chain_f32.h"
 #include "gemm_chain_i8.h"
@@ -21,10 +20,6 @@ hipError_t launch_bf16_softmax(int d_pad, int q, bool b_kl, const BmmChainArgs& 
 // ch in {32, 16}: input channels per staged chunk
 hipError_t launch_conv_f16(int c1_tiles, int ch, const ConvChainArgs& args, hipStream_t stream);
 hipError_t launch_conv_bf16(int c1_tiles, int ch, const ConvChainArgs& args, hipStream_t stream);
-// conv_chain_persist_inst.hip: persistent workgroups with both weight tensors resident in LDS;
-// c1_tiles in {1, 2}, ch in {32, 64} (all input channels, padded), c2_tiles = 8, 1x1 or 3x3 first filter
-hipError_t launch_conv_persist_f16(int c1_tiles, int ch, int c2_tiles, const ConvChainArgs& args, int grid, hipStream_t stream);
-hipError_t launch_conv_persist_bf16(int c1_tiles, int ch, int c2_tiles, const ConvChainArgs& args, int grid, hipStream_t stream);
 // W1 -> the chunked layout the chain kernel loads directly (conv_w1_chunk_bytes per chunk)
 hipError_t pack_conv_w1_f16(int c1_tiles, int ch, const ConvChainArgs& args, void* out, hipStream_t stream);
 hipError_t pack_conv_w1_bf16(int c1_tiles, int ch, const ConvChainArgs& args, void* out, hipStream_t stream);

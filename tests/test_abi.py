@@ -121,17 +121,12 @@ def test_conv_tile_choice_without_gpu(monkeypatch):
     assert tile.variant == 3022 and tile.grid_x == 32 * 14 and tile.lds_bytes <= 80 * 1024  # two workgroups per CU
     default_ws = lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc()))
     assert default_ws == 2 * 9 * 64 * 40 * 2  # two chunks of 32 input channels, [tap][c1][32 + 8]
-    # the opt-in persistent kernel: one workgroup per CU, tiles of two output rows, everything resident
+    # the opt-in persistent kernel is switched off: asking for it is refused, not silently ignored
     monkeypatch.setenv("DITTO_CONV_PERSIST", "1")
-    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc()), ctypes.byref(tile)) == _lib.OK
-    assert tile.variant == 3928 and tile.block_threads == 256 and tile.grid_x == 256 and tile.grid_y == 2
-    assert tile.lds_bytes <= 160 * 1024
-    # its workspace request also covers the kernel that less aligned pointers fall back to
-    assert lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc())) == default_ws
-    # too few tiles for two rounds, fp32 output, or more than 64 channels: the default kernel
-    for kw in (dict(N=2), dict(out_dtype=_lib.F32), dict(C1=128)):
-        assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(**kw)), ctypes.byref(tile)) == _lib.OK
-        assert tile.variant // 100 != 39, kw
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc()), ctypes.byref(tile)) == _lib.EUNSUPPORTED
+    assert b"switched off" in lib.ditto_last_error()
+    assert lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc())) == 0
+    monkeypatch.delenv("DITTO_CONV_PERSIST")
     # depthwise first convolution: persistent kernel with the matrix-core or the vector-ALU depthwise stage
     dw = dict(C0=32, H=112, W=112, C2=64, groups1=32)
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=512, **dw)), ctypes.byref(tile)) == _lib.OK

@@ -70,6 +70,11 @@ CASES_PERSISTENT = [
 ]
 
 
+PERSIST_OFF = ("the persistent conv chain kernel is switched off in the planner (DITTO_EUNSUPPORTED): it waits for "
+               "prefetch loads the compiler does not track with a hand-counted s_waitcnt and is slower than the default")
+
+
+@pytest.mark.skip(reason=PERSIST_OFF)
 @pytest.mark.parametrize("case", CASES_PERSISTENT)
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
 def test_persistent_conv_chain_vs_oracle(oracle, case, dtype, monkeypatch):
@@ -302,6 +307,7 @@ def test_conv_chain_full_size_linearity(oracle):
     assert errors(s, got)[1] <= 1e-5
 
 
+@pytest.mark.skip(reason=PERSIST_OFF)
 def test_persistent_conv_chain_full_size(oracle, monkeypatch):
     # the full configuration through the opt-in persistent kernel: two images against the checker, all
     # of them against the default kernel (two summation orders, both rounded to fp16 at the end)
