@@ -117,7 +117,10 @@ EXPORTS = [
      [ctypes.POINTER(ConvChainDesc), _P, _P, _P, ctypes.c_size_t, _P]),
     ("ditto_conv_chain_run_prepared", ctypes.c_int,
      [ctypes.POINTER(ConvChainDesc), _P, _P, _P, _P, _P, ctypes.c_size_t, _P]),
+    ("ditto_conv_chain_run_static", ctypes.c_int, [ctypes.POINTER(ConvChainDesc), _P, _P, _P, _P, _P]),
 ]
+
+STATIC_WORKSPACE_BYTES = 4 << 20  # DITTO_STATIC_WORKSPACE_BYTES
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libditto_chain.so")
 

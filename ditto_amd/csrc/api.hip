@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "bmm_chain_fp8.h"
 #include "chain_kernels.h"
@@ -819,3 +820,54 @@ int ditto_conv_chain_run_prepared(const ditto_conv_chain_desc* d, const void* x,
 }
 
 }  // extern "C"
+
+// ---- the entry point that allocates nothing -------------------------------------------------
+// Its workspace (the repacked weights of a conv chain) is a file-scope device array instead of
+// caller memory.  Every device the library runs on holds its own copy of the array at its own
+// address until the process ends; host code reaches it only through the address taken with
+// hipGetSymbolAddress on that device (the array's name is a host-side stand-in, not a device
+// address).
+static __device__ __align__(256) unsigned char scratch[DITTO_STATIC_WORKSPACE_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices];  // per device, filled at the first call on that device
+
+// Device address of `scratch` on the current device.
+int static_workspace(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(DITTO_EHIP, "hipGetDevice failed: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(DITTO_EUNSUPPORTED, "device ordinal %d beyond %d", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return fail(DITTO_EHIP, "hipGetSymbolAddress(static workspace) failed: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return DITTO_OK;
+}
+}  // namespace
+
+extern "C" int ditto_conv_chain_run_static(const ditto_conv_chain_desc* d, const void* x, const void* w1,
+                                           const void* w2, void* y, void* stream) {
+  ConvPlan plan;
+  int rc = plan_conv(d, &plan);
+  if (rc != DITTO_OK) return rc;
+  const size_t need = plan.w1p_bytes + plan.w2p_bytes;
+  if (need > (size_t)DITTO_STATIC_WORKSPACE_BYTES)
+    return fail(DITTO_EWORKSPACE, "the repacked weights take %zu bytes, the static workspace holds %zu", need,
+                (size_t)DITTO_STATIC_WORKSPACE_BYTES);
+  void* ws = nullptr;
+  if (need > 0) {  // (depthwise chains stage their filters themselves and take no workspace)
+    rc = static_workspace(&ws);
+    if (rc != DITTO_OK) return rc;
+  }
+  // every byte of the workspace that the fused kernel reads is written by the repacking kernel of the
+  // same call, ahead of it on `stream`: nothing has to be cleared between calls
+  return conv_chain_call(kConvBoth, d, x, w1, w2, y, ws, ws ? (size_t)DITTO_STATIC_WORKSPACE_BYTES : 0, stream);
+}

@@ -203,6 +203,21 @@ int ditto_conv_chain_run_prepared(const ditto_conv_chain_desc* desc, const void*
                                   const void* w2, void* y, void* workspace, size_t workspace_bytes,
                                   void* stream);
 
+/*
+ * ditto_conv_chain_run for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same kernels and results as ditto_conv_chain_run with a workspace, but the
+ * repacked weights go into a device array inside the library (DITTO_STATIC_WORKSPACE_BYTES per
+ * GPU, held until the process ends) and the call allocates nothing.
+ *   - DITTO_EWORKSPACE if ditto_conv_chain_workspace_bytes(desc) exceeds that size;
+ *   - every call on one GPU shares that GPU's array: calls that overlap on one GPU (two streams,
+ *     two threads) race; calls on one stream are ordered and safe;
+ *   - the array keeps the last call's contents; each call rewrites all it reads.
+ */
+#define DITTO_STATIC_WORKSPACE_BYTES (4u << 20)
+int ditto_conv_chain_run_static(const ditto_conv_chain_desc* desc, const void* x, const void* w1,
+                                const void* w2, void* y, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
