@@ -9,10 +9,12 @@ resident in HBM.  The headline workload is the long-sequence BMM -> softmax -> B
 peak" target is stated.  The other configurations are timed briefly and reported under
 "also".  One JSON line is printed.
 
-Timing protocol (mirrors the reference's ``time_evaluator(..., min_repeat_ms=600)`` use,
-benchmark/chimera/cuda/bmm_softmax_bmm_cuda.py:39): W untimed warm-up calls, then exactly K
-calls between two HIP events recorded on the launch stream, bracketed by device
-synchronisation.  FLOPs are the algorithmic ``2*batch*M*L*(K+N)`` (the reference counts
+Timing protocol: untimed warm-up calls until both W calls and 300 ms of device work are done (a
+fresh device needs that long to reach its steady clocks), then exactly K calls between two HIP
+events recorded on the launch stream, bracketed by device synchronisation.  Beside it,
+``roofline.min_repeat_600ms_ms`` is the mean per call over a timed region grown to at least 600 ms,
+the reference's ``time_evaluator(..., min_repeat_ms=600)`` rule
+(benchmark/chimera/cuda/bmm_softmax_bmm_cuda.py:39).  FLOPs are the algorithmic ``2*batch*M*L*(K+N)`` (the reference counts
 ``batch*M*L*(K+N)`` MACs, benchmark/chimera/cpu/bmm_bmm_cpu.py:281); softmax, casts and
 padding count zero.
 """
@@ -158,7 +160,7 @@ def make_call(w, dev, prepared=False):
     return (lambda: chain.run_bmm_chain(a, b, c, f, desc=desc)), desc
 
 
-def time_gpu(w, steps, warmup, dev, prepared=False):
+def time_gpu(w, steps, warmup, dev, prepared=False, long_run=False):
     """(ms per step over the synchronised wall clock, ms per launch from HIP events around the eager
     loop, ms per launch from a graph replay of the same loop)."""
     import torch
@@ -166,9 +168,7 @@ def time_gpu(w, steps, warmup, dev, prepared=False):
     from ditto_amd import chain
 
     call, desc = make_call(w, dev, prepared)
-    for _ in range(max(warmup, 1)):
-        call()
-    torch.cuda.synchronize()
+    warm_up(call, warmup)
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
@@ -180,7 +180,42 @@ def time_gpu(w, steps, warmup, dev, prepared=False):
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     ev_ms = e0.elapsed_time(e1) / steps
     tile = chain.select_tile(desc).to_json()
-    return wall_ms, ev_ms, graph_ms(call, steps), tile
+    return wall_ms, ev_ms, graph_ms(call, steps), tile, (min_repeat_ms(call) if long_run else None)
+
+
+WARMUP_MIN_S = 0.3
+
+
+def warm_up(call, warmup):
+    """At least ``warmup`` calls and at least WARMUP_MIN_S seconds of back-to-back device work."""
+    import torch
+
+    done, t0 = 0, time.perf_counter()
+    while done < max(warmup, 1) or time.perf_counter() - t0 < WARMUP_MIN_S:
+        for _ in range(max(warmup, 1)):
+            call()
+        torch.cuda.synchronize()
+        done += max(warmup, 1)
+
+
+def min_repeat_ms(call, min_ms=600.0):
+    """Mean ms per call over a timed region of at least ``min_ms`` (the number of calls is grown until
+    the region is long enough: TVM's ``min_repeat_ms`` rule)."""
+    import torch
+
+    n = 8
+    while True:
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        if ms >= min_ms or n >= (1 << 22):
+            return ms / n
+        n = max(n + 1, int(n * max(1.5, min_ms / max(ms, 1e-3) * 1.05)))
 
 
 def graph_ms(call, steps):
@@ -248,9 +283,9 @@ def cpu_baseline(w, budget_s=10.0, pool=24):
     }
 
 
-def run_one(name, steps, warmup, dev):
+def run_one(name, steps, warmup, dev, long_run=False):
     w = WORKLOADS[name]
-    wall_ms, ev_ms, gr_ms, tile = time_gpu(w, steps, warmup, dev)
+    wall_ms, ev_ms, gr_ms, tile, long_ms = time_gpu(w, steps, warmup, dev, long_run=long_run)
     fl, by = flops_of(w), bytes_of(w)
     short = SHORT[w["dtype"]]
     # The roofline uses the HIP-event time per launch of the eager loop (what rocprofv3's per-kernel
@@ -268,10 +303,12 @@ def run_one(name, steps, warmup, dev):
     roof["algorithmic_bytes"] = by
     roof["kernel_ms"] = k_ms
     roof["graph_replay_ms"] = gr_ms
+    if long_ms is not None:
+        roof["min_repeat_600ms_ms"] = long_ms
     if w["kind"] == "conv" and w.get("groups", 1) == 1:
         # the same step with the weight repacking done once beforehand (ditto_conv_chain_prepare +
         # ditto_conv_chain_run_prepared): what a caller with fixed weights pays per call
-        _, pev_ms, pgr_ms, _ = time_gpu(w, steps, warmup, dev, prepared=True)
+        _, pev_ms, pgr_ms, _, _ = time_gpu(w, steps, warmup, dev, prepared=True)
         roof["weights_prepared_ms"] = pev_ms
         roof["weights_prepared_graph_replay_ms"] = pgr_ms
     return w, wall_ms, ev_ms, tile, roof
@@ -307,7 +344,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    w, wall_ms, ev_ms, tile, roof = run_one(args.workload, args.steps, args.warmup, dev)
+    w, wall_ms, ev_ms, tile, roof = run_one(args.workload, args.steps, args.warmup, dev, long_run=True)
     fl = flops_of(w)
     value = fl / (wall_ms * 1e-3) / 1e12
     short = SHORT[w["dtype"]]

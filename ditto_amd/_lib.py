@@ -47,7 +47,7 @@ class BmmChainDesc(ctypes.Structure):
         ("softmax_scale", ctypes.c_float),
         ("requant_scale", ctypes.c_float),
         ("tile_variant", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("relu_out", ctypes.c_int32),
         ("batch_inner", ctypes.c_int64),
         ("a_batch_stride_outer", ctypes.c_int64),
         ("b_batch_stride_outer", ctypes.c_int64),

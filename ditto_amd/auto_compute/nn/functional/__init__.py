@@ -1,3 +1,4 @@
 from .bmm_chain import (BatchGemmGemm, BatchGemmGemmMMA, BatchGemmSoftmaxGemm,
                         BatchGemmSoftmaxGemmMMA)
 from .conv_chain import Conv1x1Conv3x3, Conv3x3Conv1x1, Depthwise3x3Conv1x1, conv_chain, conv_relu_conv
+from .elementwise import ACT_KINDS, ELEM_KINDS, ReLU, activation, elementwise

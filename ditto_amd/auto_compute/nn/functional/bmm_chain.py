@@ -88,23 +88,47 @@ def BatchGemmSoftmaxGemmMMA(query, key, value, MI=16, NI=16, KI=16, in_dtype="fl
     return F
 
 
-def BatchGemmGemmMMA(A, B, C, MI=16, NI=16, KI=16, in_dtype="float16", acc_dtype="float32", relu=False):
+def BatchGemmGemmMMA(A, B, C, MI=16, NI=16, KI=16, in_dtype="float16", acc_dtype="float32", relu=False,
+                     requant_scale=None, scale=None, out_dtype=None):
     """GEMM -> GEMM chain on given placeholders: ``F = cast(cast(A.B) . C)`` (optionally
-    ReLU on the first accumulator, as test_hyper_fusion_cpu.py:61-67)."""
+    ReLU on the first accumulator, as test_hyper_fusion_cpu.py:61-67).
+
+    int8 operands with an int32 accumulator (the ("80", "int8", "int32") row of
+    bmm_bmm_cuda.py:273-288): the middle result goes back to int8 through a *requantise* op,
+    ``saturate(round_to_nearest_even(acc * s))`` with ``s = requant_scale`` for every intermediate
+    column or ``scale[l]`` from a float32 placeholder ``scale[L]`` (the reference's chain wraps
+    with ``astype("int8")``, :116, which no kernel here implements), and ``F`` keeps the
+    accumulator type unless ``out_dtype`` says otherwise."""
     batch, M, K = A.shape
     _batch, _K, L = B.shape
     _batch2, _L, N = C.shape
     assert _batch == batch and _batch2 == batch and _K == K and _L == L, "operand shapes do not chain"
     _check_divisible(M, N, K, L, MI, NI, KI)
     D_frag = _first_gemm(A, B, batch, M, K, L, MI, NI, KI, in_dtype, acc_dtype)
-    cast = te.compute(
-        [batch, M // MI, L // NI, MI, NI], "relu" if relu else "cast", in_dtype, "relu" if relu else "cast",
-        lambda b, mo, lo, mi, li: [(D_frag, [b, mo, lo, mi, li])],
-        axis_names=["b", "mo", "lo", "mi", "li"],
-    )
-    E_frag = _second_gemm(cast, C, batch, M, L, N, N, MI, NI, KI, in_dtype, acc_dtype, pad_value=0)
+    requant = requant_scale is not None or scale is not None
+    if requant:
+        assert not relu, "a requantised middle result has no ReLU variant"
+        if scale is not None:
+            assert tuple(scale.shape) == (L,), f"scale must be [L]=[{L}], got {scale.shape}"
+        mid = te.compute(
+            [batch, M // MI, L // NI, MI, NI], "requant", in_dtype, "requant",
+            (lambda b, mo, lo, mi, li: [(D_frag, [b, mo, lo, mi, li]), (scale, [lo, li])]) if scale is not None
+            else (lambda b, mo, lo, mi, li: [(D_frag, [b, mo, lo, mi, li])]),
+            axis_names=["b", "mo", "lo", "mi", "li"],
+            attrs={"scale": None if scale is not None else float(requant_scale), "round": "nearest_even",
+                   "saturate": True},
+        )
+        out_dtype = out_dtype or acc_dtype
+    else:
+        mid = te.compute(
+            [batch, M // MI, L // NI, MI, NI], "relu" if relu else "cast", in_dtype, "relu" if relu else "cast",
+            lambda b, mo, lo, mi, li: [(D_frag, [b, mo, lo, mi, li])],
+            axis_names=["b", "mo", "lo", "mi", "li"],
+        )
+        out_dtype = out_dtype or in_dtype
+    E_frag = _second_gemm(mid, C, batch, M, L, N, N, MI, NI, KI, in_dtype, acc_dtype, pad_value=0)
     F = te.compute(
-        [batch, M, N], "F", in_dtype, "unpack_cast",
+        [batch, M, N], "F", out_dtype, "unpack_cast",
         lambda b, m, n: [(E_frag, [b, m, n])],
         axis_names=["b", "m", "n"],
     )
@@ -112,13 +136,16 @@ def BatchGemmGemmMMA(A, B, C, MI=16, NI=16, KI=16, in_dtype="float16", acc_dtype
 
 
 def BatchGemmGemm(batch=12, M=512, N=64, K=64, L=512, in_dtype="float16", acc_dtype="float32", relu=False,
-                  MI=16, NI=16, KI=16):
-    """Creates the placeholders too; returns ``([A, B, C], [F])`` like bmm_bmm_cuda.py:69-149."""
+                  MI=16, NI=16, KI=16, requant_scale=None, scale_tensor=False, out_dtype=None):
+    """Creates the placeholders too; returns ``([A, B, C], [F])`` like bmm_bmm_cuda.py:69-149.
+    int8 / int32: pass ``requant_scale`` (one scale for every intermediate column) or
+    ``scale_tensor=True`` (a fourth placeholder ``scale[L]``, float32: returns ``([A, B, C, scale], [F])``)."""
     A = te.placeholder([batch, M, K], name="A", dtype=in_dtype)
     B = te.placeholder([batch, K, L], name="B", dtype=in_dtype)
     C = te.placeholder([batch, L, N], name="C", dtype=in_dtype)
-    F = BatchGemmGemmMMA(A, B, C, MI, NI, KI, in_dtype, acc_dtype, relu)
-    return [A, B, C], [F]
+    scale = te.placeholder([L], name="scale", dtype="float32") if scale_tensor else None
+    F = BatchGemmGemmMMA(A, B, C, MI, NI, KI, in_dtype, acc_dtype, relu, requant_scale, scale, out_dtype)
+    return ([A, B, C, scale] if scale_tensor else [A, B, C]), [F]
 
 
 def BatchGemmSoftmaxGemm(batch=12, M=512, N=64, K=64, L=512, in_dtype="float16", acc_dtype="float32",

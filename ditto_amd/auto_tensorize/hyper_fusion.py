@@ -23,6 +23,10 @@ class FusionChoice:
     second_op: te.Operation
     ordered_iters: List[te.IterVar]
     attach_pos: int
+    # filled by build_fusion_choice (hyper_fusion.cc:2030-2078): the split factor and the index (position
+    # among the second op's spatial-then-reduce iteration variables) of every fused outer loop
+    secondOpOuterTilingFactors: List[int] = None
+    secondOpOuterIndices: List[int] = None
 
     def __str__(self):
         return "FusionChoice(axis=%s, pos=%d)" % (self.ordered_iters, self.attach_pos)
@@ -30,6 +34,51 @@ class FusionChoice:
 
 def fusion_choice(first_op, second_op, ordered_iters, attach_pos):
     return FusionChoice(first_op, second_op, list(ordered_iters), int(attach_pos))
+
+
+_DTYPE_BYTES = {"float32": 4, "float64": 8, "float16": 2, "bfloat16": 2, "int16": 2, "int32": 4, "int64": 8, "int8": 1}
+
+
+def build_fusion_choice(sfs, hw_param=None, dtype="float32", simple_mode=-1):
+    """The fusion choice for the two contractions of a serial fusion state whose tensorize axes
+    are registered (reference: hyper_fusion.py:271-295, hyper_fusion.cc:1974-2079).
+
+    The reference searches over tilings and loop orders of both ops with a cache-level cost model
+    (``simple_mode`` 0: full search, -1: pruned search, 1: the identity order) and returns the
+    second op's loops in the winning order followed by its tensorized loops, with ``attach_pos``
+    = the last loop the first op is computed under.  The gfx950 kernels fix tiling and order
+    themselves, so every mode returns the order all of the reference's own drivers choose by hand
+    (bmm_bmm_cuda.py:176 ``[b, m, n, rlo, mi, ni, rli], 3``; conv3x3_conv1x1_cuda.py:211
+    ``[b, no, p, mo, rlo, mi, ni, rli], 4``; conv1x1_conv3x3_cuda.py:228
+    ``[b, no, p, mo, rlo, mi, ni, rr, rs, rli], 4``): the spatial loops that are not tensorized,
+    the outermost reduce loop that is not tensorized, the tensorized spatial loops, the remaining
+    reduce loops, the tensorized reduce loop; the first op is attached under that outermost
+    reduce loop."""
+    if not getattr(sfs, "tensorize_axes", None):
+        raise ValueError("register the tensorize axes first (SerialFusionState.register_tensorize_axes)")
+    if dtype not in _DTYPE_BYTES:
+        raise ValueError("unknown dtype %s" % dtype)
+    if simple_mode not in (-1, 0, 1):
+        raise ValueError("simple_mode must be 1 (a pick without search), 0 (full search) or -1 (pruned search)")
+    op1, op2 = sfs.first_op, sfs.second_op
+    tens = sfs.tensorize_axes.get(op2, [])
+    if not tens:
+        raise ValueError("no tensorize axes registered for the second contraction %s" % op2.name)
+
+    def is_tens(iv):
+        return any(iv is t for t in tens)
+
+    spatial_nt = [iv for iv in op2.axis if not is_tens(iv)]
+    reduce_nt = [iv for iv in op2.reduce_axis if not is_tens(iv)]
+    ordered = (spatial_nt + reduce_nt[:1] + [iv for iv in op2.axis if is_tens(iv)] + reduce_nt[1:]
+               + [iv for iv in op2.reduce_axis if is_tens(iv)])
+    attach_pos = len(spatial_nt) + len(reduce_nt[:1]) - 1
+    if attach_pos < 0:
+        raise ValueError("no loop of %s is left to attach the first contraction under" % op2.name)
+    all_iters = op2.axis + op2.reduce_axis
+    outer = ordered[: attach_pos + 1]
+    return FusionChoice(op1, op2, ordered, attach_pos, [1] * len(outer),
+                        [next(i for i, v in enumerate(all_iters) if v is iv) for iv in outer])
 
 
 @dataclass
@@ -201,6 +250,10 @@ class ChainSchedule:
     relu_out: bool = False
     hw_param: HardwareParam = None
     tensorize_param: CUDATensorizeParam = None
+    requant_scale: float = 1.0       # inter_op "requant": the scale of every column ...
+    scale_tensor: bool = False       # ... unless a float32 scale[L] placeholder follows A, B, C
+    tile_variant: int = 0            # 0: the library's per-shape table; else the variant id to force
+    target: str = "hip"              # "cpu" only from tensorize_cpu / FusionContext.run, which nothing can build
 
 
 def _kinds(ops):
@@ -244,19 +297,70 @@ def _recognise(layer, state):
         return dict(kind="bmm_chain", inter_op="softmax", dims=dims, relu_out=False, in_dtype=A.dtype,
                     acc_dtype=first.output(0).dtype, out_dtype=out_t.dtype,
                     softmax_scale=state.inter_path[0].attrs.get("scale", 1.0))
-    if inter in (["cast"], ["relu"]) and epi == ["unpack_cast"]:
-        return dict(kind="bmm_chain", inter_op=inter[0], dims=dims, relu_out=False, in_dtype=A.dtype,
+    relu_out = epi == ["relu_cast"]  # an activation layer fused into the chain (chimera.graph_fusion)
+    if inter == ["requant"] and epi == ["unpack_cast"]:
+        req = state.inter_path[0]
+        if A.dtype != "int8" or first.output(0).dtype != "int32":
+            raise ValueError("a requantised middle result belongs to the int8 / int32 chain")
+        has_tensor = len(req.input_tensors) == 2
+        return dict(kind="bmm_chain", inter_op="requant", dims=dims, relu_out=False, in_dtype=A.dtype,
+                    acc_dtype="int32", out_dtype=out_t.dtype, softmax_scale=1.0,
+                    requant_scale=1.0 if has_tensor else float(req.attrs["scale"]), scale_tensor=has_tensor)
+    if inter in (["cast"], ["relu"]) and (epi == ["unpack_cast"] or relu_out):
+        if A.dtype == "int8":
+            raise NotImplementedError(
+                "the int8 chain is built with a requantised middle result (BatchGemmGemm(..., requant_scale=s)); "
+                "the wrapping astype(int8) of bmm_bmm_cuda.py:116 has no kernel here")
+        return dict(kind="bmm_chain", inter_op=inter[0], dims=dims, relu_out=relu_out, in_dtype=A.dtype,
                     acc_dtype=first.output(0).dtype, out_dtype=out_t.dtype, softmax_scale=1.0)
     raise ValueError("The fusion and tensorize decisions are not valid (inter path %s, epilogue %s)." % (inter, epi))
 
 
-def tensorize_hip(layer, state, hip_param=None, tensorize_param=None):
+def tensorize_hip(layer, state, hip_param=None, tensorize_param=None, tile_variant=0):
     """Bind a described chain to its gfx950 kernel family.  Raises ``ValueError`` for chains
-    the path does not cover, where the reference raises ``TVMError`` from a failed CHECK."""
+    the path does not cover, where the reference raises ``TVMError`` from a failed CHECK.
+    ``tile_variant`` forces a kernel variant (an id ``select_tile`` reports): the counterpart of
+    the explicit ``CUDATensorizeParam`` the reference's callers pass."""
     info = _recognise(layer, state)
-    return ChainSchedule(layer=layer, state=state, hw_param=hip_param, tensorize_param=tensorize_param, **info)
+    return ChainSchedule(layer=layer, state=state, hw_param=hip_param, tensorize_param=tensorize_param,
+                         tile_variant=int(tile_variant), **info)
 
 
 def tensorize_cuda(layer, state, cuda_param=None, tensorize_param=None):
     """Same entry point and argument list as the reference's (hyper_fusion.py:191-197)."""
     return tensorize_hip(layer, state, cuda_param, tensorize_param)
+
+
+
+@dataclass
+class CPUTensorizeParam:
+    """Loop tiling of the CPU fused nest (hyper_fusion.cc:609-642: per-op tiling factors and loop
+    orders chosen by ``buildCPUTensorizeParam``).  Kept as a record only: this build has no CPU
+    product path."""
+    firstOpTilingFactor: tuple = ()
+    firstOpLoopOrder: tuple = ()
+    secondOpTilingFactor: tuple = ()
+    secondOpLoopOrder: tuple = ()
+    parallelism: int = 1
+
+
+def build_cpu_tensorize_param(sfs, fusion_choice, hw_param, dtype):
+    """Identity tiling in the loop order of ``fusion_choice`` (reference: hyper_fusion.py:297-302)."""
+    if dtype not in _DTYPE_BYTES:
+        raise ValueError("unknown dtype %s" % dtype)
+    op1, op2 = sfs.first_op, sfs.second_op
+    n1, n2 = len(op1.axis + op1.reduce_axis), len(op2.axis + op2.reduce_axis)
+    all2 = op2.axis + op2.reduce_axis
+    order2 = tuple(next(i for i, v in enumerate(all2) if v is iv) for iv in fusion_choice.ordered_iters)
+    return CPUTensorizeParam((1,) * n1, tuple(range(n1)), (1,) * n2, order2,
+                             int(getattr(hw_param, "num_groups", 1) or 1))
+
+
+def tensorize_cpu(layer, state, cpu_param=None, tensorize_param=None):
+    """The reference lowers the chain to an x86 loop nest here (hyper_fusion.py:262-268,
+    hyper_fusion_cpu.cc:1553-1614).  This build is the gfx950 path only: the chain is recognised
+    (so descriptor errors surface as they do for the GPU flow) and a ``ChainSchedule`` marked for a
+    CPU target is returned, which ``ditto_amd.build`` refuses."""
+    sch = tensorize_hip(layer, state, cpu_param, None)
+    sch.target = "cpu"
+    return sch

@@ -42,7 +42,8 @@ class PackedIntrinsic:
 
     def __str__(self):
         return "PackedIntrinsic(load=%s; compute=%s; store=%s)" % (
-            [i.name for i in self.load_intrinsics], self.compute_intrinsic.name, self.store_intrinsic.name)
+            [i.name for i in self.load_intrinsics], self.compute_intrinsic.name,
+            self.store_intrinsic.name if self.store_intrinsic is not None else None)
 
 
 def packed_intrinsic(loads, compute, store, load_scopes, compute_scope, store_scope):
@@ -109,8 +110,8 @@ def intrinsic_match(target: te.Tensor, packed_intrin: PackedIntrinsic, restricti
         for ni in b_cands:
             for ki in k_cands:
                 if "SameRange" in restrictions:
-                    is_wmma = intr.name == "gemm"
-                    ok = ((mi.extent, ni.extent, ki.extent) == (intr.M, intr.N, intr.K)) if is_wmma else (
+                    is_mfma = intr.name.startswith("mfma_")  # wmma and CPU micro-kernel tiles match exactly
+                    ok = ((mi.extent, ni.extent, ki.extent) == (intr.M, intr.N, intr.K)) if not is_mfma else (
                         mi.extent % 16 == 0 and ni.extent % 16 == 0 and ki.extent % 16 == 0)
                     if not ok:
                         continue
@@ -118,3 +119,26 @@ def intrinsic_match(target: te.Tensor, packed_intrin: PackedIntrinsic, restricti
                 if "InnerMost" in restrictions:
                     return choices
     return choices
+
+
+def cpu_intrin(op, shape, isa, dtype, prefix=""):
+    """The CPU micro-kernel contract (reference: intrinsic.py:1675-1706): returns
+    ``(packed_intrinsic, code)``.  In the reference ``code`` is the C / assembly source of a 6 x 16
+    (AVX2) or 6 x 64 (AVX-512) register-tile kernel reached through ``call_extern("<prefix>_update")``
+    (:292-416, :646-674); here it is a one-line description, since this build has no CPU product
+    path -- the object only carries the tile shape through ``intrinsic_match`` / ``match_info``."""
+    if op not in ("gemm", "gemm_noreshape", "conv", "exp", "exp_noreshape"):
+        raise ValueError("unknown cpu intrinsic %r" % op)
+    if isa not in ("avx2", "avx512"):
+        raise ValueError("isa must be avx2 or avx512")
+    if dtype not in ("float32", "float64"):
+        raise ValueError("the CPU micro-kernels are fp32 / fp64 (intrinsic.py:283-291)")
+    if op in ("exp", "exp_noreshape"):
+        M, N = (int(x) for x in shape)
+        K = 1
+    else:
+        M, N, K = (int(x) for x in shape[:3])
+    compute = TensorIntrin("%s_update" % (prefix or op), M, N, K, dtype, dtype, "global")
+    code = "// %s micro-kernel %s (%d x %d x %d, %s, %s): described, not generated" % (op, compute.name, M, N, K,
+                                                                                     isa, dtype)
+    return packed_intrinsic([], compute, None, ["global", "global"], "global", "global"), code

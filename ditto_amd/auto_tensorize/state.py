@@ -26,8 +26,23 @@ class SerialFusionState:
         return sum(1 for op in self.ops if self.patterns[op] == pattern)
 
     def register_tensorize_axes(self, axes):
-        """``axes``: {op: [iter vars]} handed to the micro-kernel (bmm_bmm_cpu.py:165-170)."""
-        self.tensorize_axes.update(axes)
+        """``axes``: the iteration variables handed to the intrinsics, as one flat list over both
+        contractions (state.py:16, bmm_bmm_cpu.py:194-196, test_hyper_fusion.py:866-868) or as
+        ``{op: [iter vars]}``.  Every variable must belong to one of the two contractions."""
+        if isinstance(axes, dict):
+            flat = [(op, iv) for op, ivs in axes.items() for iv in ivs]
+        else:
+            flat = []
+            for iv in axes:
+                owner = [op for op in (self.first_op, self.second_op)
+                         if any(iv is v for v in op.axis + op.reduce_axis)]
+                if not owner:
+                    raise ValueError("iter var %s belongs to neither contraction of the layer" % iv.name)
+                flat.append((owner[0], iv))
+        for op, iv in flat:
+            lst = self.tensorize_axes.setdefault(op, [])
+            if not any(iv is v for v in lst):
+                lst.append(iv)
 
 
 def build_serial_fusion_state(layer):
@@ -46,3 +61,69 @@ def validate(state):
                        "should be eliminated by the frontend.\n Did you forget to use"
                        "Ditto's graph frontend?")
     return True, ""
+
+
+class FusionContext:
+    """What ``build_fusion_context`` returns in the reference: the ranked candidate schedules of the
+    CPU fused nest (state.py:34-78, hyper_fusion.cc:2182-2247).  Here a single candidate: the
+    fusion the layer's ``TensorizeHyperFusionState`` describes.  ``run`` yields a schedule marked
+    for a CPU target, which ``ditto_amd.build`` refuses -- this build has no CPU product path."""
+
+    def __init__(self, sfs, layer, state, path, hw_param, searchType, mode, dtype):
+        from .hyper_fusion import _DTYPE_BYTES
+
+        if searchType not in ("normal", "stochastic"):
+            raise ValueError("searchType must be normal or stochastic")
+        if mode not in ("survey", "best", "test"):
+            raise ValueError("mode must be survey, best or test")
+        if dtype not in _DTYPE_BYTES:
+            raise ValueError("unknown dtype %s" % dtype)
+        self.sfs, self.layer, self.state, self.path = sfs, layer, state, path
+        self.hw_param, self.searchType, self.mode, self.dtype = hw_param, searchType, mode, dtype
+        self.bytePerEle = _DTYPE_BYTES[dtype]
+        self.size = 1
+
+    def _check(self, i):
+        if not 0 <= i < self.size:
+            raise IndexError("fusion context holds %d candidate(s)" % self.size)
+
+    def run(self, i, sch=None, verbose=False):
+        from .hyper_fusion import tensorize_cpu
+
+        self._check(i)
+        out = tensorize_cpu(self.layer, self.state, self.hw_param, None)
+        if verbose:
+            print(self.state.summary(verbose=True))
+        return out
+
+    def getComputation(self, i):
+        """Multiply-accumulates of the two contractions."""
+        self._check(i)
+        total = 0
+        for op in (self.sfs.first_op, self.sfs.second_op):
+            n = 1
+            for iv in op.axis + op.reduce_axis:
+                n *= iv.extent
+            total += n
+        return total
+
+    def getFusionLevel(self, i):
+        """Index of the smallest cache level that holds the first contraction's tile under the fused
+        loops (one iteration of them), -1 if none does or the hardware record lists no caches."""
+        self._check(i)
+        fused = self.state.fused_spatial_outer_iters
+        op1 = self.sfs.first_op
+        elems = 1
+        for iv in op1.axis:
+            if not any(iv.name == f.name and iv.extent == f.extent for f in fused):
+                elems *= iv.extent
+        sizes = list(getattr(self.hw_param, "cacheSizes", None) or [])
+        for level, cap in enumerate(sizes):
+            if elems * self.bytePerEle <= cap:
+                return level
+        return -1
+
+
+def build_fusion_context(sfs, layer, state, path, hw_param, searchType="normal", mode="best", dtype="float32"):
+    """Same argument list as the reference's (state.py:34-51)."""
+    return FusionContext(sfs, layer, state, path, hw_param, searchType, mode, dtype)

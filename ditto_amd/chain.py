@@ -57,7 +57,8 @@ def _split_levels(t, name):
     return _as3d(t, name), 1, 0
 
 
-def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=1.0, tile_variant=0):
+def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=1.0, tile_variant=0,
+                   relu_out=False):
     """Fill a ``ditto_bmm_chain_desc`` from tensors A[b,M,K], B[b,K,L], C[b,L,N], F[b,M,N].
 
     B may be a transposed view of a ``[b, L, K]`` tensor (stride 1 along K); it is then
@@ -110,7 +111,7 @@ def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale
     d.softmax_scale = float(softmax_scale)
     d.requant_scale = float(requant_scale)
     d.tile_variant = int(tile_variant)
-    d.reserved = 0
+    d.relu_out = int(bool(relu_out))
     return d
 
 
@@ -126,7 +127,7 @@ def select_tile(desc):
 
 
 def run_bmm_chain(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=1.0, aux=None, desc=None,
-                  tile_variant=0):
+                  tile_variant=0, relu_out=False):
     """F[b] = epilogue(inter(A[b] . B[b]) . C[b]) as ONE kernel on the current stream.
 
     ``aux``: for ``inter_op="requant"`` an fp32 tensor of L per-column scales (``None``: use
@@ -134,7 +135,7 @@ def run_bmm_chain(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=
     lib = _lib.load()
     dev = _check_device(A, B, C, F)
     if desc is None:
-        desc = bmm_chain_desc(A, B, C, F, inter_op, softmax_scale, requant_scale, tile_variant)
+        desc = bmm_chain_desc(A, B, C, F, inter_op, softmax_scale, requant_scale, tile_variant, relu_out)
     aux_ptr = None
     if aux is not None:
         _check_device(A, aux)
@@ -186,17 +187,19 @@ def conv_chain_desc(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op
     return d
 
 
-_WORKSPACES = {}
+_WORKSPACES = {}  # device -> every scratch buffer handed out so far, the current (largest) one last
 
 
 def _workspace(dev, nbytes):
-    """A per-device scratch buffer (uint8) of at least ``nbytes``; the library writes the repacked
-    first-convolution weights there on every call, so calls on one device must not overlap."""
-    buf = _WORKSPACES.get(dev)
-    if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
-        _WORKSPACES[dev] = buf
-    return buf
+    """The shared per-device scratch buffer (uint8) of at least ``nbytes`` that ``run_conv_chain`` uses
+    when its caller passes none; the library writes the repacked first-convolution weights there on
+    every call, so such calls on one device must not overlap.  A buffer that has been handed out is
+    never freed: a HIP graph that captured a call keeps a valid pointer when a later, larger request
+    makes a new buffer current."""
+    bufs = _WORKSPACES.setdefault(dev, [])
+    if not bufs or bufs[-1].numel() < nbytes:
+        bufs.append(torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev))
+    return bufs[-1]
 
 
 def conv_chain_workspace_bytes(desc):

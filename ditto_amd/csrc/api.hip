@@ -65,7 +65,9 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
   if (d->abi_version != DITTO_CHAIN_ABI_VERSION)
     return fail(DITTO_EINVAL, "descriptor abi_version %d, library %d", d->abi_version,
                 DITTO_CHAIN_ABI_VERSION);
-  if (d->reserved != 0) return fail(DITTO_EINVAL, "descriptor field `reserved` must be 0");
+  if (d->relu_out != 0 && d->relu_out != 1) return fail(DITTO_EINVAL, "relu_out must be 0 or 1");
+  if (d->relu_out && (d->in_dtype == DITTO_I8 || d->inter_op == DITTO_INTER_SOFTMAX))
+    return fail(DITTO_EUNSUPPORTED, "relu_out is implemented for the cast / relu chains on fp16, bf16 and fp32");
   if (d->tile_variant < 0) return fail(DITTO_EINVAL, "tile_variant must be 0 or a variant id");
   if (d->batch_inner < 0 || (d->batch_inner > 0 && d->batch > 0 && d->batch % d->batch_inner != 0))
     return fail(DITTO_EINVAL, "batch_inner must be 0 or divide batch");
@@ -631,6 +633,7 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     args.mblocks = (int)((d->M + plan.tile.block_m - 1) / plan.tile.block_m);
     args.scale_log2 = d->softmax_scale * 1.4426950408889634f;
     args.relu = d->inter_op == DITTO_INTER_RELU;
+    args.relu_out = d->relu_out;
     args.out_f32 = d->out_dtype == DITTO_F32;
     const bool kl = d->b_layout == DITTO_B_KL;
     const bool sm = d->inter_op == DITTO_INTER_SOFTMAX;
@@ -666,6 +669,7 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     args.mblocks = (int)((d->M + 31) / 32);
     args.b_lk = d->b_layout == DITTO_B_LK;
     args.relu = d->inter_op == DITTO_INTER_RELU;
+    args.relu_out = d->relu_out;
     hipError_t e = ditto::launch_gemm_chain_f32(args, st);
     if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
     return DITTO_OK;

@@ -42,6 +42,7 @@ struct BmmChainArgs {
   int mblocks;       // workgroups per batch entry
   float scale_log2;  // softmax: scale * log2(e)
   int relu;          // inter = relu instead of cast (non-softmax kernels)
+  int relu_out;      // ReLU on the second accumulator before the final cast (non-softmax kernels)
   int out_f32;       // write F as fp32 instead of T
 };
 
@@ -444,8 +445,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       for (int q4 = 0; q4 < 4; ++q4) {
         const int n = 32 * t + 8 * q4 + 4 * g;
         if (n >= N) continue;
-        const float v0 = o[t][j][4 * q4 + 0] * inv, v1 = o[t][j][4 * q4 + 1] * inv;
-        const float v2 = o[t][j][4 * q4 + 2] * inv, v3 = o[t][j][4 * q4 + 3] * inv;
+        float v0 = o[t][j][4 * q4 + 0] * inv, v1 = o[t][j][4 * q4 + 1] * inv;
+        float v2 = o[t][j][4 * q4 + 2] * inv, v3 = o[t][j][4 * q4 + 3] * inv;
+        if (INTER != kInterSoftmax && p.relu_out) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); v2 = fmaxf(v2, 0.f); v3 = fmaxf(v3, 0.f); }
         const long long off = zo * p.f_bs2 + zi * p.f_bs + (long long)row * p.f_rs + n;
         if (p.out_f32) {
           f32x4 w = {v0, v1, v2, v3};

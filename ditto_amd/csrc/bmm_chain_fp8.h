@@ -383,8 +383,9 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
       for (int q4 = 0; q4 < 4; ++q4) {
         const int n = 32 * t + 8 * q4 + 4 * g;
         if (n >= N) continue;
-        const float v0 = o[t][4 * q4 + 0] * inv, v1 = o[t][4 * q4 + 1] * inv;
-        const float v2 = o[t][4 * q4 + 2] * inv, v3 = o[t][4 * q4 + 3] * inv;
+        float v0 = o[t][4 * q4 + 0] * inv, v1 = o[t][4 * q4 + 1] * inv;
+        float v2 = o[t][4 * q4 + 2] * inv, v3 = o[t][4 * q4 + 3] * inv;
+        if (INTER != kInterSoftmax && p.relu_out) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); v2 = fmaxf(v2, 0.f); v3 = fmaxf(v3, 0.f); }
         const long long off = zo * p.f_bs2 + zi * p.f_bs + (long long)row * p.f_rs + n;
         if (p.out_f32) {
           f32x4 w = {v0, v1, v2, v3};

@@ -15,6 +15,7 @@ struct F32ChainArgs {
   int mblocks;  // workgroups (32 rows each) per batch entry
   int b_lk;     // B stored [L][K]
   int relu;
+  int relu_out;  // ReLU on the output
 };
 
 int f32_chain_lds_bytes_host(int K, int N);

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void gemm_chain_f32_kernel(F32ChainArgs p) {
 #pragma unroll
     for (int i = 0; i < kMaxD / 8; ++i) {
       const int n = c8 + 8 * i;
-      if (n < N) Fg[(long long)(m0 + r) * p.f_rs + n] = acc[i];
+      if (n < N) Fg[(long long)(m0 + r) * p.f_rs + n] = p.relu_out ? fmaxf(acc[i], 0.f) : acc[i];
     }
   }
 }

@@ -12,8 +12,11 @@ shapes = common.BMM_SHAPES
 
 def main(batch=12, M=512, N=64, K=64, L=512, in_dtype="float16", acc_dtype="float32", sm="gfx950",
          only_once=False):
+    # int8 / int32: the middle result is requantised (scale 2^-10, round to nearest even, saturate)
+    # where the reference's chain wraps with astype("int8") (bmm_bmm_cuda.py:116)
+    requant = common.INT8_REQUANT_SCALE if in_dtype == "int8" else None
     ins, outs = ac.nn.functional.BatchGemmGemm(batch=batch, M=M, N=N, K=K, L=L, in_dtype=in_dtype,
-                                               acc_dtype=acc_dtype)
+                                               acc_dtype=acc_dtype, requant_scale=requant)
     try:
         layer, sch = common.describe_bmm_chain(ins, outs, in_dtype, acc_dtype, sm)
     except Exception as error:
@@ -29,7 +32,7 @@ if __name__ == "__main__":
     if args.ai:
         for ss in shapes[args.begin: args.begin + args.num]:
             print(ss, *common.cal_ai(*ss))
-    elif common.check_dtypes(args):
+    elif common.check_dtypes(args, int8_ok=True):
         costs = []
         for ss in shapes[args.begin: args.begin + args.num]:
             B, M, N, K, L = ss

@@ -72,7 +72,7 @@ def cal_ai(B, M, N, K, L):
 def describe_bmm_chain(ins, outs, in_dtype, acc_dtype, sm):
     """Steps 2-8 of the reference driver: fusion choice, intrinsic match, layer, hyper-fusion
     state, hardware table, tensorize parameters, tensorize."""
-    A, B, C = ins
+    A, B, C = ins[:3]  # (a requantised int8 chain may carry a fourth input, the scale vector)
     (F,) = outs
     E_frag = F.op.input_tensors[0]
     mid, C_ext = E_frag.op.input_tensors
@@ -86,7 +86,7 @@ def describe_bmm_chain(ins, outs, in_dtype, acc_dtype, sm):
     second_packed = at.cuda_wmma(M=16, N=16, K=16, in_dtype=in_dtype, out_dtype=acc_dtype, scope="global")
     second_match_info = at.match_info(at.intrinsic_match(E_frag, second_packed, ["InnerMost", "SameRange"])[0],
                                       second_packed)
-    layer = ac.layer([F.op], inputs=[A, B, C])
+    layer = ac.layer([F.op], inputs=list(ins))
     state = at.tensorize_hyper_fusion_state(layer, fuse_choice,
                                             {D_frag.op: first_match_info, E_frag.op: second_match_info})
     device = hw.query_hw_param(DEVICES[sm])
@@ -101,13 +101,47 @@ def describe_bmm_chain(ins, outs, in_dtype, acc_dtype, sm):
     return layer, sch
 
 
+def describe_layer(layer, sm="gfx950", tile_variant=0):
+    """Any chain layer (GEMM or conv chain, e.g. one ``chimera.graph_fusion`` produced) -> its schedule, by the
+    flow of python_test/auto_tensorize/test_hyper_fusion.py:833-880: serial fusion state, validate, intrinsic
+    match, ``register_tensorize_axes``, ``build_fusion_choice``, hyper-fusion state, tensorize."""
+    sfs = at.build_serial_fusion_state(layer)
+    ok, why = at.validate(sfs)
+    if not ok:
+        raise ValueError(why)
+    op1, op2 = sfs.first_op, sfs.second_op
+    in_dtype, acc_dtype = layer.inputs[0].dtype, op1.output(0).dtype
+    if op1.attrs.get("conv"):
+        mfma = at.hip_mfma(32, 32, 32 if in_dtype == "int8" else 16, in_dtype, acc_dtype)
+        # pixel x output channel x input channel
+        infos = {op: at.match_info([op.axis[3], op.axis[1], op.reduce_axis[0]], mfma) for op in (op1, op2)}
+    else:
+        infos = {}
+        for op, scope in ((op1, "shared"), (op2, "global")):
+            packed = at.cuda_wmma(M=16, N=16, K=16, in_dtype=in_dtype, out_dtype=acc_dtype, scope=scope)
+            infos[op] = at.match_info(at.intrinsic_match(op.output(0), packed, ["InnerMost", "SameRange"])[0], packed)
+    sfs.register_tensorize_axes([iv for mi in infos.values() for iv in mi.axis])
+    device = hw.query_hw_param(DEVICES[sm])
+    fuse_choice = at.build_fusion_choice(sfs, hw_param=device, dtype=acc_dtype, simple_mode=-1)
+    state = at.tensorize_hyper_fusion_state(layer, fuse_choice, infos)
+    return at.tensorize_hip(layer, state, device, at.cuda_tensorize_param(), tile_variant=tile_variant)
+
+
 def random_args(layer, in_dtype, n_inputs, scale=1.0, device="cuda:0"):
     """uniform(-1, 1) tensors for every schedule tensor, as the reference drivers create them."""
     import torch
 
-    dt = {"float16": torch.float16, "bfloat16": torch.bfloat16, "float32": torch.float32}[in_dtype]
+    dts = {"float16": torch.float16, "bfloat16": torch.bfloat16, "float32": torch.float32, "int8": torch.int8,
+           "int32": torch.int32}
     args = []
     for i, t in enumerate(layer.schedule_tensors):
+        dt = dts[t.dtype]
+        if dt == torch.int8:  # uniform integers in [-127, 127]
+            args.append(torch.randint(-127, 128, tuple(t.shape), dtype=torch.int8, device=device))
+            continue
+        if dt == torch.int32:
+            args.append(torch.zeros(tuple(t.shape), dtype=torch.int32, device=device))
+            continue
         x = (torch.rand(*t.shape, device=device) * 2 - 1)
         if i < n_inputs:
             x = x * scale
@@ -149,11 +183,14 @@ def base_parser(example, n_shapes, with_ai=True):
 
 
 # (sm, in_dtype, acc_dtype) combinations with a kernel on this device
-SUPPORTED_DTYPES = {("gfx950", "float16", "float32"), ("gfx950", "bfloat16", "float32")}
+# (the int8 / int32 row is the reference's ("80", "int8", "int32"), bmm_bmm_cuda.py:273-288; GEMM chain only)
+SUPPORTED_DTYPES = {("gfx950", "float16", "float32"), ("gfx950", "bfloat16", "float32"), ("gfx950", "int8", "int32")}
+# the requantisation scale the int8 driver rows use for the middle result (2^-10 for every column)
+INT8_REQUANT_SCALE = 2.0 ** -10
 
 
-def check_dtypes(args):
-    ok = (args.sm, args.in_dtype, args.acc_dtype) in SUPPORTED_DTYPES
+def check_dtypes(args, int8_ok=False):
+    ok = (args.sm, args.in_dtype, args.acc_dtype) in SUPPORTED_DTYPES and (int8_ok or args.in_dtype != "int8")
     if not ok:
         print(f"Data type not supported: sm_{args.sm}, in_dtype={args.in_dtype}, out_dtype={args.acc_dtype}.")
     return ok

@@ -45,8 +45,11 @@ class Graph:
 
 
 class GraphEngine:
-    def __init__(self, graph, built_mods, dev="cuda:0"):
+    def __init__(self, graph, built_mods, dev="cuda:0", prepare_weights=True):
         self.graph = graph
+        # conv chain layers with weights: repack the weights once per compile (set_weight compiles
+        # again) instead of on every run; weights changed in place afterwards need a new compile
+        self.prepare_weights = prepare_weights
         self.built_mods = built_mods  # {layer fingerprint: callable f(*inputs, *weights, *outputs)}
         self.dev = torch.device(dev)
         self._init = False
@@ -105,6 +108,10 @@ class GraphEngine:
             if key not in self.built_mods:
                 raise KeyError("no built function for layer %s" % layer.name)
             func = self.built_mods[key]
+            if (self.prepare_weights and len(layer.weights) == 2 and len(layer.inputs) == 1
+                    and getattr(getattr(func, "sch", None), "kind", None) == "conv_chain"):
+                # fixed weights: repack them once, here, into a workspace this layer owns
+                func = func.specialize(*self.weight_buffer[li])
             args = [*self.input_buffer[li], *self.weight_buffer[li], *self.output_buffer[li]]
             self._to_exe.append((func, args))
 

@@ -88,7 +88,9 @@ typedef struct ditto_bmm_chain_desc {
                             `ditto_tile_param.variant` id to force (the counterpart of passing
                             an explicit CUDATensorizeParam, hyper_fusion.cc:586-607);
                             DITTO_EINVAL if that variant cannot run the shape              */
-  int32_t reserved;      /* must be 0 */
+  int32_t relu_out;      /* 1: ReLU on the second accumulator before the final cast (an activation layer
+                            fused into the chain, python/ditto/chimera/graph_fusion.py:4-52); cast / relu
+                            chains on fp16, bf16, fp32; else 0 */
   /* Two-level batch (fp16/bf16 chains): batch entry z = zo * batch_inner + zi lives at
    * zo * x_batch_stride_outer + zi * x_batch_stride.  This is how an attention caller hands
    * over [batch, heads] without the reshape/transpose copies of

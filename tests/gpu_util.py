@@ -15,3 +15,9 @@ def errors(got, want):
     want = np.asarray(want, dtype=np.float64)
     d = got - want
     return float(np.abs(d).max()), float(np.linalg.norm(d) / max(np.linalg.norm(want), 1e-30))
+
+
+def report(name, mx, rel):
+    """Print the measured errors of a parity case (``pytest -s`` shows them; the figures recorded for
+    the full-size configurations come from these lines)."""
+    print("PARITY %s: max-abs %.3e rel-L2 %.3e" % (name, mx, rel), flush=True)

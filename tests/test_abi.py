@@ -79,7 +79,7 @@ def test_select_tile_and_validation_without_gpu():
         assert tile.lds_bytes <= 160 * 1024
     assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(tile_variant=1288)), ctypes.byref(tile)) == _lib.EINVAL
     assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(tile_variant=643)), ctypes.byref(tile)) == _lib.EINVAL
-    assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(reserved=1)), ctypes.byref(tile)) == _lib.EINVAL
+    assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(relu_out=2)), ctypes.byref(tile)) == _lib.EINVAL
     # the long-sequence configuration picks the 128-wide head tile
     big = _desc(in_dtype=_lib.BF16, out_dtype=_lib.BF16, batch=64, M=4096, L=4096, K=128, N=128,
                 a_row_stride=128, b_row_stride=128, c_row_stride=128, f_row_stride=128,

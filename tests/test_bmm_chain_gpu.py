@@ -5,21 +5,25 @@ the fp32/fp64 closed form on identical seeded inputs.  bf16 carries 8 significan
 rounding the softmax probabilities (as the reference does: ``exp(...).astype(in_dtype)``,
 bmm_chain.py:63-70) or the output to bf16 alone costs about 1.6e-3 rel-L2; the bf16 cases
 therefore assert 1e-3 where no bf16 rounding of P is on the path (cast chains with fp32
-output against the checker that rounds the intermediate the same way) and the quantisation
-bound 3e-3 otherwise, always with max-abs-err <= 1e-2.
+output against the checker that rounds the intermediate the same way) and the measured
+quantisation figure + 10 % otherwise, always with max-abs-err <= 1e-2.
 """
 import numpy as np
 import pytest
 import torch
 
 from ditto_amd import chain
-from tests.gpu_util import errors, to_dev, TORCH_DTYPES
+from tests.gpu_util import errors, report, to_dev, TORCH_DTYPES
 
 pytestmark = pytest.mark.gpu
 
 MAX_ABS = 1e-2
 REL_L2 = 1e-3
-REL_L2_BF16_QUANT = 3e-3
+# bf16 softmax chains (probabilities and output both rounded to bf16): the largest rel-L2 any case of this
+# file reaches is 2.36e-3 (1 x 300 x 128 x 128 x 712; the comment above the long-sequence test derives the
+# figure from the rounding floor); bound = that + 10 %.  bf16 cast / relu chains meet the stated 1e-3
+# against the checker that rounds where they round (measured: at most 1.1e-4).
+REL_L2_BF16_QUANT = 2.6e-3
 
 
 def variants(K, N):
@@ -68,6 +72,8 @@ def test_softmax_chain_vs_oracle(oracle, shape, dtype, b_layout):
             got = run_chain(A, B, C, dtype, "softmax", scale, b_layout, out_dtype, variant)
             assert np.isfinite(got).all(), variant
             mx, rel = errors(got, want)
+            if dtype == "bfloat16":
+                report("softmax bf16 %s %s variant %d out %s" % (shape, b_layout, variant, out_dtype), mx, rel)
             assert mx <= MAX_ABS, (variant, mx, rel)
             assert rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (variant, mx, rel)
 
@@ -100,9 +106,11 @@ def test_cast_chain_vs_oracle(oracle, shape, dtype, inter):
             assert mx <= MAX_ABS and rel <= REL_L2, (variant, b_layout, mx, rel)
             got = run_chain(A, B, C, dtype, inter, 1.0, b_layout, None, variant)
             mx, rel = errors(got, want)
+            if dtype == "bfloat16":
+                report("%s bf16 %s %s variant %d" % (inter, shape, b_layout, variant), mx, rel)
             # one bf16 ulp at |x| ~ 4 is 3e-2
             assert mx <= (MAX_ABS if dtype == "float16" else 4e-2), (variant, b_layout, mx, rel)
-            assert rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (variant, b_layout, mx, rel)
+            assert rel <= REL_L2, (variant, b_layout, mx, rel)
             # and the narrow output is the rounding of the fp32 output (same kernel, cast at the end)
             assert np.array_equal(got, oracle.np_round_to(got32, dtype)), (variant, b_layout)
 
@@ -184,7 +192,63 @@ def test_attention_full_size_fp16_heads(oracle):
     for variant in variants(K, N):
         got = run_chain(A, B, C, "float16", "softmax", 0.125, "LK", None, variant)
         mx, rel = errors(got, want)
+        report("attention fp16 96 x 512 x 64, variant %d" % variant, mx, rel)
         assert mx <= MAX_ABS and rel <= REL_L2, (variant, mx, rel)
+
+
+# Measured on the long-sequence configuration (64 heads of 4096 x 128, N(0,1) inputs, scale 1/sqrt(128)),
+# the same for the three kernel variants to two digits: bf16 rel-L2 2.33e-3 .. 2.35e-3 (max-abs 3.9e-4 ..
+# 4.9e-4), fp16 rel-L2 2.87e-4 .. 2.95e-4 (max-abs 4.7e-5 .. 7.0e-5).  The rel-L2 bounds are the largest
+# measured figure + 10 %; max-abs, a maximum over a million outputs, gets twice the largest figure.
+# The bf16 figure is rounding, not the online softmax: rounding N(0,1) data to bf16 costs rel-L2 1.66e-3 by
+# itself (tests/test_oracle.py::test_rounding_floor_of_the_16_bit_types), the chain rounds both the
+# probabilities and the output, and 1.66e-3 * sqrt(2) = 2.35e-3.  The fp16 run of the same shape holds the
+# online softmax itself, 64 steps and their rescales per row, to the stated 1e-3.
+MAX_ABS_BF16_LONG, REL_L2_BF16_LONG = 1.0e-3, 2.6e-3
+MAX_ABS_FP16_LONG, REL_L2_FP16_LONG = 1.4e-4, 3.25e-4
+
+
+@pytest.mark.parametrize("variant", [0, 1282, 1288])
+def test_attention_full_size_fp16_long_sequence(oracle, variant):
+    # the long-sequence shape in fp16, where the stated bar (1e-2 / 1e-3) is reachable: 64 online-softmax
+    # steps per row, every variant; three whole heads and a row block of every head against the closed form
+    batch, S, d = 64, 4096, 128
+    scale = d ** -0.5
+    dev = "cuda:0"
+    g = torch.Generator(device="cpu").manual_seed(34)
+    q = torch.randn(batch, S, d, generator=g).to(torch.float16)
+    k = torch.randn(batch, S, d, generator=g).to(torch.float16)
+    v = torch.randn(batch, S, d, generator=g).to(torch.float16)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    out = torch.full((batch, S, d), float("nan"), device=dev, dtype=torch.float16)
+    chain.run_bmm_chain(qd, kd.transpose(1, 2), vd, out, "softmax", scale, tile_variant=variant)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    qn, kn, vn = q.float().numpy(), k.float().numpy(), v.float().numpy()
+    for h in (0, 17, 63):
+        want = oracle.bmm_chain_f64(qn[h:h + 1], np.ascontiguousarray(kn[h:h + 1].transpose(0, 2, 1)), vn[h:h + 1],
+                                    inter="softmax", scale=scale)
+        mx, rel = errors(got[h:h + 1], want)
+        report("attention fp16 64 x 4096 x 128, variant %d, head %d" % (variant, h), mx, rel)
+        assert mx <= MAX_ABS and rel <= REL_L2, (h, mx, rel)                      # the stated bar
+        assert mx <= MAX_ABS_FP16_LONG and rel <= REL_L2_FP16_LONG, (h, mx, rel)  # measured + 10 %
+    rows = slice(3000, 3032)
+    want = oracle.bmm_chain_f64(np.ascontiguousarray(qn[:, rows]), np.ascontiguousarray(kn.transpose(0, 2, 1)), vn,
+                                inter="softmax", scale=scale)
+    mx, rel = errors(got[:, rows], want)
+    report("attention fp16 64 x 4096 x 128, variant %d, rows 3000-3031 of every head" % variant, mx, rel)
+    assert mx <= MAX_ABS_FP16_LONG and rel <= REL_L2_FP16_LONG, (mx, rel)
+    # scores shifted far from zero: keys scaled up make row maxima of +-40 and more in the exponent, so
+    # the running maximum is raised many times along a row
+    big = (kd.float() * 6.0).to(torch.float16)
+    chain.run_bmm_chain(qd[:2], big[:2].transpose(1, 2), vd[:2], out[:2], "softmax", scale, tile_variant=variant)
+    torch.cuda.synchronize()
+    want = oracle.bmm_chain_f64(qn[:2, :256], np.ascontiguousarray(big[:2].float().cpu().numpy().transpose(0, 2, 1)),
+                                vn[:2], inter="softmax", scale=scale)
+    mx, rel = errors(out[:2, :256].float().cpu().numpy(), want)
+    report("attention fp16 2 x 4096 x 128 with keys x 6, variant %d" % variant, mx, rel)
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
 
 
 @pytest.mark.parametrize("variant", [0, 1282, 1288])
@@ -210,12 +274,14 @@ def test_attention_full_size_bf16_long_sequence(oracle, variant):
         want = oracle.bmm_chain_f64(qn[h:h + 1], np.ascontiguousarray(kn[h:h + 1].transpose(0, 2, 1)), vn[h:h + 1],
                                     inter="softmax", scale=scale)
         mx, rel = errors(got[h:h + 1], want)
-        assert mx <= MAX_ABS and rel <= REL_L2_BF16_QUANT, (h, mx, rel)
+        report("attention bf16 64 x 4096 x 128, variant %d, head %d" % (variant, h), mx, rel)
+        assert mx <= MAX_ABS_BF16_LONG and rel <= REL_L2_BF16_LONG, (h, mx, rel)
     rows = slice(1000, 1032)  # one row block of every head (straddles no tile boundary specially)
     want = oracle.bmm_chain_f64(np.ascontiguousarray(qn[:, rows]), np.ascontiguousarray(kn.transpose(0, 2, 1)), vn,
                                 inter="softmax", scale=scale)
     mx, rel = errors(got[:, rows], want)
-    assert mx <= MAX_ABS and rel <= REL_L2_BF16_QUANT, (mx, rel)
+    report("attention bf16 64 x 4096 x 128, variant %d, rows 1000-1031 of every head" % variant, mx, rel)
+    assert mx <= MAX_ABS_BF16_LONG and rel <= REL_L2_BF16_LONG, (mx, rel)
     # values all ones -> output all ones (the normaliser is the sum of what was multiplied)
     ones = torch.ones_like(vd)
     chain.run_bmm_chain(qd, kd.transpose(1, 2), ones, out, "softmax", scale, tile_variant=variant)
@@ -263,17 +329,19 @@ def test_gemm_chain_full_size_bf16(oracle, variant):
     for h in (0, 40, 63):
         want = oracle.bmm_chain_f64(an[h:h + 1], bn[h:h + 1], cn[h:h + 1], inter="cast", round_mid="bfloat16")
         mx, rel = errors(got[h:h + 1], oracle.np_round_to(want.astype(np.float32), "bfloat16"))
-        assert rel <= REL_L2_BF16_QUANT and mx <= 4e-2, (h, mx, rel)  # one bf16 ulp at |x| ~ 4 is 3e-2
+        report("GEMM chain bf16 64 x 4096 x 128, variant %d, head %d" % (variant, h), mx, rel)
+        assert rel <= REL_L2 and mx <= 4e-2, (h, mx, rel)  # one bf16 ulp at |x| ~ 4 is 3e-2
     rows = slice(3000, 3040)
     want = oracle.bmm_chain_f64(np.ascontiguousarray(an[:, rows]), bn, cn, inter="cast", round_mid="bfloat16")
     mx, rel = errors(got[:, rows], oracle.np_round_to(want.astype(np.float32), "bfloat16"))
-    assert rel <= REL_L2_BF16_QUANT and mx <= 4e-2, (mx, rel)
+    assert rel <= REL_L2 and mx <= 4e-2, (mx, rel)
     # B = [I | 0]: the middle result is A itself (exact in bf16), so F = A . C[:K] -- one GEMM
     eye = torch.zeros(batch, K, L, dtype=torch.bfloat16, device=dev)
     eye[:, torch.arange(K), torch.arange(K)] = 1
     chain.run_bmm_chain(ad, eye, cd, out, "cast", 1.0, tile_variant=variant)
     torch.cuda.synchronize()
     want_d = torch.bmm(ad.float(), cd[:, :K].float())
+    # (against an unrounded fp32 product: the bf16 rounding of the output alone is 1.66e-3)
     assert float((out.float() - want_d).norm() / want_d.norm()) <= REL_L2_BF16_QUANT
     # rows of A permuted -> rows of F permuted, bit for bit (no cross-row state in this chain)
     perm = torch.randperm(M, generator=g).to(dev)
@@ -306,6 +374,8 @@ def test_multi_head_attention_module(oracle, dtype, cfg):
     want = oracle.bmm_chain_f64(q, np.ascontiguousarray(k.transpose(0, 2, 1)), v, inter="softmax", scale=d ** -0.5)
     want = want.reshape(batch, heads, M, d).transpose(0, 2, 1, 3).reshape(batch, M, hidden)
     mx, rel = errors(out.float().cpu().numpy(), want)
+    if dtype == "bfloat16":
+        report("multi-head attention bf16 %s" % (cfg,), mx, rel)
     assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (mx, rel)
     # same numbers as the chain on materialised per-head tensors (bit for bit: same kernel, same order)
     qd, kd, vd = (to_dev(np.ascontiguousarray(t), dtype) for t in (q, k, v))
@@ -394,3 +464,77 @@ def test_front_end_end_to_end(oracle):
     assert 0 < t.mean < 1e-2
     with pytest.raises(ValueError):
         func(*args[:3])
+
+
+def test_reference_test_flow_with_build_fusion_choice(oracle):
+    """python_test/auto_tensorize/test_hyper_fusion.py:833-910 (test_tensorize_cuda_run) against this package:
+    serial fusion state -> intrinsic match -> register_tensorize_axes -> build_fusion_choice ->
+    tensorize_hyper_fusion_state -> tensorize_cuda -> build -> time_evaluator, on the reference's own
+    uniform(-1, 1) inputs; the result is checked, which the reference's test does not do."""
+    import ditto_amd as ditto
+    from ditto_amd import auto_compute as ac, auto_tensorize as at, hardware as hw
+
+    ins, outs = ac.nn.functional.BatchGemmSoftmaxGemm()  # the reference's defaults: 12 x 512 x 64 x 64 x 512
+    layer = ac.layer([outs[0].op], inputs=ins)
+    sfs = at.build_serial_fusion_state(layer)
+    op1, op2 = sfs.first_op, sfs.second_op
+
+    def get_match_info(op, store_scope):
+        packed = at.cuda_wmma(16, 16, 16, "float16", "float32", store_scope)
+        choice = at.intrinsic_match(op.output(0), packed, ["InnerMost", "SameRange"])[0]
+        return at.match_info(choice, packed, impl="")
+
+    first_match_info = get_match_info(op1, "shared")
+    second_match_info = get_match_info(op2, "global")
+    sfs.register_tensorize_axes(list(first_match_info.axis) + list(second_match_info.axis))
+    V100 = hw.query_hw_param("gpu.cuda.V100")
+    fuse_choice = at.build_fusion_choice(sfs, hw_param=V100, dtype="float32", simple_mode=-1)
+    tensorize_state = at.tensorize_hyper_fusion_state(layer, fuse_choice, {op1: first_match_info, op2: second_match_info})
+    tensorize_param = at.cuda_tensorize_param(warp_size=32, ty_size=4, tz_size=2, input_vector_len=4, serial_y=2,
+                                              serial_z=1, block_rx=8, warp_rx=4, block_ry=1, warp_ry=4,
+                                              unroll_steps=512)
+    sch = at.tensorize_cuda(layer, tensorize_state, V100, tensorize_param)
+    func = ditto.build(sch, layer.schedule_tensors, "hip")
+    rng = np.random.default_rng(0)
+    inputs_np = [oracle.np_round_to(rng.uniform(-1, 1, [int(x) for x in y.shape]).astype(np.float32), "float16")
+                 for y in ins]
+    inputs = [to_dev(x, "float16") for x in inputs_np]
+    outputs = [torch.full(tuple(y.shape), float("nan"), device="cuda:0", dtype=torch.float16) for y in outs]
+    evaluator = func.time_evaluator(func.entry_name, None, min_repeat_ms=50)
+    cost = evaluator(*inputs, *outputs).mean * 1e3
+    assert 0 < cost < 1.0  # ms
+    want = oracle.bmm_chain_f64(*inputs_np, inter="softmax", scale=1.0)
+    mx, rel = errors(outputs[0].float().cpu().numpy(), want)
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
+    # the descriptor is filled once and reused; a forced variant travels from the schedule to the call
+    assert len(func._descs) == 1
+    sch8 = at.tensorize_hip(layer, tensorize_state, tile_variant=648)
+    f8 = ditto.build(sch8, layer.schedule_tensors, "hip")
+    f8(*inputs, *outputs)
+    torch.cuda.synchronize()
+    assert next(iter(f8._descs.values())).tile_variant == 648
+    assert errors(outputs[0].float().cpu().numpy(), want)[1] <= REL_L2
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float32"])
+def test_relu_after_the_second_contraction(oracle, dtype):
+    # relu_out: the slot a fused activation layer lands in (chimera.graph_fusion)
+    batch, M, N, K, L = 2, 200, 64, 40, 136
+    A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, dtype if dtype != "float32" else "float16", seed=9, std=0.25)
+    want = np.maximum(oracle.bmm_chain_f64(A, B, C, inter="relu", round_mid=None if dtype == "float32" else dtype), 0.0)
+    dev = "cuda:0"
+    if dtype == "float32":
+        a, b, c = (torch.from_numpy(x).to(dev) for x in (A, B, C))
+    else:
+        a, b, c = to_dev(A, dtype), to_dev(B, dtype), to_dev(C, dtype)
+    for variant in ([0] if dtype == "float32" else variants(K, N)):
+        f = torch.full((batch, M, N), float("nan"), device=dev, dtype=torch.float32)
+        chain.run_bmm_chain(a, b, c, f, "relu", tile_variant=variant, relu_out=True)
+        torch.cuda.synchronize()
+        got = f.cpu().numpy()
+        assert (got >= 0).all() and (got == 0).mean() > 0.2
+        mx, rel = errors(got, want)
+        assert mx <= MAX_ABS and rel <= REL_L2, (variant, mx, rel)
+    with pytest.raises(NotImplementedError):  # no such slot behind the softmax chain
+        chain.run_bmm_chain(a.half(), b.half(), c.half(), torch.empty(batch, M, N, device=dev, dtype=torch.float16),
+                            "softmax", relu_out=True)

@@ -4,11 +4,13 @@ import pytest
 import torch
 
 from ditto_amd import chain
-from tests.gpu_util import errors, to_dev, TORCH_DTYPES
+from tests.gpu_util import errors, report, to_dev, TORCH_DTYPES
 
 pytestmark = pytest.mark.gpu
 
-MAX_ABS, REL_L2, REL_L2_BF16_QUANT = 1e-2, 1e-3, 3e-3
+# fp16 and bf16 alike against the checker that rounds the intermediate and the output where the chain does
+# (bf16 measured: at most 1.1e-4 rel-L2, from roundings that flip on the last accumulator bits)
+MAX_ABS, REL_L2 = 1e-2, 1e-3
 
 
 def run_conv(X, W1, W2, dtype, pad1=1, stride1=1, inter="cast", relu_out=False, out_dtype=None, workspace=None,
@@ -53,7 +55,9 @@ def test_conv_chain_vs_oracle(oracle, case, dtype):
         got = run_conv(X, W1, W2, dtype, pad, stride, workspace=ws)
         assert np.array_equal(got, oracle.np_round_to(got32, dtype)), ws
         mx, rel = errors(got, oracle.np_round_to(want32, dtype))
-        assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (ws, mx, rel)
+        if dtype == "bfloat16":
+            report("conv chain bf16 %s" % (case,), mx, rel)
+        assert mx <= MAX_ABS and rel <= REL_L2, (ws, mx, rel)
 
 
 # Enough tiles of whole output rows for two rounds of persistent workgroups (at least 512), 16-bit
@@ -91,11 +95,11 @@ def test_persistent_conv_chain_vs_oracle(oracle, case, dtype, monkeypatch):
         got = run_conv(X, W1, W2, dtype, pad, stride, "relu" if relu else "cast", relu)
         assert got.shape == want32.shape and np.isfinite(got).all()
         mx, rel = errors(got, oracle.np_round_to(want32, dtype))
-        assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (relu, mx, rel)
+        assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
         # against the one-tile-per-workgroup kernel (taken when there is no workspace); their summation
         # orders differ (here two waves each sum half of the taps x channel groups)
         other = run_conv(X, W1, W2, dtype, pad, stride, "relu" if relu else "cast", relu, workspace=False)
-        assert errors(got, other)[1] <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), relu
+        assert errors(got, other)[1] <= REL_L2, relu
     # a second call right away (the halo prefetch and the stores of the first are independent of it)
     again = run_conv(X, W1, W2, dtype, pad, stride, "relu", True)
     assert np.array_equal(again, got)
@@ -180,7 +184,9 @@ def test_depthwise_conv_chain_vs_oracle(oracle, case, dtype):
         # fp32 output runs the plain kernel there and 16-bit output the persistent one: their
         # summation orders differ, so the 16-bit result is held to the oracle, not to the fp32 bits
         mx, rel = errors(got, oracle.np_round_to(want32, dtype))
-        assert mx <= MAX_ABS and rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (mx, rel)
+        if dtype == "bfloat16":
+            report("conv chain (wide second filter / depthwise) bf16 %s" % (case,), mx, rel)
+        assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
     else:
         assert np.array_equal(got, oracle.np_round_to(got32, dtype))
 

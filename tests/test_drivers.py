@@ -51,6 +51,20 @@ def test_drivers_run_one_row_each(capsys):
 
 
 @pytest.mark.gpu
+def test_int8_driver_row():
+    # the ("80", "int8", "int32") combination of bmm_bmm_cuda.py:273-288 (GEMM chain only)
+    cost = bmm_bmm.main(*common.BMM_SHAPES[1], in_dtype="int8", acc_dtype="int32")
+    assert 0 < cost < 5.0
+    out = subprocess.run([sys.executable, "-m", "ditto_amd.drivers.bmm_bmm", "--in_dtype", "int8", "--acc_dtype",
+                          "int32", "--begin", "9", "--num", "1", "--only_once"], capture_output=True, text=True,
+                         check=True).stdout.strip().splitlines()
+    assert out[-2] == "1,512,64,64,256,int8,int32,gfx950,-1"
+    out = subprocess.run([sys.executable, "-m", "ditto_amd.drivers.bmm_softmax_bmm", "--in_dtype", "int8",
+                          "--acc_dtype", "int32", "--num", "1"], capture_output=True, text=True, check=True).stdout
+    assert "Data type not supported" in out  # no int8 softmax chain
+
+
+@pytest.mark.gpu
 def test_cli_csv_format():
     out = subprocess.run([sys.executable, "-m", "ditto_amd.drivers.bmm_softmax_bmm", "--begin", "3", "--num", "1",
                           "--only_once"], capture_output=True, text=True, check=True).stdout.strip().splitlines()

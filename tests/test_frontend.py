@@ -275,3 +275,192 @@ def test_retrieve_attention_schedule_from_log(tmp_path):
             print(json.dumps({"wkl_key": key, "entry": {"record": {"variant": variant}, "value": value}}), file=f)
     sch, _ = auto_schedule.retrieve_schedule_bound_tasks(bound, opt)[key]
     assert sch.tile_variant == 648 and sch.module.num_heads == 12 and sch.module.scale == 64 ** -0.5
+
+
+def _reference_flow(ins, outs, in_dtype="float16", acc_dtype="float32"):
+    """The flow of python_test/auto_tensorize/test_hyper_fusion.py:833-880: serial fusion state ->
+    intrinsic match -> register_tensorize_axes (one flat list) -> build_fusion_choice -> state."""
+    layer = ac.layer([outs[0].op], inputs=list(ins))
+    sfs = at.build_serial_fusion_state(layer)
+    op1, op2 = sfs.first_op, sfs.second_op
+
+    def get_match_info(op, scope):
+        packed = at.cuda_wmma(16, 16, 16, in_dtype, acc_dtype, scope)
+        return at.match_info(at.intrinsic_match(op.output(0), packed, ["InnerMost", "SameRange"])[0], packed, impl="")
+
+    first, second = get_match_info(op1, "shared"), get_match_info(op2, "global")
+    sfs.register_tensorize_axes(list(first.axis) + list(second.axis))
+    fuse_choice = at.build_fusion_choice(sfs, hw_param=hw.query_hw_param("gpu.cuda.V100"), dtype="float32",
+                                         simple_mode=-1)
+    state = at.tensorize_hyper_fusion_state(layer, fuse_choice, {op1: first, op2: second})
+    return layer, sfs, fuse_choice, state
+
+
+def test_build_fusion_choice_gives_the_order_the_reference_drivers_write_by_hand():
+    # bmm_bmm_cuda.py:176 and bmm_softmax_bmm_cuda.py: [b, m, n, rlo, mi, ni, rli], 3
+    for ins, outs in (F.BatchGemmSoftmaxGemm(12, 512, 64, 64, 512), F.BatchGemmGemm(1, 512, 64, 64, 64)):
+        layer, sfs, fc, state = _reference_flow(ins, outs)
+        E_frag = outs[0].op.input_tensors[0]
+        b, m, n, mi, ni = E_frag.op.axis
+        rlo, rli = E_frag.op.reduce_axis
+        manual = at.fusion_choice(sfs.first_op, sfs.second_op, [b, m, n, rlo, mi, ni, rli], 3)
+        assert fc.first_op is manual.first_op and fc.second_op is manual.second_op
+        assert all(x is y for x, y in zip(fc.ordered_iters, manual.ordered_iters)) and len(fc.ordered_iters) == 7
+        assert fc.attach_pos == 3
+        assert fc.secondOpOuterIndices == [0, 1, 2, 5] and fc.secondOpOuterTilingFactors == [1, 1, 1, 1]
+        assert [iv.name for iv in state.fused_spatial_outer_iters] == ["b", "mo", "no"]
+        assert [iv.name for iv in state.fused_reduce_outer_iters] == ["rlo"]
+        # every search mode names the same fusion (the kernels fix tiling and order themselves)
+        for mode in (0, 1):
+            other = at.build_fusion_choice(sfs, None, "float16", mode)
+            assert all(x is y for x, y in zip(other.ordered_iters, fc.ordered_iters)) and other.attach_pos == 3
+        sch = at.tensorize_cuda(layer, state, hw.query_hw_param("gpu.hip.MI355X"), at.cuda_tensorize_param())
+        assert sch.kind == "bmm_chain"
+    # errors: axes not registered, unknown dtype, unknown mode (CHECKs of hyper_fusion.cc:1978, 1988)
+    ins, outs = F.BatchGemmGemm(1, 64, 64, 64, 64)
+    sfs = at.build_serial_fusion_state(ac.layer([outs[0].op], inputs=ins))
+    with pytest.raises(ValueError, match="register"):
+        at.build_fusion_choice(sfs, None, "float32")
+    sfs.register_tensorize_axes({sfs.second_op: list(sfs.second_op.axis[-2:]) + [sfs.second_op.reduce_axis[-1]]})
+    with pytest.raises(ValueError, match="dtype"):
+        at.build_fusion_choice(sfs, None, "complex64")
+    with pytest.raises(ValueError, match="simple_mode"):
+        at.build_fusion_choice(sfs, None, "float32", 7)
+    with pytest.raises(ValueError, match="neither contraction"):
+        sfs.register_tensorize_axes([te.reduce_axis([0, 16], "stranger")])
+
+
+def test_build_fusion_choice_on_conv_chains():
+    # the hand-written choices of conv3x3_conv1x1_cuda.py:211 ([b, no, p, mo, rlo, mi, ni, rli], 4) and
+    # conv1x1_conv3x3_cuda.py:228 ([b, no, p, mo, rlo, mi, ni, rr, rs, rli], 4) have this shape: spatial loops
+    # that are not tensorized, the outermost free reduce loop, tensorized spatial loops, the other reduce loops
+    for builder, n_red in ((F.Conv3x3Conv1x1, 3), (F.Conv1x1Conv3x3, 3)):
+        cins, couts = builder(2, 64, 56, 56, 64, 64)
+        layer = ac.layer([couts[0].op], inputs=[cins[0]], weights=cins[1:])
+        sfs = at.build_serial_fusion_state(layer)
+        op2 = sfs.second_op
+        n, k, p, q = op2.axis
+        c2, r2, s2 = op2.reduce_axis
+        sfs.register_tensorize_axes([q, k, c2])  # pixel x output channel x input channel tile
+        fc = at.build_fusion_choice(sfs, hw.query_hw_param("gpu.hip.MI355X"), "float16")
+        assert [iv.name for iv in fc.ordered_iters] == ["n", "p", "rr2", "k", "q", "rs2", "rc2"]
+        assert fc.attach_pos == 2 and fc.ordered_iters[fc.attach_pos] is r2
+
+
+def test_int8_chain_builder_and_recognition():
+    # the ("80", "int8", "int32") row of bmm_bmm_cuda.py:273-288, with the middle result requantised
+    ins, outs = F.BatchGemmGemm(1, 8192, 1024, 1024, 256, "int8", "int32", requant_scale=2.0 ** -10)
+    assert [t.dtype for t in ins] == ["int8"] * 3 and outs[0].dtype == "int32"
+    layer, sfs, fc, state = _reference_flow(ins, outs, "int8", "int32")
+    assert [o.name for o in state.inter_path] == ["requant"] and [o.name for o in state.epilogue] == ["F"]
+    sch = at.tensorize_cuda(layer, state, hw.query_hw_param("gpu.hip.MI355X"), at.cuda_tensorize_param())
+    assert (sch.kind, sch.inter_op, sch.in_dtype, sch.acc_dtype, sch.out_dtype) == (
+        "bmm_chain", "requant", "int8", "int32", "int32")
+    assert sch.requant_scale == 2.0 ** -10 and not sch.scale_tensor
+    assert sch.dims == dict(batch=1, M=8192, N=1024, K=1024, L=256)
+    # per-column scales: a fourth input placeholder, in schedule_tensors order before the output
+    ins, outs = F.BatchGemmGemm(2, 64, 64, 64, 128, "int8", "int32", scale_tensor=True)
+    assert len(ins) == 4 and ins[3].shape == (128,) and ins[3].dtype == "float32"
+    layer, sfs, fc, state = _reference_flow(ins, outs, "int8", "int32")
+    sch = at.tensorize_hip(layer, state)
+    assert sch.scale_tensor and [t.name for t in layer.schedule_tensors] == ["A", "B", "C", "scale", "F"]
+    # the reference's wrapping astype("int8") has no kernel: refused when the chain is tensorized
+    ins, outs = F.BatchGemmGemm(1, 64, 64, 64, 64, "int8", "int32")
+    layer, sfs, fc, state = _reference_flow(ins, outs, "int8", "int32")
+    with pytest.raises(NotImplementedError, match="requant"):
+        at.tensorize_hip(layer, state)
+    # tile_variant travels on the schedule
+    ins, outs = F.BatchGemmGemm(64, 4096, 128, 128, 4096, "bfloat16", "float32")
+    layer, sfs, fc, state = _reference_flow(ins, outs, "bfloat16")
+    assert at.tensorize_hip(layer, state, tile_variant=1288).tile_variant == 1288
+
+
+def test_cpu_side_names_describe_but_do_not_build():
+    # the flow of benchmark/chimera/cpu/bmm_bmm_cpu.py:118-276 up to the point where it would compile
+    ins, outs = F.BatchGemmGemm(1, 516, 64, 64, 64, "float32", "float32", MI=6, NI=16, KI=16)
+    layer = ac.layer([outs[0].op], inputs=ins)
+    sfs = at.build_serial_fusion_state(layer)
+    op1, op2 = sfs.first_op, sfs.second_op
+    packed, code = at.cpu_intrin(op="gemm_noreshape", shape=(6, 16, 16), isa="avx2", dtype="float32", prefix="gemm1")
+    assert packed.compute_intrinsic.name == "gemm1_update" and "6 x 16 x 16" in code and packed.store_intrinsic is None
+    assert str(packed).startswith("PackedIntrinsic(")
+    with pytest.raises(ValueError):
+        at.cpu_intrin("gemm", (6, 16, 16), "avx2", "float16")  # the micro-kernels are fp32 / fp64
+    infos = {}
+    for op, prefix in ((op1, "gemm1"), (op2, "gemm2")):
+        pk, cd = at.cpu_intrin("gemm_noreshape", (6, 16, 16), "avx2", "float32", prefix)
+        infos[op] = at.match_info(at.intrinsic_match(op.output(0), pk, ["SameRange"])[0], pk, cd)
+    sfs.register_tensorize_axes(list(infos[op1].axis) + list(infos[op2].axis))
+    cpu = hw.hardware_param(num_groups=16, cacheSizes=[32 * 16, 32 * 1024, 1024 * 1024, 11264 * 1024],
+                            bandwidth=[293.72, 81.72, 38.54, 13.14], coresPerCacheLevel=[1.0, 1.0, 1.0, 16.0],
+                            tensorWeight=[1.0, 2.0, 1.0, 1.0, 1.0], platform="CPU")
+    fc = at.build_fusion_choice(sfs, hw_param=cpu, dtype="float32", simple_mode=-1)
+    state = at.tensorize_hyper_fusion_state(layer, fc, infos)
+    param = at.build_cpu_tensorize_param(sfs, fc, cpu, "float32")
+    assert param.parallelism == 16 and len(param.secondOpLoopOrder) == 7
+    ctx = at.build_fusion_context(sfs, layer, state, "", hw_param=cpu, dtype="float32", searchType="stochastic",
+                                  mode="survey")
+    assert ctx.size == 1 and ctx.getComputation(0) == 516 * 64 * 64 * 2
+    # D_frag's tile under the fused loops (b, mo, no): 6 x 64 fp32 = 1.5 KB -> the 32 KB level
+    assert ctx.getFusionLevel(0) == 1
+    sch = ctx.run(0, None)
+    assert sch.target == "cpu" and sch.kind == "bmm_chain"
+    with pytest.raises(NotImplementedError, match="no CPU product path"):
+        ditto.build(sch, layer.schedule_tensors, "llvm")
+    with pytest.raises(IndexError):
+        ctx.run(1, None)
+
+
+def test_graph_fusion_folds_relu_layers_into_the_producing_chain():
+    from ditto_amd import chimera, runtime
+
+    def chain_layer(relu_mid=False):
+        ins, outs = F.BatchGemmGemm(2, 128, 64, 64, 128, relu=relu_mid)
+        return ac.layer([outs[0].op], inputs=ins, name="gemm_chain")
+
+    def relu_layer(shape, name="act"):
+        x = te.placeholder(shape, "x", "float16")
+        return ac.layer([F.ReLU(x).op], inputs=[x], name=name)
+
+    l0, act, l1 = chain_layer(), relu_layer([2, 128, 64]), chain_layer(True)
+    graph = runtime.Graph([l0, act, l1], edges={(1, 0): (0, 0), (2, 0): (1, 0)})
+    assert chimera.is_act_layer(act) and not chimera.is_act_layer(l0) and not chimera.is_elem_layer(act)
+    fused = chimera.graph_fusion(graph)
+    assert [l.name for l in fused.layers] == ["gemm_chain_relu", "gemm_chain"]
+    assert fused.edges == {(1, 0): (0, 0)} and fused.graph_outputs == [(1, 0)]
+    assert [l.name for l in graph.layers] == ["gemm_chain", "act", "gemm_chain"]  # the input graph is untouched
+    out_op = fused.layers[0].ops[0]
+    assert out_op.kind == "relu_cast" and out_op.attrs["fused_activation"] == "relu"
+    assert fused.layers[0].fingerprint != l0.fingerprint
+    # the fused layer still describes and tensorizes as a chain, now with the output ReLU
+    layer, sfs, fc, state = None, None, None, None
+    fl = fused.layers[0]
+    sfs = at.build_serial_fusion_state(fl)
+    p = at.cuda_wmma(16, 16, 16, "float16", "float32", "global")
+    infos = {op: at.match_info(at.intrinsic_match(op.output(0), p, ["InnerMost", "SameRange"])[0], p)
+             for op in (sfs.first_op, sfs.second_op)}
+    sfs.register_tensorize_axes([iv for mi in infos.values() for iv in mi.axis])
+    state = at.tensorize_hyper_fusion_state(fl, at.build_fusion_choice(sfs, None, "float16"), infos)
+    sch = at.tensorize_hip(fl, state)
+    assert (sch.inter_op, sch.relu_out) == ("cast", True)
+    # not fused: a ReLU whose input is also a graph output, one behind a softmax chain, a gelu, a residual add
+    keep = runtime.Graph([l0, act], edges={(1, 0): (0, 0)}, outputs=[(0, 0), (1, 0)])
+    assert chimera.graph_fusion(keep) is keep
+    sins, souts = F.BatchGemmSoftmaxGemm(2, 128, 64, 64, 128)
+    sl = ac.layer([souts[0].op], inputs=sins, name="attn_chain")
+    g2 = runtime.Graph([sl, relu_layer([2, 128, 64])], edges={(1, 0): (0, 0)})
+    assert chimera.graph_fusion(g2) is g2
+    x = te.placeholder([2, 128, 64], "x", "float16")
+    gelu = ac.layer([F.activation(x, "gelu").op], inputs=[x], name="gelu")
+    g3 = runtime.Graph([l0, gelu], edges={(1, 0): (0, 0)})
+    assert chimera.graph_fusion(g3) is g3
+    a, b = te.placeholder([2, 128, 64], "a", "float16"), te.placeholder([2, 128, 64], "b", "float16")
+    add = ac.layer([F.elementwise(a, b, "add").op], inputs=[a, b], name="residual")
+    assert chimera.is_elem_layer(add)
+    g4 = runtime.Graph([l0, add], edges={(1, 0): (0, 0)})
+    assert chimera.graph_fusion(g4) is g4
+    # a conv chain takes the ReLU too (its descriptor already has the output slot)
+    cins, couts = F.Conv3x3Conv1x1(2, 16, 16, 16, 32, 48)
+    cl = ac.layer([couts[0].op], inputs=[cins[0]], weights=cins[1:], name="conv_chain")
+    g5 = chimera.graph_fusion(runtime.Graph([cl, relu_layer([2, 48, 16, 16])], edges={(1, 0): (0, 0)}))
+    assert len(g5.layers) == 1 and g5.layers[0].ops[0].kind == "relu_cast" and len(g5.layers[0].weights) == 2

@@ -104,3 +104,46 @@ def test_i8_chain_rejects_bad_descriptors():
         chain.run_bmm_chain(a, b, d, e, "requant", aux=torch.ones(5, device=dev))
     with pytest.raises(ValueError):
         chain.run_bmm_chain(a, b, d, e.float(), "requant")
+
+
+def test_i8_chain_through_the_operator_api(oracle):
+    """The quantised configuration (int8 A[8192,1024], B[1024,256], D[256,1024], middle result requantised
+    at 2^-10) built the way the reference builds its chains -- BatchGemmGemm -> serial fusion state ->
+    build_fusion_choice -> tensorize_cuda -> build -> f(A, B, D, E) -- and checked bit for bit."""
+    import ditto_amd as ditto
+    from ditto_amd import auto_compute as ac, auto_tensorize as at, hardware as hw
+
+    def built(ins, outs):
+        layer = ac.layer([outs[0].op], inputs=list(ins))
+        sfs = at.build_serial_fusion_state(layer)
+        packed = at.cuda_wmma(16, 16, 16, "int8", "int32", "global")
+        infos = {op: at.match_info(at.intrinsic_match(op.output(0), packed, ["InnerMost", "SameRange"])[0], packed)
+                 for op in (sfs.first_op, sfs.second_op)}
+        sfs.register_tensorize_axes([iv for mi in infos.values() for iv in mi.axis])
+        fc = at.build_fusion_choice(sfs, hw.query_hw_param("gpu.hip.MI355X"), "int32")
+        state = at.tensorize_hyper_fusion_state(layer, fc, infos)
+        sch = at.tensorize_cuda(layer, state, hw.query_hw_param("gpu.hip.MI355X"), at.cuda_tensorize_param())
+        return ditto.build(sch, layer.schedule_tensors, "hip")
+
+    dev = "cuda:0"
+    M, K, L, N = 8192, 1024, 256, 1024
+    A, B, D, scale = oracle.make_i8_chain_inputs(M, K, L, N, seed=11)
+    func = built(*ac.nn.functional.BatchGemmGemm(1, M, N, K, L, "int8", "int32", requant_scale=2.0 ** -10))
+    a, b, d = (torch.from_numpy(x[None]).to(dev) for x in (A, B, D))
+    e = torch.full((1, M, N), -7, dtype=torch.int32, device=dev)
+    func(a, b, d, e)
+    torch.cuda.synchronize()
+    got = e.cpu().numpy()[0]
+    rows = np.r_[0:64, 4000:4100, M - 37:M]  # rows are independent: the checker runs on a sample of them
+    want = oracle.gemm_chain_i8(A[rows], B, D, scale)[0]
+    assert np.array_equal(got[rows], want)
+    assert np.array_equal(got, run_i8(A, B, D, scale))  # and all of it equals the direct C-ABI call
+    # per-column scales as a fourth input tensor
+    M2, K2, L2, N2 = 96, 256, 64, 48
+    A2, B2, D2, _ = oracle.make_i8_chain_inputs(M2, K2, L2, N2, seed=5)
+    sc = (2.0 ** -np.random.default_rng(1).integers(6, 14, L2)).astype(np.float32)
+    func2 = built(*ac.nn.functional.BatchGemmGemm(1, M2, N2, K2, L2, "int8", "int32", scale_tensor=True))
+    e2 = torch.zeros((1, M2, N2), dtype=torch.int32, device=dev)
+    func2(*(torch.from_numpy(x[None]).to(dev) for x in (A2, B2, D2)), torch.from_numpy(sc).to(dev), e2)
+    torch.cuda.synchronize()
+    assert np.array_equal(e2.cpu().numpy()[0], oracle.gemm_chain_i8(A2, B2, D2, sc)[0])

@@ -287,3 +287,13 @@ def test_conv_chain_mid_rounding(oracle):
     assert np.array_equal(Y, oracle.np_round_to(Y, "float16"))
     want = _torch_conv_chain(X, W1, W2, 1, 1, 0, 1, False, False)
     assert np.allclose(Y, want, rtol=5e-3, atol=5e-3)
+
+
+def test_rounding_floor_of_the_16_bit_types(oracle):
+    """What rounding alone costs: the figure the bf16 parity bounds of the GPU tests rest on."""
+    x = np.random.default_rng(0).standard_normal(1 << 20).astype(np.float32)
+    rel = {dt: float(np.linalg.norm(oracle.np_round_to(x, dt) - x) / np.linalg.norm(x)) for dt in ("bfloat16", "float16")}
+    assert 1.6e-3 < rel["bfloat16"] < 1.7e-3 and 2.0e-4 < rel["float16"] < 2.2e-4
+    # two independent roundings (probabilities, then output) add in quadrature
+    y = oracle.np_round_to(oracle.np_round_to(x, "bfloat16") * np.float32(1.2345), "bfloat16") / np.float32(1.2345)
+    assert 2.2e-3 < float(np.linalg.norm(y - x) / np.linalg.norm(x)) < 2.5e-3

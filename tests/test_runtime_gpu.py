@@ -127,3 +127,117 @@ def test_attention_blocks_through_task_binding_and_graph_engine(tmp_path, oracle
         for got in eng.get_outputs():
             err = np.abs(got.float().cpu().numpy() - want)
             assert err.max() <= 1e-2 and np.linalg.norm(err) / np.linalg.norm(want) <= 1e-3
+
+
+def test_graph_fusion_on_the_gpu(oracle):
+    """A ReLU layer behind a GEMM chain and one behind a conv chain are folded into the chains by
+    ``chimera.graph_fusion`` (reference: python/ditto/chimera/graph_fusion.py:4-52); the fused graph has one
+    layer per chain and gives the numbers of chain-then-ReLU."""
+    import numpy as np
+
+    from ditto_amd import chimera, te
+    from tests.gpu_util import errors, to_dev
+
+    F = ac.nn.functional
+
+    def relu_layer(shape, dtype="float16"):
+        x = te.placeholder(shape, "x", dtype)
+        return ac.layer([F.ReLU(x).op], inputs=[x], name="act")
+
+    # GEMM chain -> ReLU -> GEMM chain
+    batch, M, K, L, N = 2, 256, 64, 128, 64
+    ins0, outs0 = F.BatchGemmGemm(batch, M, N, K, L, "float16", "float32")
+    ins1, outs1 = F.BatchGemmGemm(batch, M, N, N, L, "float16", "float32", relu=True)
+    l0 = ac.layer([outs0[0].op], inputs=ins0, name="chain0")
+    l1 = ac.layer([outs1[0].op], inputs=ins1, name="chain1")
+    graph = runtime.Graph([l0, relu_layer([batch, M, N]), l1], edges={(1, 0): (0, 0), (2, 0): (1, 0)})
+    fused = chimera.graph_fusion(graph)
+    assert len(fused.layers) == 2 and fused.layers[0].ops[0].kind == "relu_cast"
+    mods = {l.fingerprint: ditto.build(common.describe_layer(l), l.schedule_tensors, "hip") for l in fused.layers}
+    assert mods[fused.layers[0].fingerprint].sch.relu_out
+    A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, "float16", seed=3, std=0.25)
+    _, B1, C1 = oracle.make_gemm_chain_inputs(batch, M, N, N, L, "float16", seed=4, std=0.25)
+    for make in (runtime.create_graph_engine, runtime.create_hip_graph_engine):
+        eng = make(fused, mods, "cuda:0")
+        eng.set_inputs([to_dev(x, "float16") for x in (A, B, C, B1, C1)])
+        eng.compile()
+        eng.run()
+        torch.cuda.synchronize()
+        mid = oracle.np_round_to(np.maximum(oracle.bmm_chain_f64(A, B, C, inter="cast", round_mid="float16"), 0.0),
+                                 "float16")
+        want = oracle.bmm_chain_f64(mid, B1, C1, inter="relu", round_mid="float16")
+        mx, rel = errors(eng.get_outputs()[0].float().cpu().numpy(), want)
+        assert mx <= 1e-2 and rel <= 2e-3, (mx, rel)  # two chains deep: one rounding flip of the first moves the second
+
+    # conv chain -> ReLU, weights as layer weights (the engine repacks them once per compile)
+    n, c0, hw_, c1, c2 = 4, 32, 28, 64, 96
+    cins, couts = F.Conv3x3Conv1x1(n, c0, hw_, hw_, c1, c2)
+    cl = ac.layer([couts[0].op], inputs=[cins[0]], weights=cins[1:], name="conv_chain")
+    cg = chimera.graph_fusion(runtime.Graph([cl, relu_layer([n, c2, hw_, hw_])], edges={(1, 0): (0, 0)}))
+    assert len(cg.layers) == 1
+    fl = cg.layers[0]
+    func = ditto.build(common.describe_layer(fl), fl.schedule_tensors, "hip")
+    assert func.sch.relu_out and func.sch.kind == "conv_chain"
+    X, W1, W2 = oracle.make_conv_chain_inputs(n, c0, hw_, hw_, c1, c2, 3, 1, "float16", seed=8)
+    want = oracle.np_round_to(oracle.conv_chain_f32(X, W1, W2, 1, 1, 0, 1, relu_mid=False, relu_out=True,
+                                                    round_mid="float16"), "float16")
+    for make in (runtime.create_graph_engine, runtime.create_hip_graph_engine):
+        eng = make(cg, {fl.fingerprint: func}, "cuda:0")
+        eng.set_inputs([to_dev(X, "float16")])
+        eng.set_weight(fl, fl.weights[0], to_dev(W1, "float16"))
+        eng.set_weight(fl, fl.weights[1], to_dev(W2, "float16"))
+        eng.compile()
+        assert eng._to_exe[0][0] is not func and eng._to_exe[0][0]._prepared is not None  # bound to these weights
+        for _ in range(2):
+            eng.run()
+        torch.cuda.synchronize()
+        got = eng.get_outputs()[0].float().cpu().numpy()
+        assert (got >= 0).all() and (got == 0).mean() > 0.2
+        mx, rel = errors(got, want)
+        assert mx <= 1e-2 and rel <= 1e-3, (mx, rel)
+        # new weights through set_weight are repacked at the next compile
+        eng.set_weight(fl, fl.weights[1], to_dev(W2 * 0.5, "float16"))
+        eng.run()
+        torch.cuda.synchronize()
+        half = oracle.np_round_to(oracle.conv_chain_f32(X, W1, oracle.np_round_to(W2 * 0.5, "float16"), 1, 1, 0, 1,
+                                                        relu_mid=False, relu_out=True, round_mid="float16"), "float16")
+        assert errors(eng.get_outputs()[0].float().cpu().numpy(), half)[1] <= 1e-3
+
+
+def test_captured_conv_chain_survives_growth_of_the_shared_workspace(oracle):
+    """A HIP graph that captured a conv chain call keeps replaying correctly after a later, larger chain made
+    the shared per-device workspace grow: buffers that were handed out are never freed, and a built function
+    owns its workspace."""
+    import numpy as np
+
+    from ditto_amd import chain
+    from tests.gpu_util import errors, to_dev
+
+    dev = "cuda:0"
+    X, W1, W2 = oracle.make_conv_chain_inputs(2, 16, 24, 24, 32, 48, 3, 1, "float16", seed=2)
+    x, w1, w2 = (to_dev(t, "float16") for t in (X, W1, W2))
+    y = torch.zeros(2, 48, 24, 24, device=dev, dtype=torch.float16)
+    chain.run_conv_chain(x, w1, w2, y)  # warm-up: sizes the shared workspace (1 MiB floor)
+    torch.cuda.synchronize()
+    want = y.clone()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        chain.run_conv_chain(x, w1, w2, y)
+    before = chain._WORKSPACES[torch.device(dev)][-1].data_ptr()
+    # a chain whose repacked weights exceed the floor: the shared workspace grows
+    bx = torch.zeros(1, 512, 8, 8, device=dev, dtype=torch.float16)
+    bw1 = torch.zeros(256, 512, 3, 3, device=dev, dtype=torch.float16)
+    bw2 = torch.zeros(32, 256, 1, 1, device=dev, dtype=torch.float16)
+    by = torch.zeros(1, 32, 8, 8, device=dev, dtype=torch.float16)
+    chain.run_conv_chain(bx, bw1, bw2, by)
+    torch.cuda.synchronize()
+    bufs = chain._WORKSPACES[torch.device(dev)]
+    assert bufs[-1].data_ptr() != before and any(b.data_ptr() == before for b in bufs)  # grown, old one kept
+    junk = [torch.full((1 << 20,), 0xAB, dtype=torch.uint8, device=dev) for _ in range(8)]  # would reuse a freed block
+    for it in range(3):
+        y.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), it
+    del junk
