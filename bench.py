@@ -32,19 +32,30 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "i8": 5000.0, "f32": 157.3}
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a copy
-# kernel of known size; see the summaries under profiles/.  None where not measured.
-MEASURED_TRAFFIC_BYTES = {
-    # FETCH_SIZE reads half of a plain copy's bytes on this device (scale factor 2.00), WRITE_SIZE all of them
-    "attn_bf16_b64_s4096_d128": int((192.48 + 64.00) * 2 ** 20),
-    "gemm_chain_bf16_b64_4096x128x4096x128": int((192.28 + 64.00) * 2 ** 20),
-    "attn_f16_b96_s512_d64": int((18.22 + 6.00) * 2 ** 20),
-    "conv_chain_f16_n32_c64_56x56_k64_k256": int((13.44 + 54.50) * 2 ** 20),
-    "gemm_chain_i8_8192x1024x256x1024": int((12.15 + 32.00) * 2 ** 20),
-    "conv1x1_conv3x3_f16_n32_c64_56x56_k64_k64": int((13.25 + 12.25) * 2 ** 20),
-    "dw3x3_conv1x1_f16_n32_c32_112x112_f16_k64": int((29.79 + 49.00) * 2 ** 20),
-    "dw3x3_conv1x1_f16_n32_c32_112x112_x1_k64": int((29.30 + 49.00) * 2 ** 20),
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a copy kernel of known
+# size (FETCH_SIZE reads half of a plain copy's bytes on this device: scale factor 2.00; WRITE_SIZE all of
+# them); the summaries are under profiles/.  Each figure belongs to the kernel variant it was measured on
+# (``tile.variant``): when the library picks another variant for the workload the figure is stale and
+# ``roofline.traffic`` is reported as null.
+MEASURED_TRAFFIC = {
+    # workload: (FETCH MiB, WRITE MiB, tile variant measured)
+    "attn_bf16_b64_s4096_d128": (192.48, 64.00, 1282),
+    "gemm_chain_bf16_b64_4096x128x4096x128": (192.28, 64.00, 1282),
+    "attn_f16_b96_s512_d64": (18.22, 6.00, 648),
+    "conv_chain_f16_n32_c64_56x56_k64_k256": (13.44, 54.50, 3022),
+    "gemm_chain_i8_8192x1024x256x1024": (12.15, 32.00, 8014),
+    "conv1x1_conv3x3_f16_n32_c64_56x56_k64_k64": (13.25, 12.25, 3521),
+    "dw3x3_conv1x1_f16_n32_c32_112x112_f16_k64": (29.79, 49.00, 4022),
+    "dw3x3_conv1x1_f16_n32_c32_112x112_x1_k64": (29.30, 49.00, 4023),
 }
+
+
+def measured_traffic(name, variant):
+    rec = MEASURED_TRAFFIC.get(name)
+    if rec is None or rec[2] != variant:
+        return None
+    return int((rec[0] + rec[1]) * 2 ** 20)
+
 
 WORKLOADS = {
     # name: kind, dtype, dims
@@ -272,7 +283,7 @@ def cpu_baseline(w, budget_s=10.0, pool=24):
         run(e)
         elapsed += time.perf_counter() - t0
         done += 1
-    return {
+    out = {
         "value": per_entry * done / elapsed / 1e12,
         "unit": "TFLOP/s",
         "cores": orc.num_threads(),
@@ -281,6 +292,67 @@ def cpu_baseline(w, budget_s=10.0, pool=24):
                   "fused CPU loop nest (oracle_bmm_chain_fused_f32), cycling over %d distinct entries, %.1f s"
                   % (done, M, L, K, N, pool, elapsed),
     }
+    out["torch_cpu"] = torch_cpu_comparator(w, entries)
+    out["config1_cpu"] = config1_cpu()
+    return out
+
+
+def torch_cpu_comparator(w, entries, budget_s=6.0):
+    """The reference's own CPU comparator (benchmark/pytorch/cpu/bmm_softmax_bmm.py:54-74): ``torch.bmm`` ->
+    softmax -> ``torch.bmm`` in fp32 on the host cores, on the same single-batch entries as the port above."""
+    import torch
+
+    M, N, K, L = w["M"], w["N"], w["K"], w["L"]
+    ts = [tuple(torch.from_numpy(x) for x in e) for e in entries[:8]]
+
+    def run(q, k, v):
+        s = torch.bmm(q, k)
+        if w["kind"] == "softmax":
+            s = torch.softmax(s * w["scale"], dim=2)
+        return torch.bmm(s, v)
+
+    run(*ts[0])
+    done, elapsed = 0, 0.0
+    while elapsed < budget_s and done < 100000:
+        t0 = time.perf_counter()
+        run(*ts[(done + 1) % len(ts)])
+        elapsed += time.perf_counter() - t0
+        done += 1
+    return {"value": 2.0 * M * L * (K + N) * done / elapsed / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "sample": "%d single-batch-entry calls of torch.bmm / softmax / torch.bmm in fp32, %.1f s" % (done, elapsed)}
+
+
+def config1_cpu(repeats=40):
+    """The CPU-sized configuration exactly (fp32, batch 1, A[512x64].B[64x64].D[64x64], N(0,1), seed 0) through
+    the fused CPU loop nest, one call per repeat with the caches flushed in between by streaming a buffer
+    larger than the last-level cache (the protocol of benchmark/chimera/cpu/bmm_bmm_cpu.py:264-269,
+    ``f_preproc="cache_flush_cpu_non_first_arg"``)."""
+    import numpy as np
+
+    from oracle import oracle as orc
+
+    rng = np.random.default_rng(0)
+    A = rng.standard_normal((1, 512, 64), dtype=np.float32)
+    B = rng.standard_normal((1, 64, 64), dtype=np.float32)
+    D = rng.standard_normal((1, 64, 64), dtype=np.float32)
+    out = np.empty((1, 512, 64), dtype=np.float32)
+    flush = np.zeros(1 << 27, dtype=np.uint8)  # 128 MiB streamed between calls
+    orc.bmm_chain_fused_f32(A, B, D, inter="cast", out=out)
+    cold, warm = [], []
+    for i in range(repeats):
+        flush += 1
+        t0 = time.perf_counter()
+        orc.bmm_chain_fused_f32(A, B, D, inter="cast", out=out)
+        cold.append(time.perf_counter() - t0)
+        t0 = time.perf_counter()
+        orc.bmm_chain_fused_f32(A, B, D, inter="cast", out=out)
+        warm.append(time.perf_counter() - t0)
+    fl = 2.0 * 512 * 64 * (64 + 64)
+    mean = sum(cold) / len(cold)
+    return {"us_per_call": mean * 1e6, "gflops": fl / mean / 1e9, "us_per_call_caches_warm": min(warm) * 1e6,
+            "cores": orc.num_threads(),
+            "sample": "%d calls of the fp32 GEMM chain 512x64.64x64.64x64 through the fused CPU loop nest, "
+                      "128 MiB streamed between calls" % repeats}
 
 
 def run_one(name, steps, warmup, dev, long_run=False):
@@ -298,7 +370,7 @@ def run_one(name, steps, warmup, dev, long_run=False):
     else:
         gbs = by / (k_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS}
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
+    roof["traffic"] = measured_traffic(name, tile["variant"])
     roof["algorithmic_flops"] = fl
     roof["algorithmic_bytes"] = by
     roof["kernel_ms"] = k_ms
