@@ -22,7 +22,9 @@ import os
 from ... import _lib, chain
 from ...hardware import query_hw_param
 
-FP_VARIANT_CODES = (1, 2, 8)  # rows-per-wave code of the fp16/bf16 chain kernels
+# kernel codes of the fp16/bf16 chain: four waves x 32 | 64 rows, eight waves x 32 rows (staggered phases,
+# software pipelined, on the 16x16x32 MFMA: the library refuses that one unless B is stored [L][K])
+FP_VARIANT_CODES = (1, 2, 8, 9, 6)
 
 
 class TuneEntry:

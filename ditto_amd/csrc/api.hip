@@ -11,6 +11,7 @@
 #include <mutex>
 
 #include "bmm_chain_fp8.h"
+#include "bmm_chain_fp8m16.h"
 #include "chain_kernels.h"
 
 namespace {
@@ -127,36 +128,47 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     plan->family = 0;
     plan->d_pad = dmax <= 64 ? 64 : 128;
     const int cus = need_device ? device_cus() : 256;
-    // Variant table (measured on MI355X, bf16 attention shapes).  With n8 = number of 256-row
-    // workgroups: the eight-wave kernel (two waves per SIMD) wins once n8 fills 3/4 of the CUs;
-    // below that the four-wave kernel with 128-row workgroups spreads over more CUs.  For
-    // head_pad 128 and n8 >= 2 CUs the two are within noise and the four-wave, 256-row kernel
-    // (half the LDS fragment traffic) is kept.
-    // Without a softmax between the contractions (nothing for a second wave to overlap) the
-    // four-wave, 256-row kernel also wins at head_pad 64 once n8 >= 2 CUs (249 vs 274 us at
-    // 64 x 4096 x 64 x 4096 x 64, bf16).
+    // Variant table (measured on MI355X, fp16 and bf16, head_pad 64 and 128).  n8 = number of 256-row
+    // workgroups.  Below 3/4 of the CUs the four-wave kernel with 128-row workgroups spreads over more
+    // CUs.  From there on eight waves (two per SIMD) win, in their software-pipelined form (9) at every
+    // size measured.  Once there are two workgroups per CU the chip runs at its power limit and the
+    // kernel on the 16x16x32 MFMA (6; B stored [L][K] only), which needs less energy per flop, is ahead
+    // (64 x 4096 x 4096 x 128 bf16: 464 vs 484 us with the softmax, 410 vs 443 us without); the
+    // exception is head_pad 64 with the softmax (306 vs 314 us).  With B stored [K][L] and no softmax
+    // (nothing for a second wave per SIMD to overlap) the four-wave, 256-row kernel stays (429 vs 443 us).
     const long long n8 = ((d->M + 255) / 256) * d->batch;
-    const bool many = n8 >= 2LL * cus && (plan->d_pad == 128 || d->inter_op != DITTO_INTER_SOFTMAX);
-    if (n8 * 4 >= 3LL * cus && !many)
-      plan->qt = 8;
-    else
-      plan->qt = (n8 >= 2LL * cus) ? 2 : 1;
+    const bool sm = d->inter_op == DITTO_INTER_SOFTMAX;
+    if (n8 >= 2LL * cus) {
+      if (d->b_layout == DITTO_B_LK)
+        plan->qt = (sm && plan->d_pad == 64) ? 9 : 6;
+      else
+        plan->qt = sm ? 9 : 2;
+    } else if (n8 * 4 >= 3LL * cus) {
+      plan->qt = 9;
+    } else {
+      plan->qt = 1;
+    }
     if (d->tile_variant != 0) {
       const int q = d->tile_variant % 10;
-      if (d->tile_variant / 10 != plan->d_pad || (q != 1 && q != 2 && q != 8))
-        return fail(DITTO_EINVAL, "tile_variant %d cannot run this shape (head_pad %d; q must be 1, 2 or 8)",
+      if (d->tile_variant / 10 != plan->d_pad || (q != 1 && q != 2 && q != 8 && q != 9 && q != 6))
+        return fail(DITTO_EINVAL, "tile_variant %d cannot run this shape (head_pad %d; q must be 1, 2, 6, 8 or 9)",
                     d->tile_variant, plan->d_pad);
+      if (q == 6 && d->b_layout != DITTO_B_LK)
+        return fail(DITTO_EINVAL, "tile_variant %d (16x16x32 MFMA kernel) takes B stored [L][K]", d->tile_variant);
       plan->qt = q;
     }
     const bool kl = d->b_layout == DITTO_B_KL;
-    const int bm = plan->qt == 8 ? 256 : 128 * plan->qt;
+    const bool eight = plan->qt >= 6;  // 6, 8, 9: eight waves owning 32 rows each
+    const int bm = eight ? 256 : 128 * plan->qt;
     ditto_tile_param& t = plan->tile;
-    t.block_threads = plan->qt == 8 ? 512 : 256;
+    t.block_threads = eight ? 512 : 256;
     t.block_m = bm;
     t.block_l = ditto::kBN;
     t.block_n = (int)d->N;
     t.head_pad = plan->d_pad;
-    if (plan->qt == 8)
+    if (plan->qt == 6)
+      t.lds_bytes = plan->d_pad == 64 ? ditto::bmm_chain8m16_lds_bytes<64>() : ditto::bmm_chain8m16_lds_bytes<128>();
+    else if (eight)
       t.lds_bytes = plan->d_pad == 64 ? (kl ? ditto::bmm_chain8_lds_bytes<64, true>() : ditto::bmm_chain8_lds_bytes<64, false>())
                                       : (kl ? ditto::bmm_chain8_lds_bytes<128, true>() : ditto::bmm_chain8_lds_bytes<128, false>());
     else

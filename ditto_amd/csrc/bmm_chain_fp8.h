@@ -21,6 +21,15 @@
 //   transposition  raw C(it+1) -> fragment-major C(it+1); raw B(it+2) -> fragment-major B(it+2)
 //   compute        waves 0-3: S(it) = B(it)^T.A^T, inter op, F^T += C(it)^T.P(it)^T
 //                  waves 4-7: inter op on S(it), F^T += C(it)^T.P(it)^T, S(it+1)
+//
+// PIPE = true is the software-pipelined form of the compute part.  Above, a wave alternates between
+// MFMA-only and vector-only phases and the overlap comes from running the two waves of a SIMD half a
+// tile apart; the phases differ in length, so the waves drift and one of them waits at every barrier.
+// Pipelined, every wave runs the SAME stream in half steps of 32 rows of the L tile, as the four-wave
+// kernel does: while the matrix pipe computes the scores of the next half, the vector ALU
+// exponentiates the current one, a few vector instructions behind every MFMA (an MFMA holds the vector
+// issue port for about 12 of its 32 cycles, which leaves the two waves of a SIMD five vector issue
+// slots per MFMA).  The waves stay level and reach the barrier together.
 #pragma once
 #include "bmm_chain_fp.h"
 
@@ -39,7 +48,7 @@ __host__ __device__ constexpr int bmm_chain8_lds_bytes() {
   return ((B_KL ? 6 : 4) + bmm_chain8_raw_c_tiles<D, B_KL>() + 2) * kBN * D * 2;
 }
 
-template <typename T, int D, int INTER, bool B_KL>
+template <typename T, int D, int INTER, bool B_KL, bool PIPE = false>
 __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef typename Elem<T>::v8 V8;
@@ -76,7 +85,7 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
   // The two waves of a SIMD (w and w+4) run half a tile apart: the "late" wave computes the
   // scores of tile it+1 at the END of step it, so its softmax of step it+1 runs while the
   // other wave's MFMAs occupy the matrix pipe, and vice versa.
-  const bool late = wave >= 4;
+  const bool late = !PIPE && wave >= 4;
 
   const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
   const int mb = lid % p.mblocks;
@@ -339,6 +348,128 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
     __syncthreads();
   };
 
+
+  // ======== pipelined form (PIPE) ========
+  // sa / sb alternate as the finished half (`cur`) and the half being computed (`nxt`); mxn is the scaled
+  // row maximum of `cur`.
+  f32x16 sa, sb;
+  float mxn = -INFINITY;
+  auto b_frag = [&](int off, int i, int st) __attribute__((always_inline)) -> V8 {
+    return B_KL ? frag_rd(off, i * NS + st) : b_frag_row(off, i, st);
+  };
+  // scores of rows past L are masked out (softmax only; the other chains see zero operands)
+  auto mask_tail = [&](f32x16& sc, int l0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int l = l0 + 8 * (r >> 2) + 4 * g + (r & 3);
+      if (l >= L) sc[r] = -INFINITY;
+    }
+  };
+  auto row_max = [&](const f32x16& sc) __attribute__((always_inline)) {
+    float mx = sc[0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sc[r]);
+    mxn = pair_max(mx) * c2;
+  };
+  // probabilities of registers [r0, r1) of the half tile
+  auto exp_range = [&](f32x16& sc, int r0, int r1) __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = r0; r < r1; ++r) sc[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[r], c2, -mrow));
+  };
+  // operand of the second contraction for sixteen rows of the L tile: registers 8 * u2 .. + 7 of the half,
+  // cast; the row sum is taken over the ROUNDED values, exactly what enters the MFMA
+  auto make_p = [&](const f32x16& sc, int u2, V8& pf) __attribute__((always_inline)) {
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[e] = sc[8 * u2 + e];
+      if (INTER != kInterSoftmax && p.relu) v[e] = fmaxf(v[e], 0.f);
+    }
+    V2 p0 = cvt2<T>(v[0], v[1]), p1 = cvt2<T>(v[2], v[3]), p2 = cvt2<T>(v[4], v[5]), p3 = cvt2<T>(v[6], v[7]);
+    if constexpr (INTER == kInterSoftmax) {
+      lsum = Elem<T>::add_pair(p0, lsum);
+      lsum = Elem<T>::add_pair(p1, lsum);
+      lsum = Elem<T>::add_pair(p2, lsum);
+      lsum = Elem<T>::add_pair(p3, lsum);
+    }
+    pf = V8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+  };
+  // One half step: consumes `cur` (half hh of tile it) and produces `nxt` (half 1 of the same tile, or
+  // half 0 of tile it + 1; past the last tile that is a tile of zeros whose scores nothing reads).
+  // NS MFMAs of the first contraction, then two sixteen-row steps x NT column tiles of the second.
+  // Of the sixteen exponentials per lane EA run behind the first contraction's MFMAs (at least the eight
+  // that the first sixteen-row step needs), the rest behind the first NT MFMAs of the second.
+  constexpr int NG = NS + 2 * NT;
+  constexpr int EA = D == 128 ? 12 : 10;
+  static_assert(EA >= 8 && EA <= 16, "the first sixteen-row step needs its eight probabilities");
+  auto half_step = [&](f32x16& cur, f32x16& nxt, int it, auto j_c, auto hh_c) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value, hh = decltype(hh_c)::value;
+    constexpr int BNX = B_USE + (hh ? (J + 1) % 4 : J) * TB;  // B tile of the next half
+    constexpr int CF = C_FRAG + (J & 1) * TB;
+    if constexpr (INTER == kInterSoftmax) {
+      // lazy rescale: raise the running maximum only when a row of the wave exceeds it by 2^kLazy
+      if (__builtin_amdgcn_ballot_w64(mxn > mrow + kLazy) != 0) {
+        const float mnew = fmaxf(mrow, mxn);
+        const float alpha = __builtin_amdgcn_exp2f(mrow - mnew);
+        mrow = mnew;
+        lsum *= alpha;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
+      }
+    }
+    V8 fr[NG];
+    auto fetch = [&](int k) __attribute__((always_inline)) {
+      fr[k] = k < NS ? b_frag(BNX, hh ^ 1, k) : frag_rd(CF, (2 * hh + (k - NS) / NT) * NT + (k - NS) % NT);
+    };
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) fetch(k);
+    V8 pf[2];
+#pragma unroll
+    for (int k = 0; k < NG; ++k) {
+      if (k + kAhead < NG) fetch(k + kAhead);
+      __builtin_amdgcn_sched_barrier(0);
+      if (k == 0) {
+        const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        nxt = Elem<T>::mfma32(fr[k], af[k], z);
+      } else if (k < NS) {
+        nxt = Elem<T>::mfma32(fr[k], af[k], nxt);
+      } else {
+        o[(k - NS) % NT] = Elem<T>::mfma32(fr[k], pf[(k - NS) / NT], o[(k - NS) % NT]);
+      }
+      if constexpr (INTER == kInterSoftmax) {
+        if (k < NS) exp_range(cur, k * EA / NS, (k + 1) * EA / NS);
+        else if (k < NS + NT) exp_range(cur, EA + (k - NS) * (16 - EA) / NT, EA + (k - NS + 1) * (16 - EA) / NT);
+      }
+      if (k == NS - 1) make_p(cur, 0, pf[0]);
+      if (k == NS + NT - 1) make_p(cur, 1, pf[1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (INTER == kInterSoftmax) {
+      const int nt = hh ? it + 1 : it;  // tile of the next half
+      if (ragged && nt == ntiles - 1) mask_tail(nxt, nt * kBN + 32 * (hh ^ 1));
+      row_max(nxt);
+    }
+  };
+  auto tile_step_pipe = [&](int it, auto j_c) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value;
+    constexpr int PAR = J & 1;
+    V8 xb[NTR], xc[NTR];
+    load_c(it + C_AHEAD, NCR == 4 ? (J + 3) % 4 : PAR);
+    load_b(it + B_AHEAD, B_KL ? (PAR ^ 1) : (J + 3) % 4);
+    if (B_KL) tr_read_b(B_LOAD + PAR * TB, xb);
+    tr_read_c(C_RAW + (NCR == 4 ? (J + 1) % 4 : (PAR ^ 1)) * TB, xc);
+    half_step(sa, sb, it, j_c, IntC<0>{});
+    if (B_KL) tr_write(B_FRAG + ((J + 2) % 4) * TB, xb);
+    tr_write(C_FRAG + (PAR ^ 1) * TB, xc);
+    half_step(sb, sa, it, j_c, IntC<1>{});
+    if (B_KL) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if (NCR == 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLD) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
+    __syncthreads();
+  };
+
   // ---- prologue: first tiles in flight, first transposition(s), the late waves' first scores
   load_b(0, 0);
   load_b(1, 1);
@@ -362,14 +493,39 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
     }
   }
   if (late) scores(IntC<B_USE>{});
+  if constexpr (PIPE) {  // scores of the very first half
+#pragma unroll
+    for (int k = 0; k < NS; ++k) {
+      const V8 bf = b_frag(B_USE, 0, k);
+      if (k == 0) {
+        const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        sa = Elem<T>::mfma32(bf, af[k], z);
+      } else {
+        sa = Elem<T>::mfma32(bf, af[k], sa);
+      }
+    }
+    if constexpr (INTER == kInterSoftmax) {
+      if (ragged && ntiles == 1) mask_tail(sa, 0);
+      row_max(sa);
+    }
+  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  for (int it = 0; it < ntiles; it += 4) {
-    tile_step(it, IntC<0>{});
-    if (it + 1 < ntiles) tile_step(it + 1, IntC<1>{});
-    if (it + 2 < ntiles) tile_step(it + 2, IntC<2>{});
-    if (it + 3 < ntiles) tile_step(it + 3, IntC<3>{});
+  if constexpr (PIPE) {
+    for (int it = 0; it < ntiles; it += 4) {
+      tile_step_pipe(it, IntC<0>{});
+      if (it + 1 < ntiles) tile_step_pipe(it + 1, IntC<1>{});
+      if (it + 2 < ntiles) tile_step_pipe(it + 2, IntC<2>{});
+      if (it + 3 < ntiles) tile_step_pipe(it + 3, IntC<3>{});
+    }
+  } else {
+    for (int it = 0; it < ntiles; it += 4) {
+      tile_step(it, IntC<0>{});
+      if (it + 1 < ntiles) tile_step(it + 1, IntC<1>{});
+      if (it + 2 < ntiles) tile_step(it + 2, IntC<2>{});
+      if (it + 3 < ntiles) tile_step(it + 3, IntC<3>{});
+    }
   }
 
   // ---- epilogue: normalise (softmax), cast, store 4 contiguous columns per lane
@@ -402,10 +558,10 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
 #endif
 }
 
-template <typename T, int D, int INTER, bool B_KL>
+template <typename T, int D, int INTER, bool B_KL, bool PIPE = false>
 hipError_t launch_bmm_chain8(const BmmChainArgs& args, hipStream_t stream) {
   constexpr int lds = bmm_chain8_lds_bytes<D, B_KL>();
-  auto kern = bmm_chain8_kernel<T, D, INTER, B_KL>;
+  auto kern = bmm_chain8_kernel<T, D, INTER, B_KL, PIPE>;
   static thread_local int configured_dev = -1;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);

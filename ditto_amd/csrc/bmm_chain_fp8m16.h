@@ -1,0 +1,529 @@
+// Eight-wave fused two-contraction chain on the 16x16x32 MFMA (see bmm_chain_fp.h for the chain and the
+// transposed formulation, bmm_chain_fp8.h for the eight-wave workgroup and the once-per-workgroup
+// transposition of the C tile into fragment-major order).
+//
+// Why another tile shape: on N(0,1) operands this device runs matrix code against its power limit, not
+// against its clock (the same kernel on zero operands is a quarter faster), so what counts is energy per
+// flop, and v_mfma_f32_16x16x32 needs about 14 % less of it than v_mfma_f32_32x32x16 (a loop of either,
+// random bf16 operands, two waves per SIMD: 16.1 against 18.9 ns per 32768 flop per SIMD): it reads and
+// writes a quarter of the accumulator registers per instruction.  A wave still owns 32 rows of A (two
+// column tiles of 16), so every operand fragment read from LDS feeds two MFMAs and LDS traffic, register
+// count and the number of direct loads are those of the 32x32x16 kernels.
+//
+// Layouts (lane = 16 * q + c, q = 0..3, c = 0..15):
+//   v_mfma_f32_16x16x32:  A[16][32]: lane holds A[c][8q .. 8q+7];  B[32][16]: lane holds B[8q .. 8q+7][c];
+//                         acc[r] = C[4q + r][c], r = 0..3.
+//   first contraction, transposed:  S^T[l][m] = sum_k B^T[l][k] A^T[k][m]
+//       A operand  = 16 rows l of the B tile (stored [L][K]: one 16-byte read per lane),
+//       B operand  = rows m of A from registers (lane: row 16j + c, 8 consecutive k),
+//       result     = lane (c, q) holds S^T[16i + 4q + r][16j + c]: four consecutive l of row m.
+//   second contraction, transposed:  F^T[n][m] = sum_l C^T[n][l] P^T[l][m] over the 32 rows of a half tile
+//       B operand  = P^T from the accumulators above: slot e < 4 is row 4q + e of the first 16-row tile,
+//                    slot e >= 4 row 4q + e - 4 of the second, i.e. contraction slot 8q + e <-> row
+//                    pi(8q + e) = 4q + e (e < 4), 16 + 4q + e - 4 (e >= 4);
+//       A operand  = C^T with its rows taken in the same order pi: lane (n = c, q) holds
+//                    C[pi(8q + e)][16t + c], e = 0..7: two transposing reads of 4 rows x 16 columns, done once
+//                    per workgroup by the wave that owns the fragment and written back fragment major.
+//
+// Softmax: a lane holds eight scores of each of two rows per half tile.  The running maximum of a row is
+// shared by its four lanes and raised lazily; whether it has to be raised is decided from the lanes' LOCAL
+// maxima (a ballot), so the usual case needs no exchange between lanes at all; the exchange
+// (v_permlane16_swap, v_permlane32_swap) runs only in the rare rescale.
+#pragma once
+#include "bmm_chain_fp8.h"
+
+namespace ditto {
+
+template <int D>
+__host__ __device__ constexpr int bmm_chain8m16_lds_bytes() {
+  // B tiles as loaded [4], raw C tiles [2 or 4], fragment-major C tiles [2]
+  return (4 + (D == 64 ? 4 : 2) + 2) * kBN * D * 2;
+}
+
+template <typename T>
+struct Mfma16;
+template <>
+struct Mfma16<f16> {
+  static __device__ __forceinline__ f32x4 run(f16x8 a, f16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma16<bf16> {
+  static __device__ __forceinline__ f32x4 run(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+// The output accumulators live in FIXED registers, v[4 i : 4 i + 3] for accumulator i, and every instruction
+// that writes them is written out in inline asm with that register as a tied operand.  Left to itself the
+// compiler gives an MFMA's result another register than the accumulator came in (it likes to reuse the first
+// operand's) and computes the rare rescale into fresh registers, so the accumulators change places and the
+// common path of every branch copies all 64 of them back, every half step.  MFMAs in inline asm are outside
+// the compiler's hazard bookkeeping: the next reader of an accumulator is its own MFMA of the next half step;
+// the rare rescale and the epilogue wait out the pipeline first (mfma_drain).
+__device__ __forceinline__ void acc_mfma(int i, bf16x8 a, bf16x8 b, f32x4 (&o)[16]) {
+  switch (i) {
+    case 0: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[0:3]}"(o[0]) : "v"(a), "v"(b)); break;
+    case 1: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[4:7]}"(o[1]) : "v"(a), "v"(b)); break;
+    case 2: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[8:11]}"(o[2]) : "v"(a), "v"(b)); break;
+    case 3: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[12:15]}"(o[3]) : "v"(a), "v"(b)); break;
+    case 4: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[16:19]}"(o[4]) : "v"(a), "v"(b)); break;
+    case 5: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[20:23]}"(o[5]) : "v"(a), "v"(b)); break;
+    case 6: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[24:27]}"(o[6]) : "v"(a), "v"(b)); break;
+    case 7: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[28:31]}"(o[7]) : "v"(a), "v"(b)); break;
+    case 8: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[32:35]}"(o[8]) : "v"(a), "v"(b)); break;
+    case 9: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[36:39]}"(o[9]) : "v"(a), "v"(b)); break;
+    case 10: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[40:43]}"(o[10]) : "v"(a), "v"(b)); break;
+    case 11: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[44:47]}"(o[11]) : "v"(a), "v"(b)); break;
+    case 12: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[48:51]}"(o[12]) : "v"(a), "v"(b)); break;
+    case 13: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[52:55]}"(o[13]) : "v"(a), "v"(b)); break;
+    case 14: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[56:59]}"(o[14]) : "v"(a), "v"(b)); break;
+    case 15: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[60:63]}"(o[15]) : "v"(a), "v"(b)); break;
+  }
+}
+__device__ __forceinline__ void acc_mfma(int i, f16x8 a, f16x8 b, f32x4 (&o)[16]) {
+  switch (i) {
+    case 0: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[0:3]}"(o[0]) : "v"(a), "v"(b)); break;
+    case 1: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[4:7]}"(o[1]) : "v"(a), "v"(b)); break;
+    case 2: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[8:11]}"(o[2]) : "v"(a), "v"(b)); break;
+    case 3: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[12:15]}"(o[3]) : "v"(a), "v"(b)); break;
+    case 4: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[16:19]}"(o[4]) : "v"(a), "v"(b)); break;
+    case 5: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[20:23]}"(o[5]) : "v"(a), "v"(b)); break;
+    case 6: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[24:27]}"(o[6]) : "v"(a), "v"(b)); break;
+    case 7: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[28:31]}"(o[7]) : "v"(a), "v"(b)); break;
+    case 8: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[32:35]}"(o[8]) : "v"(a), "v"(b)); break;
+    case 9: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[36:39]}"(o[9]) : "v"(a), "v"(b)); break;
+    case 10: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[40:43]}"(o[10]) : "v"(a), "v"(b)); break;
+    case 11: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[44:47]}"(o[11]) : "v"(a), "v"(b)); break;
+    case 12: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[48:51]}"(o[12]) : "v"(a), "v"(b)); break;
+    case 13: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[52:55]}"(o[13]) : "v"(a), "v"(b)); break;
+    case 14: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[56:59]}"(o[14]) : "v"(a), "v"(b)); break;
+    case 15: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[60:63]}"(o[15]) : "v"(a), "v"(b)); break;
+  }
+}
+__device__ __forceinline__ void acc_scale(int i, float alpha, f32x4 (&o)[16]) {
+  switch (i) {
+    case 0: asm volatile("v_mul_f32 v0, %1, v0\n\tv_mul_f32 v1, %1, v1\n\tv_mul_f32 v2, %1, v2\n\tv_mul_f32 v3, %1, v3" : "+{v[0:3]}"(o[0]) : "v"(alpha)); break;
+    case 1: asm volatile("v_mul_f32 v4, %1, v4\n\tv_mul_f32 v5, %1, v5\n\tv_mul_f32 v6, %1, v6\n\tv_mul_f32 v7, %1, v7" : "+{v[4:7]}"(o[1]) : "v"(alpha)); break;
+    case 2: asm volatile("v_mul_f32 v8, %1, v8\n\tv_mul_f32 v9, %1, v9\n\tv_mul_f32 v10, %1, v10\n\tv_mul_f32 v11, %1, v11" : "+{v[8:11]}"(o[2]) : "v"(alpha)); break;
+    case 3: asm volatile("v_mul_f32 v12, %1, v12\n\tv_mul_f32 v13, %1, v13\n\tv_mul_f32 v14, %1, v14\n\tv_mul_f32 v15, %1, v15" : "+{v[12:15]}"(o[3]) : "v"(alpha)); break;
+    case 4: asm volatile("v_mul_f32 v16, %1, v16\n\tv_mul_f32 v17, %1, v17\n\tv_mul_f32 v18, %1, v18\n\tv_mul_f32 v19, %1, v19" : "+{v[16:19]}"(o[4]) : "v"(alpha)); break;
+    case 5: asm volatile("v_mul_f32 v20, %1, v20\n\tv_mul_f32 v21, %1, v21\n\tv_mul_f32 v22, %1, v22\n\tv_mul_f32 v23, %1, v23" : "+{v[20:23]}"(o[5]) : "v"(alpha)); break;
+    case 6: asm volatile("v_mul_f32 v24, %1, v24\n\tv_mul_f32 v25, %1, v25\n\tv_mul_f32 v26, %1, v26\n\tv_mul_f32 v27, %1, v27" : "+{v[24:27]}"(o[6]) : "v"(alpha)); break;
+    case 7: asm volatile("v_mul_f32 v28, %1, v28\n\tv_mul_f32 v29, %1, v29\n\tv_mul_f32 v30, %1, v30\n\tv_mul_f32 v31, %1, v31" : "+{v[28:31]}"(o[7]) : "v"(alpha)); break;
+    case 8: asm volatile("v_mul_f32 v32, %1, v32\n\tv_mul_f32 v33, %1, v33\n\tv_mul_f32 v34, %1, v34\n\tv_mul_f32 v35, %1, v35" : "+{v[32:35]}"(o[8]) : "v"(alpha)); break;
+    case 9: asm volatile("v_mul_f32 v36, %1, v36\n\tv_mul_f32 v37, %1, v37\n\tv_mul_f32 v38, %1, v38\n\tv_mul_f32 v39, %1, v39" : "+{v[36:39]}"(o[9]) : "v"(alpha)); break;
+    case 10: asm volatile("v_mul_f32 v40, %1, v40\n\tv_mul_f32 v41, %1, v41\n\tv_mul_f32 v42, %1, v42\n\tv_mul_f32 v43, %1, v43" : "+{v[40:43]}"(o[10]) : "v"(alpha)); break;
+    case 11: asm volatile("v_mul_f32 v44, %1, v44\n\tv_mul_f32 v45, %1, v45\n\tv_mul_f32 v46, %1, v46\n\tv_mul_f32 v47, %1, v47" : "+{v[44:47]}"(o[11]) : "v"(alpha)); break;
+    case 12: asm volatile("v_mul_f32 v48, %1, v48\n\tv_mul_f32 v49, %1, v49\n\tv_mul_f32 v50, %1, v50\n\tv_mul_f32 v51, %1, v51" : "+{v[48:51]}"(o[12]) : "v"(alpha)); break;
+    case 13: asm volatile("v_mul_f32 v52, %1, v52\n\tv_mul_f32 v53, %1, v53\n\tv_mul_f32 v54, %1, v54\n\tv_mul_f32 v55, %1, v55" : "+{v[52:55]}"(o[13]) : "v"(alpha)); break;
+    case 14: asm volatile("v_mul_f32 v56, %1, v56\n\tv_mul_f32 v57, %1, v57\n\tv_mul_f32 v58, %1, v58\n\tv_mul_f32 v59, %1, v59" : "+{v[56:59]}"(o[14]) : "v"(alpha)); break;
+    case 15: asm volatile("v_mul_f32 v60, %1, v60\n\tv_mul_f32 v61, %1, v61\n\tv_mul_f32 v62, %1, v62\n\tv_mul_f32 v63, %1, v63" : "+{v[60:63]}"(o[15]) : "v"(alpha)); break;
+  }
+}
+// every MFMA issued so far has written its result (a 16x16x32 MFMA takes four passes; sixteen idle cycles
+// cover the last one and its write-back)
+__device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 7" ::: "memory"); }
+
+// maximum over the four lanes c, c + 16, c + 32, c + 48 (every lane gets it).
+// v_permlane16_swap a, b swaps the odd rows of 16 lanes of a with the even rows of b; from a == b == x,
+// max(a, b) holds max(x[row 0], x[row 1]) in rows 0 and 1 and max(x[row 2], x[row 3]) in rows 2 and 3.
+__device__ __forceinline__ float quad_max(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return pair_max(fmaxf(a, b));
+}
+__device__ __forceinline__ float quad_sum(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return pair_sum(a + b);
+}
+
+template <typename T, int D, int INTER>
+__global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef typename Elem<T>::v8 V8;
+  typedef typename Elem<T>::v4 V4;
+  typedef typename Elem<T>::v2 V2;
+  constexpr int NW = 8, BM = NW * 32;
+  constexpr int TB = kBN * D * 2;     // bytes per tile
+  constexpr int B_RB = D * 2;         // bytes per LDS row of a B tile ([L][K])
+  constexpr int B_CPR = B_RB / 16;
+  constexpr int C_RB = D * 2;
+  constexpr int C_CPR = C_RB / 16;
+  constexpr int NS = D / 32;          // k steps of the first contraction
+  constexpr int NTN = D / 16;         // column tiles of the second contraction
+  constexpr int NFRAG = 2 * NTN;      // C fragments per tile: two 32-row halves x NTN column tiles
+  constexpr int NLD = TB / 1024 / NW; // direct loads per wave per tile
+  constexpr int NTR = NFRAG / NW;     // fragments each wave transposes per tile
+  static_assert(NLD >= 1 && NTR >= 1, "tile too small for eight waves");
+  constexpr int NCR = D == 64 ? 4 : 2;
+  constexpr int B_LOAD = 0;                   // [4] row-read layout
+  constexpr int C_RAW = 4 * TB;               // [NCR]
+  constexpr int C_FRAG = C_RAW + NCR * TB;    // [2]
+  constexpr int B_AHEAD = 3;
+  constexpr int C_AHEAD = NCR == 4 ? 3 : 2;
+
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c16 = lane & 15, q = lane >> 4;
+
+  const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int mb = lid % p.mblocks;
+  const int bz = lid / p.mblocks;
+  const int zo = bz / p.batch_inner, zi = bz - zo * p.batch_inner;
+  const T* __restrict__ Ag = reinterpret_cast<const T*>(p.a) + zo * p.a_bs2 + zi * p.a_bs;
+  const T* Bg = reinterpret_cast<const T*>(p.b) + zo * p.b_bs2 + zi * p.b_bs;
+  const T* Cg = reinterpret_cast<const T*>(p.c) + zo * p.c_bs2 + zi * p.c_bs;
+  const int m_wave = mb * BM + wave * 32;
+  const int M = p.M, N = p.N, K = p.K, L = p.L;
+
+  const unsigned b_bytes = (unsigned)((long long)(L - 1) * p.b_rs + K) * 2u;
+  const unsigned c_bytes = (unsigned)((long long)(L - 1) * p.c_rs + N) * 2u;
+  const i32x4 b_rsrc = make_rsrc(Bg, b_bytes);
+  const i32x4 c_rsrc = make_rsrc(Cg, c_bytes);
+  const unsigned lds0 = (unsigned)(size_t)(DITTO_LDS char*)smem_raw;
+
+  // ---- per-lane source offsets of the direct loads (the swizzles of the other kernels)
+  int b_voff[NLD], c_voff[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; ++i) {
+    const int gi = NLD * wave + i;
+    {
+      const int row = gi * (64 / B_CPR) + lane / B_CPR, pc = lane % B_CPR;
+      const int cl = pc ^ swz_rowread<B_CPR>(row);  // rows are l, columns k
+      b_voff[i] = cl * 8 < K ? (row * p.b_rs + cl * 8) * 2 : (int)b_bytes;
+    }
+    {
+      const int row = gi * (64 / C_CPR) + lane / C_CPR, pc = lane % C_CPR;
+      const int cl = pc ^ swz_trread<C_CPR>(row);
+      c_voff[i] = cl * 8 < N ? (row * p.c_rs + cl * 8) * 2 : (int)c_bytes;
+    }
+  }
+  auto load_b = [&](int tile, int buf) __attribute__((always_inline)) {
+    const int soff = tile * kBN * p.b_rs * 2;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i)
+      lds_dma_16(b_rsrc, (unsigned)(b_voff[i] + soff), lds0 + B_LOAD + buf * TB + 1024 * (NLD * wave + i));
+  };
+  auto load_c = [&](int tile, int buf) __attribute__((always_inline)) {
+    const int soff = tile * kBN * p.c_rs * 2;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i)
+      lds_dma_16(c_rsrc, (unsigned)(c_voff[i] + soff), lds0 + C_RAW + buf * TB + 1024 * (NLD * wave + i));
+  };
+
+  // ---- per-lane LDS read addresses (bytes within a tile), loop invariant
+  // B fragment (i = 16-row tile of the 64-row L tile, st = k step): row 16 i + c, logical chunks 4 st + q
+  // (256-byte rows: the swizzle of row 16 i + c does not depend on i, so the tile index is a constant offset)
+  constexpr int NBI = B_CPR == 16 ? 1 : 4;
+  int b_ad[NBI][NS];
+#pragma unroll
+  for (int i = 0; i < NBI; ++i)
+#pragma unroll
+    for (int st = 0; st < NS; ++st)
+      b_ad[i][st] = (16 * i + c16) * B_RB + (((4 * st + q) ^ swz_rowread<B_CPR>(16 * i + c16)) * 16);
+  // Fragment-major and raw C tiles lie beyond the 64 KB an LDS instruction's offset field reaches: each
+  // region gets ONE base register, kept opaque so that the compiler folds only the small remainder into the
+  // instructions' offsets (it otherwise makes an address register per buffer and fragment, and spills)
+  int frag_ad = lane * 16 + C_FRAG;
+  asm volatile("" : "+v"(frag_ad));
+  auto b_frag = [&](int off, int i, int st) __attribute__((always_inline)) -> V8 {
+    if (NBI == 1) return *reinterpret_cast<const V8*>(smem_raw + b_ad[0][st] + (off + 16 * i * B_RB));
+    return *reinterpret_cast<const V8*>(smem_raw + b_ad[i % NBI][st] + off);
+  };
+  auto frag_rd = [&](int off, int f) __attribute__((always_inline)) -> V8 {
+    return *reinterpret_cast<const V8*>(smem_raw + frag_ad + (off - C_FRAG + 1024 * f));
+  };
+  // This wave's share of the transposition of one C tile: fragments NTR * wave .. + NTR - 1, fragment
+  // f = hh * NTN + t (hh: 32-row half, t: 16-column tile).  The 16 lanes of group q read rows
+  // 32 hh + 4 q + {0..3} (and + 16) x columns 16 t .. 16 t + 15: lane s of the group points at row s / 4,
+  // 8 bytes at column 4 (s % 4).
+  int ctr_ad[NTR], fw_ad[NTR];
+#pragma unroll
+  for (int i = 0; i < NTR; ++i) {
+    const int f = NTR * wave + i;
+    const int hh = f / NTN, t = f % NTN;
+    const int row = 32 * hh + 4 * q + (c16 >> 2);
+    const int chunk = 2 * t + ((c16 & 3) >> 1);
+    // (rows row and row + 16 share their swizzle: it depends on row % 4 only)
+    ctr_ad[i] = row * C_RB + ((chunk ^ swz_trread<C_CPR>(row)) * 16) + 8 * (c16 & 1) + C_RAW;
+    fw_ad[i] = frag_ad + 1024 * f;
+    asm volatile("" : "+v"(ctr_ad[i]), "+v"(fw_ad[i]));
+  }
+  auto tr_read_c = [&](int raw_off, V8* x) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NTR; ++i) {
+      const char* a = smem_raw + ctr_ad[i] + (raw_off - C_RAW);
+      V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(a));
+      V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(a + 16 * C_RB));
+      x[i] = concat4<V4, V8>(lo, hi);
+    }
+  };
+  auto tr_write = [&](int frag_off, const V8* x) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NTR; ++i) *reinterpret_cast<V8*>(smem_raw + fw_ad[i] + (frag_off - C_FRAG)) = x[i];
+  };
+
+  // ---- A fragments (B operand of the first contraction): lane holds A[16 j + c][32 st + 8 q .. + 7]
+  V8 af[2][NS];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int row = m_wave + 16 * j + c16;
+#pragma unroll
+    for (int st = 0; st < NS; ++st) {
+      const int col = 32 * st + 8 * q;
+      V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (row < M && col < K) v = *reinterpret_cast<const V8*>(Ag + (long long)row * p.a_rs + col);
+      af[j][st] = v;
+    }
+  }
+
+  // ---- accumulators of F^T: o[t][j][r] = F^T[16 t + 4 q + r][16 j + c]
+  // (flat: accumulator 2 t + j, pinned to v[4 (2 t + j) : +3], see acc_mfma)
+  static_assert(2 * NTN <= 16, "sixteen pinned accumulators");
+  f32x4 o[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // softmax state of the lane's two rows: running maximum (exp2 domain; the same in the four lanes of a
+  // row), the lane's share of the row sum, and the lane's LOCAL scaled maximum of the half about to be consumed
+  float mrow[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f}, mloc[2] = {-INFINITY, -INFINITY};
+  const float c2 = p.scale_log2;
+  const int ntiles = (L + kBN - 1) / kBN;
+  const bool ragged = (L % kBN) != 0;
+
+  // A half tile of scores: sc[i][j] = 16-row tile i x row tile j
+  struct Half {
+    f32x4 v[2][2];
+  };
+  Half sa, sb;
+  auto mask_tail = [&](Half& h, int l0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (l0 + 16 * i + 4 * q + r >= L) {
+          h.v[i][0][r] = -INFINITY;
+          h.v[i][1][r] = -INFINITY;
+        }
+  };
+  auto local_max = [&](const Half& h) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      float mx = h.v[0][j][0];
+#pragma unroll
+      for (int r = 1; r < 4; ++r) mx = fmaxf(mx, h.v[0][j][r]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, h.v[1][j][r]);
+      mloc[j] = mx * c2;
+    }
+  };
+  // probabilities of 16-row tile i (both rows): two registers' worth at a time would be finer, but four
+  // per call keeps the bookkeeping simple: unit u = 0..3 is (i = u / 2, j = u % 2)
+  auto exp_unit = [&](Half& h, int u) __attribute__((always_inline)) {
+    const int i = u >> 1, j = u & 1;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) h.v[i][j][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(h.v[i][j][r], c2, -mrow[j]));
+  };
+  // operand of the second contraction for row tile j: slots 0..3 from the first 16-row tile, 4..7 from the
+  // second; the row sum is taken over the ROUNDED values, exactly what enters the MFMA
+  auto make_p = [&](const Half& h, int j, V8& pf) __attribute__((always_inline)) {
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[e] = h.v[e >> 2][j][e & 3];
+      if (INTER != kInterSoftmax && p.relu) v[e] = fmaxf(v[e], 0.f);
+    }
+    V2 p0 = cvt2<T>(v[0], v[1]), p1 = cvt2<T>(v[2], v[3]), p2 = cvt2<T>(v[4], v[5]), p3 = cvt2<T>(v[6], v[7]);
+    if constexpr (INTER == kInterSoftmax) {
+      lsum[j] = Elem<T>::add_pair(p0, lsum[j]);
+      lsum[j] = Elem<T>::add_pair(p1, lsum[j]);
+      lsum[j] = Elem<T>::add_pair(p2, lsum[j]);
+      lsum[j] = Elem<T>::add_pair(p3, lsum[j]);
+    }
+    pf = V8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+  };
+  // Lazy rescale, decided without any exchange between lanes: a lane votes when its local maximum exceeds the
+  // row's running maximum by more than 2^kLazy.  Only then are the row maxima exchanged (all rows of the
+  // wave: a raised maximum must be the same in the four lanes of its row) and the accumulators rescaled.
+  auto maybe_rescale = [&]() __attribute__((always_inline)) {
+    const bool vote = mloc[0] > mrow[0] + kLazy || mloc[1] > mrow[1] + kLazy;
+    if (__builtin_amdgcn_ballot_w64(vote) != 0) {
+      mfma_drain();
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float mnew = fmaxf(mrow[j], quad_max(mloc[j]));
+        float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);  // (-inf) - (-inf) does not occur: mnew is finite
+        // A transcendental result needs one idle cycle before an ordinary vector instruction may read it.
+        // The compiler keeps that distance for its own instructions only: acc_scale's first multiply would
+        // otherwise read the register's previous content (the difference, -inf on the first rescale) in part
+        // of the lanes.
+        asm volatile("s_nop 1" : "+v"(alpha));
+        mrow[j] = mnew;
+        lsum[j] *= alpha;
+#pragma unroll
+        for (int t = 0; t < NTN; ++t) acc_scale(2 * t + j, alpha, o);
+      }
+    }
+  };
+
+  // One half step: consumes `cur` (half hh of tile it), produces `nxt` (the following half).  Fragment
+  // groups: 2 NS of the first contraction (16-row tile i of the next half x k step), then NTN of the second
+  // (column tile t); each fragment feeds the two row tiles.
+  constexpr int kAhead = 3;
+  constexpr int NGS = 2 * NS, NG = NGS + NTN;
+  auto half_step = [&](Half& cur, Half& nxt, int it, auto j_c, auto hh_c) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value, hh = decltype(hh_c)::value;
+    constexpr int BNX = B_LOAD + (hh ? (J + 1) % 4 : J) * TB;  // B tile of the next half
+    constexpr int CF = C_FRAG + (J & 1) * TB;
+    if constexpr (INTER == kInterSoftmax) maybe_rescale();
+    V8 fr[NG];
+    auto fetch = [&](int k) __attribute__((always_inline)) {
+      // first contraction: k = st * 2 + i (the two 16-row tiles of the half alternate: four accumulators in turn)
+      fr[k] = k < NGS ? b_frag(BNX, 2 * (hh ^ 1) + (k & 1), k >> 1) : frag_rd(CF, hh * NTN + (k - NGS));
+    };
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) fetch(k);
+    V8 pf[2];
+#pragma unroll
+    for (int k = 0; k < NG; ++k) {
+      if (k + kAhead < NG) fetch(k + kAhead);
+      __builtin_amdgcn_sched_barrier(0);
+      if (k < NGS) {
+        const int i = k & 1, st = k >> 1;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          if (st == 0) nxt.v[i][j] = Mfma16<T>::run(fr[k], af[j][st], f32x4{0.f, 0.f, 0.f, 0.f});
+          else nxt.v[i][j] = Mfma16<T>::run(fr[k], af[j][st], nxt.v[i][j]);
+        }
+        // the four exponential units of `cur` are spread over the first contraction's groups
+        if constexpr (INTER == kInterSoftmax) {
+          if (NGS >= 4) {
+            if (k % (NGS / 4) == 0 && k / (NGS / 4) < 4) exp_unit(cur, k / (NGS / 4));
+          } else {  // two groups only (K = 32): two units behind each
+            exp_unit(cur, 2 * k);
+            exp_unit(cur, 2 * k + 1);
+          }
+        }
+        if (k == NGS - 1) {
+          make_p(cur, 0, pf[0]);
+          make_p(cur, 1, pf[1]);
+        }
+      } else {
+        const int t = k - NGS;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc_mfma(2 * t + j, fr[k], pf[j], o);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (INTER == kInterSoftmax) {
+      const int nt = hh ? it + 1 : it;  // tile of the next half
+      if (ragged && nt == ntiles - 1) mask_tail(nxt, nt * kBN + 32 * (hh ^ 1));
+      local_max(nxt);
+    }
+  };
+  auto tile_step = [&](int it, auto j_c) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value;
+    constexpr int PAR = J & 1;
+    V8 xc[NTR];
+    // C first: the wait at the end of the step can then leave the (younger) B loads in flight
+    load_c(it + C_AHEAD, NCR == 4 ? (J + 3) % 4 : PAR);
+    load_b(it + B_AHEAD, (J + 3) % 4);
+    tr_read_c(C_RAW + (NCR == 4 ? (J + 1) % 4 : (PAR ^ 1)) * TB, xc);
+    half_step(sa, sb, it, j_c, IntC<0>{});
+    tr_write(C_FRAG + (PAR ^ 1) * TB, xc);
+    half_step(sb, sa, it, j_c, IntC<1>{});
+    if (NCR == 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLD) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
+    __syncthreads();
+  };
+
+  // ---- prologue: first tiles in flight, first transposition, scores of the very first half
+  load_b(0, 0);
+  load_b(1, 1);
+  load_c(0, 0);
+  load_c(1, 1);
+  load_b(2, 2);
+  if (NCR == 4) load_c(2, 2);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  {
+    V8 x[NTR];
+    tr_read_c(C_RAW, x);
+    tr_write(C_FRAG, x);
+  }
+#pragma unroll
+  for (int st = 0; st < NS; ++st)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const V8 bf = b_frag(B_LOAD, i, st);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (st == 0) sa.v[i][j] = Mfma16<T>::run(bf, af[j][st], f32x4{0.f, 0.f, 0.f, 0.f});
+        else sa.v[i][j] = Mfma16<T>::run(bf, af[j][st], sa.v[i][j]);
+      }
+    }
+  if constexpr (INTER == kInterSoftmax) {
+    if (ragged && ntiles == 1) mask_tail(sa, 0);
+    local_max(sa);
+  }
+  __syncthreads();
+
+  for (int it = 0; it < ntiles; it += 4) {
+    tile_step(it, IntC<0>{});
+    if (it + 1 < ntiles) tile_step(it + 1, IntC<1>{});
+    if (it + 2 < ntiles) tile_step(it + 2, IntC<2>{});
+    if (it + 3 < ntiles) tile_step(it + 3, IntC<3>{});
+  }
+
+  // ---- epilogue: normalise (softmax), cast, store 4 contiguous columns per lane
+  mfma_drain();
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    float inv = 1.f;
+    if constexpr (INTER == kInterSoftmax) inv = 1.f / quad_sum(lsum[j]);
+    const int row = m_wave + 16 * j + c16;
+    if (row >= M) continue;
+#pragma unroll
+    for (int t = 0; t < NTN; ++t) {
+      const int n = 16 * t + 4 * q;
+      if (n >= N) continue;
+      float v0 = o[2 * t + j][0] * inv, v1 = o[2 * t + j][1] * inv, v2 = o[2 * t + j][2] * inv, v3 = o[2 * t + j][3] * inv;
+      if (INTER != kInterSoftmax && p.relu_out) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); v2 = fmaxf(v2, 0.f); v3 = fmaxf(v3, 0.f); }
+      const long long off = zo * p.f_bs2 + zi * p.f_bs + (long long)row * p.f_rs + n;
+      if (p.out_f32) {
+        f32x4 w = {v0, v1, v2, v3};
+        *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.f) + off) = w;
+      } else {
+        V2 a0 = cvt2<T>(v0, v1), a1 = cvt2<T>(v2, v3);
+        V4 w = {a0[0], a0[1], a1[0], a1[1]};
+        *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.f) + off) = w;
+      }
+    }
+  }
+#else
+  (void)p;
+#endif
+}
+
+template <typename T, int D, int INTER>
+hipError_t launch_bmm_chain8m16(const BmmChainArgs& args, hipStream_t stream) {
+  constexpr int lds = bmm_chain8m16_lds_bytes<D>();
+  auto kern = bmm_chain8m16_kernel<T, D, INTER>;
+  static thread_local int configured_dev = -1;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (configured_dev != dev) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return e;
+    configured_dev = dev;
+  }
+  const unsigned grid = (unsigned)args.mblocks * (unsigned)args.batch;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, args);
+  return hipGetLastError();
+}
+
+}  // namespace ditto

@@ -2,10 +2,12 @@
 // Compiled once per pair with -DDITTO_INST_T=<f16|bf16> -DDITTO_INST_INTER=<0|2>
 // -DDITTO_INST_NAME=<symbol> so the variants build in parallel.
 #include "bmm_chain_fp8.h"
+#include "bmm_chain_fp8m16.h"
 
 namespace ditto {
 
-// q = 1 | 2: four-wave kernel, 32*q rows per wave; q = 8: eight-wave kernel
+// q = 1 | 2: four-wave kernel, 32*q rows per wave; q = 8: eight-wave kernel; q = 9: eight-wave kernel,
+// software pipelined; q = 6: eight-wave kernel on the 16x16x32 MFMA (B stored [L][K] only)
 hipError_t DITTO_INST_NAME(int d_pad, int q, bool b_kl, const BmmChainArgs& args, hipStream_t stream) {
   typedef DITTO_INST_T T;
   constexpr int I = DITTO_INST_INTER;
@@ -17,14 +19,26 @@ hipError_t DITTO_INST_NAME(int d_pad, int q, bool b_kl, const BmmChainArgs& args
   if (d_pad == DP && q == 8)                                               \
     return b_kl ? launch_bmm_chain8<T, DP, I, true>(args, stream)          \
                 : launch_bmm_chain8<T, DP, I, false>(args, stream);
+#define DITTO_CASE9(DP)                                                    \
+  if (d_pad == DP && q == 9)                                               \
+    return b_kl ? launch_bmm_chain8<T, DP, I, true, true>(args, stream)    \
+                : launch_bmm_chain8<T, DP, I, false, true>(args, stream);
+#define DITTO_CASE6(DP)                                                    \
+  if (d_pad == DP && q == 6) return b_kl ? hipErrorInvalidValue : launch_bmm_chain8m16<T, DP, I>(args, stream);
   DITTO_CASE(64, 1)
   DITTO_CASE(64, 2)
   DITTO_CASE(128, 1)
   DITTO_CASE(128, 2)
   DITTO_CASE8(64)
   DITTO_CASE8(128)
+  DITTO_CASE9(64)
+  DITTO_CASE9(128)
+  DITTO_CASE6(64)
+  DITTO_CASE6(128)
 #undef DITTO_CASE
 #undef DITTO_CASE8
+#undef DITTO_CASE9
+#undef DITTO_CASE6
   return hipErrorInvalidValue;
 }
 

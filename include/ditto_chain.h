@@ -135,8 +135,10 @@ typedef struct ditto_tile_param {
   int32_t lds_bytes;      /* dynamic LDS per workgroup                           */
   int32_t grid_x, grid_y, grid_z;
   int32_t variant;        /* kernel variant id: fp16/bf16 chains head_pad*10 + q, with
-                             q = 1|2: four waves owning 32*q rows each, q = 8: eight
-                             waves owning 32 rows each; other chains: see api.hip  */
+                             q = 1|2: four waves owning 32*q rows each; eight waves owning
+                             32 rows each: q = 8 (phases staggered between the two waves of a
+                             SIMD), q = 9 (software pipelined), q = 6 (16x16x32 MFMA, B stored
+                             [L][K] only); other chains: see api.hip  */
 } ditto_tile_param;
 
 /* ---- entry points ------------------------------------------------------- */

@@ -26,11 +26,12 @@ REL_L2 = 1e-3
 REL_L2_BF16_QUANT = 2.6e-3
 
 
-def variants(K, N):
+def variants(K, N, b_layout="LK"):
     """0 (the library's own choice) and every kernel variant that can run the head size:
-    four waves x 32 rows, four waves x 64 rows, eight waves x 32 rows."""
+    four waves x 32 rows, four waves x 64 rows, eight waves x 32 rows (staggered phases; software
+    pipelined; on the 16x16x32 MFMA, which takes B stored [L][K] only)."""
     pad = 64 if max(K, N) <= 64 else 128
-    return [0] + [pad * 10 + q for q in (1, 2, 8)]
+    return [0] + [pad * 10 + q for q in ((1, 2, 8, 9, 6) if b_layout == "LK" else (1, 2, 8, 9))]
 
 
 def run_chain(A, B, C, dtype, inter, scale=1.0, b_layout="KL", out_dtype=None, variant=0):
@@ -67,7 +68,7 @@ def test_softmax_chain_vs_oracle(oracle, shape, dtype, b_layout):
     scale = 1.0 / np.sqrt(K)
     A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, dtype, seed=100 + M)
     want = oracle.bmm_chain_f64(A, B, C, inter="softmax", scale=scale)
-    for variant in variants(K, N):
+    for variant in variants(K, N, b_layout):
         for out_dtype in (dtype, "float32"):
             got = run_chain(A, B, C, dtype, "softmax", scale, b_layout, out_dtype, variant)
             assert np.isfinite(got).all(), variant
@@ -97,8 +98,8 @@ def test_cast_chain_vs_oracle(oracle, shape, dtype, inter):
     # the checker rounds the intermediate to in_dtype exactly where the chain does
     want32 = oracle.bmm_chain_f64(A, B, C, inter=inter, round_mid=dtype)
     want = oracle.np_round_to(want32, dtype)
-    for variant in variants(K, N):
-        for b_layout in ("KL", "LK"):
+    for b_layout in ("KL", "LK"):
+        for variant in variants(K, N, b_layout):
             got32 = run_chain(A, B, C, dtype, inter, 1.0, b_layout, "float32", variant)
             mx, rel = errors(got32, want32)
             # fp32 accumulation order differs; a rounding flip of one intermediate moves the output
@@ -139,7 +140,7 @@ def test_fused_cpu_nest_agrees_with_gpu(oracle):
     assert mx <= MAX_ABS and rel <= REL_L2
 
 
-@pytest.mark.parametrize("variant", [641, 642, 648])
+@pytest.mark.parametrize("variant", [641, 642, 648, 649, 646])
 def test_softmax_invariants_on_gpu(oracle, variant):
     batch, M, N, K, L = 2, 160, 64, 64, 264
     A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, "float16", seed=9)
@@ -153,7 +154,8 @@ def test_softmax_invariants_on_gpu(oracle, variant):
                     "softmax", 0.125, "LK", "float32", variant)
     assert errors(got, base)[1] <= 5e-4
     # Q = 0 -> O = column means of V
-    zero = run_chain(np.zeros_like(A), B, C, "float16", "softmax", 0.125, "KL", "float32", variant)
+    zero = run_chain(np.zeros_like(A), B, C, "float16", "softmax", 0.125, "LK" if variant % 10 == 6 else "KL",
+                     "float32", variant)
     assert np.abs(zero - C.mean(axis=1, keepdims=True)).max() <= 1e-3
     # large scores do not overflow (the reference's exp-without-max form does)
     Ah = A.copy()
@@ -208,7 +210,7 @@ MAX_ABS_BF16_LONG, REL_L2_BF16_LONG = 1.0e-3, 2.6e-3
 MAX_ABS_FP16_LONG, REL_L2_FP16_LONG = 1.4e-4, 3.25e-4
 
 
-@pytest.mark.parametrize("variant", [0, 1282, 1288])
+@pytest.mark.parametrize("variant", [0, 1282, 1288, 1289, 1286])
 def test_attention_full_size_fp16_long_sequence(oracle, variant):
     # the long-sequence shape in fp16, where the stated bar (1e-2 / 1e-3) is reachable: 64 online-softmax
     # steps per row, every variant; three whole heads and a row block of every head against the closed form
@@ -251,7 +253,7 @@ def test_attention_full_size_fp16_long_sequence(oracle, variant):
     assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
 
 
-@pytest.mark.parametrize("variant", [0, 1282, 1288])
+@pytest.mark.parametrize("variant", [0, 1282, 1288, 1289, 1286])
 def test_attention_full_size_bf16_long_sequence(oracle, variant):
     # the bf16 configuration at its full size (64 heads of 4096 x 128).  The CPU closed form over
     # all of it would take minutes, so: every row of three heads chosen across the batch, one
@@ -308,7 +310,7 @@ def test_attention_full_size_bf16_long_sequence(oracle, variant):
     assert bool(((a - b).abs() <= 2.0 ** -7 * b.abs() + 1e-6).all())
 
 
-@pytest.mark.parametrize("variant", [0, 1281, 1288])
+@pytest.mark.parametrize("variant", [0, 1281, 1288, 1289])
 def test_gemm_chain_full_size_bf16(oracle, variant):
     # the large GEMM-chain point of the benchmark, (A.B).D with the cast between, 64 x (4096 x 128 x
     # 4096 x 128) bf16, B as [K][L] like the reference's operand.  The checker over all of it would take
@@ -527,7 +529,7 @@ def test_relu_after_the_second_contraction(oracle, dtype):
         a, b, c = (torch.from_numpy(x).to(dev) for x in (A, B, C))
     else:
         a, b, c = to_dev(A, dtype), to_dev(B, dtype), to_dev(C, dtype)
-    for variant in ([0] if dtype == "float32" else variants(K, N)):
+    for variant in ([0] if dtype == "float32" else variants(K, N, "KL")):
         f = torch.full((batch, M, N), float("nan"), device=dev, dtype=torch.float32)
         chain.run_bmm_chain(a, b, c, f, "relu", tile_variant=variant, relu_out=True)
         torch.cuda.synchronize()
