@@ -40,6 +40,17 @@ __host__ __device__ constexpr int bmm_chain8m16_lds_bytes() {
   return (4 + (D == 64 ? 4 : 2) + 2) * kBN * D * 2;
 }
 
+template <typename V8>
+struct ElemOf;
+template <>
+struct ElemOf<f16x8> {
+  typedef f16 type;
+};
+template <>
+struct ElemOf<bf16x8> {
+  typedef bf16 type;
+};
+
 template <typename T>
 struct Mfma16;
 template <>
@@ -55,76 +66,43 @@ struct Mfma16<bf16> {
   }
 };
 
-// The output accumulators live in FIXED registers, v[4 i : 4 i + 3] for accumulator i, and every instruction
-// that writes them is written out in inline asm with that register as a tied operand.  Left to itself the
+// The output accumulators live in FIXED registers, v[4 i : 4 i + 3] for accumulator i: every statement that
+// writes one is followed by an empty asm that names that register as a tied operand.  Left to itself the
 // compiler gives an MFMA's result another register than the accumulator came in (it likes to reuse the first
 // operand's) and computes the rare rescale into fresh registers, so the accumulators change places and the
-// common path of every branch copies all 64 of them back, every half step.  MFMAs in inline asm are outside
-// the compiler's hazard bookkeeping: the next reader of an accumulator is its own MFMA of the next half step;
-// the rare rescale and the epilogue wait out the pipeline first (mfma_drain).
-__device__ __forceinline__ void acc_mfma(int i, bf16x8 a, bf16x8 b, f32x4 (&o)[16]) {
+// common path of every branch copies all 64 of them back, every half step.  With source and result pinned to
+// the same register the MFMA is allocated in place.  The MFMAs themselves stay the compiler's own
+// instructions, so that it keeps its hazard bookkeeping: whatever reads an accumulator next (the rescale, the
+// epilogue, a copy the register allocator decides on) waits for the matrix pipeline as far as it must.
+__device__ __forceinline__ void acc_pin(int i, f32x4& x) {
   switch (i) {
-    case 0: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[0:3]}"(o[0]) : "v"(a), "v"(b)); break;
-    case 1: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[4:7]}"(o[1]) : "v"(a), "v"(b)); break;
-    case 2: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[8:11]}"(o[2]) : "v"(a), "v"(b)); break;
-    case 3: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[12:15]}"(o[3]) : "v"(a), "v"(b)); break;
-    case 4: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[16:19]}"(o[4]) : "v"(a), "v"(b)); break;
-    case 5: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[20:23]}"(o[5]) : "v"(a), "v"(b)); break;
-    case 6: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[24:27]}"(o[6]) : "v"(a), "v"(b)); break;
-    case 7: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[28:31]}"(o[7]) : "v"(a), "v"(b)); break;
-    case 8: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[32:35]}"(o[8]) : "v"(a), "v"(b)); break;
-    case 9: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[36:39]}"(o[9]) : "v"(a), "v"(b)); break;
-    case 10: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[40:43]}"(o[10]) : "v"(a), "v"(b)); break;
-    case 11: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[44:47]}"(o[11]) : "v"(a), "v"(b)); break;
-    case 12: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[48:51]}"(o[12]) : "v"(a), "v"(b)); break;
-    case 13: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[52:55]}"(o[13]) : "v"(a), "v"(b)); break;
-    case 14: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[56:59]}"(o[14]) : "v"(a), "v"(b)); break;
-    case 15: asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+{v[60:63]}"(o[15]) : "v"(a), "v"(b)); break;
+    case 0: asm volatile("" : "+{v[0:3]}"(x)); break;
+    case 1: asm volatile("" : "+{v[4:7]}"(x)); break;
+    case 2: asm volatile("" : "+{v[8:11]}"(x)); break;
+    case 3: asm volatile("" : "+{v[12:15]}"(x)); break;
+    case 4: asm volatile("" : "+{v[16:19]}"(x)); break;
+    case 5: asm volatile("" : "+{v[20:23]}"(x)); break;
+    case 6: asm volatile("" : "+{v[24:27]}"(x)); break;
+    case 7: asm volatile("" : "+{v[28:31]}"(x)); break;
+    case 8: asm volatile("" : "+{v[32:35]}"(x)); break;
+    case 9: asm volatile("" : "+{v[36:39]}"(x)); break;
+    case 10: asm volatile("" : "+{v[40:43]}"(x)); break;
+    case 11: asm volatile("" : "+{v[44:47]}"(x)); break;
+    case 12: asm volatile("" : "+{v[48:51]}"(x)); break;
+    case 13: asm volatile("" : "+{v[52:55]}"(x)); break;
+    case 14: asm volatile("" : "+{v[56:59]}"(x)); break;
+    case 15: asm volatile("" : "+{v[60:63]}"(x)); break;
   }
 }
-__device__ __forceinline__ void acc_mfma(int i, f16x8 a, f16x8 b, f32x4 (&o)[16]) {
-  switch (i) {
-    case 0: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[0:3]}"(o[0]) : "v"(a), "v"(b)); break;
-    case 1: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[4:7]}"(o[1]) : "v"(a), "v"(b)); break;
-    case 2: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[8:11]}"(o[2]) : "v"(a), "v"(b)); break;
-    case 3: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[12:15]}"(o[3]) : "v"(a), "v"(b)); break;
-    case 4: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[16:19]}"(o[4]) : "v"(a), "v"(b)); break;
-    case 5: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[20:23]}"(o[5]) : "v"(a), "v"(b)); break;
-    case 6: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[24:27]}"(o[6]) : "v"(a), "v"(b)); break;
-    case 7: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[28:31]}"(o[7]) : "v"(a), "v"(b)); break;
-    case 8: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[32:35]}"(o[8]) : "v"(a), "v"(b)); break;
-    case 9: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[36:39]}"(o[9]) : "v"(a), "v"(b)); break;
-    case 10: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[40:43]}"(o[10]) : "v"(a), "v"(b)); break;
-    case 11: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[44:47]}"(o[11]) : "v"(a), "v"(b)); break;
-    case 12: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[48:51]}"(o[12]) : "v"(a), "v"(b)); break;
-    case 13: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[52:55]}"(o[13]) : "v"(a), "v"(b)); break;
-    case 14: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[56:59]}"(o[14]) : "v"(a), "v"(b)); break;
-    case 15: asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+{v[60:63]}"(o[15]) : "v"(a), "v"(b)); break;
-  }
+template <typename V8>
+__device__ __forceinline__ void acc_mfma(int i, V8 a, V8 b, f32x4 (&o)[16]) {
+  o[i] = Mfma16<typename ElemOf<V8>::type>::run(a, b, o[i]);
+  acc_pin(i, o[i]);
 }
 __device__ __forceinline__ void acc_scale(int i, float alpha, f32x4 (&o)[16]) {
-  switch (i) {
-    case 0: asm volatile("v_mul_f32 v0, %1, v0\n\tv_mul_f32 v1, %1, v1\n\tv_mul_f32 v2, %1, v2\n\tv_mul_f32 v3, %1, v3" : "+{v[0:3]}"(o[0]) : "v"(alpha)); break;
-    case 1: asm volatile("v_mul_f32 v4, %1, v4\n\tv_mul_f32 v5, %1, v5\n\tv_mul_f32 v6, %1, v6\n\tv_mul_f32 v7, %1, v7" : "+{v[4:7]}"(o[1]) : "v"(alpha)); break;
-    case 2: asm volatile("v_mul_f32 v8, %1, v8\n\tv_mul_f32 v9, %1, v9\n\tv_mul_f32 v10, %1, v10\n\tv_mul_f32 v11, %1, v11" : "+{v[8:11]}"(o[2]) : "v"(alpha)); break;
-    case 3: asm volatile("v_mul_f32 v12, %1, v12\n\tv_mul_f32 v13, %1, v13\n\tv_mul_f32 v14, %1, v14\n\tv_mul_f32 v15, %1, v15" : "+{v[12:15]}"(o[3]) : "v"(alpha)); break;
-    case 4: asm volatile("v_mul_f32 v16, %1, v16\n\tv_mul_f32 v17, %1, v17\n\tv_mul_f32 v18, %1, v18\n\tv_mul_f32 v19, %1, v19" : "+{v[16:19]}"(o[4]) : "v"(alpha)); break;
-    case 5: asm volatile("v_mul_f32 v20, %1, v20\n\tv_mul_f32 v21, %1, v21\n\tv_mul_f32 v22, %1, v22\n\tv_mul_f32 v23, %1, v23" : "+{v[20:23]}"(o[5]) : "v"(alpha)); break;
-    case 6: asm volatile("v_mul_f32 v24, %1, v24\n\tv_mul_f32 v25, %1, v25\n\tv_mul_f32 v26, %1, v26\n\tv_mul_f32 v27, %1, v27" : "+{v[24:27]}"(o[6]) : "v"(alpha)); break;
-    case 7: asm volatile("v_mul_f32 v28, %1, v28\n\tv_mul_f32 v29, %1, v29\n\tv_mul_f32 v30, %1, v30\n\tv_mul_f32 v31, %1, v31" : "+{v[28:31]}"(o[7]) : "v"(alpha)); break;
-    case 8: asm volatile("v_mul_f32 v32, %1, v32\n\tv_mul_f32 v33, %1, v33\n\tv_mul_f32 v34, %1, v34\n\tv_mul_f32 v35, %1, v35" : "+{v[32:35]}"(o[8]) : "v"(alpha)); break;
-    case 9: asm volatile("v_mul_f32 v36, %1, v36\n\tv_mul_f32 v37, %1, v37\n\tv_mul_f32 v38, %1, v38\n\tv_mul_f32 v39, %1, v39" : "+{v[36:39]}"(o[9]) : "v"(alpha)); break;
-    case 10: asm volatile("v_mul_f32 v40, %1, v40\n\tv_mul_f32 v41, %1, v41\n\tv_mul_f32 v42, %1, v42\n\tv_mul_f32 v43, %1, v43" : "+{v[40:43]}"(o[10]) : "v"(alpha)); break;
-    case 11: asm volatile("v_mul_f32 v44, %1, v44\n\tv_mul_f32 v45, %1, v45\n\tv_mul_f32 v46, %1, v46\n\tv_mul_f32 v47, %1, v47" : "+{v[44:47]}"(o[11]) : "v"(alpha)); break;
-    case 12: asm volatile("v_mul_f32 v48, %1, v48\n\tv_mul_f32 v49, %1, v49\n\tv_mul_f32 v50, %1, v50\n\tv_mul_f32 v51, %1, v51" : "+{v[48:51]}"(o[12]) : "v"(alpha)); break;
-    case 13: asm volatile("v_mul_f32 v52, %1, v52\n\tv_mul_f32 v53, %1, v53\n\tv_mul_f32 v54, %1, v54\n\tv_mul_f32 v55, %1, v55" : "+{v[52:55]}"(o[13]) : "v"(alpha)); break;
-    case 14: asm volatile("v_mul_f32 v56, %1, v56\n\tv_mul_f32 v57, %1, v57\n\tv_mul_f32 v58, %1, v58\n\tv_mul_f32 v59, %1, v59" : "+{v[56:59]}"(o[14]) : "v"(alpha)); break;
-    case 15: asm volatile("v_mul_f32 v60, %1, v60\n\tv_mul_f32 v61, %1, v61\n\tv_mul_f32 v62, %1, v62\n\tv_mul_f32 v63, %1, v63" : "+{v[60:63]}"(o[15]) : "v"(alpha)); break;
-  }
+  o[i] *= alpha;
+  acc_pin(i, o[i]);
 }
-// every MFMA issued so far has written its result (a 16x16x32 MFMA takes four passes; sixteen idle cycles
-// cover the last one and its write-back)
-__device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 7" ::: "memory"); }
 
 // maximum over the four lanes c, c + 16, c + 32, c + 48 (every lane gets it).
 // v_permlane16_swap a, b swaps the odd rows of 16 lanes of a with the even rows of b; from a == b == x,
@@ -169,6 +147,16 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c16 = lane & 15, q = lane >> 4;
+  // A half step has a phase that is heavy on the vector ALU (first contraction of the coming half tile, with
+  // the exponentials of the current one between its MFMAs) and one that is MFMAs only (second contraction of
+  // the current one).  Taking the phases in the other order changes nothing measurable, and letting the two
+  // waves of a SIMD take different orders, so that one wave's exponentials meet the other's MFMAs, is slower
+  // (506 against 437 us at 64 x 4096 x 4096 x 128 on zero operands): what limits a half step is the register
+  // file's write port, which the fragments returning from LDS (four registers per 16-byte read), the vector
+  // ALU's results and the MFMAs share.  A loop of two 16x16x32 MFMAs, one ds_read_b128 and n vector
+  // instructions per wave, two waves per SIMD, takes 39, 55 and 60 cycles for n = 0, 4, 6 (34, 36 and 43
+  // without the read; 32 is the matrix pipe's own time): about four register writes per MFMA pair are free,
+  // each further one costs four cycles.  This kernel has the read and about 5.6 vector results per pair.
 
   const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
   const int mb = lid % p.mblocks;
@@ -203,13 +191,15 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
     }
   }
   auto load_b = [&](int tile, int buf) __attribute__((always_inline)) {
-    const int soff = tile * kBN * p.b_rs * 2;
+    int soff = tile * kBN * p.b_rs * 2;
+    asm volatile("" : "+s"(soff));  // one add per load, not a hoisted address register per load and tile slot
 #pragma unroll
     for (int i = 0; i < NLD; ++i)
       lds_dma_16(b_rsrc, (unsigned)(b_voff[i] + soff), lds0 + B_LOAD + buf * TB + 1024 * (NLD * wave + i));
   };
   auto load_c = [&](int tile, int buf) __attribute__((always_inline)) {
-    const int soff = tile * kBN * p.c_rs * 2;
+    int soff = tile * kBN * p.c_rs * 2;
+    asm volatile("" : "+s"(soff));
 #pragma unroll
     for (int i = 0; i < NLD; ++i)
       lds_dma_16(c_rsrc, (unsigned)(c_voff[i] + soff), lds0 + C_RAW + buf * TB + 1024 * (NLD * wave + i));
@@ -300,11 +290,12 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   };
   Half sa, sb;
   auto mask_tail = [&](Half& h, int l0) __attribute__((always_inline)) {
+    const int rem = L - l0 - 4 * q;  // rows left, counted from the lane's first (compared with constants below)
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        if (l0 + 16 * i + 4 * q + r >= L) {
+        if (16 * i + r >= rem) {
           h.v[i][0][r] = -INFINITY;
           h.v[i][1][r] = -INFINITY;
         }
@@ -326,6 +317,9 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
     const int i = u >> 1, j = u & 1;
 #pragma unroll
     for (int r = 0; r < 4; ++r) h.v[i][j][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(h.v[i][j][r], c2, -mrow[j]));
+    // keep the unit where it is called, between the MFMAs of its group: statements with side effects keep
+    // their order, plain arithmetic is otherwise free to sink to its use
+    asm volatile("" : "+v"(h.v[i][j][0]), "+v"(h.v[i][j][1]), "+v"(h.v[i][j][2]), "+v"(h.v[i][j][3]));
   };
   // operand of the second contraction for row tile j: slots 0..3 from the first 16-row tile, 4..7 from the
   // second; the row sum is taken over the ROUNDED values, exactly what enters the MFMA
@@ -351,16 +345,10 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   auto maybe_rescale = [&]() __attribute__((always_inline)) {
     const bool vote = mloc[0] > mrow[0] + kLazy || mloc[1] > mrow[1] + kLazy;
     if (__builtin_amdgcn_ballot_w64(vote) != 0) {
-      mfma_drain();
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const float mnew = fmaxf(mrow[j], quad_max(mloc[j]));
-        float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);  // (-inf) - (-inf) does not occur: mnew is finite
-        // A transcendental result needs one idle cycle before an ordinary vector instruction may read it.
-        // The compiler keeps that distance for its own instructions only: acc_scale's first multiply would
-        // otherwise read the register's previous content (the difference, -inf on the first rescale) in part
-        // of the lanes.
-        asm volatile("s_nop 1" : "+v"(alpha));
+        const float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);  // (-inf) - (-inf) does not occur: mnew is finite
         mrow[j] = mnew;
         lsum[j] *= alpha;
 #pragma unroll
@@ -479,7 +467,6 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   }
 
   // ---- epilogue: normalise (softmax), cast, store 4 contiguous columns per lane
-  mfma_drain();
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     float inv = 1.f;
