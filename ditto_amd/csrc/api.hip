@@ -268,6 +268,9 @@ struct ConvPlan {
   int dw_mode;         // 0 | 1: plain kernel (1: multiplier a multiple of 8); 2 | 3: persistent kernel,
                        // depthwise stage on the matrix cores (2) or the vector ALU (3)
   ditto::DwConvArgs dwargs;
+  bool resident;       // 1x1 -> 3x3 with at most 64 channels: persistent kernel, W2 resident in LDS
+  int res_grid;
+  ditto::ConvResidentArgs rargs;
   ditto_tile_param tile;
 };
 
@@ -430,12 +433,19 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   return DITTO_OK;
 }
 
+// DITTO_CONV_RESIDENT=0 keeps the 1x1 -> 3x3 chains on the general kernel (A/B runs, tests of that kernel)
+bool resident_off() {
+  const char* v = getenv("DITTO_CONV_RESIDENT");
+  return v && v[0] == '0';
+}
+
 bool persist_requested() {
   const char* v = getenv("DITTO_CONV_PERSIST");
   return v && v[0] == '1';
 }
 
-int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device = false, int dw_vec_cap = 8) {
+int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device = false, int dw_vec_cap = 8,
+              bool allow_resident = true) {
   if (!d) return fail(DITTO_EINVAL, "null descriptor");
   if (d->abi_version != DITTO_CHAIN_ABI_VERSION)
     return fail(DITTO_EINVAL, "descriptor abi_version %d, library %d", d->abi_version, DITTO_CHAIN_ABI_VERSION);
@@ -484,6 +494,46 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
     if (P2 <= 0 || Q2 <= 0) return fail(DITTO_EINVAL, "empty convolution output");
     if (d->N * d->C2 * P2 * Q2 > 0x7fffffffLL * 4) return fail(DITTO_EINVAL, "tensor too large");
     a.R2 = (int)d->R2; a.S2 = (int)d->S2; a.pad2 = (int)d->pad2; a.P2 = (int)P2; a.Q2 = (int)Q2;
+    // 1x1 -> 3x3 (pad 1) with at most 64 channels everywhere and rows that are whole 16-byte vectors: the
+    // persistent kernel that keeps W2 in LDS (conv_chain_resident.h), tiles of whole output rows
+    if (allow_resident && !resident_off() && d->R1 == 1 && d->S1 == 1 && d->pad1 == 0 && d->stride1 == 1 && d->R2 == 3 &&
+        d->S2 == 3 && d->pad2 == 1 && d->C0 <= ditto::kCrC && d->C1 <= ditto::kCrC && d->C2 <= ditto::kCrC &&
+        d->C0 % 8 == 0 && d->W % 8 == 0 && d->W <= 256 &&
+        d->C0 * d->H * d->W * 2 < 0x7fffffffLL) {
+      int th2 = (int)(256 / d->W);
+      if (th2 > d->H) th2 = (int)d->H;
+      while (th2 >= 1 && (ditto::conv_resident_lds_bytes(th2, (int)d->W) > 160 * 1024 ||
+                          (th2 + 2) * d->W > 64 * ditto::kCrMaxLoads))
+        --th2;
+      if (th2 >= 1) {
+        const int cus = need_device ? device_cus() : 256;
+        ditto::ConvResidentArgs& r = plan->rargs;
+        r.N = (int)d->N; r.C0 = (int)d->C0; r.H = (int)d->H; r.W = (int)d->W; r.C1 = (int)d->C1; r.C2 = (int)d->C2;
+        r.TH2 = th2;
+        r.tiles_h = (int)((d->H + th2 - 1) / th2);
+        r.ntiles = r.N * r.tiles_h;
+        r.relu_mid = d->inter_op == DITTO_INTER_RELU;
+        r.relu_out = d->relu_out != 0;
+        r.out_f32 = d->out_dtype == DITTO_F32;
+        plan->resident = true;
+        plan->res_grid = r.ntiles < cus ? r.ntiles : cus;
+        plan->px2 = 1;
+        plan->w1p_bytes = 0;
+        plan->w2p_bytes = ditto::kCrW2Bytes;
+        ditto_tile_param& t = plan->tile;
+        t.block_threads = 512;
+        t.block_m = th2 * (int)d->W;
+        t.block_l = ditto::kCrC;
+        t.block_n = (int)d->C2;
+        t.head_pad = ditto::kCrC;
+        t.lds_bytes = ditto::conv_resident_lds_bytes(th2, (int)d->W);
+        t.grid_x = plan->res_grid;
+        t.grid_y = th2;
+        t.grid_z = (int)d->W;
+        t.variant = 3600 + th2;  // persistent, W2 resident in LDS; th2 output rows per tile
+        return DITTO_OK;
+      }
+    }
     a.TW2 = (int)Q2;
     while ((a.TW2 + a.S2 - 1) * a.R2 > slots) a.TW2 = (a.TW2 + 1) / 2;
     a.TW = a.TW2 + a.S2 - 1;
@@ -729,7 +779,13 @@ int ditto_conv_chain_select_tile(const ditto_conv_chain_desc* desc, ditto_tile_p
 size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
   ConvPlan plan;
   if (plan_conv(desc, &plan) != DITTO_OK) return 0;
-  return plan.w1p_bytes + plan.w2p_bytes;
+  size_t need = plan.w1p_bytes + plan.w2p_bytes;
+  if (plan.resident) {  // a call with pointers the resident kernel cannot take falls back to the general one
+    ConvPlan general;
+    if (plan_conv(desc, &general, false, 8, false) == DITTO_OK && general.w1p_bytes + general.w2p_bytes > need)
+      need = general.w1p_bytes + general.w2p_bytes;
+  }
+  return need;
 }
 
 }  // extern "C"
@@ -745,6 +801,38 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
   int rc = plan_conv(d, &plan, true, x && aligned(x, 16) ? 8 : 4);
   if (rc != DITTO_OK) return rc;
   if (((phase & kConvCompute) && (!x || !y)) || !w1 || !w2) return fail(DITTO_EINVAL, "null data pointer");
+  if (plan.resident) {
+    // 16-byte direct loads of X and W1 fragments, stores of 4 pixels
+    const bool ok = aligned(w1, 16) && (!(phase & kConvCompute) || (aligned(x, 16) && aligned(y, plan.rargs.out_f32 ? 16 : 8)));
+    if (!ok && phase == kConvBoth) {
+      rc = plan_conv(d, &plan, true, 4, false);  // the general kernel takes any element-aligned pointer
+      if (rc != DITTO_OK) return rc;
+    } else if (!ok) {
+      return fail(DITTO_EINVAL, "misaligned data pointer: this shape runs with x, w1 16-byte and y 8-byte (fp32: 16-byte) aligned "
+                                "(its prepared weights are in the resident kernel's layout)");
+    }
+  }
+  if (plan.resident) {
+    if (!workspace) return fail(DITTO_EWORKSPACE, "this conv chain needs the workspace (%zu bytes)", plan.w2p_bytes);
+    if (workspace_bytes < plan.w2p_bytes)
+      return fail(DITTO_EWORKSPACE, "workspace of %zu bytes, need %zu", workspace_bytes, plan.w2p_bytes);
+    if (!aligned(workspace, 16)) return fail(DITTO_EINVAL, "workspace must be 16-byte aligned");
+    ditto::ConvResidentArgs r = plan.rargs;
+    r.x = x;
+    r.w1 = w1;
+    r.w2f = workspace;
+    r.y = y;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const bool f16 = d->in_dtype == DITTO_F16;
+    hipError_t e = hipSuccess;
+    if (phase & kConvPrepare)
+      e = f16 ? ditto::pack_conv_w2_resident_f16(w2, workspace, r.C1, r.C2, st)
+              : ditto::pack_conv_w2_resident_bf16(w2, workspace, r.C1, r.C2, st);
+    if (e == hipSuccess && (phase & kConvCompute))
+      e = f16 ? ditto::launch_conv_resident_f16(r, plan.res_grid, st) : ditto::launch_conv_resident_bf16(r, plan.res_grid, st);
+    if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
+    return DITTO_OK;
+  }
   if (!aligned(x, 2) || !aligned(w1, 2) || !aligned(w2, 8) || !aligned(y, 4))
     return fail(DITTO_EINVAL, "misaligned data pointer");
   if (phase != kConvBoth && !plan.dw && !workspace)

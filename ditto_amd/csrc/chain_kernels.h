@@ -4,6 +4,7 @@
 
 #include "bmm_chain_fp.h"
 #include "conv_chain.h"
+#include "conv_chain_resident.h"
 #include "dw_conv_chain.h"
 #include "gemm_chain_f32.h"
 #include "gemm_chain_i8.h"
@@ -28,6 +29,11 @@ hipError_t launch_conv2_f16(int c1_tiles, int px2, const ConvChainArgs& args, hi
 hipError_t launch_conv2_bf16(int c1_tiles, int px2, const ConvChainArgs& args, hipStream_t stream);
 hipError_t pack_conv_w2_f16(int c1_tiles, const ConvChainArgs& args, void* out1, void* out2, hipStream_t stream);
 hipError_t pack_conv_w2_bf16(int c1_tiles, const ConvChainArgs& args, void* out1, void* out2, hipStream_t stream);
+// 1x1 -> 3x3 with at most 64 channels: persistent kernel, W2 resident in LDS (conv_chain_resident.h)
+hipError_t launch_conv_resident_f16(const ConvResidentArgs& args, int grid, hipStream_t stream);
+hipError_t launch_conv_resident_bf16(const ConvResidentArgs& args, int grid, hipStream_t stream);
+hipError_t pack_conv_w2_resident_f16(const void* w2, void* out, int C1, int C2, hipStream_t stream);
+hipError_t pack_conv_w2_resident_bf16(const void* w2, void* out, int C1, int C2, hipStream_t stream);
 // depthwise first convolution (dw_conv_chain.h); c2_tiles in {1, 2, 4, 8}; mode 0 | 1: plain kernel,
 // vector-ALU depthwise stage (1: multiplier a multiple of 8); 2: persistent kernel, MFMA depthwise
 // stage (multiplier a multiple of 16); 3: persistent kernel, vector-ALU stage (3x3, multiplier 1, 2, 4, 8)

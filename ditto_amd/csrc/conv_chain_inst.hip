@@ -1,6 +1,7 @@
 // Instantiates the conv chain kernels for one element type.
-// Compiled with -DDITTO_INST_T=<f16|bf16> and -DDITTO_{INST,PACK,INST2,PACK2}_NAME=<symbol>.
+// Compiled with -DDITTO_INST_T=<f16|bf16> and -DDITTO_{INST,PACK,INST2,PACK2,RES,PACKRES,DW}_NAME=<symbol>.
 #include "conv_chain.h"
+#include "conv_chain_resident.h"
 #include "dw_conv_chain.h"
 
 namespace ditto {
@@ -33,6 +34,14 @@ hipError_t DITTO_INST2_NAME(int c1_tiles, int px2, const ConvChainArgs& args, hi
 
 hipError_t DITTO_PACK2_NAME(int c1_tiles, const ConvChainArgs& args, void* out1, void* out2, hipStream_t stream) {
   return launch_pack_conv_w12<DITTO_INST_T>(args, 32 * c1_tiles, 32, out1, out2, stream);
+}
+
+// 1x1 first, 3x3 second convolution, at most 64 channels: persistent kernel with W2 resident in LDS
+hipError_t DITTO_RES_NAME(const ConvResidentArgs& args, int grid, hipStream_t stream) {
+  return launch_conv_chain_resident<DITTO_INST_T>(args, grid, stream);
+}
+hipError_t DITTO_PACKRES_NAME(const void* w2, void* out, int C1, int C2, hipStream_t stream) {
+  return pack_conv_w2_resident<DITTO_INST_T>(w2, out, C1, C2, stream);
 }
 
 // depthwise first convolution: c2_tiles in {1, 2, 4, 8} (32 output channels each); mode 0 | 1: plain

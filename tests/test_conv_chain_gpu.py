@@ -114,6 +114,10 @@ CASES_3X3_SECOND = [
     (1, 16, 12, 150, 16, 1, 0, 1, 16, 3, 1),   # wider than one tile
     (1, 16, 16, 16, 32, 3, 1, 1, 32, 3, 0),    # unpadded second convolution
     (2, 24, 30, 30, 64, 3, 1, 1, 128, 3, 1),   # conv3x3 -> conv3x3, 64 intermediate channels, C0 % 32 != 0
+    # 1x1 -> 3x3 with rows of whole 16-byte vectors and at most 64 channels: the persistent kernel with W2 in LDS
+    (1, 32, 21, 24, 48, 1, 0, 1, 40, 3, 1),    # channel counts that are no multiples of 32; a partial last tile
+    (1, 8, 9, 8, 8, 1, 0, 1, 8, 3, 1),         # one small tile
+    (3, 64, 7, 128, 16, 1, 0, 1, 64, 3, 1),    # two output rows per tile
 ]
 
 
@@ -132,6 +136,35 @@ def test_conv_chain_with_wide_second_filter(oracle, case, dtype):
     assert np.array_equal(got, oracle.np_round_to(got32, dtype))
     with pytest.raises(ValueError):  # this variant cannot run without its workspace
         run_conv(X, W1, W2, dtype, pad1, stride1, workspace=False, pad2=pad2)
+
+
+def test_resident_conv_chain_over_several_rounds(oracle, monkeypatch):
+    """More tiles than CUs: every persistent workgroup walks over more than one tile.  Checked against the
+    general kernel (which streams W2 per workgroup) on the same inputs, both against the oracle on a slice."""
+    N, C0, H, W, C1, C2 = 20, 64, 56, 56, 64, 64
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, 1, 3, "float16", seed=5, w_std=0.05)
+    x, w1, w2 = to_dev(X, "float16"), to_dev(W1, "float16"), to_dev(W2, "float16")
+    y = torch.full((N, C2, H, W), float("nan"), device=x.device, dtype=torch.float16)
+    desc = chain.conv_chain_desc(x, w1, w2, y, 0, 1, 1, 1, "relu", False)
+    tile = chain.select_tile(desc)
+    assert tile.variant == 3604 and tile.block_threads == 512 and tile.lds_bytes <= 160 * 1024
+    chain.run_conv_chain(x, w1, w2, y, desc=desc)
+    torch.cuda.synchronize()
+    got = y.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    monkeypatch.setenv("DITTO_CONV_RESIDENT", "0")
+    y2 = torch.full_like(y, float("nan"))
+    desc2 = chain.conv_chain_desc(x, w1, w2, y2, 0, 1, 1, 1, "relu", False)
+    assert chain.select_tile(desc2).variant // 100 == 35
+    chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
+    torch.cuda.synchronize()
+    monkeypatch.delenv("DITTO_CONV_RESIDENT")
+    mx, rel = errors(got, y2.float().cpu().numpy())
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
+    for n in (0, 13, 19):  # first, a middle and the last image (the last one is the second tile of its workgroup)
+        want = oracle.conv_chain_f32(X[n:n + 1], W1, W2, 0, 1, 1, 1, relu_mid=True, relu_out=False, round_mid="float16")
+        mx, rel = errors(got[n:n + 1], want)
+        assert mx <= MAX_ABS and rel <= REL_L2, (n, mx, rel)
 
 
 CASES_DEPTHWISE = [
