@@ -803,12 +803,12 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
   if (((phase & kConvCompute) && (!x || !y)) || !w1 || !w2) return fail(DITTO_EINVAL, "null data pointer");
   if (plan.resident) {
     // 16-byte direct loads of X and W1 fragments, stores of 4 pixels
-    const bool ok = aligned(w1, 16) && (!(phase & kConvCompute) || (aligned(x, 16) && aligned(y, plan.rargs.out_f32 ? 16 : 8)));
+    const bool ok = aligned(w1, 16) && (!(phase & kConvCompute) || (aligned(x, 16) && aligned(y, 16)));
     if (!ok && phase == kConvBoth) {
       rc = plan_conv(d, &plan, true, 4, false);  // the general kernel takes any element-aligned pointer
       if (rc != DITTO_OK) return rc;
     } else if (!ok) {
-      return fail(DITTO_EINVAL, "misaligned data pointer: this shape runs with x, w1 16-byte and y 8-byte (fp32: 16-byte) aligned "
+      return fail(DITTO_EINVAL, "misaligned data pointer: this shape runs with x, w1 and y 16-byte aligned "
                                 "(its prepared weights are in the resident kernel's layout)");
     }
   }

@@ -17,8 +17,8 @@
 //        second convolution's padding; rows outside the image are zero because X was)
 //   second convolution (MFMA row = pixel):  out[px][c2] = sum_tap mid[px + tap][c1] . W2[tap][c1][c2]
 //        A = 16-byte reads of mid, B = 16-byte reads of the resident W2 fragments
-//        result: a lane holds 4 consecutive pixels of one output channel per register group: 8-byte stores
-//        (16-byte for fp32 output) straight from registers, no turn-around.
+//        result: with the MFMA rows dealt to the pixels in the right order a lane holds 16 consecutive pixels
+//        of one output channel: 16-byte stores straight from registers, no turn-around.
 //
 // While the second convolution of a tile runs, the direct loads of the next tile's X rows are in flight
 // (the raw X buffer is free once the first convolution is done).  Two barriers per tile.
@@ -118,18 +118,10 @@ __global__ __launch_bounds__(512) void conv_chain_resident_kernel(ConvResidentAr
     }
   };
 
-  // ---- prologue: W2 fragments into LDS, zero columns of the intermediate tile, W1 fragments, first X tile
-  {
-    const i32x4 w2_rsrc = make_rsrc(p.w2f, (unsigned)kCrW2Bytes);
-#pragma unroll
-    for (int j = 0; j < kCrW2Bytes / 1024 / 8; ++j)
-      lds_dma_16(w2_rsrc, (unsigned)(1024 * (wave + 8 * j) + 16 * lane), lds0 + 1024 * (wave + 8 * j));
-    // pixels (row, 0) and (row, W + 1) of every row: 2 * rows_mid pixels of 128 bytes = 8 pieces of 16 each
-    for (int i = tid; i < 2 * rows_mid * 8; i += 512) {
-      const int px = i >> 3, row = px >> 1, col = (px & 1) ? W + 1 : 0;
-      *reinterpret_cast<i32x4*>(Ms + (row * MW + col) * 128 + (i & 7) * 16) = i32x4{0, 0, 0, 0};
-    }
-  }
+  // ---- prologue: first X tile, W1 fragments, W2 fragments into LDS (waited for only before the first second
+  // convolution), zero columns of the intermediate tile
+  int tile = (int)xcd_remap(blockIdx.x, gridDim.x);
+  if (tile < p.ntiles) load_x(tile);
   // A operand of the first convolution: lane (ln, g) holds W1[32 c1t + ln][16 kk + 8 g .. + 7]
   V8 w1f[2][NKK];
 #pragma unroll
@@ -141,6 +133,18 @@ __global__ __launch_bounds__(512) void conv_chain_resident_kernel(ConvResidentAr
       if (c1 < p.C1 && c0 < p.C0) v = *reinterpret_cast<const V8*>(W1g + (long long)c1 * p.C0 + c0);
       w1f[c1t][kk] = v;
     }
+  constexpr int kW2Loads = kCrW2Bytes / 1024 / 8;  // per wave
+  {
+    const i32x4 w2_rsrc = make_rsrc(p.w2f, (unsigned)kCrW2Bytes);
+#pragma unroll
+    for (int j = 0; j < kW2Loads; ++j)
+      lds_dma_16(w2_rsrc, (unsigned)(1024 * (wave + 8 * j) + 16 * lane), lds0 + 1024 * (wave + 8 * j));
+    // pixels (row, 0) and (row, W + 1) of every row: 2 * rows_mid pixels of 128 bytes = 8 pieces of 16 each
+    for (int i = tid; i < 2 * rows_mid * 8; i += 512) {
+      const int px = i >> 3, row = px >> 1, col = (px & 1) ? W + 1 : 0;
+      *reinterpret_cast<i32x4*>(Ms + (row * MW + col) * 128 + (i & 7) * 16) = i32x4{0, 0, 0, 0};
+    }
+  }
 
   // ---- per-lane addresses, the same for every tile
   // first convolution: pixel tile t = wave + 8 u of the intermediate tile, slot = 32 t + ln
@@ -160,10 +164,13 @@ __global__ __launch_bounds__(512) void conv_chain_resident_kernel(ConvResidentAr
     // tile's last pixel keeps its read address: the 16 lanes of a group transpose among themselves, and what
     // it reads lies in the next channel's run or the intermediate tile, inside LDS either way)
   }
-  // second convolution: output slot 32 wave + ln; address of the lane's pixel at tap (r, s), chunk XOR
+  // second convolution: MFMA row ln = 8 i + 4 g' + e of the wave's pixel tile stands for output slot
+  // 32 wave + 16 g' + 4 i + e, so that the accumulator registers of a lane (rows 8 i + 4 g + e, i and e = 0..3) are
+  // 16 consecutive pixels: two 16-byte stores per lane and column tile.  Address of the lane's pixel at tap
+  // (r, s), chunk XOR
   int m_rd[kCrTaps], m_x7[kCrTaps];
   {
-    const int slot = 32 * wave + ln;
+    const int slot = 32 * wave + 16 * ((ln >> 2) & 1) + 4 * (ln >> 3) + (ln & 3);
     const int sl = slot < npo ? slot : 0;
     const int ph = sl / W, pw = sl - ph * W;
 #pragma unroll
@@ -176,17 +183,29 @@ __global__ __launch_bounds__(512) void conv_chain_resident_kernel(ConvResidentAr
       }
   }
   const int w2_rd = lane * 16;
-  // output: register group i of column tile ct holds pixels 32 wave + 8 i + 4 g + {0..3} of channel 32 ct + ln
-  const int o_slot = 32 * wave + 4 * g;
+  // output: registers 4 i + e of column tile ct hold pixels 32 wave + 16 g + 4 i + e of channel 32 ct + ln
+  const int o_slot = 32 * wave + 16 * g;
 
-  int tile = (int)xcd_remap(blockIdx.x, gridDim.x);
-  if (tile < p.ntiles) load_x(tile);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // loads return in order: the X rows (and W1) are there once only the W2 loads, issued last, are outstanding
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kW2Loads) : "memory");
   __syncthreads();
+  bool w2_pending = true;
 
   for (; tile < p.ntiles; tile += gridDim.x) {
     const int n = tile / p.tiles_h, r0 = (tile - n * p.tiles_h) * TH2;
-    // ---- first convolution over the tile's rows (with halo), result to LDS
+    // ---- first convolution over the tile's rows (with halo), result to LDS; all fragments are read first
+    V8 xf[2][NKK];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      if (32 * (wave + 8 * u) < npm) {
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk) {
+          const char* q = Xs + x_rd[u] + 16 * kk * rwb;
+          V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
+          V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(q + 4 * rwb));
+          xf[u][kk] = concat4<V4, V8>(lo, hi);
+        }
+      }
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       if (32 * (wave + 8 * u) < npm) {
@@ -196,14 +215,9 @@ __global__ __launch_bounds__(512) void conv_chain_resident_kernel(ConvResidentAr
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[c][r] = 0.f;
 #pragma unroll
-        for (int kk = 0; kk < NKK; ++kk) {
-          const char* q = Xs + x_rd[u] + 16 * kk * rwb;
-          V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(q));
-          V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(q + 4 * rwb));
-          const V8 xf = concat4<V4, V8>(lo, hi);
+        for (int kk = 0; kk < NKK; ++kk)
 #pragma unroll
-          for (int c = 0; c < 2; ++c) acc[c] = Elem<T>::mfma32(w1f[c][kk], xf, acc[c]);
-        }
+          for (int c = 0; c < 2; ++c) acc[c] = Elem<T>::mfma32(w1f[c][kk], xf[u][kk], acc[c]);
         if (m_ok[u]) {
           const int x7 = (m_wr[u] >> 7) & 7;
 #pragma unroll
@@ -219,28 +233,50 @@ __global__ __launch_bounds__(512) void conv_chain_resident_kernel(ConvResidentAr
         }
       }
     }
+    if (w2_pending) {  // first tile: the W2 fragments
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      w2_pending = false;
+    }
     __syncthreads();  // intermediate tile complete; raw X buffer free
     if (tile + (int)gridDim.x < p.ntiles) load_x(tile + gridDim.x);
 
     // ---- second convolution: 32 output pixels x 64 channels per wave
+    f32x16 o[2];
     if (32 * wave < npo) {
-      f32x16 o[2];
 #pragma unroll
       for (int c = 0; c < 2; ++c)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[c][r] = 0.f;
+      // step = (tap, k step): one fragment of the intermediate tile, two of W2, two MFMAs; fragments are
+      // fetched kAhead steps before their MFMAs
+      constexpr int NSTEP = kCrTaps * NKK, kAhead = 3;
+      V8 mf[NSTEP], wf[NSTEP][2];
+      auto fetch = [&](int st) __attribute__((always_inline)) {
+        const int tap = st / NKK, kk = st % NKK;
+        mf[st] = *reinterpret_cast<const V8*>(Ms + m_rd[tap] + ((((2 * kk + g) << 4)) ^ m_x7[tap]));
 #pragma unroll
-      for (int tap = 0; tap < kCrTaps; ++tap)
+        for (int c = 0; c < 2; ++c) wf[st][c] = *reinterpret_cast<const V8*>(smem_raw + w2_rd + (st * 2 + c) * 1024);
+      };
 #pragma unroll
-        for (int kk = 0; kk < NKK; ++kk) {
-          const V8 mf = *reinterpret_cast<const V8*>(Ms + m_rd[tap] + ((((2 * kk + g) << 4)) ^ m_x7[tap]));
+      for (int st = 0; st < kAhead; ++st) fetch(st);
 #pragma unroll
-          for (int c = 0; c < 2; ++c) {
-            const V8 wf = *reinterpret_cast<const V8*>(smem_raw + w2_rd + ((tap * NKK + kk) * 2 + c) * 1024);
-            o[c] = Elem<T>::mfma32(mf, wf, o[c]);
-          }
-        }
-      // ---- output: 4 consecutive pixels of one channel per register group
+      for (int st = 0; st < NSTEP; ++st) {
+        if (st + kAhead < NSTEP) fetch(st + kAhead);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < 2; ++c) o[c] = Elem<T>::mfma32(mf[st], wf[st][c], o[c]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // The next tile's X rows (issued before this convolution) have landed, the previous tile's stores too.
+    // Behind this barrier every wave is done with the intermediate tile and X is complete: the next tile's
+    // first convolution may start while other waves still issue the stores below, which nobody waits for.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    if (32 * wave < npo) {
+      // ---- output: 16 consecutive pixels of one channel per lane and column tile, 8 per store (fp32: 4)
       const long long y0 = (long long)n * p.C2 * plane + (long long)r0 * W;
       const int rows_left = H - r0;  // output rows of this tile inside the image
       const int lim = (rows_left < TH2 ? rows_left : TH2) * W;
@@ -248,25 +284,29 @@ __global__ __launch_bounds__(512) void conv_chain_resident_kernel(ConvResidentAr
       for (int c = 0; c < 2; ++c) {
         const int c2 = 32 * c + ln;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int s4 = o_slot + 8 * i;
-          if (c2 < p.C2 && s4 < lim) {
-            float v0 = o[c][4 * i], v1 = o[c][4 * i + 1], v2 = o[c][4 * i + 2], v3 = o[c][4 * i + 3];
-            if (p.relu_out) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); v2 = fmaxf(v2, 0.f); v3 = fmaxf(v3, 0.f); }
-            const long long off = y0 + (long long)c2 * plane + s4;
+        for (int hh = 0; hh < 2; ++hh) {
+          const int s8 = o_slot + 8 * hh;  // W is a multiple of 8: the 8 pixels are in one row, inside the tile or not
+          if (c2 < p.C2 && s8 < lim) {
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              v[e] = o[c][8 * hh + e];
+              if (p.relu_out) v[e] = fmaxf(v[e], 0.f);
+            }
+            const long long off = y0 + (long long)c2 * plane + s8;
             if (p.out_f32) {
-              *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.y) + off) = f32x4{v0, v1, v2, v3};
+              float* dst = reinterpret_cast<float*>(p.y) + off;
+              *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+              *reinterpret_cast<f32x4*>(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
             } else {
-              const V2 a0 = cvt2<T>(v0, v1), a1 = cvt2<T>(v2, v3);
-              const V4 w = {a0[0], a0[1], a1[0], a1[1]};
-              *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.y) + off) = w;
+              const V2 a0 = cvt2<T>(v[0], v[1]), a1 = cvt2<T>(v[2], v[3]), a2 = cvt2<T>(v[4], v[5]), a3 = cvt2<T>(v[6], v[7]);
+              const V8 w = {a0[0], a0[1], a1[0], a1[1], a2[0], a2[1], a3[0], a3[1]};
+              *reinterpret_cast<V8*>(reinterpret_cast<T*>(p.y) + off) = w;
             }
           }
         }
       }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();  // next tile's X rows have landed; every wave is done with the intermediate tile
   }
 #else
   (void)p;
