@@ -125,10 +125,11 @@ def bytes_of(w):
     return eb * w["batch"] * (w["M"] * w["K"] + w["K"] * w["L"] + w["L"] * w["N"] + w["M"] * w["N"])
 
 
-def make_call(w, dev, prepared=False):
+def make_call(w, dev, prepared=False, zero=False):
     """Synthetic inputs resident on the device and a zero-argument callable that runs one step.
     ``prepared`` (conv chains that take a workspace): the weights are repacked once, outside the
-    step, as the reference's drivers are handed host-packed weights; the step is the fused kernel alone."""
+    step, as the reference's drivers are handed host-packed weights; the step is the fused kernel alone.
+    ``zero`` (BMM chains): all-zero operands, the same instructions on data that toggles nothing."""
     import torch
 
     from ditto_amd import chain
@@ -166,6 +167,8 @@ def make_call(w, dev, prepared=False):
         b = torch.randn(w["batch"], w["L"], w["K"], generator=g).to(dt).to(dev).transpose(1, 2)
     else:
         b = (torch.randn(w["batch"], w["K"], w["L"], generator=g) * std).to(dt).to(dev)
+    if zero:
+        a.zero_(), b.zero_(), c.zero_()
     f = torch.empty(w["batch"], w["M"], w["N"], dtype=dt, device=dev)
     desc = chain.bmm_chain_desc(a, b, c, f, w["kind"], w["scale"])
     return (lambda: chain.run_bmm_chain(a, b, c, f, desc=desc)), desc
@@ -377,6 +380,12 @@ def run_one(name, steps, warmup, dev, long_run=False):
     roof["graph_replay_ms"] = gr_ms
     if long_ms is not None:
         roof["min_repeat_600ms_ms"] = long_ms
+    if long_run and w["bound"] == "mfma" and w["kind"] in ("softmax", "cast"):
+        # The same launch on all-zero operands: the same instruction stream without the switching activity of
+        # real data.  The gap to kernel_ms is what the device's power management takes on N(0,1) operands.
+        zcall, _ = make_call(w, dev, zero=True)
+        warm_up(zcall, warmup)
+        roof["zero_operand_kernel_ms"] = min_repeat_ms(zcall, 200.0)
     if w["kind"] == "conv" and w.get("groups", 1) == 1:
         # the same step with the weight repacking done once beforehand (ditto_conv_chain_prepare +
         # ditto_conv_chain_run_prepared): what a caller with fixed weights pays per call
