@@ -464,9 +464,9 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
   const bool second_1x1 = d->R2 == 1 && d->S2 == 1 && d->pad2 == 0;
   if (d->stride2 != 1) return fail(DITTO_EUNSUPPORTED, "the second convolution must have stride 1");
   if (!dw) {
-    if (!second_1x1 && (d->R2 > 3 || d->S2 > 3 || d->C1 > 64))
+    if (!second_1x1 && (d->R2 > 3 || d->S2 > 3 || d->C1 > 128))
       return fail(DITTO_EUNSUPPORTED,
-                  "a second convolution larger than 1x1 takes filters up to 3x3 and at most 64 intermediate channels");
+                  "a second convolution larger than 1x1 takes filters up to 3x3 and at most 128 intermediate channels");
     if (d->C1 % 8) return fail(DITTO_EINVAL, "C1 must be a multiple of 8");
     if (d->C1 > 256) return fail(DITTO_EUNSUPPORTED, "C1=%lld: at most 256 intermediate channels", (long long)d->C1);
   }

@@ -24,7 +24,7 @@ hipError_t launch_conv_bf16(int c1_tiles, int ch, const ConvChainArgs& args, hip
 // W1 -> the chunked layout the chain kernel loads directly (conv_w1_chunk_bytes per chunk)
 hipError_t pack_conv_w1_f16(int c1_tiles, int ch, const ConvChainArgs& args, void* out, hipStream_t stream);
 hipError_t pack_conv_w1_bf16(int c1_tiles, int ch, const ConvChainArgs& args, void* out, hipStream_t stream);
-// second convolution larger than 1x1 (32-channel chunks; c1_tiles in {1, 2}; px2 in {1, 2})
+// second convolution larger than 1x1 (32-channel chunks; c1_tiles in {1, 2, 4}; px2 in {1, 2})
 hipError_t launch_conv2_f16(int c1_tiles, int px2, const ConvChainArgs& args, hipStream_t stream);
 hipError_t launch_conv2_bf16(int c1_tiles, int px2, const ConvChainArgs& args, hipStream_t stream);
 hipError_t pack_conv_w2_f16(int c1_tiles, const ConvChainArgs& args, void* out1, void* out2, hipStream_t stream);

@@ -118,6 +118,9 @@ CASES_3X3_SECOND = [
     (1, 32, 21, 24, 48, 1, 0, 1, 40, 3, 1),    # channel counts that are no multiples of 32; a partial last tile
     (1, 8, 9, 8, 8, 1, 0, 1, 8, 3, 1),         # one small tile
     (3, 64, 7, 128, 16, 1, 0, 1, 64, 3, 1),    # two output rows per tile
+    # more than 64 intermediate channels (general kernel, four tiles of 32)
+    (1, 32, 20, 24, 128, 1, 0, 1, 64, 3, 1),   # conv1x1 -> conv3x3, 128 intermediate channels
+    (1, 16, 14, 14, 96, 3, 1, 1, 40, 3, 1),    # conv3x3 -> conv3x3, 96 intermediate channels
 ]
 
 
