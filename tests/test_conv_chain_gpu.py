@@ -289,9 +289,9 @@ def test_conv_chain_rejects_what_it_cannot_fuse():
     with pytest.raises(NotImplementedError):  # 5x5 second filter
         chain.run_conv_chain(x, w1, torch.zeros(32, 32, 5, 5, device="cuda:0", dtype=torch.float16),
                              torch.zeros(1, 32, 14, 14, device="cuda:0", dtype=torch.float16), 0, 1, 2, 1)
-    w1b = torch.zeros(128, 16, 1, 1, device="cuda:0", dtype=torch.float16)
-    with pytest.raises(NotImplementedError):  # 3x3 second filter over more than 64 intermediate channels
-        chain.run_conv_chain(x, w1b, torch.zeros(32, 128, 3, 3, device="cuda:0", dtype=torch.float16),
+    w1b = torch.zeros(160, 16, 1, 1, device="cuda:0", dtype=torch.float16)
+    with pytest.raises(NotImplementedError):  # 3x3 second filter over more than 128 intermediate channels
+        chain.run_conv_chain(x, w1b, torch.zeros(32, 160, 3, 3, device="cuda:0", dtype=torch.float16),
                              torch.zeros(1, 32, 14, 14, device="cuda:0", dtype=torch.float16), 0, 1, 1, 1)
 
 
