@@ -266,8 +266,10 @@ struct ConvPlan {
   bool dw;             // depthwise first convolution: dwargs / c2_tiles / dw_shared describe the launch
   int c2_tiles;
   int dw_mode;         // 0 | 1: plain kernel (1: multiplier a multiple of 8); 2 | 3: persistent kernel,
-                       // depthwise stage on the matrix cores (2) or the vector ALU (3)
+                       // depthwise stage on the matrix cores (2) or the vector ALU (3); 4: the row-streaming
+                       // kernel (rowargs)
   ditto::DwConvArgs dwargs;
+  ditto::DwRowsArgs rowargs;
   bool resident;       // 1x1 -> 3x3 with at most 64 channels: persistent kernel, W2 resident in LDS
   int res_grid;
   ditto::ConvResidentArgs rargs;
@@ -278,9 +280,17 @@ struct ConvPlan {
 // dw_mode 2 | 3: the persistent kernel, depthwise stage on the matrix cores (multipliers that are
 // multiples of 16) or on the vector ALU (3x3, multiplier 1, 2, 4, 8); dw_mode 0 | 1: the plain
 // kernel for what is left (1: multiples of 8, 0: 1, 2, 4).
+// dw_mode 4: the row-streaming kernel (dw_rows.h) for multiplier 1, 3x3, pad 1, stride 1, at most 32 input and
+// 64 output channels, image rows of whole 16-byte vectors and at most 128 pixels, 16-bit output.
 // vec_cap: the widest halo vector (elements) the pointer of this call allows; 8 when planning without one.
+// DITTO_DW_ROWS=0 keeps such shapes on the persistent kernel (A/B runs, tests of that kernel).
+bool dw_rows_off() {
+  const char* v = getenv("DITTO_DW_ROWS");
+  return v && v[0] == '0';
+}
+
 int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvPlan* plan, bool need_device,
-                 bool allow_dwv = true, int vec_cap = 8) {
+                 bool allow_dwv = true, int vec_cap = 8, bool allow_rows = true) {
   if (d->C1 % d->C0) return fail(DITTO_EINVAL, "depthwise: C1 must be a multiple of C0");
   const long long mult = d->C1 / d->C0;
   const long long RS = d->R1 * d->S1;
@@ -301,6 +311,47 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   if (d->C1 > 32768) return fail(DITTO_EUNSUPPORTED, "depthwise chain: at most 32768 intermediate channels");
   memset(plan, 0, sizeof(*plan));
   plan->dw = true;
+  if (allow_rows && vec_cap >= 8 && !dw_rows_off() && mult == 1 && d->R1 == 3 && d->S1 == 3 && d->pad1 == 1 &&
+      d->stride1 == 1 && d->C0 <= ditto::kDwRowsC && d->C2 <= 64 && d->W % 8 == 0 && d->W <= 128 &&
+      d->out_dtype != DITTO_F32 && d->H * d->W * 64 < 0x7fffffffLL) {
+    // Bands of whole output rows, one workgroup each: all input rows of a band stay in LDS.  Among the
+    // band heights that fit, the one with the fewest row steps on the busiest CU (a band costs its rows
+    // plus the two halo rows plus about three steps of start-up).
+    const int cus = need_device ? device_cus() : 256;
+    int band_max = 0;
+    while (band_max < d->H && ditto::dw_rows_lds_bytes((int)d->W, band_max + 1) <= 160 * 1024) ++band_max;
+    if (band_max >= 1) {
+      long long best = -1;
+      int best_nb = 0;
+      const int nb_min = (int)((d->H + band_max - 1) / band_max);
+      for (int nb = nb_min; nb <= d->H && nb < nb_min + 64; ++nb) {
+        const int band = (int)((d->H + nb - 1) / nb);
+        const long long wgs = d->N * ((d->H + band - 1) / band);
+        const long long cost = ((wgs + cus - 1) / cus) * (band + 5);
+        if (best < 0 || cost < best) { best = cost; best_nb = nb; }
+      }
+      ditto::DwRowsArgs& r = plan->rowargs;
+      r.N = (int)d->N; r.C0 = (int)d->C0; r.H = (int)d->H; r.W = (int)d->W; r.C2 = (int)d->C2;
+      r.band = (int)((d->H + best_nb - 1) / best_nb);
+      r.bands = (int)((d->H + r.band - 1) / r.band);
+      r.relu_mid = d->inter_op == DITTO_INTER_RELU;
+      r.relu_out = d->relu_out != 0;
+      plan->dw_mode = 4;
+      plan->c2_tiles = 2;
+      ditto_tile_param& t = plan->tile;
+      t.block_threads = 64 * ditto::kDwRowsWaves;
+      t.block_m = r.band * r.W;
+      t.block_l = ditto::kDwRowsC;
+      t.block_n = 64;
+      t.head_pad = 0;
+      t.lds_bytes = ditto::dw_rows_lds_bytes(r.W, r.band);
+      t.grid_x = r.N * r.bands;
+      t.grid_y = r.band;
+      t.grid_z = r.W;
+      t.variant = 4000 + 20 + 4;
+      return DITTO_OK;
+    }
+  }
   plan->dw_mode = dwv ? 3 : mfma ? 2 : mult % 8 == 0 ? 1 : 0;
   const int c2t = d->C2 <= 32 ? 1 : d->C2 <= 64 ? 2 : d->C2 <= 128 ? 4 : 8;
   const int pxw = mfma ? ditto::dw_mfma_pxw(c2t) : c2t == 8 ? 1 : 2;
@@ -408,7 +459,7 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   a.relu_mid = d->inter_op == DITTO_INTER_RELU;
   a.relu_out = d->relu_out != 0;
   a.out_f32 = d->out_dtype == DITTO_F32;
-  if (dwv && !a.wide) return plan_dw_conv(d, P, Q, plan, need_device, false, vec_cap);  // that variant needs the wide stores
+  if (dwv && !a.wide) return plan_dw_conv(d, P, Q, plan, need_device, false, vec_cap, false);  // that variant needs the wide stores
   plan->c2_tiles = c2t;
   ditto_tile_param& t = plan->tile;
   t.block_threads = 256 * groups;
@@ -445,7 +496,7 @@ bool persist_requested() {
 }
 
 int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device = false, int dw_vec_cap = 8,
-              bool allow_resident = true) {
+              bool allow_resident = true, bool allow_dw_rows = true) {  // allow_dw_rows: y takes 16-byte stores
   if (!d) return fail(DITTO_EINVAL, "null descriptor");
   if (d->abi_version != DITTO_CHAIN_ABI_VERSION)
     return fail(DITTO_EINVAL, "descriptor abi_version %d, library %d", d->abi_version, DITTO_CHAIN_ABI_VERSION);
@@ -478,7 +529,8 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
   if (d->N * d->C0 * d->H * d->W > 0x7fffffffLL * 4 || d->N * d->C2 * P * Q > 0x7fffffffLL * 4 ||
       d->H > 65535 || d->W > 65535 || d->N > 65535 || d->C0 > 65535 || d->C2 > 65535)
     return fail(DITTO_EINVAL, "tensor too large");
-  if (dw) return plan_dw_conv(d, P, Q, plan, need_device, true, dw_vec_cap);
+  // (a y that is not 16-byte aligned rules out both kernels that only store 16-byte vectors)
+  if (dw) return plan_dw_conv(d, P, Q, plan, need_device, allow_dw_rows, dw_vec_cap, allow_dw_rows);
   memset(plan, 0, sizeof(*plan));
   const int c1t = d->C1 <= 32 ? 1 : d->C1 <= 64 ? 2 : d->C1 <= 128 ? 4 : 8;
   const int pxw = c1t == 8 ? 1 : 2;
@@ -798,7 +850,8 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
                     void* y, void* workspace, size_t workspace_bytes, void* stream) {
   ConvPlan plan;
   // (depthwise chains: 16-byte halo vectors only for a 16-byte aligned x; the tile query assumes one)
-  int rc = plan_conv(d, &plan, true, x && aligned(x, 16) ? 8 : 4);
+  // (the row-streaming depthwise kernel moves 16-byte vectors of x and y)
+  int rc = plan_conv(d, &plan, true, x && aligned(x, 16) ? 8 : 4, true, !y || aligned(y, 16));
   if (rc != DITTO_OK) return rc;
   if (((phase & kConvCompute) && (!x || !y)) || !w1 || !w2) return fail(DITTO_EINVAL, "null data pointer");
   if (plan.resident) {
@@ -839,6 +892,17 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
     return fail(DITTO_EWORKSPACE, "prepared weights live in the workspace: none given");
   if (plan.dw) {
     if (!(phase & kConvCompute)) return DITTO_OK;  // nothing to prepare: the kernel stages the filters itself
+    if (plan.dw_mode == 4) {
+      ditto::DwRowsArgs r = plan.rowargs;
+      r.x = x;
+      r.w1 = w1;
+      r.w2 = w2;
+      r.y = y;
+      hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+      hipError_t e = d->in_dtype == DITTO_F16 ? ditto::launch_dw_rows_f16(r, st) : ditto::launch_dw_rows_bf16(r, st);
+      if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
+      return DITTO_OK;
+    }
     if (!aligned(w2, 16)) return fail(DITTO_EINVAL, "misaligned data pointer");
     ditto::DwConvArgs a = plan.dwargs;
     // less aligned pointers: narrower halo loads (the LDS layout stays valid) while the chunk still

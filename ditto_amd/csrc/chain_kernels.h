@@ -6,6 +6,7 @@
 #include "conv_chain.h"
 #include "conv_chain_resident.h"
 #include "dw_conv_chain.h"
+#include "dw_rows.h"
 #include "gemm_chain_f32.h"
 #include "gemm_chain_i8.h"
 
@@ -39,5 +40,8 @@ hipError_t pack_conv_w2_resident_bf16(const void* w2, void* out, int C1, int C2,
 // stage (multiplier a multiple of 16); 3: persistent kernel, vector-ALU stage (3x3, multiplier 1, 2, 4, 8)
 hipError_t launch_dw_conv_f16(int c2_tiles, int mode, const DwConvArgs& args, hipStream_t stream);
 hipError_t launch_dw_conv_bf16(int c2_tiles, int mode, const DwConvArgs& args, hipStream_t stream);
+// depthwise 3x3 (multiplier 1) -> 1x1, at most 32 -> 64 channels, rows of at most 128 pixels (dw_rows.h)
+hipError_t launch_dw_rows_f16(const DwRowsArgs& args, hipStream_t stream);
+hipError_t launch_dw_rows_bf16(const DwRowsArgs& args, hipStream_t stream);
 
 }  // namespace ditto

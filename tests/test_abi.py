@@ -137,12 +137,22 @@ def test_conv_tile_choice_without_gpu(monkeypatch):
     assert b"switched off" in lib.ditto_last_error()
     assert lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc())) == 0
     monkeypatch.delenv("DITTO_CONV_PERSIST")
-    # depthwise first convolution: persistent kernel with the matrix-core or the vector-ALU depthwise stage
+    # depthwise first convolution: persistent kernel with the matrix-core depthwise stage; at multiplier 1 the
+    # row-streaming kernel (bands of 14 rows: one workgroup per CU, nine waves) for up to 32 -> 64 channels and
+    # the persistent kernel with the vector-ALU stage beyond
     dw = dict(C0=32, H=112, W=112, C2=64, groups1=32)
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=512, **dw)), ctypes.byref(tile)) == _lib.OK
     assert tile.variant == 4022 and tile.grid_x == 256
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=32, **dw)), ctypes.byref(tile)) == _lib.OK
+    assert (tile.variant, tile.grid_x, tile.grid_y, tile.block_threads) == (4024, 256, 14, 576)
+    assert tile.lds_bytes <= 160 * 1024
+    monkeypatch.setenv("DITTO_DW_ROWS", "0")
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=32, **dw)), ctypes.byref(tile)) == _lib.OK
     assert tile.variant == 4023
+    monkeypatch.delenv("DITTO_DW_ROWS")
+    dw = dict(C0=64, H=56, W=56, C2=128, groups1=64)
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=64, **dw)), ctypes.byref(tile)) == _lib.OK
+    assert tile.variant == 4043
 
 
 def test_run_rejects_bad_arguments_before_touching_the_device():

@@ -197,6 +197,9 @@ CASES_DEPTHWISE = [
     (1, 128, 8, 8, 2, 3, 1, 1, 256),     # 256 output channels
 ]
 DW_VECTOR_ALU_CASES = [c for c in CASES_DEPTHWISE if c[4] in (1, 2, 4, 8) and ((c[3] + 2 * c[6] - 3) // c[7] + 1) % 8 == 0]
+# factor 1, stride 1, at most 32 -> 64 channels, rows of whole 16-byte vectors up to 128 pixels: the
+# row-streaming kernel takes these when the output is 16-bit
+DW_ROWS_CASES = [c for c in DW_VECTOR_ALU_CASES if c[4] == 1 and c[7] == 1 and c[1] <= 32 and c[8] <= 64 and c[3] <= 128]
 
 
 @pytest.mark.parametrize("case", CASES_DEPTHWISE)
@@ -239,7 +242,76 @@ def test_small_factor_cases_run_the_persistent_kernel(case):
     P, Q = (H + 2 * pad - R) // stride + 1, (W + 2 * pad - R) // stride + 1
     y = torch.empty(N, C2, P, Q, device=dev, dtype=torch.float16)
     desc = chain.conv_chain_desc(x, w1, w2, y, pad, stride, 0, 1, "cast", False, C0)
-    assert chain.select_tile(desc).variant % 10 == 3
+    assert chain.select_tile(desc).variant % 10 == (4 if case in DW_ROWS_CASES else 3)
+
+
+CASES_DW_ROWS = [
+    # N, C0, H, W, C2: depthwise 3x3 (factor 1, pad 1, stride 1) -> 1x1 on the row-streaming kernel
+    (2, 32, 112, 112, 64),   # MobileNet-V1's first separable block: 7 load instructions per row, many bands
+    (1, 32, 56, 56, 64),     # half-filled last load instruction of a row (224 of 256 lanes)
+    (3, 7, 9, 8, 64),        # one strip per row, odd channel count, fewer rows than a band
+    (1, 24, 5, 128, 40),     # the widest row; output channels that do not fill their tiles
+    (2, 16, 33, 40, 24),     # a last band shorter than the others
+    (1, 32, 19, 72, 64),
+    (40, 8, 16, 16, 16),     # more workgroups than CUs with many bands
+]
+
+
+@pytest.mark.parametrize("case", CASES_DW_ROWS)
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_row_streaming_depthwise_chain(oracle, case, dtype, monkeypatch):
+    """The row-streaming kernel against the oracle and against the persistent kernel on the same inputs
+    (both accumulate in fp32 in different orders: held to the workload tolerance, not to the bits)."""
+    N, C0, H, W, C2 = case
+    rng = np.random.default_rng(C0 + C2 + W)
+    X = oracle.np_round_to(rng.standard_normal((N, C0, H, W)).astype(np.float32), dtype)
+    W1 = oracle.np_round_to(rng.standard_normal((C0, 1, 3, 3)).astype(np.float32) * 0.3, dtype)
+    W2 = oracle.np_round_to(rng.standard_normal((C2, C0, 1, 1)).astype(np.float32) * 0.2, dtype)
+    x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
+    for relu in (False, True):
+        y = torch.full((N, C2, H, W), float("nan"), device=x.device, dtype=x.dtype)
+        desc = chain.conv_chain_desc(x, w1, w2, y, 1, 1, 0, 1, "relu" if relu else "cast", relu, C0)
+        assert chain.select_tile(desc).variant == 4024
+        chain.run_conv_chain(x, w1, w2, y, desc=desc)
+        torch.cuda.synchronize()
+        got = y.float().cpu().numpy()
+        assert np.isfinite(got).all()
+        want = oracle.conv_chain_f32(X, W1, W2, 1, 1, 0, 1, relu_mid=relu, relu_out=relu, round_mid=dtype, groups1=C0)
+        mx, rel = errors(got, oracle.np_round_to(want, dtype))
+        if dtype == "bfloat16" and relu:
+            report("conv chain (wide second filter / depthwise) bf16 rows %s" % (case,), mx, rel)
+        assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
+        monkeypatch.setenv("DITTO_DW_ROWS", "0")
+        y2 = torch.full_like(y, float("nan"))
+        desc2 = chain.conv_chain_desc(x, w1, w2, y2, 1, 1, 0, 1, "relu" if relu else "cast", relu, C0)
+        assert chain.select_tile(desc2).variant % 10 != 4
+        chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
+        torch.cuda.synchronize()
+        monkeypatch.delenv("DITTO_DW_ROWS")
+        mx, rel = errors(got, y2.float().cpu().numpy())
+        assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
+
+
+def test_row_streaming_kernel_steps_aside_for_less_aligned_pointers(oracle):
+    """x or y not 16-byte aligned: the call runs on the persistent kernel instead (same result within tolerance)."""
+    N, C0, H, W, C2 = 1, 16, 16, 24, 32
+    rng = np.random.default_rng(3)
+    X = oracle.np_round_to(rng.standard_normal((N, C0, H, W)).astype(np.float32), "float16")
+    W1 = oracle.np_round_to(rng.standard_normal((C0, 1, 3, 3)).astype(np.float32) * 0.3, "float16")
+    W2 = oracle.np_round_to(rng.standard_normal((C2, C0, 1, 1)).astype(np.float32) * 0.2, "float16")
+    x, w1, w2 = to_dev(X, "float16"), to_dev(W1, "float16"), to_dev(W2, "float16")
+    want = oracle.np_round_to(oracle.conv_chain_f32(X, W1, W2, 1, 1, 0, 1, round_mid="float16", groups1=C0), "float16")
+    xbuf = torch.zeros(x.numel() + 8, device=x.device, dtype=torch.float16)
+    ybuf = torch.zeros(N * C2 * H * W + 8, device=x.device, dtype=torch.float16)
+    for xo, yo in ((0, 0), (4, 0), (0, 4), (1, 2)):
+        xs = xbuf[xo:xo + x.numel()].view_as(x)
+        xs.copy_(x)
+        ys = ybuf[yo:yo + N * C2 * H * W].view(N, C2, H, W)
+        ys.fill_(float("nan"))
+        chain.run_conv_chain(xs, w1, w2, ys, groups1=C0)
+        torch.cuda.synchronize()
+        mx, rel = errors(ys.float().cpu().numpy(), want)
+        assert mx <= MAX_ABS and rel <= REL_L2, (xo, yo, mx, rel)
 
 
 def test_depthwise_chain_with_less_aligned_pointers(oracle):
