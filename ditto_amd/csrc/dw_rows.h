@@ -16,10 +16,13 @@
 //    the strip's three input rows in registers (10 values each) and reads only the new row per step,
 //    one step ahead; 8 pixels x 3 rows x (one v_dot2 + one multiply-add) in fp32; the cast row goes to
 //    LDS as mid[pixel][32 channels] (16-byte chunks XOR-swizzled by pixel group, double buffered).
-//  * 1x1 stage of the previous row, same step: out[pixel][c2] = mid[pixel][:] . W2[c2][:] is ONE
-//    16x16x32 MFMA per 16 pixels x 16 output channels (W2 fragment resident in registers).  The MFMA
-//    rows of two tiles are dealt to the pixels so that a lane ends with 8 consecutive pixels of one
-//    output channel: one 16-byte store per lane, no turn-around.
+//  * 1x1 stage of the previous row, same step, on four waves of their own (16 output channels each,
+//    W2 fragment resident in registers): out^T[c2][pixel] = W2[c2][:] . mid[pixel][:] is ONE 16x16x32
+//    MFMA per 16 output channels x 16 pixels.  MFMA column j of tile t is pixel 8 j + t, so after the
+//    eight tiles of a row a lane holds 8 consecutive pixels of each of its 4 channels and the 16 lanes
+//    of a column group write 256 contiguous bytes of a channel with one 16-byte store each, no
+//    turn-around.  (Stores whose neighbouring lanes hit different 128-byte lines run at half the
+//    device's write bandwidth; waves that wait in the store queue do nothing else here.)
 //  One barrier per output row.
 //
 // Non-finite inputs behave as in the reference (every product is of values inside the 3x3 window).
@@ -39,13 +42,13 @@ struct DwRowsArgs {
 };
 
 constexpr int kDwRowsC = 32;        // input channels (padded)
-constexpr int kDwRowsWaves = 9;     // eight compute waves + the loader
+constexpr int kDwRowsWaves = 13;    // eight depthwise waves, four 1x1 / store waves, the loader
 constexpr int kDwRowsMaxAhead = 12; // input rows the loader keeps in flight at most
 
 __host__ __device__ constexpr int dw_rows_ni(int W) { return (W + 15) / 16; }
-// LDS: 16 bytes, band + 2 row slots of NI KB, 16 bytes, two intermediate rows of 64 bytes per pixel
+// LDS: 16 bytes, band + 2 row slots of NI KB, 16 bytes, two intermediate rows of 128 pixel slots of 64 bytes
 __host__ __device__ constexpr int dw_rows_lds_bytes(int W, int band) {
-  return 32 + (band + 2) * 1024 * dw_rows_ni(W) + 2 * ((W + 31) / 32 * 32) * 64;
+  return 32 + (band + 2) * 1024 * dw_rows_ni(W) + 2 * 128 * 64;
 }
 
 // wait until at most k rows of NI load instructions each are outstanding
@@ -84,7 +87,6 @@ __global__ __launch_bounds__(64 * kDwRowsWaves) void dw_rows_kernel(DwRowsArgs p
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int W = p.W, H = p.H, S = W >> 3;
-  const int Wp = (W + 31) & ~31;
   const unsigned wg = xcd_remap(blockIdx.x, gridDim.x);
   const int n = (int)wg / p.bands, y0 = ((int)wg - n * p.bands) * p.band;
   const int nout = H - y0 < p.band ? H - y0 : p.band;  // output rows of this band
@@ -94,7 +96,7 @@ __global__ __launch_bounds__(64 * kDwRowsWaves) void dw_rows_kernel(DwRowsArgs p
   char* const mids = rows + (p.band + 2) * SLOT + 16;
   const unsigned lds0 = (unsigned)(size_t)(DITTO_LDS char*)smem_raw;
 
-  if (wave == 8) {
+  if (wave == 12) {
     // ======================= loader wave =======================
     // instruction i of a row: lane l brings 16 bytes of job 64 i + l = channel * S + strip
     const i32x4 rsrc = make_rsrc_uniform(reinterpret_cast<const T*>(p.x) + (long long)n * p.C0 * plane,
@@ -115,6 +117,8 @@ __global__ __launch_bounds__(64 * kDwRowsWaves) void dw_rows_kernel(DwRowsArgs p
     constexpr int AH = 63 / NI < kDwRowsMaxAhead ? 63 / NI : kDwRowsMaxAhead;
     int issued = 0;
     while (issued < nin && issued < AH) issue(issued++);
+    dw_rows_wait<NI>(issued - 3 > 0 ? issued - 3 : 0);  // input rows 0, 1, 2: what the depthwise waves start from
+    __syncthreads();
     for (int r = 0; r <= nout; ++r) {
       // the compute waves read input row r + 3 during step r (one step ahead of its use)
       const int need = r + 3 < nin - 1 ? r + 3 : nin - 1;
@@ -131,8 +135,60 @@ __global__ __launch_bounds__(64 * kDwRowsWaves) void dw_rows_kernel(DwRowsArgs p
     return;
   }
 
-  // ======================= compute waves =======================
-  // ---- depthwise role: job = (channel c, strip of 8 pixels)
+  if (wave >= 8) {
+    // ======================= 1x1 / store waves =======================
+    const int c2q = wave - 8;
+    const int j = lane & 15, kg = lane >> 4;
+    // A operand: lane (m, kg) holds W2[16 c2q + m][8 kg .. + 7]
+    V8 wf;
+    {
+      const T* W2g = reinterpret_cast<const T*>(p.w2);
+      const int c2 = 16 * c2q + j;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int ch = 8 * kg + e;
+        wf[e] = (c2 < p.C2 && ch < p.C0) ? W2g[(long long)c2 * p.C0 + ch] : (T)0.f;
+      }
+    }
+    // B operand of tile t: lane (j, kg) reads channels 8 kg .. + 7 of pixel 8 j + t (slot 16 t + j)
+    const int b_rd = 64 * j + 16 * (kg ^ ((j >> 2) & 3));
+    // result: register i of tile t is out[c2 = 16 c2q + 4 kg + i][pixel 8 j + t]
+    unsigned y_vo[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c2 = 16 * c2q + 4 * kg + i;
+      y_vo[i] = (c2 < p.C2 && 8 * j < W) ? (unsigned)(c2 * (int)plane * 2 + 16 * j) : kOut;
+    }
+    const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<T*>(p.y) + (long long)n * p.C2 * plane, 0, (int)(p.C2 * plane * 2), 0x00020000);
+    __syncthreads();
+    for (int r = 0; r <= nout; ++r) {
+      __syncthreads();  // mid row r - 1 is written
+      if (r == 0) continue;
+      const char* const mr = mids + ((r - 1) & 1) * (128 * 64) + b_rd;
+      V8 bf[8];
+#pragma unroll
+      for (int t = 0; t < 8; ++t) bf[t] = *reinterpret_cast<const V8*>(mr + 1024 * t);
+      f32x4 o[8];
+      const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int t = 0; t < 8; ++t) o[t] = Elem<T>::mfma16(wf, bf[t], z);
+      const unsigned soff = (unsigned)((y0 + r - 1) * W * 2);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) v[t] = p.relu_out ? fmaxf(o[t][i], 0.f) : o[t][i];
+        const V2 q0 = cvt2<T>(v[0], v[1]), q1 = cvt2<T>(v[2], v[3]), q2 = cvt2<T>(v[4], v[5]), q3 = cvt2<T>(v[6], v[7]);
+        const V8 px8 = {q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, px8), y_rsrc, y_vo[i], soff, 0);
+      }
+    }
+    return;
+  }
+
+  // ======================= depthwise waves =======================
+  // job = (channel c, strip of 8 pixels)
   const int job = 64 * wave + lane;
   const bool dw_wave = wave < NI;  // wave-uniform
   const int c = job / S, strip = job - c * S;
@@ -183,83 +239,32 @@ __global__ __launch_bounds__(64 * kDwRowsWaves) void dw_rows_kernel(DwRowsArgs p
       acc[2 * m + 1] = Elem<T>::dot2(dm, w01[rr], fmaf(lo(m < 3 ? v.d[m + 1] : v.r), w2f[rr], acc[2 * m + 1]));
     }
   };
-  // intermediate row: mid[pixel][32 channels], 16-byte chunk ch of pixel px at chunk ch ^ ((px >> 3) & 3)
-  const int mid_wr = strip * 8 * 64 + 16 * ((c >> 3) ^ (strip & 3)) + 2 * (c & 7);
-
-  // ---- 1x1 role: 16 output channels (c2q), pixels 64 pt64 .. + 63 as two tiles of 32
-  const int c2q = wave >> 1, pt64 = wave & 1;
-  const int m16 = lane & 15, kg = lane >> 4;
-  const int c2 = 16 * c2q + m16;
-  V8 wf;
-  {
-    const T* W2g = reinterpret_cast<const T*>(p.w2);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int ch = 8 * kg + e;
-      wf[e] = (c2 < p.C2 && ch < p.C0) ? W2g[(long long)c2 * p.C0 + ch] : (T)0.f;
-    }
-  }
-  // A fragments: MFMA row m of the first MFMA of a tile is pixel 8 (m / 4) + m % 4 of the tile, of the
-  // second one that pixel + 4; lane (m, kg) reads the pixel's channels 8 kg .. + 7
-  int a_rd[2];
-  unsigned y_vo[2];
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int pt = 2 * pt64 + h;
-    const int px = 32 * pt + 8 * (m16 >> 2) + (m16 & 3);
-    a_rd[h] = px * 64 + 16 * (kg ^ ((m16 >> 2) & 3));
-    const int px_out = 32 * pt + 8 * kg;  // the lane's 8 consecutive output pixels
-    y_vo[h] = (c2 < p.C2 && px_out < W) ? (unsigned)(c2 * (int)plane * 2 + px_out * 2) : kOut;
-  }
-  const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      reinterpret_cast<T*>(p.y) + (long long)n * p.C2 * plane, 0, (int)(p.C2 * plane * 2), 0x00020000);
+  // intermediate row: pixel 8 j + t lives in slot 16 t + j (64 bytes: 32 channels), its 16-byte chunk ch at
+  // chunk ch ^ ((j >> 2) & 3): the 16 lanes of an MFMA operand read (fixed t, j = 0..15) hit every bank once
+  const int mid_wr = 64 * strip + 16 * ((c >> 3) ^ ((strip >> 2) & 3)) + 2 * (c & 7);
 
   Row r0, r1, r2, nx;
+  __syncthreads();  // input rows 0, 1, 2 have landed
+  if (dw_wave) {
+    r1 = read_row(0);
+    r2 = read_row(1);
+    nx = read_row(2);
+  }
   for (int r = 0; r <= nout; ++r) {
-    __syncthreads();  // input rows <= r + 3 have landed; mid row r - 1 is written, mid row r - 2 is read
+    __syncthreads();  // input rows <= r + 3 have landed; mid row r - 2 has been consumed
     if (dw_wave && r < nout) {
-      if (r == 0) {
-        r0 = read_row(0);
-        r1 = read_row(1);
-        r2 = read_row(2);
-      } else {
-        r0 = r1;
-        r1 = r2;
-        r2 = nx;
-      }
+      r0 = r1;
+      r1 = r2;
+      r2 = nx;
       if (r + 3 < nin) nx = read_row(r + 3);
       float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       dw_accumulate(r0, 0, acc);
       dw_accumulate(r1, 1, acc);
       dw_accumulate(r2, 2, acc);
       if (dw_on) {
-        T* const mw = reinterpret_cast<T*>(mids + (r & 1) * Wp * 64 + mid_wr);
+        T* const mw = reinterpret_cast<T*>(mids + (r & 1) * (128 * 64) + mid_wr);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) mw[32 * i] = (T)(p.relu_mid ? fmaxf(acc[i], 0.f) : acc[i]);
-      }
-    }
-    if (r >= 1) {
-      const char* const mr = mids + ((r - 1) & 1) * Wp * 64;
-      const unsigned soff = (unsigned)((y0 + r - 1) * W * 2);
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        if (32 * (2 * pt64 + h) >= W) continue;  // wave-uniform
-        const V8 a1 = *reinterpret_cast<const V8*>(mr + a_rd[h]);
-        const V8 a2 = *reinterpret_cast<const V8*>(mr + a_rd[h] + 4 * 64);
-        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-        f32x4 o1 = Elem<T>::mfma16(a1, wf, z);
-        f32x4 o2 = Elem<T>::mfma16(a2, wf, z);
-        if (p.relu_out) {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            o1[j] = fmaxf(o1[j], 0.f);
-            o2[j] = fmaxf(o2[j], 0.f);
-          }
-        }
-        const V2 q0 = cvt2<T>(o1[0], o1[1]), q1 = cvt2<T>(o1[2], o1[3]);
-        const V2 q2 = cvt2<T>(o2[0], o2[1]), q3 = cvt2<T>(o2[2], o2[3]);
-        const V8 px8 = {q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, px8), y_rsrc, y_vo[h], soff, 0);
+        for (int i = 0; i < 8; ++i) mw[512 * i] = (T)(p.relu_mid ? fmaxf(acc[i], 0.f) : acc[i]);
       }
     }
   }

@@ -144,7 +144,7 @@ def test_conv_tile_choice_without_gpu(monkeypatch):
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=512, **dw)), ctypes.byref(tile)) == _lib.OK
     assert tile.variant == 4022 and tile.grid_x == 256
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=32, **dw)), ctypes.byref(tile)) == _lib.OK
-    assert (tile.variant, tile.grid_x, tile.grid_y, tile.block_threads) == (4024, 256, 14, 576)
+    assert (tile.variant, tile.grid_x, tile.grid_y, tile.block_threads) == (4024, 256, 14, 832)
     assert tile.lds_bytes <= 160 * 1024
     monkeypatch.setenv("DITTO_DW_ROWS", "0")
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=32, **dw)), ctypes.byref(tile)) == _lib.OK
