@@ -43,6 +43,8 @@ UNITS = [
     ("conv_bf16", "conv_chain_inst.hip", ["-DDITTO_INST_T=bf16", "-DDITTO_INST_NAME=launch_conv_bf16", "-DDITTO_PACK_NAME=pack_conv_w1_bf16",
                                             "-DDITTO_INST2_NAME=launch_conv2_bf16", "-DDITTO_PACK2_NAME=pack_conv_w2_bf16", "-DDITTO_DW_NAME=launch_dw_conv_bf16",
                                             "-DDITTO_RES_NAME=launch_conv_resident_bf16", "-DDITTO_PACKRES_NAME=pack_conv_w2_resident_bf16"]),
+    ("conv_rows_f16", "conv_rows_inst.hip", ["-DDITTO_INST_T=f16", "-DDITTO_CONVROWS_NAME=launch_conv_rows_f16"]),
+    ("conv_rows_bf16", "conv_rows_inst.hip", ["-DDITTO_INST_T=bf16", "-DDITTO_CONVROWS_NAME=launch_conv_rows_bf16"]),
     ("dw_rows_f16", "dw_rows_inst.hip", ["-DDITTO_INST_T=f16", "-DDITTO_DWROWS_NAME=launch_dw_rows_f16"]),
     ("dw_rows_bf16", "dw_rows_inst.hip", ["-DDITTO_INST_T=bf16", "-DDITTO_DWROWS_NAME=launch_dw_rows_bf16"]),
     ("fp_f16_cast", "bmm_chain_fp_inst.hip",

@@ -273,6 +273,9 @@ struct ConvPlan {
   bool resident;       // 1x1 -> 3x3 with at most 64 channels: persistent kernel, W2 resident in LDS
   int res_grid;
   ditto::ConvResidentArgs rargs;
+  bool rows31;         // 3x3 -> 1x1 with at most 64 -> 64 -> 256 channels: the row pipeline (cvargs), W1 fragments
+                       // in the workspace
+  ditto::ConvRowsArgs cvargs;
   ditto_tile_param tile;
 };
 
@@ -490,6 +493,12 @@ bool resident_off() {
   return v && v[0] == '0';
 }
 
+// DITTO_CONV_ROWS=0 keeps the 3x3 -> 1x1 chains on the general kernel (A/B runs, tests of that kernel)
+bool conv_rows_off() {
+  const char* v = getenv("DITTO_CONV_ROWS");
+  return v && v[0] == '0';
+}
+
 bool persist_requested() {
   const char* v = getenv("DITTO_CONV_PERSIST");
   return v && v[0] == '1';
@@ -622,6 +631,51 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
     t.grid_z = a.TW2;
     t.variant = 3500 + c1t * 10 + plan->px2;  // second convolution through LDS
     return DITTO_OK;
+  }
+  // 3x3 (pad 1, stride 1) -> 1x1 with at most 64 input and intermediate and 256 output channels, image rows of
+  // whole 16-byte vectors up to 64 pixels, 16-bit output: the row pipeline (conv_rows.h).  Bands of whole
+  // output rows, one workgroup each; a band's rows are all in flight at once, which bounds its height.
+  if (allow_resident && !conv_rows_off() && !persist_requested() && d->R1 == 3 && d->S1 == 3 && d->pad1 == 1 &&
+      d->stride1 == 1 && d->C0 <= ditto::kCvrC && d->C1 <= ditto::kCvrC && d->C2 <= 256 && d->W % 8 == 0 && d->W <= 64 &&
+      d->out_dtype != DITTO_F32 && d->C0 * d->H * d->W * 2 < 0x7fffffffLL && d->C2 * d->H * d->W * 2 < 0x7fffffffLL) {
+    const int cus = need_device ? device_cus() : 256;
+    int band_max = ditto::conv_rows_band_max((int)d->W);
+    if (band_max > d->H) band_max = (int)d->H;
+    while (band_max >= 1 && ditto::conv_rows_lds_bytes((int)d->W, band_max) > 160 * 1024) --band_max;
+    if (band_max >= 1) {
+      // fewest steps of two rows on the busiest CU (a band costs its steps plus about three of start-up)
+      long long best = -1;
+      int best_nb = 0;
+      const int nb_min = (int)((d->H + band_max - 1) / band_max);
+      for (int nb = nb_min; nb <= d->H && nb < nb_min + 64; ++nb) {
+        const int band = (int)((d->H + nb - 1) / nb);
+        const long long wgs = d->N * ((d->H + band - 1) / band);
+        const long long cost = ((wgs + cus - 1) / cus) * ((band + 1) / 2 + 3);
+        if (best < 0 || cost <= best) { best = cost; best_nb = nb; }  // ties: the split that fills more CUs
+      }
+      ditto::ConvRowsArgs& r = plan->cvargs;
+      r.N = (int)d->N; r.C0 = (int)d->C0; r.H = (int)d->H; r.W = (int)d->W; r.C1 = (int)d->C1; r.C2 = (int)d->C2;
+      r.band = (int)((d->H + best_nb - 1) / best_nb);
+      r.bands = (int)((d->H + r.band - 1) / r.band);
+      r.relu_mid = d->inter_op == DITTO_INTER_RELU;
+      r.relu_out = d->relu_out != 0;
+      plan->rows31 = true;
+      plan->c1_tiles = 2;
+      plan->w1p_bytes = ditto::kCvrW1Bytes;
+      plan->w2p_bytes = 0;
+      ditto_tile_param& t = plan->tile;
+      t.block_threads = 64 * ditto::kCvrWaves;
+      t.block_m = r.band * r.W;
+      t.block_l = ditto::kCvrC;
+      t.block_n = (int)d->C2;
+      t.head_pad = ditto::kCvrC;
+      t.lds_bytes = ditto::conv_rows_lds_bytes(r.W, r.band);
+      t.grid_x = r.N * r.bands;
+      t.grid_y = r.band;
+      t.grid_z = r.W;
+      t.variant = 3700 + r.band;  // row pipeline; output rows per workgroup
+      return DITTO_OK;
+    }
   }
   // The persistent variant (conv_chain_persist.h: W1 resident in LDS, W2 in registers, one workgroup per
   // CU walking over the tiles) is switched off: it waits for its prefetched halo tile with a hand-counted
@@ -832,7 +886,7 @@ size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
   ConvPlan plan;
   if (plan_conv(desc, &plan) != DITTO_OK) return 0;
   size_t need = plan.w1p_bytes + plan.w2p_bytes;
-  if (plan.resident) {  // a call with pointers the resident kernel cannot take falls back to the general one
+  if (plan.resident || plan.rows31) {  // a call with pointers these kernels cannot take falls back to the general one
     ConvPlan general;
     if (plan_conv(desc, &general, false, 8, false) == DITTO_OK && general.w1p_bytes + general.w2p_bytes > need)
       need = general.w1p_bytes + general.w2p_bytes;
@@ -864,6 +918,37 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
       return fail(DITTO_EINVAL, "misaligned data pointer: this shape runs with x, w1 and y 16-byte aligned "
                                 "(its prepared weights are in the resident kernel's layout)");
     }
+  }
+  if (plan.rows31) {
+    // 16-byte direct loads of X, W2 fragments and output stores; W1 as MFMA fragments in the workspace
+    const bool ok = aligned(w2, 16) && workspace && workspace_bytes >= plan.w1p_bytes && aligned(workspace, 16) &&
+                    (!(phase & kConvCompute) || (aligned(x, 16) && aligned(y, 16)));
+    if (!ok && phase == kConvBoth) {
+      rc = plan_conv(d, &plan, true, 4, false);  // the general kernel: any element-aligned pointer, workspace optional
+      if (rc != DITTO_OK) return rc;
+    } else if (!ok) {
+      if (!workspace || workspace_bytes < plan.w1p_bytes)
+        return fail(DITTO_EWORKSPACE, "prepared weights live in the workspace: need %zu bytes", plan.w1p_bytes);
+      return fail(DITTO_EINVAL, "misaligned data pointer: this shape runs with x, w2, y and the workspace 16-byte "
+                                "aligned (its prepared weights are in the row pipeline's layout)");
+    }
+  }
+  if (plan.rows31) {
+    ditto::ConvRowsArgs r = plan.cvargs;
+    r.x = x;
+    r.w1f = workspace;
+    r.w2 = w2;
+    r.y = y;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const bool f16 = d->in_dtype == DITTO_F16;
+    hipError_t e = hipSuccess;
+    if (phase & kConvPrepare)  // W1 [C1][C0][3][3] into fragments: the same layout as the resident kernel's W2
+      e = f16 ? ditto::pack_conv_w2_resident_f16(w1, workspace, r.C0, r.C1, st)
+              : ditto::pack_conv_w2_resident_bf16(w1, workspace, r.C0, r.C1, st);
+    if (e == hipSuccess && (phase & kConvCompute))
+      e = f16 ? ditto::launch_conv_rows_f16(r, st) : ditto::launch_conv_rows_bf16(r, st);
+    if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
+    return DITTO_OK;
   }
   if (plan.resident) {
     if (!workspace) return fail(DITTO_EWORKSPACE, "this conv chain needs the workspace (%zu bytes)", plan.w2p_bytes);

@@ -5,6 +5,7 @@
 #include "bmm_chain_fp.h"
 #include "conv_chain.h"
 #include "conv_chain_resident.h"
+#include "conv_rows.h"
 #include "dw_conv_chain.h"
 #include "dw_rows.h"
 #include "gemm_chain_f32.h"
@@ -35,6 +36,9 @@ hipError_t launch_conv_resident_f16(const ConvResidentArgs& args, int grid, hipS
 hipError_t launch_conv_resident_bf16(const ConvResidentArgs& args, int grid, hipStream_t stream);
 hipError_t pack_conv_w2_resident_f16(const void* w2, void* out, int C1, int C2, hipStream_t stream);
 hipError_t pack_conv_w2_resident_bf16(const void* w2, void* out, int C1, int C2, hipStream_t stream);
+// 3x3 -> 1x1 with at most 64 -> 64 -> 256 channels, rows of at most 64 pixels: the row pipeline (conv_rows.h)
+hipError_t launch_conv_rows_f16(const ConvRowsArgs& args, hipStream_t stream);
+hipError_t launch_conv_rows_bf16(const ConvRowsArgs& args, hipStream_t stream);
 // depthwise first convolution (dw_conv_chain.h); c2_tiles in {1, 2, 4, 8}; mode 0 | 1: plain kernel,
 // vector-ALU depthwise stage (1: multiplier a multiple of 8); 2: persistent kernel, MFMA depthwise
 // stage (multiplier a multiple of 16); 3: persistent kernel, vector-ALU stage (3x3, multiplier 1, 2, 4, 8)

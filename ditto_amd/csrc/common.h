@@ -79,6 +79,18 @@ __device__ __forceinline__ typename Elem<T>::v2 cvt2(float a, float b) {
   return __builtin_convertvector(v, typename Elem<T>::v2);
 }
 
+// ReLU of packed fp16 / bf16 values after the conversion (rounding keeps the sign, so relu(round(x)) =
+// round(relu(x))): as signed 16-bit integers the negative values are exactly those with the sign bit, so one
+// packed integer max against zero per two values does it for either format (v_pk_max_i16).
+template <typename V>
+__device__ __forceinline__ V relu_packed(V v) {
+  typedef __attribute__((ext_vector_type(sizeof(V) / 2))) short S;
+  S s = __builtin_bit_cast(S, v);
+  const S z = {};
+  s = __builtin_elementwise_max(s, z);
+  return __builtin_bit_cast(V, s);
+}
+
 // LDS transpose read (gfx950 ds_read_b64_tr_b16).  Within each group of 16
 // lanes, lane i receives for j=0..3 the 16-bit element (i%4) of the 64-bit
 // word addressed by lane 4*j + i/4 of the same group.  If lane s of a group
@@ -148,6 +160,12 @@ __device__ __forceinline__ i32x4 make_rsrc_uniform(const void* base, unsigned by
              __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
   return r;
 }
+
+// Workgroup barrier for waves that hand data to each other through LDS: waits for this wave's own LDS
+// accesses first.  Spelled out because the compiler's own wait in front of __syncthreads() has been seen
+// missing behind LDS writes under divergent control flow at a loop's end (the next wave then read a slot
+// before the write had landed).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // Workgroups are dealt round-robin to the 8 XCDs (each with a private L2) by
 // linear id.  Remap so that ids that are neighbours in the logical order (and

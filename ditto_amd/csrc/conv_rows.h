@@ -1,0 +1,314 @@
+// conv(3x3, pad 1, stride 1) -> cast|relu -> conv(1x1) on NCHW fp16 / bf16 tensors with at most 64 input
+// and intermediate channels, at most 256 output channels and image rows of at most 64 pixels (whole
+// 16-byte vectors), 16-bit output: the bottleneck block of a ResNet-50 at 56 x 56.
+//
+// Reference chain: benchmark/chimera/cuda/conv_relu_conv_relu... / testing/hyper_fusion/
+// conv_relu_conv_relu_fuse_hw_cuda.py (conv3x3 -> conv1x1, the second GEMM consuming the first one's tile).
+//
+// The chain is bound by its output traffic (256 channels out for 64 in), so the kernel is built as a
+// pipeline over image rows whose stages run on waves of their own inside one workgroup, and the output
+// stores start as soon as the first rows are through instead of after the whole tile:
+//
+//  * A workgroup owns a band of output rows of one image.  Waves 0..3 issue ALL input rows of the band
+//    (band + 2, a quarter each) as direct global -> LDS loads at kernel start ([channel][W] per row; rows
+//    outside the image are out of range and arrive as zeros) together with their W1 fragments, wait for
+//    them once, and issue no memory instruction afterwards.  The wave that loaded a row turns it round
+//    into Xt[pixel + 1][64 channels] (a ring of 6 rows with a zero pixel left and right, 16-byte chunks
+//    XOR-swizzled by pixel pair so that 16 consecutive pixels cover every LDS bank once) with the
+//    transposing LDS read, one step before the row is needed.
+//  * Step k = output rows 2k, 2k + 1.  First convolution on waves 0..3 = (row, half of the intermediate
+//    channels): mid^T[c1][pixel] = W1 . X as 36 x 2 MFMAs 32x32x16 with the wave's 36 W1 fragments
+//    RESIDENT IN REGISTERS (loaded once from the repacked copy in the workspace) and the pixel
+//    fragments read from Xt at the tap's offset; the cast result goes to LDS as mid[pixel][64]
+//    (double buffered).
+//  * Second convolution of the previous step on waves 4..7 (64 output channels each, W2 fragments in
+//    registers, one wave per SIMD next to a first-convolution wave): out^T[c2][pixel] = W2 . mid as
+//    16x16x32 MFMAs whose column j of tile t is pixel 8 j + t of the step, so a lane ends with 8
+//    consecutive pixels of each of its 4 channels and the 16 lanes of a column group store whole runs
+//    of a channel row with one 16-byte store each.
+//  One barrier per step; the only waves that wait for memory after the prologue are waves 4..7, in the
+//  store queue.
+#pragma once
+#include "common.h"
+
+namespace ditto {
+
+struct ConvRowsArgs {
+  const void* x;    // [N][C0][H][W]
+  const void* w1f;  // W1 as MFMA fragments [tap][c0 / 16][c1 / 32][lane][8] (pack_conv_w2_resident's layout)
+  const void* w2;   // [C2][C1]
+  void* y;          // [N][C2][H][W]
+  int N, C0, H, W, C1, C2;
+  int band, bands;  // output rows per workgroup, workgroups per image
+  int relu_mid, relu_out;
+};
+
+constexpr int kCvrC = 64;      // input / intermediate channels (padded)
+constexpr int kCvrWaves = 8;   // four load / first-convolution waves, four second-convolution / store waves
+constexpr int kCvrRing = 6;    // rows of the transposed ring
+constexpr int kCvrW1Bytes = 9 * kCvrC * kCvrC * 2;
+
+// LDS: band + 2 raw rows of 128 W bytes, the ring of transposed rows, two intermediate steps of 2 W pixels
+__host__ __device__ constexpr int conv_rows_lds_bytes(int W, int band) {
+  return (band + 2) * 128 * W + kCvrRing * (W + 2) * 128 + 2 * (2 * W) * 128;
+}
+// a wave keeps its quarter of the band's rows in flight at once, W / 8 load instructions per row, next to the 36
+// loads of its W1 fragments: stay well inside the 6-bit outstanding-load counter
+__host__ __device__ constexpr int conv_rows_band_max(int W) { return 4 * (24 / (W / 8)) - 2; }
+
+template <typename T, int NI>
+__global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef typename Elem<T>::v8 V8;
+  typedef typename Elem<T>::v4 V4;
+  typedef typename Elem<T>::v2 V2;
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  constexpr unsigned kOut = 0x7fffffffu;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 31, g = lane >> 5;
+  const int Wi = p.W, H = p.H;
+  const int MW = Wi + 2, SJ = Wi >> 2;  // pixels of a transposed row; strips of 8 pixels in a step of two rows
+  const int RAWROW = 128 * Wi, XTROW = MW * 128, MIDBUF = 2 * Wi * 128;
+  const unsigned wg = xcd_remap(blockIdx.x, gridDim.x);
+  const int n = (int)wg / p.bands, y0 = ((int)wg - n * p.bands) * p.band;
+  const int nout = H - y0 < p.band ? H - y0 : p.band;
+  const int nin = nout + 2;
+  const int nsteps = (nout + 1) >> 1;
+  const long long plane = (long long)H * Wi;
+  char* const raw = smem_raw;
+  char* const Xt = raw + (p.band + 2) * RAWROW;
+  char* const mid = Xt + kCvrRing * XTROW;
+  const unsigned lds0 = (unsigned)(size_t)(DITTO_LDS char*)smem_raw;
+
+  if (wave >= 4) {
+    // ======================= second convolution / stores =======================
+    const int hh = wave - 4;  // output channels 64 hh .. 64 hh + 63
+    const int j = lane & 15, kg = lane >> 4;
+    // A operand: lane (m, kg) holds W2[64 hh + 16 ct + m][32 ks + 8 kg .. + 7]
+    V8 w2f[4][2];
+    {
+      const T* W2g = reinterpret_cast<const T*>(p.w2);
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const int c2 = 64 * hh + 16 * ct + j, k0 = 32 * ks + 8 * kg;
+          V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+          if (c2 < p.C2 && k0 < p.C1) v = *reinterpret_cast<const V8*>(W2g + (long long)c2 * p.C1 + k0);
+          w2f[ct][ks] = v;
+        }
+    }
+    // B operand of tile t: lane (j, kg) reads channels 32 ks + 8 kg .. + 7 of pixel 8 j + t of the step
+    // (slot SJ t + j, chunk index XORed with (j >> 1) & 7)
+    const int jc = j < SJ ? j : 0;
+    const int b_rd = jc * 128, b_x = (jc >> 1) & 7;
+    // the lane's 8 output pixels 8 j .. 8 j + 7 of the step: row 8 j / W of the two, column 8 j % W
+    const int S8 = Wi >> 3;
+    const int prow = j / S8, pcol = 8 * (j - prow * S8);
+    const unsigned y_lane = (unsigned)((64 * hh + 4 * kg) * (int)plane * 2 + (prow * Wi + pcol) * 2);
+    const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<T*>(p.y) + (long long)n * p.C2 * plane, 0, (int)(p.C2 * plane * 2), 0x00020000);
+    for (int k = 0; k <= nsteps; ++k) {
+      lds_barrier();  // the intermediate rows of step k - 1 are written
+      if (k == 0 || 64 * hh >= p.C2) continue;
+      const int s = k - 1;
+      const char* const mr = mid + (s & 1) * MIDBUF + b_rd;
+      V8 bf[2][8];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) bf[ks][t] = *reinterpret_cast<const V8*>(mr + SJ * t * 128 + (((4 * ks + kg) ^ b_x) << 4));
+      const bool row_ok = j < SJ && 2 * s + prow < nout;
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct) {
+        if (64 * hh + 16 * ct >= p.C2) break;  // wave-uniform
+        f32x4 o[8];
+        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < 8; ++t) o[t] = Elem<T>::mfma16(w2f[ct][0], bf[0][t], z);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) o[t] = Elem<T>::mfma16(w2f[ct][1], bf[1][t], o[t]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const V2 q0 = cvt2<T>(o[0][i], o[1][i]), q1 = cvt2<T>(o[2][i], o[3][i]);
+          const V2 q2 = cvt2<T>(o[4][i], o[5][i]), q3 = cvt2<T>(o[6][i], o[7][i]);
+          V8 px8 = {q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
+          if (p.relu_out) px8 = relu_packed(px8);
+          const int c2 = 64 * hh + 16 * ct + 4 * kg + i;
+          const unsigned vo = (row_ok && c2 < p.C2) ? y_lane : kOut;
+          const unsigned soff = (unsigned)((y0 + 2 * s) * Wi * 2 + (16 * ct + i) * (int)plane * 2);
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, px8), y_rsrc, vo, soff, 0);
+        }
+      }
+    }
+    return;
+  }
+
+  // ======================= loads, transposition and first convolution =======================
+  const int rho = wave & 1, c1t = wave >> 1;
+  // ---- this wave's input rows: q = wave, wave + 4, ... (all issued at once; the wave issues no other
+  // memory instruction after its prologue, so its counter waits are exact)
+  const int S8 = Wi >> 3;  // 16-byte pieces per channel row
+  {
+    const i32x4 rsrc = make_rsrc_uniform(reinterpret_cast<const T*>(p.x) + (long long)n * p.C0 * plane,
+                                         (unsigned)(p.C0 * plane * 2));
+#pragma unroll 1
+    for (int q = wave; q < nin; q += 4) {
+      const int y = y0 - 1 + q;
+      const bool ok = y >= 0 && y < H;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int job = 64 * i + lane, c = job / S8, piece = job - c * S8;  // channels >= C0 are out of range
+        const unsigned vo = ok ? (unsigned)(c * (int)plane * 2 + piece * 16 + y * Wi * 2) : kOut;
+        lds_dma_16(rsrc, vo, lds0 + q * RAWROW + 1024 * i);
+      }
+    }
+  }
+  // the zero pixels left and right of every ring row
+  if (wave == 0)
+    for (int i = lane; i < kCvrRing * 2 * 8; i += 64) {
+      const int row = i >> 4, side = (i >> 3) & 1, piece = i & 7;
+      *reinterpret_cast<i32x4*>(Xt + row * XTROW + (side ? (Wi + 1) * 128 : 0) + piece * 16) = i32x4{0, 0, 0, 0};
+    }
+  // the wave's fragments of W1: step st = (tap, kk), lane (ln, g) holds W1[32 c1t + ln][16 kk + 8 g .. + 7][tap]
+  constexpr int NSTEP = 36;
+  V8 w1f[NSTEP];
+  {
+    const char* w = reinterpret_cast<const char*>(p.w1f) + c1t * 1024 + lane * 16;
+#pragma unroll
+    for (int st = 0; st < NSTEP; ++st) w1f[st] = *reinterpret_cast<const V8*>(w + st * 2048);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // W1 fragments and this wave's rows: from here on LDS only
+  // raw row q -> ring slot q % 6: unit (pixel tile t of 32, 16 channels kk): the lane receives channels
+  // 16 kk + 8 g .. + 7 of pixel 32 t + ln (two transposing reads) and writes them as one 16-byte chunk
+  const int i16 = lane & 15, h = (lane >> 4) & 1;
+  const int ntile = (Wi + 31) >> 5;
+  auto transpose_row = [&](int q) __attribute__((always_inline)) {
+    const char* const src = raw + q * RAWROW;
+    char* const dst = Xt + (q % kCvrRing) * XTROW;
+    // per pixel tile: its reads first (one LDS round trip), then the writes
+#pragma unroll 1
+    for (int t = 0; t < ntile; ++t) {
+      V8 v[4];
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const char* rd = src + (16 * kk + 8 * g + (i16 >> 2)) * (2 * Wi) + (32 * t + 16 * h + 4 * (i16 & 3)) * 2;
+        const V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(rd));
+        const V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(rd + 4 * 2 * Wi));
+        v[kk] = concat4<V4, V8>(lo, hi);
+      }
+      const int px = 32 * t + ln, col = px + 1;
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk)
+        if (px < Wi) *reinterpret_cast<V8*>(dst + col * 128 + (((2 * kk + g) ^ ((col >> 1) & 7)) << 4)) = v[kk];
+    }
+  };
+  if (wave < nin) transpose_row(wave);  // rows 0 .. 3: what step 0 reads
+
+  // pixel tiles pt = 0, 1: column ln of the MFMA is pixel 32 pt + ln of the row; pixels past the row read pixel 0.
+  // Ring rows are whole multiples of 128 bytes, so a fragment's address is (row + xb) ^ (chunk << 4) with
+  // xb = column * 128 | swizzle << 4; likewise the intermediate pixel's chunk is at (buffer + mb) ^ (chunk << 4)
+  int xb[2][3], mb[2];
+  bool px_ok[2];
+#pragma unroll
+  for (int pt = 0; pt < 2; ++pt) {
+    const int px = 32 * pt + ln;
+    px_ok[pt] = px < Wi;
+    const int pxc = px_ok[pt] ? px : 0;
+#pragma unroll
+    for (int ds = 0; ds < 3; ++ds) {
+      const int col = pxc + ds;
+      xb[pt][ds] = col * 128 | (((col >> 1) & 7) << 4);
+    }
+    // pixel of the step: slot SJ t + j with 8 j + t = W rho + px
+    const int pp = Wi * rho + pxc, jj = pp >> 3, tt = pp & 7;
+    mb[pt] = (SJ * tt + jj) * 128 | (((jj >> 1) & 7) << 4) | 8 * g;
+  }
+  for (int k = 0; k <= nsteps; ++k) {
+    lds_barrier();  // the transposed rows of step k are there; the buffer of step k - 2 has been read
+    // rows 2k + 4, 2k + 5 for the next step (their ring slots were last read in step k - 1): the wave that loaded them
+    {
+      const int q = 2 * k + 4 + (wave & 1);
+      if ((q & 3) == wave && q < nin) transpose_row(q);
+    }
+    const int r = 2 * k + rho;
+    if (k == nsteps || r >= nout) continue;
+    int rowoff[3];
+#pragma unroll
+    for (int dr = 0; dr < 3; ++dr) rowoff[dr] = ((r + dr) % kCvrRing) * XTROW;
+    f32x16 acc[2];
+#pragma unroll
+    for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[pt][e] = 0.f;
+    constexpr int kAhead = 3;
+    V8 xf[NSTEP][2];
+    auto fetch = [&](int st) __attribute__((always_inline)) {
+      const int tap = st >> 2, kk = st & 3, dr = tap / 3, ds = tap - 3 * dr;
+#pragma unroll
+      for (int pt = 0; pt < 2; ++pt)
+        xf[st][pt] = *reinterpret_cast<const V8*>(Xt + ((rowoff[dr] + xb[pt][ds]) ^ ((2 * kk + g) << 4)));
+    };
+#pragma unroll
+    for (int st = 0; st < kAhead; ++st) fetch(st);
+#pragma unroll
+    for (int st = 0; st < NSTEP; ++st) {
+      if (st + kAhead < NSTEP) fetch(st + kAhead);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int pt = 0; pt < 2; ++pt) acc[pt] = Elem<T>::mfma32(w1f[st], xf[st][pt], acc[pt]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // acc[pt][4 i + e] = mid[c1 = 32 c1t + 8 i + 4 g + e][pixel]: 8 bytes into chunk 4 c1t + i of the pixel
+    char* const mw = mid + (k & 1) * MIDBUF;  // (both buffers start on multiples of 128 bytes)
+#pragma unroll
+    for (int pt = 0; pt < 2; ++pt) {
+      if (!px_ok[pt]) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const V2 a0 = cvt2<T>(acc[pt][4 * i], acc[pt][4 * i + 1]), a1 = cvt2<T>(acc[pt][4 * i + 2], acc[pt][4 * i + 3]);
+        V4 w = {a0[0], a0[1], a1[0], a1[1]};
+        if (p.relu_mid) w = relu_packed(w);
+        *reinterpret_cast<V4*>(mw + (mb[pt] ^ ((4 * c1t + i) << 4))) = w;
+      }
+    }
+  }
+#else
+  (void)p;
+#endif
+}
+
+template <typename T, int NI>
+hipError_t launch_conv_rows_ni(const ConvRowsArgs& args, hipStream_t stream) {
+  const int lds = conv_rows_lds_bytes(args.W, args.band);
+  auto kern = conv_rows_kernel<T, NI>;
+  static thread_local int configured_dev = -1;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (configured_dev != dev) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return e;
+    configured_dev = dev;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)(args.N * args.bands)), dim3(64 * kCvrWaves), lds, stream, args);
+  return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_conv_rows(const ConvRowsArgs& args, hipStream_t stream) {
+  switch (args.W / 8) {
+    case 1: return launch_conv_rows_ni<T, 1>(args, stream);
+    case 2: return launch_conv_rows_ni<T, 2>(args, stream);
+    case 3: return launch_conv_rows_ni<T, 3>(args, stream);
+    case 4: return launch_conv_rows_ni<T, 4>(args, stream);
+    case 5: return launch_conv_rows_ni<T, 5>(args, stream);
+    case 6: return launch_conv_rows_ni<T, 6>(args, stream);
+    case 7: return launch_conv_rows_ni<T, 7>(args, stream);
+    case 8: return launch_conv_rows_ni<T, 8>(args, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace ditto

@@ -118,14 +118,14 @@ __global__ __launch_bounds__(64 * kDwRowsWaves) void dw_rows_kernel(DwRowsArgs p
     int issued = 0;
     while (issued < nin && issued < AH) issue(issued++);
     dw_rows_wait<NI>(issued - 3 > 0 ? issued - 3 : 0);  // input rows 0, 1, 2: what the depthwise waves start from
-    __syncthreads();
+    lds_barrier();
     for (int r = 0; r <= nout; ++r) {
       // the compute waves read input row r + 3 during step r (one step ahead of its use)
       const int need = r + 3 < nin - 1 ? r + 3 : nin - 1;
       int k = issued - 1 - need;  // rows that may still be outstanding
       if (k < 0) k = 0;
       dw_rows_wait<NI>(k);
-      __syncthreads();
+      lds_barrier();
       while (issued < nin && k < AH) {
         issue(issued++);
         ++k;
@@ -161,9 +161,9 @@ __global__ __launch_bounds__(64 * kDwRowsWaves) void dw_rows_kernel(DwRowsArgs p
     }
     const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         reinterpret_cast<T*>(p.y) + (long long)n * p.C2 * plane, 0, (int)(p.C2 * plane * 2), 0x00020000);
-    __syncthreads();
+    lds_barrier();
     for (int r = 0; r <= nout; ++r) {
-      __syncthreads();  // mid row r - 1 is written
+      lds_barrier();  // mid row r - 1 is written
       if (r == 0) continue;
       const char* const mr = mids + ((r - 1) & 1) * (128 * 64) + b_rd;
       V8 bf[8];
@@ -244,14 +244,14 @@ __global__ __launch_bounds__(64 * kDwRowsWaves) void dw_rows_kernel(DwRowsArgs p
   const int mid_wr = 64 * strip + 16 * ((c >> 3) ^ ((strip >> 2) & 3)) + 2 * (c & 7);
 
   Row r0, r1, r2, nx;
-  __syncthreads();  // input rows 0, 1, 2 have landed
+  lds_barrier();  // input rows 0, 1, 2 have landed
   if (dw_wave) {
     r1 = read_row(0);
     r2 = read_row(1);
     nx = read_row(2);
   }
   for (int r = 0; r <= nout; ++r) {
-    __syncthreads();  // input rows <= r + 3 have landed; mid row r - 2 has been consumed
+    lds_barrier();  // input rows <= r + 3 have landed; mid row r - 2 has been consumed
     if (dw_wave && r < nout) {
       r0 = r1;
       r1 = r2;

@@ -127,10 +127,23 @@ def test_conv_tile_choice_without_gpu(monkeypatch):
     lib = _lib.load()
     tile = _lib.TileParam()
     monkeypatch.delenv("DITTO_CONV_PERSIST", raising=False)
+    # the workload shape runs on the row pipeline: bands of 7 output rows, one workgroup per CU, seven waves
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc()), ctypes.byref(tile)) == _lib.OK
+    assert (tile.variant, tile.grid_x, tile.grid_y, tile.block_threads) == (3707, 256, 7, 512)
+    assert tile.lds_bytes <= 160 * 1024
+    rows_ws = lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc()))
+    # W1 as MFMA fragments takes 9 * 64 * 64 * 2 bytes; the query covers the general kernel too, which a call
+    # with less aligned pointers falls back to
+    assert rows_ws == max(9 * 64 * 64 * 2, 2 * 9 * 64 * 40 * 2)
+    # fp32 output, wider rows or more channels stay on the general kernel, and so does everything with DITTO_CONV_ROWS=0
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(out_dtype=_lib.F32)), ctypes.byref(tile)) == _lib.OK
+    assert tile.variant == 3022
+    monkeypatch.setenv("DITTO_CONV_ROWS", "0")
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc()), ctypes.byref(tile)) == _lib.OK
     assert tile.variant == 3022 and tile.grid_x == 32 * 14 and tile.lds_bytes <= 80 * 1024  # two workgroups per CU
     default_ws = lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc()))
     assert default_ws == 2 * 9 * 64 * 40 * 2  # two chunks of 32 input channels, [tap][c1][32 + 8]
+    monkeypatch.delenv("DITTO_CONV_ROWS")
     # the opt-in persistent kernel is switched off: asking for it is refused, not silently ignored
     monkeypatch.setenv("DITTO_CONV_PERSIST", "1")
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc()), ctypes.byref(tile)) == _lib.EUNSUPPORTED

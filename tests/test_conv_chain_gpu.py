@@ -40,6 +40,13 @@ CASES = [
 ]
 
 
+def rows_pipeline_shape(case):
+    """3x3 (pad 1, stride 1) -> 1x1, at most 64 -> 64 -> 256 channels, rows of whole 16-byte vectors up to 64 pixels:
+    with a 16-bit output and a workspace these run on the row pipeline."""
+    N, C0, H, W, C1, R, pad, stride, C2 = case
+    return R == 3 and pad == 1 and stride == 1 and C0 <= 64 and C1 <= 64 and C2 <= 256 and W % 8 == 0 and W <= 64
+
+
 @pytest.mark.parametrize("case", CASES)
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
 def test_conv_chain_vs_oracle(oracle, case, dtype):
@@ -53,11 +60,63 @@ def test_conv_chain_vs_oracle(oracle, case, dtype):
         mx, rel = errors(got32, want32)
         assert mx <= MAX_ABS and rel <= REL_L2, (ws, mx, rel)
         got = run_conv(X, W1, W2, dtype, pad, stride, workspace=ws)
-        assert np.array_equal(got, oracle.np_round_to(got32, dtype)), ws
+        if not (ws is None and rows_pipeline_shape(case)):
+            # (with a workspace that shape runs on the row pipeline, whose summation order is its own)
+            assert np.array_equal(got, oracle.np_round_to(got32, dtype)), ws
         mx, rel = errors(got, oracle.np_round_to(want32, dtype))
         if dtype == "bfloat16":
             report("conv chain bf16 %s" % (case,), mx, rel)
         assert mx <= MAX_ABS and rel <= REL_L2, (ws, mx, rel)
+
+
+CASES_ROWS_PIPELINE = [
+    # N, C0, H, W, C1, C2: conv3x3 (pad 1, stride 1) -> conv1x1 on the row pipeline
+    (2, 64, 56, 56, 64, 256),   # the workload's shape, 2 images: bands of 7 rows (3 steps of two rows and one of one)
+    (1, 64, 9, 64, 64, 256),    # the widest row (two full pixel tiles, 16 strips per step); bands of 5
+    (3, 24, 11, 8, 40, 72),     # one strip per row, channel counts that fill no tile, a short last band
+    (1, 16, 1, 16, 8, 16),      # a single output row
+    (2, 48, 30, 40, 32, 136),   # the second store wave takes 8 of its 128 channels
+    (40, 8, 12, 24, 16, 32),    # more workgroups than CUs
+]
+
+
+@pytest.mark.parametrize("case", CASES_ROWS_PIPELINE)
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_conv_chain_row_pipeline(oracle, case, dtype, monkeypatch):
+    """The row pipeline against the oracle and against the general kernel on the same inputs (different
+    summation orders: held to the workload tolerance), through run and through prepare + run_prepared."""
+    N, C0, H, W, C1, C2 = case
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, 3, 1, dtype, seed=C0 + C2 + W, w_std=0.05)
+    x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
+    for relu in (False, True):
+        inter = "relu" if relu else "cast"
+        y = torch.full((N, C2, H, W), float("nan"), device=x.device, dtype=x.dtype)
+        desc = chain.conv_chain_desc(x, w1, w2, y, 1, 1, 0, 1, inter, relu)
+        assert chain.select_tile(desc).variant // 100 == 37
+        chain.run_conv_chain(x, w1, w2, y, desc=desc)
+        torch.cuda.synchronize()
+        got = y.float().cpu().numpy()
+        assert np.isfinite(got).all()
+        want = oracle.conv_chain_f32(X, W1, W2, 1, 1, 0, 1, relu_mid=relu, relu_out=relu, round_mid=dtype)
+        mx, rel = errors(got, oracle.np_round_to(want, dtype))
+        if dtype == "bfloat16" and relu:
+            report("conv chain bf16 row pipeline %s" % (case,), mx, rel)
+        assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
+        # prepared weights: same bits as the one-call form
+        ws = chain.prepare_conv_chain(desc, w1, w2)
+        y1 = torch.full_like(y, float("nan"))
+        chain.run_conv_chain(x, w1, w2, y1, desc=desc, workspace=ws, prepared=True)
+        torch.cuda.synchronize()
+        assert torch.equal(y1, y), relu
+        monkeypatch.setenv("DITTO_CONV_ROWS", "0")
+        y2 = torch.full_like(y, float("nan"))
+        desc2 = chain.conv_chain_desc(x, w1, w2, y2, 1, 1, 0, 1, inter, relu)
+        assert chain.select_tile(desc2).variant // 100 != 37
+        chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
+        torch.cuda.synchronize()
+        monkeypatch.delenv("DITTO_CONV_ROWS")
+        mx, rel = errors(got, y2.float().cpu().numpy())
+        assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
 
 
 # Enough tiles of whole output rows for two rounds of persistent workgroups (at least 512), 16-bit
