@@ -9,10 +9,11 @@
 // pipeline over image rows whose stages run on waves of their own inside one workgroup, and the output
 // stores start as soon as the first rows are through instead of after the whole tile:
 //
-//  * A workgroup owns a band of output rows of one image.  Waves 0..3 issue ALL input rows of the band
-//    (band + 2, a quarter each) as direct global -> LDS loads at kernel start ([channel][W] per row; rows
-//    outside the image are out of range and arrive as zeros) together with their W1 fragments, wait for
-//    them once, and issue no memory instruction afterwards.  The wave that loaded a row turns it round
+//  * A workgroup owns a band of output rows of one image.  ALL input rows of the band (band + 2) are
+//    issued at kernel start as direct global -> LDS loads ([channel][W] per row; rows outside the image
+//    are out of range and arrive as zeros): rows 0..3 by waves 0..3 ahead of their W1 fragments, rows
+//    4 and 5 by waves 4 and 5, the rest by waves 6 and 7 - waves 4..7 have nothing to store before step 1
+//    and wait for their rows before then, so every counter wait is exact.  Waves 0..3 turn the rows round
 //    into Xt[pixel + 1][64 channels] (a ring of 6 rows with a zero pixel left and right, 16-byte chunks
 //    XOR-swizzled by pixel pair so that 16 consecutive pixels cover every LDS bank once) with the
 //    transposing LDS read, one step before the row is needed.
@@ -52,9 +53,9 @@ constexpr int kCvrW1Bytes = 9 * kCvrC * kCvrC * 2;
 __host__ __device__ constexpr int conv_rows_lds_bytes(int W, int band) {
   return (band + 2) * 128 * W + kCvrRing * (W + 2) * 128 + 2 * (2 * W) * 128;
 }
-// a wave keeps its quarter of the band's rows in flight at once, W / 8 load instructions per row, next to the 36
-// loads of its W1 fragments: stay well inside the 6-bit outstanding-load counter
-__host__ __device__ constexpr int conv_rows_band_max(int W) { return 4 * (24 / (W / 8)) - 2; }
+// waves 6 and 7 keep half each of the band's rows from the seventh on in flight at once, W / 8 load instructions
+// per row, next to the 8 loads of their W2 fragments: stay inside the 6-bit outstanding-load counter
+__host__ __device__ constexpr int conv_rows_band_max(int W) { return 2 * (48 / (W / 8)) + 4; }
 
 template <typename T, int NI>
 __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs p) {
@@ -81,9 +82,33 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
   char* const mid = Xt + kCvrRing * XTROW;
   const unsigned lds0 = (unsigned)(size_t)(DITTO_LDS char*)smem_raw;
 
+  // direct global -> LDS load of input row q of the band (band-relative; image row y0 - 1 + q)
+  const i32x4 x_rsrc = make_rsrc_uniform(reinterpret_cast<const T*>(p.x) + (long long)n * p.C0 * plane,
+                                         (unsigned)(p.C0 * plane * 2));
+  auto issue_row = [&](int q) __attribute__((always_inline)) {
+    const int S8 = Wi >> 3;  // 16-byte pieces per channel row
+    const int y = y0 - 1 + q;
+    const bool ok = y >= 0 && y < H;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int job = 64 * i + lane, c = job / S8, piece = job - c * S8;  // channels >= C0 are out of range
+      const unsigned vo = ok ? (unsigned)(c * (int)plane * 2 + piece * 16 + y * Wi * 2) : kOut;
+      lds_dma_16(x_rsrc, vo, lds0 + q * RAWROW + 1024 * i);
+    }
+  };
+
   if (wave >= 4) {
     // ======================= second convolution / stores =======================
     const int hh = wave - 4;  // output channels 64 hh .. 64 hh + 63
+    // Before their first store (step 1) these waves bring the input rows from the fifth on (rows 0 .. 3 are the
+    // other waves'): rows 4 and 5, turned round during step 0, by waves 4 and 5, which wait for them before the
+    // first barrier; the rest, turned round from step 1 on, by waves 6 and 7, which wait before the second.
+    if (hh < 2) {
+      if (4 + hh < nin) issue_row(4 + hh);
+    } else {
+#pragma unroll 1
+      for (int q = 4 + hh; q < nin; q += 2) issue_row(q);
+    }
     const int j = lane & 15, kg = lane >> 4;
     // A operand: lane (m, kg) holds W2[64 hh + 16 ct + m][32 ks + 8 kg .. + 7]
     V8 w2f[4][2];
@@ -110,6 +135,7 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
     const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         reinterpret_cast<T*>(p.y) + (long long)n * p.C2 * plane, 0, (int)(p.C2 * plane * 2), 0x00020000);
     for (int k = 0; k <= nsteps; ++k) {
+      if (k == (hh < 2 ? 0 : 1)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's rows (and W2 fragments)
       lds_barrier();  // the intermediate rows of step k - 1 are written
       if (k == 0 || 64 * hh >= p.C2) continue;
       const int s = k - 1;
@@ -147,24 +173,9 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
 
   // ======================= loads, transposition and first convolution =======================
   const int rho = wave & 1, c1t = wave >> 1;
-  // ---- this wave's input rows: q = wave, wave + 4, ... (all issued at once; the wave issues no other
-  // memory instruction after its prologue, so its counter waits are exact)
-  const int S8 = Wi >> 3;  // 16-byte pieces per channel row
-  {
-    const i32x4 rsrc = make_rsrc_uniform(reinterpret_cast<const T*>(p.x) + (long long)n * p.C0 * plane,
-                                         (unsigned)(p.C0 * plane * 2));
-#pragma unroll 1
-    for (int q = wave; q < nin; q += 4) {
-      const int y = y0 - 1 + q;
-      const bool ok = y >= 0 && y < H;
-#pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const int job = 64 * i + lane, c = job / S8, piece = job - c * S8;  // channels >= C0 are out of range
-        const unsigned vo = ok ? (unsigned)(c * (int)plane * 2 + piece * 16 + y * Wi * 2) : kOut;
-        lds_dma_16(rsrc, vo, lds0 + q * RAWROW + 1024 * i);
-      }
-    }
-  }
+  // ---- this wave's input row of the first step: q = wave (the later rows come through waves 4 .. 7); the wave
+  // issues no other memory instruction after its prologue
+  if (wave < nin) issue_row(wave);
   // the zero pixels left and right of every ring row
   if (wave == 0)
     for (int i = lane; i < kCvrRing * 2 * 8; i += 64) {
@@ -179,7 +190,7 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
 #pragma unroll
     for (int st = 0; st < NSTEP; ++st) w1f[st] = *reinterpret_cast<const V8*>(w + st * 2048);
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // W1 fragments and this wave's rows: from here on LDS only
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NSTEP) : "memory");  // the row (issued ahead of the W1 fragments) has landed
   // raw row q -> ring slot q % 6: unit (pixel tile t of 32, 16 channels kk): the lane receives channels
   // 16 kk + 8 g .. + 7 of pixel 32 t + ln (two transposing reads) and writes them as one 16-byte chunk
   const int i16 = lane & 15, h = (lane >> 4) & 1;
@@ -227,7 +238,8 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
   }
   for (int k = 0; k <= nsteps; ++k) {
     lds_barrier();  // the transposed rows of step k are there; the buffer of step k - 2 has been read
-    // rows 2k + 4, 2k + 5 for the next step (their ring slots were last read in step k - 1): the wave that loaded them
+    // rows 2k + 4, 2k + 5 for the next step (their ring slots were last read in step k - 1; they landed before
+    // barrier k: rows 4, 5 before the first one, the rest before the second)
     {
       const int q = 2 * k + 4 + (wave & 1);
       if ((q & 3) == wave && q < nin) transpose_row(q);

@@ -181,7 +181,7 @@ __global__ __launch_bounds__(64 * kDwRowsWaves) void dw_rows_kernel(DwRowsArgs p
         for (int t = 0; t < 8; ++t) v[t] = p.relu_out ? fmaxf(o[t][i], 0.f) : o[t][i];
         const V2 q0 = cvt2<T>(v[0], v[1]), q1 = cvt2<T>(v[2], v[3]), q2 = cvt2<T>(v[4], v[5]), q3 = cvt2<T>(v[6], v[7]);
         const V8 px8 = {q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, px8), y_rsrc, y_vo[i], soff, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, px8), y_rsrc, y_vo[i], soff, kStoreWriteThrough);
       }
     }
     return;
