@@ -68,3 +68,32 @@ def test_depthwise_kernels_with_wide_stores_use_no_scratch_and_no_flat_accesses(
     assert len(wide) >= 24  # 4 output widths x (3x3 | other filters | four vector-ALU multipliers)
     for name, v in wide.items():
         assert v["vgpr_spill_count"] == 0 and v["private_segment_fixed_size"] == 0, (name, v)
+
+
+@pytest.mark.parametrize("unit_name", ["conv_rows_f16", "dw_rows_f16"])
+def test_row_kernels_use_no_scratch_and_wait_for_lds_before_every_barrier(tmp_path, unit_name):
+    """The row kernels hand data between waves through LDS and count their outstanding loads by hand:
+
+    * no scratch: a spill reload is a memory instruction the counted ``s_waitcnt vmcnt`` of the loading waves does
+      not know of, and in the storing waves it would wait for every output store in flight;
+    * every ``s_barrier`` directly behind ``s_waitcnt lgkmcnt(0)``: the compiler's own wait in front of a barrier
+      was missing behind LDS writes under divergent control flow (a cold first launch then read three pixel slots
+      before the write had landed), so the kernels spell the pair out."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not available")
+    unit = [u for u in build_ext.UNITS if u[0] == unit_name][0]
+    out = tmp_path / "rows.s"
+    flags = [f for f in build_ext.HIPCC_FLAGS if f != "-fPIC"]
+    cmd = [hipcc, *flags, "--cuda-device-only", "-S", *unit[2], os.path.join(CSRC, unit[1]), "-o", str(out)]
+    subprocess.run(cmd, check=True, capture_output=True)
+    text = out.read_text()
+    md = {k: v for k, v in kernel_metadata(text).items() if "rows_kernel" in k}
+    assert len(md) == 8  # one instantiation per row width class
+    for name, v in md.items():
+        assert v["vgpr_spill_count"] == 0 and v["private_segment_fixed_size"] == 0, (name, v)
+    lines = [l.strip() for l in text.split("\n") if l.strip() and not l.strip().startswith((";", "."))]
+    barriers = [i for i, l in enumerate(lines) if l.startswith("s_barrier")]
+    assert len(barriers) >= 8 * 3
+    for i in barriers:
+        assert lines[i - 1].startswith("s_waitcnt lgkmcnt(0)"), lines[i - 3:i + 1]
