@@ -173,6 +173,13 @@ constexpr int kStoreWriteThrough = 17;
 // missing behind LDS writes under divergent control flow at a loop's end (the next wave then read a slot
 // before the write had landed).
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// __syncthreads() behind an explicit wait for this wave's own LDS accesses, for the same reason: the generated
+// code of the tile kernels had barriers that a wave with all lanes masked off in the store blocks could reach with
+// its turn-around writes still in flight.
+__device__ __forceinline__ void wg_sync() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+}
 
 // Workgroups are dealt round-robin to the 8 XCDs (each with a private L2) by
 // linear id.  Remap so that ids that are neighbours in the logical order (and

@@ -248,7 +248,7 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
   if (x_prefetch) xv_load(0, t_chg, t_gi, t_ri, tid < xtasks);
 
   for (int c0 = 0, chunk = 0; c0 < p.C0; c0 += CH, ++chunk) {
-    __syncthreads();  // everyone is done reading the previous chunk
+    wg_sync();  // everyone is done reading the previous chunk
     if (p.w1p) {
       // the W1 chunk streams into LDS while the halo tile is staged through registers below
       for (int j = wave; j * 1024 < w1_bytes; j += 4) {
@@ -309,7 +309,7 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
       }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    wg_sync();
     if (x_prefetch && c0 + CH < p.C0) xv_load(c0 + CH, t_chg, t_gi, t_ri, tid < xtasks);  // in flight during the MFMAs
     if (PX2 == 0 && w2_prefetch && c0 + CH >= p.C0) {
 #pragma unroll
@@ -358,7 +358,7 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
                    w2_lds + (stage & 1) * w2_buf + j * 1024);
       }
     };
-    __syncthreads();  // the first convolution's LDS is no longer read
+    wg_sync();  // the first convolution's LDS is no longer read
     w2_issue(0);
     // intermediate -> LDS: inter op, cast, zero outside the first convolution's output (that is the
     // second one's padding); 4 consecutive channels per register quad
@@ -401,7 +401,7 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
         const int r = stage % p.R2, sc = stage / p.R2;
         const int c2b = sc / nch2, ch = sc % nch2;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();  // this stage's rows have landed; everyone is done with the previous ones
+        wg_sync();  // this stage's rows have landed; everyone is done with the previous ones
         if (stage + 1 < nstage) w2_issue(stage + 1);
         if (ch == 0 && r == 0) {
 #pragma unroll
@@ -515,14 +515,14 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
       }
 
   for (int cb = 0; cb < p.C2; cb += c2blk) {
-    __syncthreads();  // the LDS region is free (first convolution / previous block done)
+    wg_sync();  // the LDS region is free (first convolution / previous block done)
     if (w2_prefetch && cb == 0) {
 #pragma unroll
       for (int k = 0; k < 8; ++k) w2_store(tid + 256 * k, xr[k]);
     } else {
       for (int e = tid; e < c2blk * VPR; e += 256) w2_store(e, w2_load(cb, e));
     }
-    __syncthreads();
+    wg_sync();
     for (int ct = 0; ct * 32 < c2blk && cb + ct * 32 < p.C2; ++ct) {
       const T* wr = W2s + (32 * ct + ln) * W2S + 4 * g;  // A operand row of this lane
       f32x16 o[PXW];

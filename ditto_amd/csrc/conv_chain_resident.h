@@ -188,7 +188,7 @@ __global__ __launch_bounds__(512) void conv_chain_resident_kernel(ConvResidentAr
 
   // loads return in order: the X rows (and W1) are there once only the W2 loads, issued last, are outstanding
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kW2Loads) : "memory");
-  __syncthreads();
+  wg_sync();
   bool w2_pending = true;
 
   for (; tile < p.ntiles; tile += gridDim.x) {
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(512) void conv_chain_resident_kernel(ConvResidentAr
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       w2_pending = false;
     }
-    __syncthreads();  // intermediate tile complete; raw X buffer free
+    wg_sync();  // intermediate tile complete; raw X buffer free
     if (tile + (int)gridDim.x < p.ntiles) load_x(tile + gridDim.x);
 
     // ---- second convolution: 32 output pixels x 64 channels per wave

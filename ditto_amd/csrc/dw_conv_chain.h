@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void dw_conv_chain_kernel(DwConvArgs p) {
   const long long hw = (long long)p.H * p.W;
   for (int c0 = 0; c0 < p.C0; c0 += p.chx) {
     const int cm_base = c0 * p.mult;  // first intermediate channel of the chunk
-    __syncthreads();
+    wg_sync();
     // ---- halo tile, natural layout: a wave owns (channel, row) pairs, lanes run along w
     stage_halo<T>(Xs, Xg, p, c0, h0, w0, tid);
     // ---- depthwise filters of the chunk: [cm][16], taps >= R*S zero
@@ -172,7 +172,7 @@ __global__ __launch_bounds__(256) void dw_conv_chain_kernel(DwConvArgs p) {
       }
       *reinterpret_cast<V8*>(W2s + c2 * W2S + 8 * v8) = v;
     }
-    __syncthreads();
+    wg_sync();
 
     for (int ks = 0; ks * 16 < CM; ++ks) {
       const int cm0 = 16 * ks + 8 * g;  // chunk-relative first intermediate channel of this lane
@@ -501,7 +501,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
     for (int chunk = 0; chunk < nchunks; ++chunk) {
       const int c0 = chunk * p.chx;
       const int cm_base = c0 * p.mult;
-      __syncthreads();  // every wave is done with the previous halo tiles (and filters, if restaged)
+      wg_sync();  // every wave is done with the previous halo tiles (and filters, if restaged)
       xstore();
       if (!weights_staged || nchunks > 1) {
         weights_staged = true;
@@ -515,7 +515,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
             *reinterpret_cast<V8*>(W2s + 8 * e) = v;
           }
         }
-        __syncthreads();
+        wg_sync();
         // ... and are regrouped into A-operand entries: row m = 16 * hgrp + 8a + 4gg + b of a block is
         // its intermediate channel 16 * hgrp + 8gg + 4a + b (DWV: two entries per intermediate channel)
         for (int e = tid; e < nblk * 64; e += NT) {
@@ -534,7 +534,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
                          raw[6] | (raw[7] << 16)};
         }
         if (tid == 0) W1h[zero_entry] = uint4{0, 0, 0, 0};
-        __syncthreads();
+        wg_sync();
         const int nv = CM / 8;  // 16-byte vectors per row of the W2 chunk (C1 is a multiple of 16 here)
         const float inv_nv = 1.0f / (float)nv;
         for (int e0 = tid; e0 < C2p * nv; e0 += 4 * NT) {
@@ -555,7 +555,7 @@ __global__ __launch_bounds__(256 * NG) void dw_conv_mfma_kernel(DwConvArgs p) {
             if (dst[u] >= 0) *reinterpret_cast<V8*>(W2s + dst[u]) = v[u];
         }
       }
-      __syncthreads();
+      wg_sync();
       // the next (tile, chunk) travels while this one is computed
       if (chunk + 1 < nchunks) xload(tile, c0 + p.chx);
       else if (tile_next >= 0) xload(tile_next, 0);

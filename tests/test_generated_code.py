@@ -1,4 +1,5 @@
-"""Compiler-output checks for the depthwise chain (no GPU).
+"""Compiler-output checks (no GPU): the depthwise chain's register and address-space properties, and for every
+kernel that no workgroup barrier is reached with the wave's own LDS accesses still in flight.
 
 Two properties of the generated code decide the speed of the persistent depthwise kernel and are
 invisible in its results:
@@ -36,6 +37,106 @@ def kernel_metadata(asm_text):
     return out
 
 
+def barriers_with_lds_in_flight(asm_text):
+    """[(kernel, instruction index)] of every ``s_barrier`` that some path through the kernel reaches while an LDS
+    access of the same wave may still be outstanding.  A forward may-analysis over the kernel's control-flow graph:
+    the state is the sequence of LDS (and scalar-load) instructions issued since the counter last read zero,
+    ``s_waitcnt lgkmcnt(N)`` keeps the newest N of them, joins take the longer sequence."""
+    import collections
+    found = []
+    cur, body = None, []
+    kernels = []
+    for line in asm_text.split("\n"):
+        m = re.match(r"^(_Z\w+):", line)
+        if m and "kernel" in m.group(1):
+            cur, body = m.group(1), []
+            continue
+        if cur is not None:
+            if line.startswith(".Lfunc_end"):
+                kernels.append((cur, body))
+                cur = None
+            else:
+                body.append(line)
+
+    def join(a, b):
+        if a is None:
+            return b
+        n = max(len(a), len(b))
+        a, b = (0,) * (n - len(a)) + a, (0,) * (n - len(b)) + b
+        return tuple(x | y for x, y in zip(a, b))
+
+    for name, body in kernels:
+        ins, labels = [], {}
+        for raw in body:
+            t = raw.strip()
+            if not t or t.startswith(";"):
+                continue
+            m = re.match(r"^(\.LBB\w+):", t)
+            if m:
+                labels[m.group(1)] = len(ins)
+                continue
+            if t.startswith("."):
+                continue
+            ins.append(t.split(";")[0].strip())
+        n = len(ins)
+        succ = [[] for _ in range(n)]
+        for i, t in enumerate(ins):
+            op = t.split()[0]
+            if op == "s_branch":
+                succ[i].append(labels[t.split()[1]])
+            elif op.startswith("s_cbranch"):
+                succ[i].append(labels[t.split()[1]])
+                if i + 1 < n:
+                    succ[i].append(i + 1)
+            elif op not in ("s_endpgm", "s_setpc_b64") and i + 1 < n:
+                succ[i].append(i + 1)
+        state = [None] * n
+        state[0] = ()
+        work = collections.deque([0])
+        while work:
+            i = work.popleft()
+            s, t = state[i], ins[i]
+            op = t.split()[0]
+            if op.startswith("ds_"):
+                s = (s + (1,))[-16:]
+            elif op.startswith(("s_load", "s_buffer_load")):
+                s = (s + (2,))[-16:]
+            elif op == "s_waitcnt":
+                m = re.search(r"lgkmcnt\((\d+)\)", t)
+                if m:
+                    keep = int(m.group(1))
+                    s = s[len(s) - keep:] if keep < len(s) else s
+                    if keep == 0:
+                        s = ()
+            for j in succ[i]:
+                ns = join(state[j], s)
+                if ns != state[j]:
+                    state[j] = ns
+                    work.append(j)
+        found += [(name, i) for i, t in enumerate(ins) if t.startswith("s_barrier") and state[i] and 1 in
+                  [k & 1 for k in state[i]]]
+    return found
+
+
+def test_barrier_analysis_on_a_small_kernel():
+    text = """
+_Z6kernelv:
+	ds_write_b32 v0, v1
+	s_cbranch_execz .LBB0_2
+	ds_read_b32 v2, v0
+	s_waitcnt lgkmcnt(0)
+.LBB0_2:
+	s_barrier
+	ds_write_b32 v0, v1
+	s_waitcnt lgkmcnt(0)
+	s_barrier
+	s_endpgm
+.Lfunc_end0:
+"""
+    # the first barrier is reachable over the branch with the write still in flight, the second is not
+    assert barriers_with_lds_in_flight(text) == [("_Z6kernelv", 4)]
+
+
 def test_kernel_metadata_parser():
     text = """
     .name:           _ZN5ditto1aEv
@@ -68,6 +169,10 @@ def test_depthwise_kernels_with_wide_stores_use_no_scratch_and_no_flat_accesses(
     assert len(wide) >= 24  # 4 output widths x (3x3 | other filters | four vector-ALU multipliers)
     for name, v in wide.items():
         assert v["vgpr_spill_count"] == 0 and v["private_segment_fixed_size"] == 0, (name, v)
+    # every conv kernel of the unit: no barrier that a wave can reach with its own LDS accesses in flight (the
+    # kernels wait explicitly in front of their barriers; a wave with all lanes masked off in the store blocks
+    # used to reach the tile loop's barrier with its turn-around writes outstanding)
+    assert barriers_with_lds_in_flight(text) == []
 
 
 @pytest.mark.parametrize("unit_name", ["conv_rows_f16", "dw_rows_f16"])
@@ -97,3 +202,17 @@ def test_row_kernels_use_no_scratch_and_wait_for_lds_before_every_barrier(tmp_pa
     assert len(barriers) >= 8 * 3
     for i in barriers:
         assert lines[i - 1].startswith("s_waitcnt lgkmcnt(0)"), lines[i - 3:i + 1]
+    assert barriers_with_lds_in_flight(text) == []
+
+
+@pytest.mark.parametrize("unit_name", ["gemm_chain_i8", "gemm_chain_f32", "fp_bf16_softmax", "fp_f16_cast"])
+def test_no_barrier_with_lds_accesses_in_flight(tmp_path, unit_name):
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not available")
+    unit = [u for u in build_ext.UNITS if u[0] == unit_name][0]
+    out = tmp_path / "unit.s"
+    flags = [f for f in build_ext.HIPCC_FLAGS if f != "-fPIC"]
+    cmd = [hipcc, *flags, "--cuda-device-only", "-S", *unit[2], os.path.join(CSRC, unit[1]), "-o", str(out)]
+    subprocess.run(cmd, check=True, capture_output=True)
+    assert barriers_with_lds_in_flight(out.read_text()) == []
