@@ -637,7 +637,14 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
   // output rows, one workgroup each; a band's rows are all in flight at once, which bounds its height.
   if (allow_resident && !conv_rows_off() && !persist_requested() && d->R1 == 3 && d->S1 == 3 && d->pad1 == 1 &&
       d->stride1 == 1 && d->C0 <= ditto::kCvrC && d->C1 <= ditto::kCvrC && d->C2 <= 256 && d->W % 8 == 0 && d->W <= 64 &&
-      d->out_dtype != DITTO_F32 && d->C0 * d->H * d->W * 2 < 0x7fffffffLL && d->C2 * d->H * d->W * 2 < 0x7fffffffLL) {
+      d->out_dtype != DITTO_F32 && d->C0 * d->H * d->W * 2 < 0x7fffffffLL && d->C2 * d->H * d->W * 2 < 0x7fffffffLL &&
+      // where it pays (measured against the general kernel): the pipeline pads C0 and C1 to 64, and its gain is the
+      // output stream under the compute - wide outputs - or, with few images, more workgroups than the general
+      // kernel's tiles of 256 pixels (32 x 32 x 56 x 56 -> 32 -> 128: 16.4 against 12.3 us; 64 -> 64 -> 64: a tie;
+      // one image 64 -> 64 -> 256: 8.9 against 15.6 us)
+      (d->C0 > 32 || d->C1 > 32) &&
+      (d->C2 >= 192 || d->N * ((P + (256 / d->W > 0 ? 256 / d->W : 1) - 1) / (256 / d->W > 0 ? 256 / d->W : 1)) <
+                           (need_device ? device_cus() : 256))) {
     const int cus = need_device ? device_cus() : 256;
     int band_max = ditto::conv_rows_band_max((int)d->W);
     if (band_max > d->H) band_max = (int)d->H;

@@ -138,6 +138,13 @@ def test_conv_tile_choice_without_gpu(monkeypatch):
     # fp32 output, wider rows or more channels stay on the general kernel, and so does everything with DITTO_CONV_ROWS=0
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(out_dtype=_lib.F32)), ctypes.byref(tile)) == _lib.OK
     assert tile.variant == 3022
+    # ... and narrow outputs with enough images to fill the CUs with the general kernel's tiles (measured slower there)
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C2=128)), ctypes.byref(tile)) == _lib.OK
+    assert tile.variant == 3022
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C2=128, N=8)), ctypes.byref(tile)) == _lib.OK
+    assert tile.variant // 100 == 37
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C0=32, C1=32)), ctypes.byref(tile)) == _lib.OK
+    assert tile.variant // 100 == 30
     monkeypatch.setenv("DITTO_CONV_ROWS", "0")
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc()), ctypes.byref(tile)) == _lib.OK
     assert tile.variant == 3022 and tile.grid_x == 32 * 14 and tile.lds_bytes <= 80 * 1024  # two workgroups per CU

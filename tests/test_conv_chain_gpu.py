@@ -44,7 +44,10 @@ def rows_pipeline_shape(case):
     """3x3 (pad 1, stride 1) -> 1x1, at most 64 -> 64 -> 256 channels, rows of whole 16-byte vectors up to 64 pixels:
     with a 16-bit output and a workspace these run on the row pipeline."""
     N, C0, H, W, C1, R, pad, stride, C2 = case
-    return R == 3 and pad == 1 and stride == 1 and C0 <= 64 and C1 <= 64 and C2 <= 256 and W % 8 == 0 and W <= 64
+    fits = R == 3 and pad == 1 and stride == 1 and C0 <= 64 and C1 <= 64 and C2 <= 256 and W % 8 == 0 and W <= 64
+    # ... and where it pays: more than 32 channels somewhere before the output, and a wide output or few images
+    rows_per_tile = max(1, 256 // W)
+    return fits and max(C0, C1) > 32 and (C2 >= 192 or N * -(-H // rows_per_tile) < 256)
 
 
 @pytest.mark.parametrize("case", CASES)
@@ -74,9 +77,9 @@ CASES_ROWS_PIPELINE = [
     (2, 64, 56, 56, 64, 256),   # the workload's shape, 2 images: bands of 7 rows (3 steps of two rows and one of one)
     (1, 64, 9, 64, 64, 256),    # the widest row (two full pixel tiles, 16 strips per step); bands of 5
     (3, 24, 11, 8, 40, 72),     # one strip per row, channel counts that fill no tile, a short last band
-    (1, 16, 1, 16, 8, 16),      # a single output row
-    (2, 48, 30, 40, 32, 136),   # the second store wave takes 8 of its 128 channels
-    (40, 8, 12, 24, 16, 32),    # more workgroups than CUs
+    (1, 16, 1, 16, 40, 16),     # a single output row
+    (2, 48, 30, 40, 32, 136),   # the third store wave takes 8 of its 64 channels, the fourth none
+    (40, 8, 12, 24, 48, 32),    # many images of few rows
 ]
 
 
