@@ -163,9 +163,10 @@ __device__ __forceinline__ i32x4 make_rsrc_uniform(const void* base, unsigned by
 
 // Cache policy for streamed output stores (buffer-store aux bits sc0 | sc1): write-through.  Left dirty in L2 a
 // large output is written back in a burst after the last wave has finished; written through it streams to memory
-// while the kernel still computes.  Worth 15 % on the depthwise row kernel (17.0 -> 14.4 us per call); on the
-// conv3x3 -> conv1x1 row pipeline it shortened graph replays (21 -> 19.6 us) but lengthened back-to-back eager
-// launches (22.9 -> 26.5 us), so that kernel keeps the default policy; the non-temporal hint was slower on both.
+// while the kernel still computes.  Worth 15 % on the depthwise row kernel (17.0 -> 14.4 us per call) and 11 % on
+// the conv3x3 -> conv1x1 row pipeline (21.7 -> 19.2 us) once that kernel's store windows ended on whole 128-byte
+// lines - with half-written lines the two halves went out separately and back-to-back launches got slower
+// (22.9 -> 26.5 us); the non-temporal hint was slower on both.
 constexpr int kStoreWriteThrough = 17;
 
 // Workgroup barrier for waves that hand data to each other through LDS: waits for this wave's own LDS

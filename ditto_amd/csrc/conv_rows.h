@@ -21,12 +21,13 @@
 //    channels): mid^T[c1][pixel] = W1 . X as 36 x 2 MFMAs 32x32x16 with the wave's 36 W1 fragments
 //    RESIDENT IN REGISTERS (loaded once from the repacked copy in the workspace) and the pixel
 //    fragments read from Xt at the tap's offset; the cast result goes to LDS as mid[pixel][64]
-//    (double buffered).
+//    (three buffers).
 //  * Second convolution of the previous step on waves 4..7 (64 output channels each, W2 fragments in
 //    registers, one wave per SIMD next to a first-convolution wave): out^T[c2][pixel] = W2 . mid as
-//    16x16x32 MFMAs whose column j of tile t is pixel 8 j + t of the step, so a lane ends with 8
-//    consecutive pixels of each of its 4 channels and the 16 lanes of a column group store whole runs
-//    of a channel row with one 16-byte store each.
+//    16x16x32 MFMAs whose column j of tile t is pixel 8 j + t of a window of the band's pixels, so a lane
+//    ends with 8 consecutive pixels of each of its 4 channels and the 16 lanes of a column group store
+//    256 contiguous bytes of a channel plane with one 16-byte store each; the windows end on whole
+//    128-byte lines.
 //  One barrier per step; the only waves that wait for memory after the prologue are waves 4..7, in the
 //  store queue.
 #pragma once
@@ -49,9 +50,9 @@ constexpr int kCvrWaves = 8;   // four load / first-convolution waves, four seco
 constexpr int kCvrRing = 6;    // rows of the transposed ring
 constexpr int kCvrW1Bytes = 9 * kCvrC * kCvrC * 2;
 
-// LDS: band + 2 raw rows of 128 W bytes, the ring of transposed rows, two intermediate steps of 2 W pixels
+// LDS: band + 2 raw rows of 128 W bytes, the ring of transposed rows, three intermediate steps of 2 W pixels
 __host__ __device__ constexpr int conv_rows_lds_bytes(int W, int band) {
-  return (band + 2) * 128 * W + kCvrRing * (W + 2) * 128 + 2 * (2 * W) * 128;
+  return (band + 2) * 128 * W + kCvrRing * (W + 2) * 128 + 3 * (2 * W) * 128;
 }
 // waves 6 and 7 keep half each of the band's rows from the seventh on in flight at once, W / 8 load instructions
 // per row, next to the 8 loads of their W2 fragments: stay inside the 6-bit outstanding-load counter
@@ -124,49 +125,63 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
           w2f[ct][ks] = v;
         }
     }
-    // B operand of tile t: lane (j, kg) reads channels 32 ks + 8 kg .. + 7 of pixel 8 j + t of the step
-    // (slot SJ t + j, chunk index XORed with (j >> 1) & 7)
-    const int jc = j < SJ ? j : 0;
-    const int b_rd = jc * 128, b_x = (jc >> 1) & 7;
-    // the lane's 8 output pixels 8 j .. 8 j + 7 of the step: row 8 j / W of the two, column 8 j % W
-    const int S8 = Wi >> 3;
-    const int prow = j / S8, pcol = 8 * (j - prow * S8);
-    const unsigned y_lane = (unsigned)((64 * hh + 4 * kg) * (int)plane * 2 + (prow * Wi + pcol) * 2);
+    // The band's output pixels, row after row, are one contiguous run of every channel plane.  After step s the
+    // wave stores the pixels up to the last whole 128-byte line of what is computed (the rest waits for the next
+    // step; with rows of 112 bytes every other line would else be written in two halves, 3 us apart, and go out to
+    // memory twice), in windows of 128 pixels: MFMA column j of tile t is pixel w0 + 8 j + t of the band, so a
+    // lane ends with 8 consecutive pixels of each of its 4 channels and 16 lanes write 256 contiguous bytes.
+    // The pixel lives in the intermediate buffer of its own step (slot SJ t + jj, chunk XORed with (jj >> 1) & 7),
+    // this step's or the one before: three buffers.
+    const int WB = 2 * Wi;                       // pixels of a step
+    const int align = WB >= 64 ? 64 : 8;         // window ends on whole lines where a step spans one
+    const int A0 = y0 * Wi;                      // the band's first pixel inside a channel plane
     const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         reinterpret_cast<T*>(p.y) + (long long)n * p.C2 * plane, 0, (int)(p.C2 * plane * 2), 0x00020000);
+    int ws = 0;  // first pixel of the band not stored yet
     for (int k = 0; k <= nsteps; ++k) {
       if (k == (hh < 2 ? 0 : 1)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's rows (and W2 fragments)
       lds_barrier();  // the intermediate rows of step k - 1 are written
       if (k == 0 || 64 * hh >= p.C2) continue;
       const int s = k - 1;
-      const char* const mr = mid + (s & 1) * MIDBUF + b_rd;
-      V8 bf[2][8];
+      const int ce = (2 * (s + 1) < nout ? 2 * (s + 1) : nout) * Wi;  // pixels computed so far
+      const int we = k == nsteps ? ce : ((A0 + ce) / align) * align - A0;
+      for (int w0 = ws; w0 < we; w0 += 128) {
+        const int q = w0 + 8 * j;                  // the lane's 8 pixels q .. q + 7
+        const bool on = q < we;
+        const int qc = on ? q : w0;
+        const int sq = qc >= s * WB ? s : s - 1;   // the step that computed them
+        const int jj = (qc - sq * WB) >> 3;
+        const char* const mr = mid + (sq % 3) * MIDBUF + jj * 128;
+        const int b_x = (jj >> 1) & 7;
+        V8 bf[2][8];
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks)
+        for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-        for (int t = 0; t < 8; ++t) bf[ks][t] = *reinterpret_cast<const V8*>(mr + SJ * t * 128 + (((4 * ks + kg) ^ b_x) << 4));
-      const bool row_ok = j < SJ && 2 * s + prow < nout;
+          for (int t = 0; t < 8; ++t) bf[ks][t] = *reinterpret_cast<const V8*>(mr + SJ * t * 128 + (((4 * ks + kg) ^ b_x) << 4));
+        const unsigned y_lane = (unsigned)((64 * hh + 4 * kg) * (int)plane * 2 + (A0 + qc) * 2);
 #pragma unroll
-      for (int ct = 0; ct < 4; ++ct) {
-        if (64 * hh + 16 * ct >= p.C2) break;  // wave-uniform
-        f32x4 o[8];
-        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+        for (int ct = 0; ct < 4; ++ct) {
+          if (64 * hh + 16 * ct >= p.C2) break;  // wave-uniform
+          f32x4 o[8];
+          const f32x4 z = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int t = 0; t < 8; ++t) o[t] = Elem<T>::mfma16(w2f[ct][0], bf[0][t], z);
+          for (int t = 0; t < 8; ++t) o[t] = Elem<T>::mfma16(w2f[ct][0], bf[0][t], z);
 #pragma unroll
-        for (int t = 0; t < 8; ++t) o[t] = Elem<T>::mfma16(w2f[ct][1], bf[1][t], o[t]);
+          for (int t = 0; t < 8; ++t) o[t] = Elem<T>::mfma16(w2f[ct][1], bf[1][t], o[t]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const V2 q0 = cvt2<T>(o[0][i], o[1][i]), q1 = cvt2<T>(o[2][i], o[3][i]);
-          const V2 q2 = cvt2<T>(o[4][i], o[5][i]), q3 = cvt2<T>(o[6][i], o[7][i]);
-          V8 px8 = {q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
-          if (p.relu_out) px8 = relu_packed(px8);
-          const int c2 = 64 * hh + 16 * ct + 4 * kg + i;
-          const unsigned vo = (row_ok && c2 < p.C2) ? y_lane : kOut;
-          const unsigned soff = (unsigned)((y0 + 2 * s) * Wi * 2 + (16 * ct + i) * (int)plane * 2);
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, px8), y_rsrc, vo, soff, 0);
+          for (int i = 0; i < 4; ++i) {
+            const V2 q0 = cvt2<T>(o[0][i], o[1][i]), q1 = cvt2<T>(o[2][i], o[3][i]);
+            const V2 q2 = cvt2<T>(o[4][i], o[5][i]), q3 = cvt2<T>(o[6][i], o[7][i]);
+            V8 px8 = {q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
+            if (p.relu_out) px8 = relu_packed(px8);
+            const int c2 = 64 * hh + 16 * ct + 4 * kg + i;
+            const unsigned vo = (on && c2 < p.C2) ? y_lane : kOut;
+            const unsigned soff = (unsigned)((16 * ct + i) * (int)plane * 2);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, px8), y_rsrc, vo, soff, kStoreWriteThrough);
+          }
         }
       }
+      if (we > ws) ws = we;
     }
     return;
   }
@@ -273,7 +288,7 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
       __builtin_amdgcn_sched_barrier(0);
     }
     // acc[pt][4 i + e] = mid[c1 = 32 c1t + 8 i + 4 g + e][pixel]: 8 bytes into chunk 4 c1t + i of the pixel
-    char* const mw = mid + (k & 1) * MIDBUF;  // (both buffers start on multiples of 128 bytes)
+    char* const mw = mid + (k % 3) * MIDBUF;  // (the buffers start on multiples of 128 bytes)
 #pragma unroll
     for (int pt = 0; pt < 2; ++pt) {
       if (!px_ok[pt]) continue;
