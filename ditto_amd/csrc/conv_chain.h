@@ -173,6 +173,7 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
   // ---- set-up of the second convolution (1x1).  W2 is staged through the LDS the first
   // convolution has finished with, as many rows (output channels) at a time as fit, rows zero-padded to C1p.
   const long long plane = (long long)p.P * p.Q;
+  const bool y_small = (long long)p.C2 * plane * 2 < 0x7fffffffLL;  // an image's output within a 32-bit buffer offset
   T* const W2s = reinterpret_cast<T*>(smem_raw);
   const int lds_elems = conv_chain_lds_bytes(p.rows_in, p.cols_in, RS, C1p, CH) / 2;
   // Output path.  A lane holds ONE pixel per register, so storing from registers means 2-byte
@@ -566,8 +567,18 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
           const int c2 = cb + 32 * ct + ch;
           const int slot = SLW * wave + 8 * sv;
           const V8 px = *reinterpret_cast<const V8*>(Os + ch * OSS + 8 * sv);
-          if (c2 < p.C2 && slot < nvalid)
-            __builtin_nontemporal_store(px, reinterpret_cast<V8*>(reinterpret_cast<T*>(p.y) + ((long long)n * p.C2 + c2) * plane + p0 * p.Q + slot));
+          if (c2 < p.C2 && slot < nvalid) {
+            // write-through (the output streams to memory while the kernel computes: 25.1 -> 23.4 us on the
+            // 32 x 64 x 56 x 56 -> 64 -> 256 shape); images past the 32-bit buffer offset keep the streaming store
+            if (y_small) {
+              const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(
+                  reinterpret_cast<T*>(p.y) + (long long)n * p.C2 * plane, 0, 0x7fffffff, 0x00020000);
+              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, px), yr,
+                                                     (unsigned)(((long long)c2 * plane + p0 * p.Q + slot) * 2), 0, kStoreWriteThrough);
+            } else {
+              __builtin_nontemporal_store(px, reinterpret_cast<V8*>(reinterpret_cast<T*>(p.y) + ((long long)n * p.C2 + c2) * plane + p0 * p.Q + slot));
+            }
+          }
         }
       } else {
 #pragma unroll
