@@ -432,19 +432,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     if (it + 3 < ntiles) tile_step(it + 3, IntC<3>{});
   }
 
-  // ---- epilogue: normalise (softmax), cast, store 4 contiguous columns per lane
+  // ---- epilogue: normalise (softmax), cast, store: by rows through LDS (free by now) where the output allows
+  // (store_tile_rows), else 4 contiguous columns per lane from registers
+  const bool by_rows = !p.out_f32 && (N & 7) == 0 && (p.f_rs & 7) == 0 && (p.f_bs & 7) == 0 && (p.f_bs2 & 7) == 0 &&
+                       (reinterpret_cast<size_t>(p.f) & 15) == 0;  // wave-uniform
+  static_assert(4 * (32 * QT) * tile_row_bytes<D>() <= bmm_chain_lds_bytes<D>(), "the parked rows need the staged tiles' LDS");
+  if (by_rows) wg_sync();  // every wave is done with the staged tiles
+  char* const tw = smem_raw + wave * (32 * QT) * tile_row_bytes<D>();
 #pragma unroll
   for (int j = 0; j < QT; ++j) {
     float inv = 1.f;
     if constexpr (INTER == kInterSoftmax) inv = 1.f / pair_sum(lsum[j]);
     const int row = m_wave + 32 * j + ln;
-    if (row >= M) continue;
+    if (!by_rows && row >= M) continue;
 #pragma unroll
     for (int t = 0; t < D / 32; ++t)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         const int n = 32 * t + 8 * q4 + 4 * g;
-        if (n >= N) continue;
+        if (!by_rows && n >= N) continue;
         float v0 = o[t][j][4 * q4 + 0] * inv, v1 = o[t][j][4 * q4 + 1] * inv;
         float v2 = o[t][j][4 * q4 + 2] * inv, v3 = o[t][j][4 * q4 + 3] * inv;
         if (INTER != kInterSoftmax && p.relu_out) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); v2 = fmaxf(v2, 0.f); v3 = fmaxf(v3, 0.f); }
@@ -455,10 +461,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         } else {
           V2 a0 = cvt2<T>(v0, v1), a1 = cvt2<T>(v2, v3);
           V4 w = {a0[0], a0[1], a1[0], a1[1]};
-          *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.f) + off) = w;
+          if (by_rows) *reinterpret_cast<V4*>(tw + (32 * j + ln) * tile_row_bytes<D>() + n * 2) = w;
+          else *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.f) + off) = w;
         }
       }
   }
+  if (by_rows)
+    store_tile_rows<T, D, 32 * QT>(tw, reinterpret_cast<T*>(p.f) + zo * p.f_bs2 + zi * p.f_bs + (long long)m_wave * p.f_rs,
+                                   p.f_rs, M - m_wave, N, lane);
 #else
   (void)p;
 #endif

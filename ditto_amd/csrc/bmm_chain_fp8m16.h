@@ -466,17 +466,24 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
     if (it + 3 < ntiles) tile_step(it + 3, IntC<3>{});
   }
 
-  // ---- epilogue: normalise (softmax), cast, store 4 contiguous columns per lane
+  // ---- epilogue: normalise (softmax), cast, store: by rows through LDS (free by now) where the output allows
+  // (store_tile_rows), else 4 contiguous columns per lane from registers
+  const bool by_rows = !p.out_f32 && (N & 7) == 0 && (p.f_rs & 7) == 0 && (p.f_bs & 7) == 0 && (p.f_bs2 & 7) == 0 &&
+                       (reinterpret_cast<size_t>(p.f) & 15) == 0;  // wave-uniform
+  constexpr int kRowBytes = tile_row_bytes<D>();
+  static_assert(8 * (32) * tile_row_bytes<D>() <= bmm_chain8m16_lds_bytes<D>(), "the parked rows need the staged tiles' LDS");
+  if (by_rows) wg_sync();  // every wave is done with the staged tiles
+  char* const tw = smem_raw + wave * 32 * kRowBytes;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     float inv = 1.f;
     if constexpr (INTER == kInterSoftmax) inv = 1.f / quad_sum(lsum[j]);
     const int row = m_wave + 16 * j + c16;
-    if (row >= M) continue;
+    if (!by_rows && row >= M) continue;
 #pragma unroll
     for (int t = 0; t < NTN; ++t) {
       const int n = 16 * t + 4 * q;
-      if (n >= N) continue;
+      if (!by_rows && n >= N) continue;
       float v0 = o[2 * t + j][0] * inv, v1 = o[2 * t + j][1] * inv, v2 = o[2 * t + j][2] * inv, v3 = o[2 * t + j][3] * inv;
       if (INTER != kInterSoftmax && p.relu_out) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); v2 = fmaxf(v2, 0.f); v3 = fmaxf(v3, 0.f); }
       const long long off = zo * p.f_bs2 + zi * p.f_bs + (long long)row * p.f_rs + n;
@@ -486,10 +493,14 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
       } else {
         V2 a0 = cvt2<T>(v0, v1), a1 = cvt2<T>(v2, v3);
         V4 w = {a0[0], a0[1], a1[0], a1[1]};
-        *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.f) + off) = w;
+        if (by_rows) *reinterpret_cast<V4*>(tw + (16 * j + c16) * kRowBytes + n * 2) = w;
+        else *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.f) + off) = w;
       }
     }
   }
+  if (by_rows)
+    store_tile_rows<T, D, 32>(tw, reinterpret_cast<T*>(p.f) + zo * p.f_bs2 + zi * p.f_bs + (long long)m_wave * p.f_rs, p.f_rs,
+                              M - m_wave, N, lane);
 #else
   (void)p;
 #endif

@@ -182,6 +182,28 @@ __device__ __forceinline__ void wg_sync() {
   __syncthreads();
 }
 
+// Output path of the BMM chain kernels.  A lane holds 4 contiguous columns of several tiles of one row and
+// neighbouring lanes hold different rows: stored from registers that is 8 bytes per 128-byte line and lane, the slowest
+// pattern of the store path (14 us of the 64 x 4096 x 128 attention launch; 16 bytes per line and lane move 2.9 TB/s
+// over the device, 64 contiguous bytes and more per group of lanes 6 - 7 TB/s).  With a 16-bit output whose rows are
+// whole 16-byte vectors a wave instead parks its ROWS x D tile in LDS, [row][2 D + 16 bytes] (the 16: the rows one
+// write instruction touches spread over the banks), and this stores it row by row, 16 bytes per lane.
+template <int D>
+__host__ __device__ constexpr int tile_row_bytes() { return 2 * D + 16; }
+
+template <typename T, int D, int ROWS>
+__device__ __forceinline__ void store_tile_rows(const char* tw, T* f0, long long f_rs, int rows_valid, int N, int lane) {
+  typedef typename Elem<T>::v8 V8;
+  constexpr int CPR = D / 8;  // 16-byte chunks per row
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the reads are this wave's own writes of other lanes
+#pragma unroll
+  for (int i = 0; i < ROWS * CPR / 64; ++i) {
+    const int v = 64 * i + lane, r = v / CPR, ch = v - r * CPR;
+    const V8 x = *reinterpret_cast<const V8*>(tw + r * tile_row_bytes<D>() + ch * 16);
+    if (r < rows_valid && 8 * ch < N) *reinterpret_cast<V8*>(f0 + (long long)r * f_rs + 8 * ch) = x;
+  }
+}
+
 // Workgroups are dealt round-robin to the 8 XCDs (each with a private L2) by
 // linear id.  Remap so that ids that are neighbours in the logical order (and
 // share operands) land on the same XCD.

@@ -420,6 +420,15 @@ def test_strided_views_and_errors():
     chain.run_bmm_chain(a, bt.transpose(1, 2), c, f, "softmax", 0.125)
     ref = torch.softmax(a.float() @ bt.float().transpose(1, 2) * 0.125, -1) @ c.float()
     assert (f.float() - ref).abs().max().item() <= MAX_ABS
+    # the output as a slice too.  Rows that all start on 16 bytes (row stride 96) leave through LDS as whole rows,
+    # others (row stride 100) are stored from registers, four columns per lane: every variant gives the same bits
+    for variant in variants(64, 64, "LK"):
+        chain.run_bmm_chain(a, bt.transpose(1, 2), c, f, "softmax", 0.125, tile_variant=variant)
+        for width in (96, 100):
+            big_f = torch.full((2, 128, width), float("nan"), device=dev, dtype=torch.float16)
+            chain.run_bmm_chain(a, bt.transpose(1, 2), c, big_f[:, :, 8:72], "softmax", 0.125, tile_variant=variant)
+            assert torch.equal(big_f[:, :, 8:72], f), (variant, width)
+            assert torch.isnan(big_f[:, :, :8]).all() and torch.isnan(big_f[:, :, 72:]).all(), (variant, width)
     with pytest.raises(ValueError):
         chain.run_bmm_chain(a[:, :, :60], bt[:, :, :60].transpose(1, 2), c, f, "softmax", 0.125)
     with pytest.raises(ValueError):

@@ -199,7 +199,7 @@ def test_row_kernels_use_no_scratch_and_wait_for_lds_before_every_barrier(tmp_pa
         assert v["vgpr_spill_count"] == 0 and v["private_segment_fixed_size"] == 0, (name, v)
     lines = [l.strip() for l in text.split("\n") if l.strip() and not l.strip().startswith((";", "."))]
     barriers = [i for i, l in enumerate(lines) if l.startswith("s_barrier")]
-    assert len(barriers) >= 8 * 3
+    assert len(barriers) >= 8 * 2  # the loop barrier of each wave role
     for i in barriers:
         assert lines[i - 1].startswith("s_waitcnt lgkmcnt(0)"), lines[i - 3:i + 1]
     assert barriers_with_lds_in_flight(text) == []
