@@ -47,6 +47,8 @@ UNITS = [
     ("conv_rows_bf16", "conv_rows_inst.hip", ["-DDITTO_INST_T=bf16", "-DDITTO_CONVROWS_NAME=launch_conv_rows_bf16"]),
     ("dw_rows_f16", "dw_rows_inst.hip", ["-DDITTO_INST_T=f16", "-DDITTO_DWROWS_NAME=launch_dw_rows_f16"]),
     ("dw_rows_bf16", "dw_rows_inst.hip", ["-DDITTO_INST_T=bf16", "-DDITTO_DWROWS_NAME=launch_dw_rows_bf16"]),
+    ("dw16_rows_f16", "dw16_rows_inst.hip", ["-DDITTO_INST_T=f16", "-DDITTO_DW16ROWS_NAME=launch_dw16_rows_f16"]),
+    ("dw16_rows_bf16", "dw16_rows_inst.hip", ["-DDITTO_INST_T=bf16", "-DDITTO_DW16ROWS_NAME=launch_dw16_rows_bf16"]),
     ("fp_f16_cast", "bmm_chain_fp_inst.hip",
      ["-DDITTO_INST_T=f16", "-DDITTO_INST_INTER=0", "-DDITTO_INST_NAME=launch_f16_cast", *FP_CHAIN_FLAGS]),
     ("fp_f16_softmax", "bmm_chain_fp_inst.hip",

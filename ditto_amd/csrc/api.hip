@@ -267,9 +267,10 @@ struct ConvPlan {
   int c2_tiles;
   int dw_mode;         // 0 | 1: plain kernel (1: multiplier a multiple of 8); 2 | 3: persistent kernel,
                        // depthwise stage on the matrix cores (2) or the vector ALU (3); 4: the row-streaming
-                       // kernel (rowargs)
+                       // kernel (rowargs); 5: the row-streaming kernel for multiplier 16 (row16args)
   ditto::DwConvArgs dwargs;
   ditto::DwRowsArgs rowargs;
+  ditto::Dw16RowsArgs row16args;
   bool resident;       // 1x1 -> 3x3 with at most 64 channels: persistent kernel, W2 resident in LDS
   int res_grid;
   ditto::ConvResidentArgs rargs;
@@ -287,8 +288,15 @@ struct ConvPlan {
 // 64 output channels, image rows of whole 16-byte vectors and at most 128 pixels, 16-bit output.
 // vec_cap: the widest halo vector (elements) the pointer of this call allows; 8 when planning without one.
 // DITTO_DW_ROWS=0 keeps such shapes on the persistent kernel (A/B runs, tests of that kernel).
+// dw_mode 5: the row-streaming kernel for multiplier 16 (dw16_rows.h): 3x3, pad 1, stride 1, an even number of at
+// most 32 input channels, at most 64 output channels, image rows of whole 16-byte vectors whose ring of row slots
+// fits beside the filters in LDS, 16-bit output.  DITTO_DW16_ROWS=0 keeps such shapes on the persistent kernel.
 bool dw_rows_off() {
   const char* v = getenv("DITTO_DW_ROWS");
+  return v && v[0] == '0';
+}
+bool dw16_rows_off() {
+  const char* v = getenv("DITTO_DW16_ROWS");
   return v && v[0] == '0';
 }
 
@@ -354,6 +362,48 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
       t.variant = 4000 + 20 + 4;
       return DITTO_OK;
     }
+  }
+  if (allow_rows && vec_cap >= 8 && !dw16_rows_off() && mult == 16 && d->R1 == 3 && d->S1 == 3 && d->pad1 == 1 &&
+      d->stride1 == 1 && d->C0 <= 32 && d->C0 % 2 == 0 && d->C2 <= 64 && d->W % 8 == 0 && d->W >= 8 &&
+      ditto::dw16_rows_ni((int)d->C0, (int)d->W) <= 8 &&
+      ditto::dw16_rows_lds_bytes((int)d->C0, (int)d->W) <= 160 * 1024 && d->out_dtype != DITTO_F32 &&
+      d->H * d->W < (1 << 20)) {
+    // Bands of whole output rows, one workgroup each, whose pixels eight waves take as one stream of 32-pixel
+    // tiles: the band height with the fewest tiles on the busiest SIMD (waves w and w + 4 share one) over the
+    // rounds of workgroups, a workgroup's start-up counted as three tiles.
+    const int cus = need_device ? device_cus() : 256;
+    long long best = -1;
+    int best_band = 1;
+    for (int nb = 1; nb <= d->H; ++nb) {
+      const int band = (int)((d->H + nb - 1) / nb);
+      if (nb > 1 && band == (int)((d->H + nb - 2) / (nb - 1))) continue;
+      const long long wgs = d->N * ((d->H + band - 1) / band);
+      const long long ntiles = (band * d->W + 31) / 32;
+      const long long busiest = ntiles / 8 + (ntiles % 8 > 0) + ntiles / 8 + (ntiles % 8 > 4);
+      const long long cost = ((wgs + cus - 1) / cus) * (busiest + 3);
+      if (best < 0 || cost <= best) { best = cost; best_band = band; }
+    }
+    ditto::Dw16RowsArgs& r = plan->row16args;
+    r.N = (int)d->N; r.C0 = (int)d->C0; r.H = (int)d->H; r.W = (int)d->W; r.C2 = (int)d->C2;
+    r.band = best_band;
+    r.bands = (int)((d->H + r.band - 1) / r.band);
+    r.ring = ditto::dw16_rows_ring(r.W);
+    r.relu_mid = d->inter_op == DITTO_INTER_RELU;
+    r.relu_out = d->relu_out != 0;
+    plan->dw_mode = 5;
+    plan->c2_tiles = 2;
+    ditto_tile_param& t = plan->tile;
+    t.block_threads = 64 * ditto::kDw16Waves;
+    t.block_m = r.band * r.W;
+    t.block_l = (int)d->C1;
+    t.block_n = 64;
+    t.head_pad = 0;
+    t.lds_bytes = ditto::dw16_rows_lds_bytes(r.C0, r.W);
+    t.grid_x = r.N * r.bands;
+    t.grid_y = r.band;
+    t.grid_z = r.W;
+    t.variant = 4000 + 20 + 5;
+    return DITTO_OK;
   }
   plan->dw_mode = dwv ? 3 : mfma ? 2 : mult % 8 == 0 ? 1 : 0;
   const int c2t = d->C2 <= 32 ? 1 : d->C2 <= 64 ? 2 : d->C2 <= 128 ? 4 : 8;
@@ -992,6 +1042,17 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
       r.y = y;
       hipStream_t st = reinterpret_cast<hipStream_t>(stream);
       hipError_t e = d->in_dtype == DITTO_F16 ? ditto::launch_dw_rows_f16(r, st) : ditto::launch_dw_rows_bf16(r, st);
+      if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
+      return DITTO_OK;
+    }
+    if (plan.dw_mode == 5) {
+      ditto::Dw16RowsArgs r = plan.row16args;
+      r.x = x;
+      r.w1 = w1;
+      r.w2 = w2;
+      r.y = y;
+      hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+      hipError_t e = d->in_dtype == DITTO_F16 ? ditto::launch_dw16_rows_f16(r, st) : ditto::launch_dw16_rows_bf16(r, st);
       if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
       return DITTO_OK;
     }

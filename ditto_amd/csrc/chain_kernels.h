@@ -8,6 +8,7 @@
 #include "conv_rows.h"
 #include "dw_conv_chain.h"
 #include "dw_rows.h"
+#include "dw16_rows.h"
 #include "gemm_chain_f32.h"
 #include "gemm_chain_i8.h"
 
@@ -47,5 +48,8 @@ hipError_t launch_dw_conv_bf16(int c2_tiles, int mode, const DwConvArgs& args, h
 // depthwise 3x3 (multiplier 1) -> 1x1, at most 32 -> 64 channels, rows of at most 128 pixels (dw_rows.h)
 hipError_t launch_dw_rows_f16(const DwRowsArgs& args, hipStream_t stream);
 hipError_t launch_dw_rows_bf16(const DwRowsArgs& args, hipStream_t stream);
+// depthwise 3x3 (multiplier 16) -> 1x1, at most 32 -> 512 -> 64 channels, rows of at most 120 pixels (dw16_rows.h)
+hipError_t launch_dw16_rows_f16(const Dw16RowsArgs& args, hipStream_t stream);
+hipError_t launch_dw16_rows_bf16(const Dw16RowsArgs& args, hipStream_t stream);
 
 }  // namespace ditto

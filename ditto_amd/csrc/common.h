@@ -91,6 +91,20 @@ __device__ __forceinline__ V relu_packed(V v) {
   return __builtin_bit_cast(V, s);
 }
 
+// The same with the switch in a register: thr = relu_packed_threshold(on) is zero (ReLU) or the most negative
+// 16-bit integer in every half (identity), so a run-time flag costs no select.
+__device__ __forceinline__ unsigned relu_packed_threshold(bool on) { return on ? 0u : 0x80008000u; }
+template <typename V>
+__device__ __forceinline__ V relu_packed(V v, unsigned thr) {
+  typedef __attribute__((ext_vector_type(sizeof(V) / 2))) short S;
+  typedef __attribute__((ext_vector_type(sizeof(V) / 4))) unsigned U;
+  U t;
+  for (unsigned i = 0; i < sizeof(V) / 4; ++i) t[i] = thr;
+  S s = __builtin_bit_cast(S, v);
+  s = __builtin_elementwise_max(s, __builtin_bit_cast(S, t));
+  return __builtin_bit_cast(V, s);
+}
+
 // LDS transpose read (gfx950 ds_read_b64_tr_b16).  Within each group of 16
 // lanes, lane i receives for j=0..3 the 16-bit element (i%4) of the 64-bit
 // word addressed by lane 4*j + i/4 of the same group.  If lane s of a group

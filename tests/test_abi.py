@@ -161,8 +161,14 @@ def test_conv_tile_choice_without_gpu(monkeypatch):
     # row-streaming kernel (bands of 14 rows: one workgroup per CU, nine waves) for up to 32 -> 64 channels and
     # the persistent kernel with the vector-ALU stage beyond
     dw = dict(C0=32, H=112, W=112, C2=64, groups1=32)
+    # (sixteen outputs per input channel: the row-streaming kernel for that factor, bands of 14 rows too, nine waves)
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=512, **dw)), ctypes.byref(tile)) == _lib.OK
+    assert (tile.variant, tile.grid_x, tile.grid_y, tile.block_threads) == (4025, 256, 14, 576)
+    assert tile.lds_bytes <= 160 * 1024
+    monkeypatch.setenv("DITTO_DW16_ROWS", "0")
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=512, **dw)), ctypes.byref(tile)) == _lib.OK
     assert tile.variant == 4022 and tile.grid_x == 256
+    monkeypatch.delenv("DITTO_DW16_ROWS")
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=32, **dw)), ctypes.byref(tile)) == _lib.OK
     assert (tile.variant, tile.grid_x, tile.grid_y, tile.block_threads) == (4024, 256, 14, 832)
     assert tile.lds_bytes <= 160 * 1024

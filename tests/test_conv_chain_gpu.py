@@ -354,6 +354,55 @@ def test_row_streaming_depthwise_chain(oracle, case, dtype, monkeypatch):
         assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
 
 
+CASES_DW16_ROWS = [
+    # N, C0, H, W, C2: depthwise 3x3 (factor 16, pad 1, stride 1) -> 1x1 on the row-streaming kernel for that factor
+    (2, 32, 112, 112, 64),   # the reference's MobileNet row: 49 tiles per band, rows of 15 chunks, ring of 8 rows
+    (1, 32, 56, 56, 64),     # tiles that span two image rows; ring of 16 rows
+    (3, 6, 9, 24, 40),       # few channels, output channels that do not fill their tiles, a band of every row
+    (1, 24, 5, 120, 40),     # the widest row
+    (2, 16, 33, 40, 24),     # a last band shorter than the others, a last tile that is not full
+    (1, 32, 19, 72, 64),
+    (40, 8, 16, 16, 16),     # many small images
+]
+
+
+@pytest.mark.parametrize("case", CASES_DW16_ROWS)
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_row_streaming_depthwise_chain_factor_16(oracle, case, dtype, monkeypatch):
+    """The row-streaming kernel for sixteen outputs per input channel against the oracle and against the tiled
+    kernel on the same inputs (the same MFMAs in the same order: the same bits)."""
+    N, C0, H, W, C2 = case
+    C1 = 16 * C0
+    rng = np.random.default_rng(C0 + C2 + W)
+    X = oracle.np_round_to(rng.standard_normal((N, C0, H, W)).astype(np.float32), dtype)
+    W1 = oracle.np_round_to(rng.standard_normal((C1, 1, 3, 3)).astype(np.float32) * 0.3, dtype)
+    # (W2 small enough that the sums over up to 512 intermediate channels stay below 2: one bf16 step there is
+    # 2^-7, inside the absolute bound)
+    W2 = oracle.np_round_to(rng.standard_normal((C2, C1, 1, 1)).astype(np.float32) * 0.02, dtype)
+    x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
+    for relu in (False, True):
+        y = torch.full((N, C2, H, W), float("nan"), device=x.device, dtype=x.dtype)
+        desc = chain.conv_chain_desc(x, w1, w2, y, 1, 1, 0, 1, "relu" if relu else "cast", relu, C0)
+        assert chain.select_tile(desc).variant == 4025
+        chain.run_conv_chain(x, w1, w2, y, desc=desc)
+        torch.cuda.synchronize()
+        got = y.float().cpu().numpy()
+        assert np.isfinite(got).all()
+        want = oracle.conv_chain_f32(X, W1, W2, 1, 1, 0, 1, relu_mid=relu, relu_out=relu, round_mid=dtype, groups1=C0)
+        mx, rel = errors(got, oracle.np_round_to(want, dtype))
+        if dtype == "bfloat16" and relu:
+            report("conv chain (wide second filter / depthwise) bf16 rows x16 %s" % (case,), mx, rel)
+        assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
+        monkeypatch.setenv("DITTO_DW16_ROWS", "0")
+        y2 = torch.full_like(y, float("nan"))
+        desc2 = chain.conv_chain_desc(x, w1, w2, y2, 1, 1, 0, 1, "relu" if relu else "cast", relu, C0)
+        assert chain.select_tile(desc2).variant % 10 == 2
+        chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
+        torch.cuda.synchronize()
+        monkeypatch.delenv("DITTO_DW16_ROWS")
+        assert torch.equal(y, y2), (relu, errors(got, y2.float().cpu().numpy()))
+
+
 def test_row_streaming_kernel_steps_aside_for_less_aligned_pointers(oracle):
     """x or y not 16-byte aligned: the call runs on the persistent kernel instead (same result within tolerance)."""
     N, C0, H, W, C2 = 1, 16, 16, 24, 32
