@@ -369,8 +369,8 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
       ditto::dw16_rows_lds_bytes((int)d->C0, (int)d->W) <= 160 * 1024 && d->out_dtype != DITTO_F32 &&
       d->H * d->W < (1 << 20)) {
     // Bands of whole output rows, one workgroup each, whose pixels eight waves take as one stream of 32-pixel
-    // tiles: the band height with the fewest tiles on the busiest SIMD (waves w and w + 4 share one) over the
-    // rounds of workgroups, a workgroup's start-up counted as three tiles.
+    // tiles: the band height with the fewest tiles on the busiest SIMD (waves w and w + 4 share one) over
+    // the rounds of workgroups, a workgroup's start-up counted as three tiles.
     const int cus = need_device ? device_cus() : 256;
     long long best = -1;
     int best_band = 1;
@@ -379,7 +379,8 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
       if (nb > 1 && band == (int)((d->H + nb - 2) / (nb - 1))) continue;
       const long long wgs = d->N * ((d->H + band - 1) / band);
       const long long ntiles = (band * d->W + 31) / 32;
-      const long long busiest = ntiles / 8 + (ntiles % 8 > 0) + ntiles / 8 + (ntiles % 8 > 4);
+      const long long q = ntiles / ditto::kDw16Compute, rem = ntiles % ditto::kDw16Compute;
+      const long long busiest = 2 * q + (rem > 0) + (rem > 4);
       const long long cost = ((wgs + cus - 1) / cus) * (busiest + 3);
       if (best < 0 || cost <= best) { best = cost; best_band = band; }
     }

@@ -11,19 +11,22 @@
 //
 //  * A workgroup owns a band of output rows of one image and takes its pixels as ONE stream (an NCHW plane is
 //    contiguous, so 32 consecutive pixels of the stream are 64 contiguous bytes of every output channel,
-//    whatever rows they lie in).  Eight compute waves take the 32-pixel tiles of the stream round-robin; with
-//    14 rows of 112 pixels that is 49 tiles per workgroup and 256 workgroups, i.e. 12 or 13 tiles on every SIMD
-//    of the device (16 x 16 tiles: 7 rounds of workgroups for 6.1 rounds of work).
+//    whatever rows they lie in).  Eight compute waves take the 32-pixel tiles of the stream round-robin, a round
+//    of eight tiles between two barriers; with 14 rows of 112 pixels that is 49 tiles per workgroup and 256
+//    workgroups (16 x 16 tiles: 7 rounds of workgroups for 6.1 rounds of work).
 //  * Input rows arrive in a ring of LDS row slots, [channel][W + 8] per row (the 16-byte gap behind every
 //    channel row is written as zeros and serves as the right border of its channel and the left border of the
 //    next; rows above and below the image are out of range and arrive as zeros), brought by a loader wave that
 //    does nothing else: direct global -> LDS loads, counted exactly.  There is no halo staging through
-//    registers, no border arithmetic and one barrier per round of eight tiles; the loader refills the slots of
-//    rows that no tile of the current round reads while the round computes.
+//    registers and no border arithmetic; the loader refills the slots of rows that no tile of the current round
+//    reads while the round computes.
 //  * The filters are staged once: W2 by direct loads (one per row), the depthwise filters regrouped into
-//    operand entries straight from memory.
+//    operand entries straight from memory (taps 0..7 as 16-byte entries, the ninth as a dword: its MFMA's other
+//    operand registers are zeros that never change).
 //  * MFMA row i of a tile is pixel 16 ((i >> 2) & 1) + 4 (i >> 3) + (i & 3), so a lane ends up with 16
 //    consecutive pixels of one output channel: two 16-byte stores, no turn-around through LDS.
+//  * A block's work is laid out so that no two MFMAs of a wave stand back to back: conversions, tap shifts and
+//    LDS reads sit between them (operands double buffered), pinned there with empty asm statements.
 //
 // Non-finite inputs: as in dw_conv_mfma_kernel the zero blocks of the block-diagonal operand multiply the taps
 // of the block's other input channel, so an infinity there becomes NaN in this channel's intermediates.
@@ -43,17 +46,19 @@ struct Dw16RowsArgs {
   int relu_mid, relu_out;
 };
 
-constexpr int kDw16Waves = 9;      // eight compute waves and the loader
+constexpr int kDw16Compute = 8;    // compute waves, two per SIMD
+constexpr int kDw16Waves = kDw16Compute + 1;  // and the loader
 constexpr int kDw16W2S = 512 + 8;  // elements per W2 row in LDS
-constexpr int kDw16Round = 8 * 32; // pixels per round
+constexpr int kDw16Round = kDw16Compute * 32;  // pixels per round
 
 __host__ __device__ constexpr int dw16_rows_cpc(int W) { return W / 8 + 1; }  // 16-byte chunks per channel row
 __host__ __device__ constexpr int dw16_rows_ni(int C0, int W) { return (C0 * dw16_rows_cpc(W) + 63) / 64; }
-// rows that two consecutive rounds read: the rows 512 consecutive pixels can touch, and one above and below
+// rows that two consecutive rounds read: the rows that many consecutive pixels can touch, and one above and below
 __host__ __device__ constexpr int dw16_rows_ring(int W) { return (2 * kDw16Round + W - 2) / W + 1 + 2; }
-// LDS: 16 zero bytes, the ring, operand entries of the depthwise filters (+ 64 zero entries), W2
+// LDS: 16 zero bytes, the ring, operand entries of the depthwise filters (taps 0..7: 16 bytes, the ninth: 4 bytes;
+// 32 rows per block of two input channels and 32 zero rows), W2
 __host__ __device__ constexpr int dw16_rows_lds_bytes(int C0, int W) {
-  return 16 + dw16_rows_ring(W) * 1024 * dw16_rows_ni(C0, W) + (((C0 + 1) / 2) * 64 + 64) * 16 + 64 * kDw16W2S * 2;
+  return 16 + dw16_rows_ring(W) * 1024 * dw16_rows_ni(C0, W) + (((C0 + 1) / 2) * 32 + 32) * (16 + 4) + 64 * kDw16W2S * 2;
 }
 
 // operand slot k of a lane's nine taps: r0s0 r0s1 r1s0 r1s1 r2s0 r2s1 r0s2 r1s2 | r2s2 (one dword pair per filter
@@ -88,7 +93,7 @@ __device__ __forceinline__ void dw16_rows_wait(int k) {
 #undef DITTO_DW16_CASE
 }
 
-template <typename T, int NI>
+template <typename T, int NI, bool RELU>
 __global__ __launch_bounds__(64 * kDw16Waves) void dw16_rows_kernel(Dw16RowsArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef typename Elem<T>::v8 V8;
@@ -106,13 +111,14 @@ __global__ __launch_bounds__(64 * kDw16Waves) void dw16_rows_kernel(Dw16RowsArgs
   const int nout = H - y0 < p.band ? H - y0 : p.band;  // output rows of this band
   const int nin = nout + 2;                            // input rows y0 - 1 .. y0 + nout
   const int npx = nout * W;                            // pixels of the band's stream
-  const int ntiles = (npx + 31) >> 5, nrounds = (ntiles + 7) >> 3;
+  const int ntiles = (npx + 31) >> 5, nrounds = (ntiles + kDw16Compute - 1) / kDw16Compute;
   const long long plane = (long long)H * W;
   const unsigned lds0 = (unsigned)(size_t)(DITTO_LDS char*)smem_raw;
   char* const rows = smem_raw + 16;
   uint4* const W1h = reinterpret_cast<uint4*>(rows + ring * SLOT);
-  const int zero_entry = nblk * 64;
-  T* const W2s = reinterpret_cast<T*>(W1h + zero_entry + 64);
+  const int zero_entry = nblk * 32;
+  unsigned* const A2h = reinterpret_cast<unsigned*>(W1h + zero_entry + 32);
+  T* const W2s = reinterpret_cast<T*>(A2h + zero_entry + 32);
   const float inv_w = 1.0f / (float)W, inv_ring = 1.0f / (float)ring;
   // last input row (band relative: row k is image row y0 - 1 + k) that round rd reads
   auto last_row = [&](int rd) __attribute__((always_inline)) {
@@ -121,7 +127,7 @@ __global__ __launch_bounds__(64 * kDw16Waves) void dw16_rows_kernel(Dw16RowsArgs
     return (int)(((float)e + 0.5f) * inv_w) + 2;  // exact: the host keeps H * W below 2^20
   };
 
-  if (wave == 8) {
+  if (wave == kDw16Compute) {
     // ======================= loader wave =======================
     // instruction i of a row: lane l brings 16 bytes of job 64 i + l = channel * CPC + chunk
     const i32x4 rsrc = make_rsrc_uniform(reinterpret_cast<const T*>(p.x) + (long long)n * p.C0 * plane,
@@ -179,46 +185,49 @@ __global__ __launch_bounds__(64 * kDw16Waves) void dw16_rows_kernel(Dw16RowsArgs
     const i32x4 w2_rsrc = make_rsrc_uniform(p.w2, (unsigned)(p.C2 * p.C0 * 16 * 2));
     const unsigned row_bytes = (unsigned)(p.C0 * 16 * 2);
     const unsigned w2_lds = (unsigned)(size_t)(DITTO_LDS char*)W2s;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int c2 = 8 * wave + i;
+    for (int c2 = wave; c2 < 64; c2 += kDw16Compute) {
       const unsigned vo = (c2 < p.C2 && 16u * lane < row_bytes) ? c2 * row_bytes + 16u * lane : kOut;
       lds_dma_16(w2_rsrc, vo, w2_lds + (unsigned)(c2 * kDw16W2S * 2));
     }
     // depthwise filters as A-operand entries: row m = 16 h + 8 a + 4 gg + b of a block is its intermediate
     // channel 16 h + 8 gg + 4 a + b, so that accumulator registers 8 s .. 8 s + 7 of a lane are 8 consecutive
-    // channels; entry (blk, half, m): taps 8 half .. 8 half + 7 in gather order
+    // channels; entry (blk, m): taps 0 .. 7 in gather order, and the ninth tap in a table of its own
     const unsigned short* W1g = reinterpret_cast<const unsigned short*>(p.w1);
     const int C1 = 16 * p.C0;
-    for (int e = tid; e < nblk * 64; e += 512) {
-      const int m = e & 31, half = (e >> 5) & 1, blk = e >> 6;
+    for (int e = tid; e < nblk * 32; e += 64 * kDw16Compute) {
+      const int m = e & 31, blk = e >> 5;
       const int mm = m & 15;
       const int cml = 32 * blk + 16 * (m >> 4) + 8 * ((mm >> 2) & 1) + 4 * (mm >> 3) + (mm & 3);
-      unsigned raw[8];
+      unsigned raw[9];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int tap = dw16_tap_of_k(8 * half + i);
-        raw[i] = (tap < 9 && cml < C1) ? W1g[cml * 9 + tap] : 0u;
-      }
+      for (int i = 0; i < 9; ++i) raw[i] = cml < C1 ? W1g[cml * 9 + dw16_tap_of_k(i)] : 0u;
       W1h[e] = uint4{raw[0] | (raw[1] << 16), raw[2] | (raw[3] << 16), raw[4] | (raw[5] << 16), raw[6] | (raw[7] << 16)};
+      A2h[e] = raw[8];
     }
-    if (tid < 64) W1h[zero_entry + tid] = uint4{0, 0, 0, 0};
+    if (tid < 32) {
+      W1h[zero_entry + tid] = uint4{0, 0, 0, 0};
+      A2h[zero_entry + tid] = 0;
+    }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
-  // A-operand entries of this lane: its own half of the block diagonal (entries 64 blk + ln and + 32), zeros else
+  // A-operand entries of this lane: its own half of the block diagonal, zeros else
+  // (byte offsets from the start of LDS: 32-bit address arithmetic)
   const bool own_half = (ln >> 4) == g;
-  const int a_base = own_half ? 16 * ln : 16 * zero_entry, a_step = own_half ? 1024 : 0;
-  const unsigned relu_thr = relu_packed_threshold(p.relu_mid != 0);
+  const int w1h_off = 16 + ring * SLOT, a2h_off = w1h_off + (zero_entry + 32) * 16, w2s_off = a2h_off + (zero_entry + 32) * 4;
+  const int a1_base = w1h_off + (own_half ? 16 * ln : 16 * zero_entry);
+  const int a2_base = a2h_off + (own_half ? 4 * ln : 4 * zero_entry);
+  const int own_mask = own_half ? -1 : 0;  // block blk's entries: + 512 blk (+ 128 blk) bytes for the lanes that have any
   // pixel of this lane inside a tile (as a column of the depthwise MFMA and a row of the 1x1 MFMA)
   const int pix = 16 * ((ln >> 2) & 1) + 4 * (ln >> 3) + (ln & 3);
   const int cs2 = 2 * CS;
   const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       reinterpret_cast<T*>(p.y) + (long long)n * p.C2 * plane, 0, (int)(p.C2 * plane * 2), 0x00020000);
   const int last = nblk - 1;
+  const int w2_ln = w2s_off + ln * kDw16W2S * 2 + 16 * g;  // this lane's row and k group inside a 32-row tile of W2
 
   for (int rd = 0; rd < nrounds; ++rd) {
     lds_barrier();  // the rows this round reads have landed (round 0: the filters are staged)
-    const int tile = 8 * rd + wave;
+    const int tile = kDw16Compute * rd + wave;
     if (tile >= ntiles) continue;  // wave-uniform
     // ---- the lane's pixel: row yy of the band, column x; its taps' dword pairs in the three ring rows
     int pl = 32 * tile + pix;
@@ -238,78 +247,100 @@ __global__ __launch_bounds__(64 * kDw16Waves) void dw16_rows_kernel(Dw16RowsArgs
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
-    V8 a1n, a2n, b1n, b2n, wf[2][2], pf[2];
-    auto load_w2 = [&](int blk) __attribute__((always_inline)) {
+    V8 a1n, b1n, wf[2][2][2], pf[2][2];
+    // operands of the ninth tap's MFMA: only the first of their four registers ever changes
+    u32x4 a2u = {0u, 0u, 0u, 0u}, b2u = {0u, 0u, 0u, 0u};
+    unsigned d0[3], d1[3];
+    auto load_w2 = [&](int blk, int buf) __attribute__((always_inline)) {
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int s = 0; s < 2; ++s)
-          wf[t][s] = *reinterpret_cast<const V8*>(W2s + (32 * t + ln) * kDw16W2S + 32 * blk + 16 * s + 8 * g);
+          wf[buf][t][s] = *reinterpret_cast<const V8*>(smem_raw + (w2_ln + 64 * blk) + (32 * t * kDw16W2S * 2 + 32 * s));
     };
     auto load_a = [&](int blk) __attribute__((always_inline)) {
-      const char* a = reinterpret_cast<const char*>(W1h) + (a_base + blk * a_step);
-      a1n = *reinterpret_cast<const V8*>(a);
-      a2n = *reinterpret_cast<const V8*>(a + 512);
+      a1n = *reinterpret_cast<const V8*>(smem_raw + (a1_base + ((blk << 9) & own_mask)));
+      a2u[0] = *reinterpret_cast<const unsigned*>(smem_raw + (a2_base + ((blk << 7) & own_mask)));
+      asm volatile("" : "+v"(a2u));  // in place: the other three registers stay the zeros they are
     };
-    auto load_b = [&](int blk) __attribute__((always_inline)) {
-      unsigned p01[3], t2[3];
+    // the taps of block blk: the dword pairs are read early (read_b) and shifted into operand order late (make_b)
+    auto read_b = [&](int blk) __attribute__((always_inline)) {
 #pragma unroll
       for (int r = 0; r < 3; ++r) {
         const unsigned* xw = reinterpret_cast<const unsigned*>(smem_raw + (xa[r] + blk * cs2));
-        const unsigned d0 = xw[0], d1 = xw[1];
-        p01[r] = __builtin_amdgcn_alignbit(d1, d0, sh);  // columns x - 1, x
-        t2[r] = __builtin_amdgcn_alignbit(0u, d1, sh);   // column x + 1 in the low half
+        d0[r] = xw[0];
+        d1[r] = xw[1];
       }
-      const uint4 b1r = {p01[0], p01[1], p01[2], __builtin_amdgcn_perm(t2[1], t2[0], 0x05040100u)};
-      const uint4 b2r = {t2[2] & 0xffffu, 0u, 0u, 0u};
+    };
+    auto make_b = [&]() __attribute__((always_inline)) {
+      unsigned p01[3], t2[3];
+#pragma unroll
+      for (int r = 0; r < 3; ++r) {
+        p01[r] = __builtin_amdgcn_alignbit(d1[r], d0[r], sh);  // columns x - 1, x
+        t2[r] = __builtin_amdgcn_alignbit(0u, d1[r], sh);      // column x + 1 in the low half
+      }
+      const u32x4 b1r = {p01[0], p01[1], p01[2], __builtin_amdgcn_perm(t2[1], t2[0], 0x05040100u)};
       b1n = __builtin_bit_cast(V8, b1r);
-      b2n = __builtin_bit_cast(V8, b2r);
+      b2u[0] = t2[2] & 0xffffu;
+      // (plain arithmetic is free to sink to its use: the empty asm keeps it here, between two MFMAs)
+      asm volatile("" : "+v"(b1n), "+v"(b2u));
     };
-    auto depthwise = [&]() __attribute__((always_inline)) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-      acc = Elem<T>::mfma32(a1n, b1n, acc);
-      acc = Elem<T>::mfma32(a2n, b2n, acc);
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    auto depthwise_a = [&]() __attribute__((always_inline)) { acc = Elem<T>::mfma32(a1n, b1n, zero16); };
+    auto depthwise_b = [&]() __attribute__((always_inline)) {
+      acc = Elem<T>::mfma32(__builtin_bit_cast(V8, a2u), __builtin_bit_cast(V8, b2u), acc);
     };
-    auto convert = [&]() __attribute__((always_inline)) {
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const V2 c0v = cvt2<T>(acc[8 * s + 0], acc[8 * s + 1]), c1v = cvt2<T>(acc[8 * s + 2], acc[8 * s + 3]);
-        const V2 c2v = cvt2<T>(acc[8 * s + 4], acc[8 * s + 5]), c3v = cvt2<T>(acc[8 * s + 6], acc[8 * s + 7]);
-        pf[s] = V8{c0v[0], c0v[1], c1v[0], c1v[1], c2v[0], c2v[1], c3v[0], c3v[1]};
-        pf[s] = relu_packed(pf[s], relu_thr);
-      }
+    auto convert = [&](int s, int buf) __attribute__((always_inline)) {  // half s of the block in `acc`
+      const V2 c0v = cvt2<T>(acc[8 * s + 0], acc[8 * s + 1]), c1v = cvt2<T>(acc[8 * s + 2], acc[8 * s + 3]);
+      const V2 c2v = cvt2<T>(acc[8 * s + 4], acc[8 * s + 5]), c3v = cvt2<T>(acc[8 * s + 6], acc[8 * s + 7]);
+      pf[buf][s] = V8{c0v[0], c0v[1], c1v[0], c1v[1], c2v[0], c2v[1], c3v[0], c3v[1]};
+      if (RELU) pf[buf][s] = relu_packed(pf[buf][s]);
+      asm volatile("" : "+v"(pf[buf][s]));
     };
-    auto pointwise = [&]() __attribute__((always_inline)) {
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {  // rows = pixels, columns = output channels
-        o[t] = Elem<T>::mfma32(pf[0], wf[t][0], o[t]);
-        o[t] = Elem<T>::mfma32(pf[1], wf[t][1], o[t]);
-      }
+    // rows = pixels, columns = output channels
+    auto pointwise = [&](int t, int s, int buf) __attribute__((always_inline)) {
+      o[t] = Elem<T>::mfma32(pf[buf][s], wf[buf][t][s], o[t]);
     };
-    // Software pipeline over blocks of 32 intermediate channels (two input channels): while the 1x1 MFMAs of
-    // block b issue (operand pf already converted), the depthwise result of b + 1 matures in `acc`; then it is
-    // converted and the depthwise MFMAs of b + 2 start.  Blocks past the end recompute the last one.
+#define DITTO_SB __builtin_amdgcn_sched_barrier(0)
+    // Software pipeline over blocks of 32 intermediate channels (two input channels): while the 1x1 MFMAs of block b
+    // issue, the depthwise result of b + 1 is converted (into the other operand buffer), the taps of b + 2 are
+    // shifted into place and the depthwise MFMAs of b + 2 follow; the taps of b + 3 are read between those two.
+    // Blocks past the end recompute the last one.
+    auto clampb = [&](int b) __attribute__((always_inline)) { return b < last ? b : last; };
     load_a(0);
-    load_w2(0);
-    load_b(0);
-    depthwise();
-    convert();
-    load_a(last < 1 ? last : 1);
-    load_b(last < 1 ? last : 1);
-    depthwise();
-    for (int blk = 0; blk < nblk; ++blk) {
-      const int nxt = blk < last ? blk + 1 : last, nx2 = blk + 2 < last ? blk + 2 : last;
-      load_a(nx2);
-      load_b(nx2);
-      __builtin_amdgcn_sched_barrier(0);
-      pointwise();
-      __builtin_amdgcn_sched_barrier(0);
-      load_w2(nxt);
-      convert();    // block nxt
-      depthwise();  // block nx2
-      __builtin_amdgcn_sched_barrier(0);
+    load_w2(0, 0);
+    read_b(0);
+    make_b();
+    read_b(clampb(1));
+    depthwise_a();
+    depthwise_b();
+    load_a(clampb(1));
+    convert(0, 0);
+    convert(1, 0);
+    make_b();
+    read_b(clampb(2));
+    depthwise_a();
+    depthwise_b();
+    DITTO_SB;
+    for (int blk = 0; blk < nblk; blk += 2) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {  // (unrolled by two: the operand buffers alternate)
+        const int b = blk + u;
+        if (b >= nblk) break;
+        const int cur = u, oth = u ^ 1;
+        load_a(clampb(b + 2));
+        load_w2(clampb(b + 1), oth);
+        DITTO_SB;
+        pointwise(0, 0, cur); DITTO_SB; convert(0, oth); DITTO_SB;
+        pointwise(1, 0, cur); DITTO_SB; convert(1, oth); DITTO_SB;
+        pointwise(0, 1, cur); DITTO_SB; make_b(); DITTO_SB;
+        pointwise(1, 1, cur); DITTO_SB;
+        depthwise_a(); DITTO_SB;
+        read_b(clampb(b + 3)); DITTO_SB;
+        depthwise_b(); DITTO_SB;
+      }
     }
+#undef DITTO_SB
     // ---- output: o[t][i] = out[pixel 16 g + i of the tile][c2 = 32 t + ln]
     const int px0 = 32 * tile + 16 * g;
     const unsigned soff = (unsigned)((y0 * W + 32 * tile) * 2);  // wave-uniform part of the address
@@ -334,10 +365,10 @@ __global__ __launch_bounds__(64 * kDw16Waves) void dw16_rows_kernel(Dw16RowsArgs
 #endif
 }
 
-template <typename T, int NI>
+template <typename T, int NI, bool RELU>
 hipError_t launch_dw16_rows_ni(const Dw16RowsArgs& args, hipStream_t stream) {
   const int lds = dw16_rows_lds_bytes(args.C0, args.W);
-  auto kern = dw16_rows_kernel<T, NI>;
+  auto kern = dw16_rows_kernel<T, NI, RELU>;
   static thread_local int configured_dev = -1;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -354,14 +385,14 @@ hipError_t launch_dw16_rows_ni(const Dw16RowsArgs& args, hipStream_t stream) {
 template <typename T>
 hipError_t launch_dw16_rows(const Dw16RowsArgs& args, hipStream_t stream) {
   switch (dw16_rows_ni(args.C0, args.W)) {
-    case 1: return launch_dw16_rows_ni<T, 1>(args, stream);
-    case 2: return launch_dw16_rows_ni<T, 2>(args, stream);
-    case 3: return launch_dw16_rows_ni<T, 3>(args, stream);
-    case 4: return launch_dw16_rows_ni<T, 4>(args, stream);
-    case 5: return launch_dw16_rows_ni<T, 5>(args, stream);
-    case 6: return launch_dw16_rows_ni<T, 6>(args, stream);
-    case 7: return launch_dw16_rows_ni<T, 7>(args, stream);
-    case 8: return launch_dw16_rows_ni<T, 8>(args, stream);
+    case 1: return args.relu_mid ? launch_dw16_rows_ni<T, 1, true>(args, stream) : launch_dw16_rows_ni<T, 1, false>(args, stream);
+    case 2: return args.relu_mid ? launch_dw16_rows_ni<T, 2, true>(args, stream) : launch_dw16_rows_ni<T, 2, false>(args, stream);
+    case 3: return args.relu_mid ? launch_dw16_rows_ni<T, 3, true>(args, stream) : launch_dw16_rows_ni<T, 3, false>(args, stream);
+    case 4: return args.relu_mid ? launch_dw16_rows_ni<T, 4, true>(args, stream) : launch_dw16_rows_ni<T, 4, false>(args, stream);
+    case 5: return args.relu_mid ? launch_dw16_rows_ni<T, 5, true>(args, stream) : launch_dw16_rows_ni<T, 5, false>(args, stream);
+    case 6: return args.relu_mid ? launch_dw16_rows_ni<T, 6, true>(args, stream) : launch_dw16_rows_ni<T, 6, false>(args, stream);
+    case 7: return args.relu_mid ? launch_dw16_rows_ni<T, 7, true>(args, stream) : launch_dw16_rows_ni<T, 7, false>(args, stream);
+    case 8: return args.relu_mid ? launch_dw16_rows_ni<T, 8, true>(args, stream) : launch_dw16_rows_ni<T, 8, false>(args, stream);
   }
   return hipErrorInvalidValue;
 }
