@@ -31,6 +31,7 @@
 // issue port for about 12 of its 32 cycles, which leaves the two waves of a SIMD five vector issue
 // slots per MFMA).  The waves stay level and reach the barrier together.
 #pragma once
+#include <type_traits>
 #include "bmm_chain_fp.h"
 
 namespace ditto {
@@ -212,6 +213,24 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
       af[s] = v;
     }
   }
+  // Pre-scaled softmax (fp16, pipelined kernel): A is multiplied by scale * log2(e) ONCE, here, and the first MFMA
+  // of every score tile starts from minus the row's running maximum instead of zero, so the accumulator already
+  // holds the exponent: a score then costs its v_exp_f32 and nothing else (the multiply-add in front of it was a
+  // sixth of the vector work that bounds this kernel at head dimension 64: 13.9 -> 12.7 us per call on
+  // 96 x 512 x 64).  The price is one more fp16 rounding of A (2^-11 relative: rel-L2 of the result
+  // 2.9e-4 -> 3.5e-4 at 4096 x 128); bf16 would pay 2^-9 there (2.3e-3 -> 2.9e-3) and stays on the exact form.
+  // (head dimension 64 only: at 128 the sixteen more registers do not fit without scratch)
+  constexpr bool PRE = PIPE && INTER == kInterSoftmax && std::is_same<T, f16>::value && D <= 64;
+  if constexpr (PRE) {
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const V2 q2 = cvt2<T>((float)af[s][e] * p.scale_log2, (float)af[s][e + 1] * p.scale_log2);
+        af[s][e] = q2[0];
+        af[s][e + 1] = q2[1];
+      }
+  }
 
   // ---- accumulators of F^T: o[t][r] = F^T[32t + 8(r/4) + 4g + r%4][ln]
   f32x16 o[NT];
@@ -219,7 +238,10 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
-  float mrow = -INFINITY, lsum = 0.f;
+  // (pre-scaled form: scores are kept relative to the running maximum, which starts at zero and is set from the
+  // first half tile; negm = sixteen copies of minus that maximum, the accumulator a score tile starts from)
+  float mrow = PRE ? 0.f : -INFINITY, lsum = 0.f;
+  f32x16 negm = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const float c2 = p.scale_log2;
   const int ntiles = (L + kBN - 1) / kBN;
   const bool ragged = (L % kBN) != 0;
@@ -369,12 +391,13 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
     float mx = sc[0];
 #pragma unroll
     for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sc[r]);
-    mxn = pair_max(mx) * c2;
+    mxn = PRE ? pair_max(mx) : pair_max(mx) * c2;  // (pre-scaled: already an exponent, relative to mrow)
   };
   // probabilities of registers [r0, r1) of the half tile
   auto exp_range = [&](f32x16& sc, int r0, int r1) __attribute__((always_inline)) {
 #pragma unroll
-    for (int r = r0; r < r1; ++r) sc[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[r], c2, -mrow));
+    for (int r = r0; r < r1; ++r)
+      sc[r] = PRE ? __builtin_amdgcn_exp2f(sc[r]) : __builtin_amdgcn_exp2f(__builtin_fmaf(sc[r], c2, -mrow));
   };
   // operand of the second contraction for sixteen rows of the L tile: registers 8 * u2 .. + 7 of the half,
   // cast; the row sum is taken over the ROUNDED values, exactly what enters the MFMA
@@ -406,7 +429,28 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
     constexpr int J = decltype(j_c)::value, hh = decltype(hh_c)::value;
     constexpr int BNX = B_USE + (hh ? (J + 1) % 4 : J) * TB;  // B tile of the next half
     constexpr int CF = C_FRAG + (J & 1) * TB;
-    if constexpr (INTER == kInterSoftmax) {
+    if constexpr (PRE) {
+      // The same lazy rescale on relative scores: `cur` and mxn were computed against the present maximum.  The very
+      // first half tile sets the maximum (whatever its sign; nothing is accumulated yet), later ones only raise it.
+      const bool first = hh == 0 && it == 0;
+      if (first || __builtin_amdgcn_ballot_w64(mxn > kLazy) != 0) {
+        const float d = first ? mxn : fmaxf(mxn, 0.f);
+        mrow += d;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          cur[r] -= d;
+          negm[r] = -mrow;
+        }
+        if (!first) {
+          const float alpha = __builtin_amdgcn_exp2f(-d);
+          lsum *= alpha;
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
+        }
+      }
+    } else if constexpr (INTER == kInterSoftmax) {
       // lazy rescale: raise the running maximum only when a row of the wave exceeds it by 2^kLazy
       if (__builtin_amdgcn_ballot_w64(mxn > mrow + kLazy) != 0) {
         const float mnew = fmaxf(mrow, mxn);
@@ -432,7 +476,7 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
       __builtin_amdgcn_sched_barrier(0);
       if (k == 0) {
         const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        nxt = Elem<T>::mfma32(fr[k], af[k], z);
+        nxt = Elem<T>::mfma32(fr[k], af[k], PRE ? negm : z);
       } else if (k < NS) {
         nxt = Elem<T>::mfma32(fr[k], af[k], nxt);
       } else {

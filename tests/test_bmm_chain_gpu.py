@@ -165,6 +165,38 @@ def test_softmax_invariants_on_gpu(oracle, variant):
     assert np.isfinite(hot).all() and errors(hot, want)[0] <= MAX_ABS
 
 
+@pytest.mark.parametrize("variant", [0, 641, 642, 648, 649, 646])
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_running_maximum_paths(oracle, variant, dtype):
+    """What the lazily raised row maximum has to survive: every score far below zero from the first key on (the
+    maximum starts negative), and keys sorted so that every tile of 64 brings a row maximum far above the last
+    (a rescale per tile), with ragged M and L.  (The fp16 kernel that pre-scales A keeps scores relative to the
+    maximum; the others subtract it per score.)"""
+    batch, M, N, K, L = 2, 200, 64, 64, 456
+    rng = np.random.default_rng(5)
+    A = rng.standard_normal((batch, M, K)).astype(np.float32)
+    B = rng.standard_normal((batch, K, L)).astype(np.float32)
+    C = rng.standard_normal((batch, L, N)).astype(np.float32)
+    A[:, :, 0] = 4.0
+    cases = {}
+    Bn = B.copy()
+    Bn[:, 0, :] = -24.0                               # q0 k0 = -96: every score around -96 * scale
+    cases["all far below zero"] = Bn
+    Br = B.copy()
+    Br[:, 0, :] = np.linspace(-20.0, 20.0, L)         # the maximum climbs by about 11 per tile at scale 1
+    cases["rising"] = Br
+    Bf = B.copy()
+    Bf[:, 0, :] = np.linspace(20.0, -20.0, L)         # and the other way: later tiles far below the maximum
+    cases["falling"] = Bf
+    for name, Bx in cases.items():
+        Ar, Bxr, Cr = (oracle.np_round_to(t, dtype) for t in (A, Bx, C))
+        got = run_chain(Ar, Bxr, Cr, dtype, "softmax", 1.0, "LK", "float32", variant)
+        want = oracle.bmm_chain_f64(Ar, Bxr, Cr, inter="softmax", scale=1.0)
+        mx, rel = errors(got, want)
+        assert np.isfinite(got).all(), name
+        assert mx <= MAX_ABS and rel <= (REL_L2_BF16_QUANT if dtype == "bfloat16" else REL_L2), (name, mx, rel)
+
+
 def test_reference_semantics_on_reference_inputs(oracle):
     # the reference's own check: uniform(-1,1) inputs, scale 1, its exp / ones-column / divide
     # form vs torch softmax at rtol = atol = 0.1 (testing/hyper_fusion/bmm_softmax_bmm_wmma_...py:552-587)
