@@ -181,8 +181,8 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
   if (in == DITTO_F32) {
     if (d->acc_dtype != DITTO_F32 || d->out_dtype != DITTO_F32)
       return fail(DITTO_EINVAL, "the fp32 chain accumulates and outputs fp32");
-    if (d->inter_op != DITTO_INTER_CAST && d->inter_op != DITTO_INTER_RELU)
-      return fail(DITTO_EUNSUPPORTED, "the fp32 chain takes inter_op cast or relu");
+    if (d->inter_op != DITTO_INTER_CAST && d->inter_op != DITTO_INTER_RELU && d->inter_op != DITTO_INTER_SOFTMAX)
+      return fail(DITTO_EUNSUPPORTED, "the fp32 chain takes inter_op cast, relu or softmax");
     if (d->tile_variant != 0) return fail(DITTO_EINVAL, "the fp32 chain has a single variant (tile_variant must be 0)");
     if (d->K > ditto::f32_chain_max_dim() || d->N > ditto::f32_chain_max_dim())
       return fail(DITTO_EUNSUPPORTED, "the fp32 chain supports K, N up to %d", ditto::f32_chain_max_dim());
@@ -896,6 +896,8 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     args.b_lk = d->b_layout == DITTO_B_LK;
     args.relu = d->inter_op == DITTO_INTER_RELU;
     args.relu_out = d->relu_out;
+    args.softmax = d->inter_op == DITTO_INTER_SOFTMAX;
+    args.scale_log2 = d->softmax_scale * 1.4426950408889634f;
     hipError_t e = ditto::launch_gemm_chain_f32(args, st);
     if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
     return DITTO_OK;

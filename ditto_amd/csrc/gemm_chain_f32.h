@@ -16,6 +16,8 @@ struct F32ChainArgs {
   int b_lk;     // B stored [L][K]
   int relu;
   int relu_out;  // ReLU on the output
+  int softmax;   // inter path: softmax over L of scale * (A.B)
+  float scale_log2;  // softmax: scale * log2(e)
 };
 
 int f32_chain_lds_bytes_host(int K, int N);

@@ -1,10 +1,13 @@
-// fp32 GEMM -> cast|relu -> GEMM chain  F = inter(A.B).C  for the reference's fp32, CPU-sized
-// configuration (python_test/auto_tensorize/test_hyper_fusion.py:16-21: 512x64 . 64x64 . 64x64).
+// fp32 GEMM -> cast|relu|softmax -> GEMM chain  F = inter(A.B).C  for the reference's fp32, CPU-sized
+// configurations (python_test/auto_tensorize/test_hyper_fusion.py:16-21: 512x64 . 64x64 . 64x64; the fp32
+// BMM -> softmax -> BMM of benchmark/chimera/cpu/bmm_softmax_bmm.py:64-170).
 //
 // That configuration is plumbing, not a hot path (0.5 MFLOP per row block), so this kernel is
 // plain fp32 FMAs over LDS tiles: a workgroup owns 32 rows of A for one batch entry, walks L in
 // tiles of 64, keeps the 32x64 intermediate tile in LDS and its 32xN slice of F in registers.
-// Sums run over k, then l, in ascending order in fp32.
+// Sums run over k, then l, in ascending order in fp32.  Softmax is the online form over the tiles of L: the eight
+// threads of a row share its running maximum (exchanged by lane shuffles), each keeps the sum of its own
+// probabilities, and the row's slice of F is rescaled when the maximum rises.
 #include "gemm_chain_f32.h"
 
 namespace ditto {
@@ -41,6 +44,9 @@ __global__ __launch_bounds__(256) void gemm_chain_f32_kernel(F32ChainArgs p) {
 #pragma unroll
   for (int i = 0; i < kMaxD / 8; ++i) acc[i] = 0.f;
 
+  float mrow = -INFINITY, lsum = 0.f;  // softmax: running maximum (exp2 domain), this thread's share of the row sum
+  const float c2 = p.scale_log2;
+
   for (int l0 = 0; l0 < L; l0 += kBL) {
     __syncthreads();
     for (int e = tid; e < K * kBL; e += 256) {
@@ -55,14 +61,40 @@ __global__ __launch_bounds__(256) void gemm_chain_f32_kernel(F32ChainArgs p) {
       Cs[l * (N + 1) + n] = l0 + l < L ? Cg[(long long)(l0 + l) * p.c_rs + n] : 0.f;
     }
     __syncthreads();
+    float sv[kBL / 8];
 #pragma unroll
     for (int j = 0; j < kBL / 8; ++j) {
       const int l = c8 + 8 * j;
       float s = 0.f;
       for (int k = 0; k < K; ++k) s = __builtin_fmaf(As[r * (K + 1) + k], Bs[k * (kBL + 1) + l], s);
       if (p.relu) s = fmaxf(s, 0.f);
-      Ms[r * (kBL + 1) + l] = s;
+      sv[j] = s;
     }
+    if (p.softmax) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < kBL / 8; ++j) {
+        sv[j] = l0 + c8 + 8 * j < L ? sv[j] * c2 : -INFINITY;  // keys past L take no part
+        mx = fmaxf(mx, sv[j]);
+      }
+      // the row's eight threads are eight consecutive lanes
+      mx = fmaxf(mx, __shfl_xor(mx, 1));
+      mx = fmaxf(mx, __shfl_xor(mx, 2));
+      mx = fmaxf(mx, __shfl_xor(mx, 4));
+      const float mnew = fmaxf(mrow, mx);  // finite: every tile holds at least one key
+      const float alpha = exp2f(mrow - mnew);
+      mrow = mnew;
+      lsum *= alpha;
+#pragma unroll
+      for (int i = 0; i < kMaxD / 8; ++i) acc[i] *= alpha;
+#pragma unroll
+      for (int j = 0; j < kBL / 8; ++j) {
+        sv[j] = exp2f(sv[j] - mnew);
+        lsum += sv[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kBL / 8; ++j) Ms[r * (kBL + 1) + c8 + 8 * j] = sv[j];
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < kMaxD / 8; ++i) {
@@ -74,11 +106,18 @@ __global__ __launch_bounds__(256) void gemm_chain_f32_kernel(F32ChainArgs p) {
       }
     }
   }
+  float inv = 1.f;
+  if (p.softmax) {
+    lsum += __shfl_xor(lsum, 1);
+    lsum += __shfl_xor(lsum, 2);
+    lsum += __shfl_xor(lsum, 4);
+    inv = 1.f / lsum;
+  }
   if (m0 + r < M) {
 #pragma unroll
     for (int i = 0; i < kMaxD / 8; ++i) {
       const int n = c8 + 8 * i;
-      if (n < N) Fg[(long long)(m0 + r) * p.f_rs + n] = p.relu_out ? fmaxf(acc[i], 0.f) : acc[i];
+      if (n < N) Fg[(long long)(m0 + r) * p.f_rs + n] = p.relu_out ? fmaxf(acc[i] * inv, 0.f) : acc[i] * inv;
     }
   }
 }

@@ -172,8 +172,9 @@ size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc);
  *             NULL to use desc->requant_scale for every column.  Other chains: NULL
  *   f       : output (device), must not alias an input
  * in_dtype DITTO_F16 / DITTO_BF16: the MFMA chains (cast, relu, softmax);
- * DITTO_F32: the reference's fp32 configuration
- * (python_test/auto_tensorize/test_hyper_fusion.py:16-21), cast / relu, K, N <= 128;
+ * DITTO_F32: the reference's fp32 configurations
+ * (python_test/auto_tensorize/test_hyper_fusion.py:16-21; the fp32 BMM -> softmax -> BMM of
+ * benchmark/chimera/cpu/bmm_softmax_bmm.py:64-170), cast / relu / softmax, K, N <= 128;
  * DITTO_I8: the requantised chain.
  */
 int ditto_bmm_chain_run(const ditto_bmm_chain_desc* desc, const void* a, const void* b,

@@ -117,18 +117,19 @@ def test_cast_chain_vs_oracle(oracle, shape, dtype, inter):
 
 
 @pytest.mark.parametrize("shape", [(1, 512, 64, 64, 64), (3, 100, 24, 40, 72), (2, 64, 128, 128, 200)])
-@pytest.mark.parametrize("inter", ["cast", "relu"])
+@pytest.mark.parametrize("inter", ["cast", "relu", "softmax"])
 def test_fp32_chain_vs_oracle(oracle, shape, inter):
-    # the reference's fp32, CPU-sized configuration (first shape) and ragged ones, fp32 end to end
+    # the reference's fp32, CPU-sized configuration (first shape) and ragged ones, fp32 end to end; softmax: the
+    # fp32 BMM -> softmax -> BMM of the reference's CPU benchmark (benchmark/chimera/cpu/bmm_softmax_bmm.py:64-170)
     batch, M, N, K, L = shape
-    A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, "float32", seed=300 + M, std=0.25)
-    want = oracle.bmm_chain_f64(A, B, C, inter=inter)
+    std = 1.0 if inter == "softmax" else 0.25
+    A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, "float32", seed=300 + M, std=std)
+    scale = 0.5 if inter == "softmax" else 1.0
+    want = oracle.bmm_chain_f64(A, B, C, inter=inter, scale=scale)
     for b_layout in ("KL", "LK"):
-        got = run_chain(A, B, C, "float32", inter, 1.0, b_layout)
+        got = run_chain(A, B, C, "float32", inter, scale, b_layout)
         mx, rel = errors(got, want)
         assert mx <= 1e-4 and rel <= 1e-5, (b_layout, mx, rel)  # fp32 sums of <= 200 terms
-    with pytest.raises(NotImplementedError):
-        run_chain(A, B, C, "float32", "softmax", 1.0)
 
 
 def test_fused_cpu_nest_agrees_with_gpu(oracle):
