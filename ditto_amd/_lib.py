@@ -13,9 +13,9 @@ ABI_VERSION = 1
 OK, EINVAL, EUNSUPPORTED, EHIP, EWORKSPACE = 0, -1, -2, -3, -4
 
 # ditto_dtype
-F16, BF16, F32, I8, I32 = 0, 1, 2, 3, 4
-DTYPE_CODES = {"float16": F16, "bfloat16": BF16, "float32": F32, "int8": I8, "int32": I32}
-DTYPE_BYTES = {F16: 2, BF16: 2, F32: 4, I8: 1, I32: 4}
+F16, BF16, F32, I8, I32, F64 = 0, 1, 2, 3, 4, 5
+DTYPE_CODES = {"float16": F16, "bfloat16": BF16, "float32": F32, "int8": I8, "int32": I32, "float64": F64}
+DTYPE_BYTES = {F16: 2, BF16: 2, F32: 4, I8: 1, I32: 4, F64: 8}
 
 # ditto_inter_op
 INTER_CAST, INTER_RELU, INTER_SOFTMAX, INTER_REQUANT = 0, 1, 2, 3

@@ -16,6 +16,7 @@ _TORCH_CODES = {
     torch.float16: _lib.F16,
     torch.bfloat16: _lib.BF16,
     torch.float32: _lib.F32,
+    torch.float64: _lib.F64,
     torch.int8: _lib.I8,
     torch.int32: _lib.I32,
 }
@@ -89,7 +90,7 @@ def bmm_chain_desc(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale
     d = _lib.BmmChainDesc()
     d.abi_version = _lib.ABI_VERSION
     d.in_dtype = _code(A)
-    d.acc_dtype = _lib.I32 if A.dtype == torch.int8 else _lib.F32
+    d.acc_dtype = _lib.I32 if A.dtype == torch.int8 else _lib.F64 if A.dtype == torch.float64 else _lib.F32
     d.out_dtype = _code(F)
     d.inter_op = INTER_OPS[inter_op] if isinstance(inter_op, str) else int(inter_op)
     if B.stride(2) == 1 or L == 1:

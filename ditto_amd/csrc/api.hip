@@ -178,9 +178,9 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     t.variant = plan->d_pad * 10 + plan->qt;
     return DITTO_OK;
   }
-  if (in == DITTO_F32) {
-    if (d->acc_dtype != DITTO_F32 || d->out_dtype != DITTO_F32)
-      return fail(DITTO_EINVAL, "the fp32 chain accumulates and outputs fp32");
+  if (in == DITTO_F32 || in == DITTO_F64) {
+    if (d->acc_dtype != in || d->out_dtype != in)
+      return fail(DITTO_EINVAL, "the fp32 / fp64 chain accumulates and outputs its input type");
     if (d->inter_op != DITTO_INTER_CAST && d->inter_op != DITTO_INTER_RELU && d->inter_op != DITTO_INTER_SOFTMAX)
       return fail(DITTO_EUNSUPPORTED, "the fp32 chain takes inter_op cast, relu or softmax");
     if (d->tile_variant != 0) return fail(DITTO_EINVAL, "the fp32 chain has a single variant (tile_variant must be 0)");
@@ -196,13 +196,13 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     ditto_tile_param& t = plan->tile;
     t.block_threads = 256;
     t.block_m = 32;
-    t.block_l = 64;
     t.block_n = (int)d->N;
     t.head_pad = 0;
-    t.lds_bytes = ditto::f32_chain_lds_bytes_host((int)d->K, (int)d->N);
+    t.block_l = in == DITTO_F64 ? 32 : 64;
+    t.lds_bytes = ditto::f32_chain_lds_bytes_host((int)d->K, (int)d->N, in == DITTO_F64);
     t.grid_x = (int)(((d->M + 31) / 32) * d->batch);
     t.grid_y = t.grid_z = 1;
-    t.variant = 1000;  // fp32 FMA chain
+    t.variant = in == DITTO_F64 ? 1001 : 1000;  // fp32 / fp64 FMA chain
     return DITTO_OK;
   }
   if (in == DITTO_I8) {
@@ -875,10 +875,11 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
   }
   if (plan.family == 1) {
     ditto::F32ChainArgs args;
-    args.a = static_cast<const float*>(a);
-    args.b = static_cast<const float*>(b);
-    args.c = static_cast<const float*>(c);
-    args.f = static_cast<float*>(f);
+    args.a = a;
+    args.b = b;
+    args.c = c;
+    args.f = f;
+    args.f64 = d->in_dtype == DITTO_F64;
     args.a_bs = d->a_batch_stride;
     args.b_bs = d->b_batch_stride;
     args.c_bs = d->c_batch_stride;
@@ -897,7 +898,7 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     args.relu = d->inter_op == DITTO_INTER_RELU;
     args.relu_out = d->relu_out;
     args.softmax = d->inter_op == DITTO_INTER_SOFTMAX;
-    args.scale_log2 = d->softmax_scale * 1.4426950408889634f;
+    args.softmax_scale = d->softmax_scale;
     hipError_t e = ditto::launch_gemm_chain_f32(args, st);
     if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
     return DITTO_OK;

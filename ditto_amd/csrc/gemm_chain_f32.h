@@ -1,14 +1,14 @@
-// Arguments and launcher of the fp32 GEMM chain kernel (gemm_chain_f32.hip).
+// Arguments and launcher of the fp32 / fp64 GEMM chain kernel (gemm_chain_f32.hip).
 #pragma once
 #include <hip/hip_runtime.h>
 
 namespace ditto {
 
 struct F32ChainArgs {
-  const float* a;
-  const float* b;
-  const float* c;
-  float* f;
+  const void* a;  // float or double (f64)
+  const void* b;
+  const void* c;
+  void* f;
   long long a_bs, b_bs, c_bs, f_bs;  // batch strides, elements
   int a_rs, b_rs, c_rs, f_rs;        // row strides, elements
   int M, N, K, L, batch;
@@ -17,10 +17,11 @@ struct F32ChainArgs {
   int relu;
   int relu_out;  // ReLU on the output
   int softmax;   // inter path: softmax over L of scale * (A.B)
-  float scale_log2;  // softmax: scale * log2(e)
+  float softmax_scale;
+  int f64;       // elements are doubles
 };
 
-int f32_chain_lds_bytes_host(int K, int N);
+int f32_chain_lds_bytes_host(int K, int N, int f64);
 int f32_chain_max_dim();  // largest K and N the kernel takes
 hipError_t launch_gemm_chain_f32(const F32ChainArgs& args, hipStream_t stream);
 

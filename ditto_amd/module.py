@@ -9,7 +9,8 @@ import torch
 from . import chain
 from .auto_tensorize.hyper_fusion import ChainSchedule
 
-_TORCH = {"float16": torch.float16, "bfloat16": torch.bfloat16, "float32": torch.float32, "int8": torch.int8,
+_TORCH = {"float16": torch.float16, "bfloat16": torch.bfloat16, "float32": torch.float32, "float64": torch.float64,
+          "int8": torch.int8,
           "int32": torch.int32}
 
 

@@ -42,7 +42,8 @@ typedef enum ditto_dtype {
   DITTO_BF16 = 1,
   DITTO_F32 = 2,
   DITTO_I8 = 3,
-  DITTO_I32 = 4
+  DITTO_I32 = 4,
+  DITTO_F64 = 5
 } ditto_dtype;
 
 /* The op on the single path between the two contractions
@@ -172,7 +173,7 @@ size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc);
  *             NULL to use desc->requant_scale for every column.  Other chains: NULL
  *   f       : output (device), must not alias an input
  * in_dtype DITTO_F16 / DITTO_BF16: the MFMA chains (cast, relu, softmax);
- * DITTO_F32: the reference's fp32 configurations
+ * DITTO_F32 / DITTO_F64 (the ("80", "float64", "float64") row): the reference's fp32 configurations
  * (python_test/auto_tensorize/test_hyper_fusion.py:16-21; the fp32 BMM -> softmax -> BMM of
  * benchmark/chimera/cpu/bmm_softmax_bmm.py:64-170), cast / relu / softmax, K, N <= 128;
  * DITTO_I8: the requantised chain.

@@ -132,6 +132,39 @@ def test_fp32_chain_vs_oracle(oracle, shape, inter):
         assert mx <= 1e-4 and rel <= 1e-5, (b_layout, mx, rel)  # fp32 sums of <= 200 terms
 
 
+@pytest.mark.parametrize("shape", [(1, 512, 64, 64, 64), (3, 100, 24, 40, 72), (2, 64, 128, 128, 200)])
+@pytest.mark.parametrize("inter", ["cast", "relu", "softmax"])
+def test_fp64_chain_vs_oracle(oracle, shape, inter):
+    # the reference's ("80", "float64", "float64") row (benchmark/chimera/cuda/bmm_bmm_cuda.py:273-288): doubles end
+    # to end, held to the fp64 closed form at 1e-12
+    batch, M, N, K, L = shape
+    rng = np.random.default_rng(400 + M)
+    std = 1.0 if inter == "softmax" else 0.25
+    A, B, C = (rng.standard_normal(sh) * std for sh in ((batch, M, K), (batch, K, L), (batch, L, N)))
+    scale = 0.5 if inter == "softmax" else 1.0
+    mid = A @ B  # (the checker returns single precision: the closed form in numpy doubles here)
+    if inter == "relu":
+        mid = np.maximum(mid, 0.0)
+    elif inter == "softmax":
+        e = np.exp(mid * scale - (mid * scale).max(axis=-1, keepdims=True))
+        mid = e / e.sum(axis=-1, keepdims=True)
+    want = mid @ C
+    assert errors(want, oracle.bmm_chain_f64(A, B, C, inter=inter, scale=scale))[1] <= 1e-6
+    a, c = torch.from_numpy(A).cuda(), torch.from_numpy(C).cuda()
+    for b_layout in ("KL", "LK"):
+        b = torch.from_numpy(np.ascontiguousarray(B.transpose(0, 2, 1))).cuda().transpose(1, 2) if b_layout == "LK" \
+            else torch.from_numpy(B).cuda()
+        f = torch.full((batch, M, N), float("nan"), device="cuda:0", dtype=torch.float64)
+        desc = chain.bmm_chain_desc(a, b, c, f, inter, scale)
+        assert chain.select_tile(desc).variant == 1001
+        chain.run_bmm_chain(a, b, c, f, inter, scale)
+        torch.cuda.synchronize()
+        got = f.cpu().numpy()
+        assert np.abs(got - want).max() <= 1e-12 * max(1.0, np.abs(want).max()), (b_layout, np.abs(got - want).max())
+    with pytest.raises(ValueError):  # mixed types are refused
+        chain.run_bmm_chain(a, b, c, torch.empty(batch, M, N, device="cuda:0", dtype=torch.float32), inter, scale)
+
+
 def test_fused_cpu_nest_agrees_with_gpu(oracle):
     # the CPU baseline (the fused loop nest restatement) and the GPU kernel compute the same chain
     A, B, C = oracle.make_gemm_chain_inputs(1, 512, 64, 64, 64, "float16", seed=7, std=0.25)
