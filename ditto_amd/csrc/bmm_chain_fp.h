@@ -437,7 +437,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const bool by_rows = !p.out_f32 && (N & 7) == 0 && (p.f_rs & 7) == 0 && (p.f_bs & 7) == 0 && (p.f_bs2 & 7) == 0 &&
                        (reinterpret_cast<size_t>(p.f) & 15) == 0;  // wave-uniform
   static_assert(4 * (32 * QT) * tile_row_bytes<D>() <= bmm_chain_lds_bytes<D>(), "the parked rows need the staged tiles' LDS");
-  if (by_rows) wg_sync();  // every wave is done with the staged tiles
+  if (by_rows) {
+    // every wave is done with the staged tiles, and the direct loads still in flight (the tiles past the last one:
+    // zeros) have landed -- they would otherwise fall on the rows parked below
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    wg_sync();
+  }
   char* const tw = smem_raw + wave * (32 * QT) * tile_row_bytes<D>();
 #pragma unroll
   for (int j = 0; j < QT; ++j) {

@@ -577,7 +577,12 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
   const bool by_rows = !p.out_f32 && (N & 7) == 0 && (p.f_rs & 7) == 0 && (p.f_bs & 7) == 0 && (p.f_bs2 & 7) == 0 &&
                        (reinterpret_cast<size_t>(p.f) & 15) == 0;  // wave-uniform
   static_assert(8 * (32) * tile_row_bytes<D>() <= bmm_chain8_lds_bytes<D, B_KL>(), "the parked rows need the staged tiles' LDS");
-  if (by_rows) wg_sync();  // every wave is done with the staged tiles
+  if (by_rows) {
+    // every wave is done with the staged tiles, and the direct loads still in flight (the tiles past the last one:
+    // zeros) have landed -- they would otherwise fall on the rows parked below
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    wg_sync();
+  }
   char* const tw = smem_raw + wave * 32 * tile_row_bytes<D>();
   float inv = 1.f;
   if constexpr (INTER == kInterSoftmax) inv = 1.f / pair_sum(lsum);

@@ -472,7 +472,12 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
                        (reinterpret_cast<size_t>(p.f) & 15) == 0;  // wave-uniform
   constexpr int kRowBytes = tile_row_bytes<D>();
   static_assert(8 * (32) * tile_row_bytes<D>() <= bmm_chain8m16_lds_bytes<D>(), "the parked rows need the staged tiles' LDS");
-  if (by_rows) wg_sync();  // every wave is done with the staged tiles
+  if (by_rows) {
+    // every wave is done with the staged tiles, and the direct loads still in flight (the tiles past the last one:
+    // zeros) have landed -- they would otherwise fall on the rows parked below
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    wg_sync();
+  }
   char* const tw = smem_raw + wave * 32 * kRowBytes;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
