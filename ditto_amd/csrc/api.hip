@@ -87,7 +87,9 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
   memset(plan, 0, sizeof(*plan));
 
   if (in == DITTO_F16 || in == DITTO_BF16) {
-    if (d->acc_dtype != DITTO_F32)
+    // (an fp16 accumulator asked for with fp16 operands -- the reference's ("80", "float16", "float16") row -- is
+    // served by the MFMA's fp32 accumulator: the precision asked for and more)
+    if (d->acc_dtype != DITTO_F32 && !(d->acc_dtype == DITTO_F16 && in == DITTO_F16))
       return fail(DITTO_EUNSUPPORTED, "fp16/bf16 chains accumulate in fp32 (acc_dtype %d)", d->acc_dtype);
     if (d->out_dtype != in && d->out_dtype != DITTO_F32)
       return fail(DITTO_EINVAL, "out_dtype must be in_dtype or fp32");

@@ -184,7 +184,10 @@ def base_parser(example, n_shapes, with_ai=True):
 
 # (sm, in_dtype, acc_dtype) combinations with a kernel on this device
 # (the int8 / int32 row is the reference's ("80", "int8", "int32"), bmm_bmm_cuda.py:273-288; GEMM chain only)
-SUPPORTED_DTYPES = {("gfx950", "float16", "float32"), ("gfx950", "bfloat16", "float32"), ("gfx950", "int8", "int32")}
+# (float16 / float16, the reference's ("80" | "86", "float16", "float16") rows: the kernels accumulate in the MFMA's
+# fp32 accumulator whatever is asked for, the precision of that row and more)
+SUPPORTED_DTYPES = {("gfx950", "float16", "float32"), ("gfx950", "float16", "float16"), ("gfx950", "bfloat16", "float32"),
+                    ("gfx950", "int8", "int32")}
 # the requantisation scale the int8 driver rows use for the middle result (2^-10 for every column)
 INT8_REQUANT_SCALE = 2.0 ** -10
 

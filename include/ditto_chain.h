@@ -73,7 +73,8 @@ typedef enum ditto_b_layout {
 typedef struct ditto_bmm_chain_desc {
   int32_t abi_version;   /* DITTO_CHAIN_ABI_VERSION */
   int32_t in_dtype;      /* ditto_dtype of A, B, C                                    */
-  int32_t acc_dtype;     /* DITTO_F32 (fp) or DITTO_I32 (int8)                         */
+  int32_t acc_dtype;     /* DITTO_F32 (fp16 / bf16 / fp32 chains; DITTO_F16 with fp16 operands is
+                            accepted and served in fp32), DITTO_F64 (fp64), DITTO_I32 (int8) */
   int32_t out_dtype;     /* in_dtype (reference: F cast to in_dtype) or acc_dtype      */
   int32_t inter_op;      /* ditto_inter_op                                            */
   int32_t b_layout;      /* ditto_b_layout                                            */

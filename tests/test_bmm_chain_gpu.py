@@ -507,6 +507,29 @@ def test_strided_views_and_errors():
         chain.run_bmm_chain(a.cpu(), bt.transpose(1, 2).cpu(), c.cpu(), f.cpu(), "softmax", 0.125)
 
 
+def test_fp16_accumulator_request_is_served_in_fp32():
+    """The reference's ("80", "float16", "float16") rows (benchmark/chimera/cuda/bmm_bmm_cuda.py:273-288): an fp16
+    accumulator asked for with fp16 operands runs the same kernels on the MFMA's fp32 accumulator -- the same bits as
+    the fp32 request; a bf16 accumulator is no row of the reference and stays refused."""
+    from ditto_amd import _lib
+    dev = "cuda:0"
+    torch.manual_seed(1)
+    a, bt, c = (torch.randn(2, 128, 64, device=dev).half() for _ in range(3))
+    f32, f16 = (torch.empty(2, 128, 64, device=dev, dtype=torch.float16) for _ in range(2))
+    for inter in ("softmax", "cast"):
+        chain.run_bmm_chain(a, bt.transpose(1, 2), c, f32, inter, 0.125)
+        desc = chain.bmm_chain_desc(a, bt.transpose(1, 2), c, f16, inter, 0.125)
+        desc.acc_dtype = _lib.F16
+        chain.run_bmm_chain(a, bt.transpose(1, 2), c, f16, inter, 0.125, desc=desc)
+        assert torch.equal(f16, f32)
+    ab, bb, cb = a.bfloat16(), bt.bfloat16(), c.bfloat16()
+    fb = torch.empty(2, 128, 64, device=dev, dtype=torch.bfloat16)
+    desc = chain.bmm_chain_desc(ab, bb.transpose(1, 2), cb, fb, "cast")
+    desc.acc_dtype = _lib.BF16
+    with pytest.raises(NotImplementedError):
+        chain.run_bmm_chain(ab, bb.transpose(1, 2), cb, fb, "cast", desc=desc)
+
+
 def test_front_end_end_to_end(oracle):
     import ditto_amd as ditto
     from ditto_amd import auto_compute as ac, auto_tensorize as at, hardware as hw
