@@ -131,8 +131,8 @@ def random_args(layer, in_dtype, n_inputs, scale=1.0, device="cuda:0"):
     """uniform(-1, 1) tensors for every schedule tensor, as the reference drivers create them."""
     import torch
 
-    dts = {"float16": torch.float16, "bfloat16": torch.bfloat16, "float32": torch.float32, "int8": torch.int8,
-           "int32": torch.int32}
+    dts = {"float16": torch.float16, "bfloat16": torch.bfloat16, "float32": torch.float32, "float64": torch.float64,
+           "int8": torch.int8, "int32": torch.int32}
     args = []
     for i, t in enumerate(layer.schedule_tensors):
         dt = dts[t.dtype]
@@ -186,8 +186,9 @@ def base_parser(example, n_shapes, with_ai=True):
 # (the int8 / int32 row is the reference's ("80", "int8", "int32"), bmm_bmm_cuda.py:273-288; GEMM chain only)
 # (float16 / float16, the reference's ("80" | "86", "float16", "float16") rows: the kernels accumulate in the MFMA's
 # fp32 accumulator whatever is asked for, the precision of that row and more)
+# (float64 / float64: the plain-FMA kernel on doubles, head dimensions up to 128)
 SUPPORTED_DTYPES = {("gfx950", "float16", "float32"), ("gfx950", "float16", "float16"), ("gfx950", "bfloat16", "float32"),
-                    ("gfx950", "int8", "int32")}
+                    ("gfx950", "float64", "float64"), ("gfx950", "int8", "int32")}
 # the requantisation scale the int8 driver rows use for the middle result (2^-10 for every column)
 INT8_REQUANT_SCALE = 2.0 ** -10
 

@@ -24,7 +24,7 @@ def test_cli_ai_and_unsupported_dtype():
                          capture_output=True, text=True, check=True).stdout
     assert out.strip() == "(12, 512, 64, 64, 512) 256.0 56.888888888888886"
     out = subprocess.run([sys.executable, "-m", "ditto_amd.drivers.bmm_softmax_bmm", "--in_dtype", "float64",
-                          "--acc_dtype", "float64", "--num", "1"], capture_output=True, text=True, check=True).stdout
+                          "--acc_dtype", "float32", "--num", "1"], capture_output=True, text=True, check=True).stdout
     assert "Data type not supported" in out and "cost" not in out
 
 
