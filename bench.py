@@ -244,15 +244,23 @@ def graph_ms(call, steps):
         with torch.cuda.graph(g):
             for _ in range(steps):
                 call()
+        t0 = time.perf_counter()
         g.replay()
+        torch.cuda.synchronize()
+        # the capture leaves the device idle for a while: replay for about WARMUP_MIN_S first (a graph of a few
+        # steps is otherwise timed on clocks that are still coming up), then time as many replays again
+        reps = max(1, int(WARMUP_MIN_S / max(time.perf_counter() - t0, 1e-6)))
+        for _ in range(reps):
+            g.replay()
         torch.cuda.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         e0.record()
-        g.replay()
+        for _ in range(reps):
+            g.replay()
         e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / steps
+        return e0.elapsed_time(e1) / (steps * reps)
     except Exception:  # capture unsupported: the eager figure stands alone
         torch.cuda.synchronize()
         return None
