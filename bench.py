@@ -44,7 +44,7 @@ MEASURED_TRAFFIC = {
     "attn_f16_b96_s512_d64": (18.21, 6.00, 649),
     "conv_chain_f16_n32_c64_56x56_k64_k256": (13.30, 50.00, 3707),
     "gemm_chain_i8_8192x1024x256x1024": (12.15, 32.00, 8014),
-    "conv1x1_conv3x3_f16_n32_c64_56x56_k64_k64": (13.26, 12.25, 3604),
+    "conv1x1_conv3x3_f16_n32_c64_56x56_k64_k64": (13.10, 12.50, 3807),
     "dw3x3_conv1x1_f16_n32_c32_112x112_f16_k64": (29.18, 49.50, 4025),
     "dw3x3_conv1x1_f16_n32_c32_112x112_x1_k64": (24.64, 49.00, 4024),
 }

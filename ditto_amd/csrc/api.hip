@@ -276,6 +276,8 @@ struct ConvPlan {
   bool resident;       // 1x1 -> 3x3 with at most 64 channels: persistent kernel, W2 resident in LDS
   int res_grid;
   ditto::ConvResidentArgs rargs;
+  bool rows13;         // 1x1 -> 3x3 with at most 64 channels everywhere: the same pipeline (cvargs.f13), W2 fragments
+                       // in the workspace
   bool rows31;         // 3x3 -> 1x1 with at most 64 -> 64 -> 256 channels: the row pipeline (cvargs), W1 fragments
                        // in the workspace
   ditto::ConvRowsArgs cvargs;
@@ -608,6 +610,55 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
     if (P2 <= 0 || Q2 <= 0) return fail(DITTO_EINVAL, "empty convolution output");
     if (d->N * d->C2 * P2 * Q2 > 0x7fffffffLL * 4) return fail(DITTO_EINVAL, "tensor too large");
     a.R2 = (int)d->R2; a.S2 = (int)d->S2; a.pad2 = (int)d->pad2; a.P2 = (int)P2; a.Q2 = (int)Q2;
+    // 1x1 -> 3x3 (pad 1) with at most 64 channels everywhere, 16-bit output and image rows of whole 16-byte
+    // vectors up to 64 pixels: the row pipeline with the 1x1 convolution in its transposing stage (conv_rows.h)
+    if (allow_resident && !conv_rows_off() && !resident_off() && d->R1 == 1 && d->S1 == 1 && d->pad1 == 0 &&
+        d->stride1 == 1 && d->R2 == 3 && d->S2 == 3 && d->pad2 == 1 && d->C0 <= ditto::kCvrC && d->C1 <= ditto::kCvrC &&
+        d->C2 <= ditto::kCvrC && d->C0 % 8 == 0 && d->W % 8 == 0 && d->W <= 64 && d->out_dtype != DITTO_F32 &&
+        d->C0 * d->H * d->W * 2 < 0x7fffffffLL) {
+      const int cus = need_device ? device_cus() : 256;
+      int band_max = ditto::conv_rows_band_max((int)d->W);
+      if (band_max > d->H) band_max = (int)d->H;
+      while (band_max >= 1 && ditto::conv_rows_lds_bytes((int)d->W, band_max, true) > 160 * 1024) --band_max;
+      if (band_max >= 1) {
+        // fewest steps of two rows on the busiest CU (a band costs its steps plus about three of start-up)
+        long long best = -1;
+        int best_nb = 0;
+        const int nb_min = (int)((d->H + band_max - 1) / band_max);
+        for (int nb = nb_min; nb <= d->H && nb < nb_min + 64; ++nb) {
+          const int band = (int)((d->H + nb - 1) / nb);
+          const long long wgs = d->N * ((d->H + band - 1) / band);
+          const long long cost = ((wgs + cus - 1) / cus) * ((band + 1) / 2 + 3);
+          if (best < 0 || cost <= best) { best = cost; best_nb = nb; }  // ties: the split that fills more CUs
+        }
+        ditto::ConvRowsArgs& r = plan->cvargs;
+        r.N = (int)d->N; r.C0 = (int)d->C0; r.H = (int)d->H; r.W = (int)d->W;
+        r.Cm = (int)d->C1; r.C1 = (int)d->C2; r.C2 = (int)d->C2;
+        r.band = (int)((d->H + best_nb - 1) / best_nb);
+        r.bands = (int)((d->H + r.band - 1) / r.band);
+        r.f13 = 1;
+        r.relu_pre = d->inter_op == DITTO_INTER_RELU;
+        r.relu_mid = d->relu_out != 0;
+        r.relu_out = 0;
+        plan->rows13 = true;
+        plan->c1_tiles = 2;
+        plan->px2 = 1;
+        plan->w1p_bytes = 0;
+        plan->w2p_bytes = ditto::kCvrW1Bytes;
+        ditto_tile_param& t = plan->tile;
+        t.block_threads = 64 * ditto::kCvrWaves;
+        t.block_m = r.band * r.W;
+        t.block_l = ditto::kCvrC;
+        t.block_n = (int)d->C2;
+        t.head_pad = ditto::kCvrC;
+        t.lds_bytes = ditto::conv_rows_lds_bytes(r.W, r.band, true);
+        t.grid_x = r.N * r.bands;
+        t.grid_y = r.band;
+        t.grid_z = r.W;
+        t.variant = 3800 + r.band;  // row pipeline, 1x1 first; output rows per workgroup
+        return DITTO_OK;
+      }
+    }
     // 1x1 -> 3x3 (pad 1) with at most 64 channels everywhere and rows that are whole 16-byte vectors: the
     // persistent kernel that keeps W2 in LDS (conv_chain_resident.h), tiles of whole output rows
     if (allow_resident && !resident_off() && d->R1 == 1 && d->S1 == 1 && d->pad1 == 0 && d->stride1 == 1 && d->R2 == 3 &&
@@ -949,7 +1000,7 @@ size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
   ConvPlan plan;
   if (plan_conv(desc, &plan) != DITTO_OK) return 0;
   size_t need = plan.w1p_bytes + plan.w2p_bytes;
-  if (plan.resident || plan.rows31) {  // a call with pointers these kernels cannot take falls back to the general one
+  if (plan.resident || plan.rows31 || plan.rows13) {  // a call with pointers these kernels cannot take falls back to the general one
     ConvPlan general;
     if (plan_conv(desc, &general, false, 8, false) == DITTO_OK && general.w1p_bytes + general.w2p_bytes > need)
       need = general.w1p_bytes + general.w2p_bytes;
@@ -981,6 +1032,38 @@ int conv_chain_call(int phase, const ditto_conv_chain_desc* d, const void* x, co
       return fail(DITTO_EINVAL, "misaligned data pointer: this shape runs with x, w1 and y 16-byte aligned "
                                 "(its prepared weights are in the resident kernel's layout)");
     }
+  }
+  if (plan.rows13) {
+    // 16-byte direct loads of X, W1 fragments and output stores; W2 as MFMA fragments in the workspace
+    const bool ok = aligned(w1, 16) && workspace && workspace_bytes >= plan.w2p_bytes && aligned(workspace, 16) &&
+                    (!(phase & kConvCompute) || (aligned(x, 16) && aligned(y, 16)));
+    if (!ok && phase == kConvBoth) {
+      rc = plan_conv(d, &plan, true, 4, false);  // the general kernel: any element-aligned pointer, workspace optional
+      if (rc != DITTO_OK) return rc;
+    } else if (!ok) {
+      if (!workspace || workspace_bytes < plan.w2p_bytes)
+        return fail(DITTO_EWORKSPACE, "prepared weights live in the workspace: need %zu bytes", plan.w2p_bytes);
+      return fail(DITTO_EINVAL, "misaligned data pointer: this shape runs with x, w1, y and the workspace 16-byte "
+                                "aligned (its prepared weights are in the row pipeline's layout)");
+    }
+  }
+  if (plan.rows13) {
+    ditto::ConvRowsArgs r = plan.cvargs;
+    r.x = x;
+    r.w1x = w1;
+    r.w1f = workspace;
+    r.w2 = nullptr;
+    r.y = y;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const bool f16 = d->in_dtype == DITTO_F16;
+    hipError_t e = hipSuccess;
+    if (phase & kConvPrepare)  // W2 [C2][C1][3][3] into fragments
+      e = f16 ? ditto::pack_conv_w2_resident_f16(w2, workspace, r.Cm, r.C2, st)
+              : ditto::pack_conv_w2_resident_bf16(w2, workspace, r.Cm, r.C2, st);
+    if (e == hipSuccess && (phase & kConvCompute))
+      e = f16 ? ditto::launch_conv_rows_f16(r, st) : ditto::launch_conv_rows_bf16(r, st);
+    if (e != hipSuccess) return fail(DITTO_EHIP, "kernel launch failed: %s", hipGetErrorString(e));
+    return DITTO_OK;
   }
   if (plan.rows31) {
     // 16-byte direct loads of X, W2 fragments and output stores; W1 as MFMA fragments in the workspace

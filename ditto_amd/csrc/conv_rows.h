@@ -1,6 +1,8 @@
 // conv(3x3, pad 1, stride 1) -> cast|relu -> conv(1x1) on NCHW fp16 / bf16 tensors with at most 64 input
 // and intermediate channels, at most 256 output channels and image rows of at most 64 pixels (whole
-// 16-byte vectors), 16-bit output: the bottleneck block of a ResNet-50 at 56 x 56.
+// 16-byte vectors), 16-bit output: the bottleneck block of a ResNet-50 at 56 x 56.  With the template flag F13
+// the same pipeline runs conv(1x1) -> cast|relu -> conv(3x3, pad 1) with at most 64 channels everywhere (described
+// at the kernel).
 //
 // Reference chain: benchmark/chimera/cuda/conv_relu_conv_relu... / testing/hyper_fusion/
 // conv_relu_conv_relu_fuse_hw_cuda.py (conv3x3 -> conv1x1, the second GEMM consuming the first one's tile).
@@ -43,6 +45,11 @@ struct ConvRowsArgs {
   int N, C0, H, W, C1, C2;
   int band, bands;  // output rows per workgroup, workgroups per image
   int relu_mid, relu_out;
+  // conv(1x1) -> cast|relu -> conv(3x3, pad 1) through the same pipeline (see F13 below): w1x the 1x1 weights
+  // [Cm][C0], relu_pre the ReLU between the two; w1f then holds the 3x3 weights [C1][Cm][3][3] as fragments,
+  // C1 = C2 the output channels (at most 64), relu_mid the ReLU of the output
+  const void* w1x;
+  int f13, Cm, relu_pre;
 };
 
 constexpr int kCvrC = 64;      // input / intermediate channels (padded)
@@ -51,14 +58,26 @@ constexpr int kCvrRing = 6;    // rows of the transposed ring
 constexpr int kCvrW1Bytes = 9 * kCvrC * kCvrC * 2;
 
 // LDS: band + 2 raw rows of 128 W bytes, the ring of transposed rows, three intermediate steps of 2 W pixels
-__host__ __device__ constexpr int conv_rows_lds_bytes(int W, int band) {
-  return (band + 2) * 128 * W + kCvrRing * (W + 2) * 128 + 3 * (2 * W) * 128;
+// (and, for the 1x1 -> 3x3 chain, the 1x1 weights as 8 fragments of 1 KB)
+constexpr int kCvrW1xBytes = 2 * 4 * 1024;
+__host__ __device__ constexpr int conv_rows_lds_bytes(int W, int band, bool f13 = false) {
+  return (band + 2) * 128 * W + kCvrRing * (W + 2) * 128 + 3 * (2 * W) * 128 + (f13 ? kCvrW1xBytes : 0);
 }
 // waves 6 and 7 keep half each of the band's rows from the seventh on in flight at once, W / 8 load instructions
 // per row, next to the 8 loads of their W2 fragments: stay inside the 6-bit outstanding-load counter
 __host__ __device__ constexpr int conv_rows_band_max(int W) { return 2 * (48 / (W / 8)) + 4; }
 
-template <typename T, int NI>
+// F13: the chain conv(1x1) -> cast|relu -> conv(3x3, pad 1) with at most 64 channels everywhere (the reference's
+// benchmark/chimera/cuda/conv1x1_conv3x3_cuda.py row).  The 3x3 convolution takes the place of the pipeline's first
+// convolution, so its input - the 1x1 convolution's result - is what the ring of transposed rows has to hold:
+// instead of only turning a raw row round, waves 0..3 multiply the transposed fragments by the 1x1 weights
+// (fragments in LDS, 8 MFMAs 32x32x16 per 32 pixels) and write the cast result into the ring; rows outside the
+// image arrive as zeros and stay zeros, which is the 3x3 convolution's padding.  The pipeline's second stage
+// has no convolution left: waves 4..7 take 16 output channels each and multiply by an identity fragment, which
+// leaves the values as they are (one 16-bit rounding, done where the 3x3 result is cast) and gives the
+// 8-consecutive-pixel store layout.  (A non-finite output value turns the other channels of its pixel that share
+// the fragment into NaN: 0 x inf.)
+template <typename T, int NI, bool F13>
 __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef typename Elem<T>::v8 V8;
@@ -81,6 +100,7 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
   char* const raw = smem_raw;
   char* const Xt = raw + (p.band + 2) * RAWROW;
   char* const mid = Xt + kCvrRing * XTROW;
+  char* const w1x = mid + 3 * MIDBUF;  // F13: fragment (ct, kk) of the 1x1 weights at ((4 ct + kk) * 64 + lane) * 16
   const unsigned lds0 = (unsigned)(size_t)(DITTO_LDS char*)smem_raw;
 
   // direct global -> LDS load of input row q of the band (band-relative; image row y0 - 1 + q)
@@ -98,12 +118,74 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
     }
   };
 
+  // raw row q -> ring slot q % 6: unit (pixel tile t of 32, 16 channels kk): the lane receives channels
+  // 16 kk + 8 g .. + 7 of pixel 32 t + ln (two transposing reads) and writes them as one 16-byte chunk
+  const int i16 = lane & 15, h = (lane >> 4) & 1;
+  const int ntile = (Wi + 31) >> 5;
+  // (F13: pixel tiles t0, t0 + tstep, .. only, so that two waves can share a row)
+  auto transpose_row = [&](int q, int t0, int tstep) __attribute__((always_inline)) {
+    const char* const src = raw + q * RAWROW;
+    char* const dst = Xt + (q % kCvrRing) * XTROW;
+    // per pixel tile: its reads first (one LDS round trip), then the writes
+#pragma unroll 1
+    for (int t = t0; t < ntile; t += tstep) {
+      V8 v[4];
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const char* rd = src + (16 * kk + 8 * g + (i16 >> 2)) * (2 * Wi) + (32 * t + 16 * h + 4 * (i16 & 3)) * 2;
+        const V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(rd));
+        const V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(rd + 4 * 2 * Wi));
+        v[kk] = concat4<V4, V8>(lo, hi);
+      }
+      const int px = 32 * t + ln, col = px + 1;
+      if (F13) {
+        // the 1x1 convolution of the 32 pixels: a[ct][4 i + e] = mid channel 32 ct + 8 i + 4 g + e of pixel px,
+        // 8 bytes into chunk 4 ct + i of the pixel
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) {
+          f32x16 a;
+#pragma unroll
+          for (int e = 0; e < 16; ++e) a[e] = 0.f;
+#pragma unroll
+          for (int kk = 0; kk < 4; ++kk)
+            a = Elem<T>::mfma32(*reinterpret_cast<const V8*>(w1x + ((4 * ct + kk) * 64 + lane) * 16), v[kk], a);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const V2 a0 = cvt2<T>(a[4 * i], a[4 * i + 1]), a1 = cvt2<T>(a[4 * i + 2], a[4 * i + 3]);
+            V4 w = {a0[0], a0[1], a1[0], a1[1]};
+            if (p.relu_pre) w = relu_packed(w);
+            if (px < Wi) *reinterpret_cast<V4*>(dst + col * 128 + (((4 * ct + i) ^ ((col >> 1) & 7)) << 4) + 8 * g) = w;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+          if (px < Wi) *reinterpret_cast<V8*>(dst + col * 128 + (((2 * kk + g) ^ ((col >> 1) & 7)) << 4)) = v[kk];
+      }
+    }
+  };
+
   if (wave >= 4) {
     // ======================= second convolution / stores =======================
-    const int hh = wave - 4;  // output channels 64 hh .. 64 hh + 63
+    const int hh = wave - 4;  // output channels 64 hh .. 64 hh + 63 (F13: 16 hh .. 16 hh + 15)
+    constexpr int NCT = F13 ? 1 : 4;
+    const int cb = F13 ? 16 * hh : 64 * hh;
     // Before their first store (step 1) these waves bring the input rows from the fifth on (rows 0 .. 3 are the
     // other waves'): rows 4 and 5, turned round during step 0, by waves 4 and 5, which wait for them before the
     // first barrier; the rest, turned round from step 1 on, by waves 6 and 7, which wait before the second.
+    // F13: waves 4 and 5 first fetch the 1x1 weights, four of the eight fragments each - lane (ln, g) holds
+    // W1x[32 ct + ln][16 kk + 8 g .. + 7] of fragment (ct, kk) - and put them into LDS once they are there
+    V8 wx[4];
+    if (F13 && hh < 2) {
+      const T* W1g = reinterpret_cast<const T*>(p.w1x);
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const int c1 = 32 * hh + ln, c0 = 16 * kk + 8 * g;
+        V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (c1 < p.Cm && c0 < p.C0) v = *reinterpret_cast<const V8*>(W1g + (long long)c1 * p.C0 + c0);
+        wx[kk] = v;
+      }
+    }
     if (hh < 2) {
       if (4 + hh < nin) issue_row(4 + hh);
     } else {
@@ -112,18 +194,31 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
     }
     const int j = lane & 15, kg = lane >> 4;
     // A operand: lane (m, kg) holds W2[64 hh + 16 ct + m][32 ks + 8 kg .. + 7]
-    V8 w2f[4][2];
+    V8 w2f[NCT][2];
     {
       const T* W2g = reinterpret_cast<const T*>(p.w2);
 #pragma unroll
-      for (int ct = 0; ct < 4; ++ct)
+      for (int ct = 0; ct < NCT; ++ct)
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-          const int c2 = 64 * hh + 16 * ct + j, k0 = 32 * ks + 8 * kg;
+          const int c2 = cb + 16 * ct + j, k0 = 32 * ks + 8 * kg;
           V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-          if (c2 < p.C2 && k0 < p.C1) v = *reinterpret_cast<const V8*>(W2g + (long long)c2 * p.C1 + k0);
+          if (F13) {  // row c2 of the identity
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = k0 + e == c2 ? (T)1.0f : (T)0.0f;
+          } else if (c2 < p.C2 && k0 < p.C1) {
+            v = *reinterpret_cast<const V8*>(W2g + (long long)c2 * p.C1 + k0);
+          }
           w2f[ct][ks] = v;
         }
+    }
+    if (F13) {
+      if (hh < 2) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NI) : "memory");  // (at most the row's loads are still on their way)
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) *reinterpret_cast<V8*>(w1x + ((4 * hh + kk) * 64 + lane) * 16) = wx[kk];
+      }
+      lds_barrier();  // the 1x1 weights are in LDS
     }
     // The band's output pixels, row after row, are one contiguous run of every channel plane.  After step s the
     // wave stores the pixels up to the last whole 128-byte line of what is computed (the rest waits for the next
@@ -141,7 +236,14 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
     for (int k = 0; k <= nsteps; ++k) {
       if (k == (hh < 2 ? 0 : 1)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's rows (and W2 fragments)
       lds_barrier();  // the intermediate rows of step k - 1 are written
-      if (k == 0 || 64 * hh >= p.C2) continue;
+      if (F13) {
+        // rows 2k + 4, 2k + 5 for the next step (their ring slots were last read in step k - 1; they landed before
+        // barrier k): here, next to the other waves' MFMA loop, two waves per row where it has two pixel tiles
+        const int q = 2 * k + 4 + (hh & 1);
+        const bool share = ntile == 2;
+        if (q < nin && (share || hh < 2)) transpose_row(q, share ? hh >> 1 : 0, share ? 2 : 1);
+      }
+      if (k == 0 || cb >= p.C2) continue;
       const int s = k - 1;
       const int ce = (2 * (s + 1) < nout ? 2 * (s + 1) : nout) * Wi;  // pixels computed so far
       const int we = k == nsteps ? ce : ((A0 + ce) / align) * align - A0;
@@ -158,10 +260,10 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
           for (int t = 0; t < 8; ++t) bf[ks][t] = *reinterpret_cast<const V8*>(mr + SJ * t * 128 + (((4 * ks + kg) ^ b_x) << 4));
-        const unsigned y_lane = (unsigned)((64 * hh + 4 * kg) * (int)plane * 2 + (A0 + qc) * 2);
+        const unsigned y_lane = (unsigned)((cb + 4 * kg) * (int)plane * 2 + (A0 + qc) * 2);
 #pragma unroll
-        for (int ct = 0; ct < 4; ++ct) {
-          if (64 * hh + 16 * ct >= p.C2) break;  // wave-uniform
+        for (int ct = 0; ct < NCT; ++ct) {
+          if (cb + 16 * ct >= p.C2) break;  // wave-uniform
           f32x4 o[8];
           const f32x4 z = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -174,7 +276,7 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
             const V2 q2 = cvt2<T>(o[4][i], o[5][i]), q3 = cvt2<T>(o[6][i], o[7][i]);
             V8 px8 = {q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
             if (p.relu_out) px8 = relu_packed(px8);
-            const int c2 = 64 * hh + 16 * ct + 4 * kg + i;
+            const int c2 = cb + 16 * ct + 4 * kg + i;
             const unsigned vo = (on && c2 < p.C2) ? y_lane : kOut;
             const unsigned soff = (unsigned)((16 * ct + i) * (int)plane * 2);
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, px8), y_rsrc, vo, soff, kStoreWriteThrough);
@@ -206,31 +308,8 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
     for (int st = 0; st < NSTEP; ++st) w1f[st] = *reinterpret_cast<const V8*>(w + st * 2048);
   }
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NSTEP) : "memory");  // the row (issued ahead of the W1 fragments) has landed
-  // raw row q -> ring slot q % 6: unit (pixel tile t of 32, 16 channels kk): the lane receives channels
-  // 16 kk + 8 g .. + 7 of pixel 32 t + ln (two transposing reads) and writes them as one 16-byte chunk
-  const int i16 = lane & 15, h = (lane >> 4) & 1;
-  const int ntile = (Wi + 31) >> 5;
-  auto transpose_row = [&](int q) __attribute__((always_inline)) {
-    const char* const src = raw + q * RAWROW;
-    char* const dst = Xt + (q % kCvrRing) * XTROW;
-    // per pixel tile: its reads first (one LDS round trip), then the writes
-#pragma unroll 1
-    for (int t = 0; t < ntile; ++t) {
-      V8 v[4];
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        const char* rd = src + (16 * kk + 8 * g + (i16 >> 2)) * (2 * Wi) + (32 * t + 16 * h + 4 * (i16 & 3)) * 2;
-        const V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(rd));
-        const V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(rd + 4 * 2 * Wi));
-        v[kk] = concat4<V4, V8>(lo, hi);
-      }
-      const int px = 32 * t + ln, col = px + 1;
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk)
-        if (px < Wi) *reinterpret_cast<V8*>(dst + col * 128 + (((2 * kk + g) ^ ((col >> 1) & 7)) << 4)) = v[kk];
-    }
-  };
-  if (wave < nin) transpose_row(wave);  // rows 0 .. 3: what step 0 reads
+  if (F13) lds_barrier();  // waves 4 and 5 have put the 1x1 weights into LDS
+  if (wave < nin) transpose_row(wave, 0, 1);  // rows 0 .. 3: what step 0 reads
 
   // pixel tiles pt = 0, 1: column ln of the MFMA is pixel 32 pt + ln of the row; pixels past the row read pixel 0.
   // Ring rows are whole multiples of 128 bytes, so a fragment's address is (row + xb) ^ (chunk << 4) with
@@ -254,10 +333,10 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
   for (int k = 0; k <= nsteps; ++k) {
     lds_barrier();  // the transposed rows of step k are there; the buffer of step k - 2 has been read
     // rows 2k + 4, 2k + 5 for the next step (their ring slots were last read in step k - 1; they landed before
-    // barrier k: rows 4, 5 before the first one, the rest before the second)
-    {
+    // barrier k: rows 4, 5 before the first one, the rest before the second); F13: the other waves do it
+    if (!F13) {
       const int q = 2 * k + 4 + (wave & 1);
-      if ((q & 3) == wave && q < nin) transpose_row(q);
+      if ((q & 3) == wave && q < nin) transpose_row(q, 0, 1);
     }
     const int r = 2 * k + rho;
     if (k == nsteps || r >= nout) continue;
@@ -269,7 +348,7 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
     for (int pt = 0; pt < 2; ++pt)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[pt][e] = 0.f;
-    constexpr int kAhead = 3;
+    constexpr int kAhead = F13 ? 5 : 3;
     V8 xf[NSTEP][2];
     auto fetch = [&](int st) __attribute__((always_inline)) {
       const int tap = st >> 2, kk = st & 3, dr = tap / 3, ds = tap - 3 * dr;
@@ -306,10 +385,10 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
 #endif
 }
 
-template <typename T, int NI>
+template <typename T, int NI, bool F13>
 hipError_t launch_conv_rows_ni(const ConvRowsArgs& args, hipStream_t stream) {
-  const int lds = conv_rows_lds_bytes(args.W, args.band);
-  auto kern = conv_rows_kernel<T, NI>;
+  const int lds = conv_rows_lds_bytes(args.W, args.band, F13);
+  auto kern = conv_rows_kernel<T, NI, F13>;
   static thread_local int configured_dev = -1;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -326,14 +405,22 @@ hipError_t launch_conv_rows_ni(const ConvRowsArgs& args, hipStream_t stream) {
 template <typename T>
 hipError_t launch_conv_rows(const ConvRowsArgs& args, hipStream_t stream) {
   switch (args.W / 8) {
-    case 1: return launch_conv_rows_ni<T, 1>(args, stream);
-    case 2: return launch_conv_rows_ni<T, 2>(args, stream);
-    case 3: return launch_conv_rows_ni<T, 3>(args, stream);
-    case 4: return launch_conv_rows_ni<T, 4>(args, stream);
-    case 5: return launch_conv_rows_ni<T, 5>(args, stream);
-    case 6: return launch_conv_rows_ni<T, 6>(args, stream);
-    case 7: return launch_conv_rows_ni<T, 7>(args, stream);
-    case 8: return launch_conv_rows_ni<T, 8>(args, stream);
+    case 1: return args.f13 ? launch_conv_rows_ni<T, 1, true>(args, stream)
+                            : launch_conv_rows_ni<T, 1, false>(args, stream);
+    case 2: return args.f13 ? launch_conv_rows_ni<T, 2, true>(args, stream)
+                            : launch_conv_rows_ni<T, 2, false>(args, stream);
+    case 3: return args.f13 ? launch_conv_rows_ni<T, 3, true>(args, stream)
+                            : launch_conv_rows_ni<T, 3, false>(args, stream);
+    case 4: return args.f13 ? launch_conv_rows_ni<T, 4, true>(args, stream)
+                            : launch_conv_rows_ni<T, 4, false>(args, stream);
+    case 5: return args.f13 ? launch_conv_rows_ni<T, 5, true>(args, stream)
+                            : launch_conv_rows_ni<T, 5, false>(args, stream);
+    case 6: return args.f13 ? launch_conv_rows_ni<T, 6, true>(args, stream)
+                            : launch_conv_rows_ni<T, 6, false>(args, stream);
+    case 7: return args.f13 ? launch_conv_rows_ni<T, 7, true>(args, stream)
+                            : launch_conv_rows_ni<T, 7, false>(args, stream);
+    case 8: return args.f13 ? launch_conv_rows_ni<T, 8, true>(args, stream)
+                            : launch_conv_rows_ni<T, 8, false>(args, stream);
   }
   return hipErrorInvalidValue;
 }

@@ -202,7 +202,8 @@ int ditto_conv_chain_run(const ditto_conv_chain_desc* desc, const void* x, const
  *   ditto_conv_chain_run_prepared : only the fused kernel, reading the workspace a prepare call
  *                                   (same descriptor, same w1 / w2) has filled; the workspace is
  *                                   read-only here, so such calls may overlap.  w1 / w2 must still
- *                                   be passed (a 1x1 second convolution reads w2 directly).
+ *                                   be passed (a 1x1 second convolution reads w2 directly, a
+ *                                   1x1 first convolution in front of a 3x3 one w1).
  * DITTO_EWORKSPACE if the chain takes a workspace and none (or too small a one) is given. */
 int ditto_conv_chain_prepare(const ditto_conv_chain_desc* desc, const void* w1, const void* w2,
                              void* workspace, size_t workspace_bytes, void* stream);

@@ -186,6 +186,13 @@ CASES_3X3_SECOND = [
 ]
 
 
+def rows13_shape(N, C0, W, C1, R1, pad1, stride1, C2, R2, pad2):
+    """1x1 -> 3x3 (pad 1), at most 64 channels everywhere, rows of whole 16-byte vectors up to 64 pixels: with a
+    16-bit output these run on the row pipeline with the 1x1 convolution in its transposing stage."""
+    return (R1 == 1 and pad1 == 0 and stride1 == 1 and R2 == 3 and pad2 == 1 and max(C0, C1, C2) <= 64 and
+            C0 % 8 == 0 and W % 8 == 0 and W <= 64)
+
+
 @pytest.mark.parametrize("case", CASES_3X3_SECOND)
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
 def test_conv_chain_with_wide_second_filter(oracle, case, dtype):
@@ -198,14 +205,61 @@ def test_conv_chain_with_wide_second_filter(oracle, case, dtype):
         mx, rel = errors(got32, want32)
         assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
     got = run_conv(X, W1, W2, dtype, pad1, stride1, "relu", True, None, None, pad2)
-    assert np.array_equal(got, oracle.np_round_to(got32, dtype))
+    if rows13_shape(N, C0, W, C1, R1, pad1, stride1, C2, R2, pad2):
+        # (with a 16-bit output that shape runs on the row pipeline, whose summation order is its own)
+        mx, rel = errors(got, oracle.np_round_to(want32, dtype))
+        assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
+    else:
+        assert np.array_equal(got, oracle.np_round_to(got32, dtype))
     with pytest.raises(ValueError):  # this variant cannot run without its workspace
         run_conv(X, W1, W2, dtype, pad1, stride1, workspace=False, pad2=pad2)
+
+
+CASES_ROWS13 = [
+    # N, C0, H, W, C1, C2
+    (2, 64, 56, 56, 64, 64),    # the reference's ResNet-50 row (conv1x1_conv3x3_cuda.py:348-350), 2 images
+    (1, 32, 21, 24, 48, 40),    # channel counts that are no multiples of 32, an odd number of rows, one pixel tile
+    (1, 8, 9, 8, 8, 8),         # the smallest rows
+    (3, 16, 7, 64, 64, 24),     # the widest rows; fewer output channels than one store wave's 16 times two
+    (1, 64, 5, 40, 32, 64),     # two pixel tiles, the second one partial
+    (40, 24, 30, 48, 56, 16),   # more bands than CUs; only the first store wave has channels
+    (1, 40, 1, 16, 64, 64),     # a single image row
+]
+
+
+@pytest.mark.parametrize("case", CASES_ROWS13)
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_row_pipeline_conv1x1_conv3x3(oracle, case, dtype, monkeypatch):
+    """conv1x1 -> conv3x3 (pad 1) through the row pipeline: against the oracle, and against the kernel that keeps
+    W2 in LDS on the same inputs."""
+    N, C0, H, W, C1, C2 = case
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, 1, 3, dtype, seed=C0 + C2 + H, w_std=0.05)
+    x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
+    y = torch.empty((N, C2, H, W), device=x.device, dtype=TORCH_DTYPES[dtype])
+    tile = chain.select_tile(chain.conv_chain_desc(x, w1, w2, y, 0, 1, 1, 1, "relu", False))
+    assert tile.variant // 100 == 38 and tile.block_threads == 512 and tile.lds_bytes <= 160 * 1024
+    for relu_mid, relu_out in ((False, False), (True, False), (False, True), (True, True)):
+        inter = "relu" if relu_mid else "cast"
+        want = oracle.np_round_to(oracle.conv_chain_f32(X, W1, W2, 0, 1, 1, 1, relu_mid=relu_mid, relu_out=relu_out,
+                                                        round_mid=dtype), dtype)
+        got = run_conv(X, W1, W2, dtype, 0, 1, inter, relu_out, None, None, 1)
+        assert got.shape == want.shape and np.isfinite(got).all()
+        mx, rel = errors(got, want)
+        assert mx <= MAX_ABS and rel <= REL_L2, (relu_mid, relu_out, mx, rel)
+        again = run_conv(X, W1, W2, dtype, 0, 1, inter, relu_out, None, None, 1)
+        assert np.array_equal(again, got)
+    monkeypatch.setenv("DITTO_CONV_ROWS", "0")
+    assert chain.select_tile(chain.conv_chain_desc(x, w1, w2, y, 0, 1, 1, 1, "relu", False)).variant // 100 == 36
+    other = run_conv(X, W1, W2, dtype, 0, 1, "relu", True, None, None, 1)
+    monkeypatch.delenv("DITTO_CONV_ROWS")
+    mx, rel = errors(got, other)
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
 
 
 def test_resident_conv_chain_over_several_rounds(oracle, monkeypatch):
     """More tiles than CUs: every persistent workgroup walks over more than one tile.  Checked against the
     general kernel (which streams W2 per workgroup) on the same inputs, both against the oracle on a slice."""
+    monkeypatch.setenv("DITTO_CONV_ROWS", "0")  # (else the shape runs on the row pipeline)
     N, C0, H, W, C1, C2 = 20, 64, 56, 56, 64, 64
     X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, 1, 3, "float16", seed=5, w_std=0.05)
     x, w1, w2 = to_dev(X, "float16"), to_dev(W1, "float16"), to_dev(W2, "float16")

@@ -194,8 +194,9 @@ def test_row_kernels_use_no_scratch_and_wait_for_lds_before_every_barrier(tmp_pa
     subprocess.run(cmd, check=True, capture_output=True)
     text = out.read_text()
     md = {k: v for k, v in kernel_metadata(text).items() if "rows_kernel" in k}
-    # one instantiation per row width class (the kernel for sixteen outputs per channel: with and without ReLU)
-    assert len(md) == (16 if unit_name == "dw16_rows_f16" else 8)
+    # one instantiation per row width class (the kernel for sixteen outputs per channel: with and without ReLU;
+    # the conv pipeline: 3x3 first and 1x1 first)
+    assert len(md) == (8 if unit_name == "dw_rows_f16" else 16)
     for name, v in md.items():
         assert v["vgpr_spill_count"] == 0 and v["private_segment_fixed_size"] == 0, (name, v)
     lines = [l.strip() for l in text.split("\n") if l.strip() and not l.strip().startswith((";", "."))]
