@@ -141,14 +141,19 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
       if (F13) {
         // the 1x1 convolution of the 32 pixels: a[ct][4 i + e] = mid channel 32 ct + 8 i + 4 g + e of pixel px,
         // 8 bytes into chunk 4 ct + i of the pixel
+        f32x16 a2[2];
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) a2[ct][e] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+          for (int ct = 0; ct < 2; ++ct)
+            a2[ct] = Elem<T>::mfma32(*reinterpret_cast<const V8*>(w1x + ((4 * ct + kk) * 64 + lane) * 16), v[kk], a2[ct]);
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) {
-          f32x16 a;
-#pragma unroll
-          for (int e = 0; e < 16; ++e) a[e] = 0.f;
-#pragma unroll
-          for (int kk = 0; kk < 4; ++kk)
-            a = Elem<T>::mfma32(*reinterpret_cast<const V8*>(w1x + ((4 * ct + kk) * 64 + lane) * 16), v[kk], a);
+          const f32x16 a = a2[ct];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const V2 a0 = cvt2<T>(a[4 * i], a[4 * i + 1]), a1 = cvt2<T>(a[4 * i + 2], a[4 * i + 3]);
@@ -168,23 +173,26 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
   if (wave >= 4) {
     // ======================= second convolution / stores =======================
     const int hh = wave - 4;  // output channels 64 hh .. 64 hh + 63 (F13: 16 hh .. 16 hh + 15)
-    constexpr int NCT = F13 ? 1 : 4;
-    const int cb = F13 ? 16 * hh : 64 * hh;
+    // (F13: the identity's rows 16 hh .. + 15 are zero outside the 32-channel block hh / 2: one k step)
+    constexpr int NCT = F13 ? 1 : 4, NKS = F13 ? 1 : 2;
+    const int cb = F13 ? 16 * hh : 64 * hh, ks0 = F13 ? hh >> 1 : 0;
     // Before their first store (step 1) these waves bring the input rows from the fifth on (rows 0 .. 3 are the
     // other waves'): rows 4 and 5, turned round during step 0, by waves 4 and 5, which wait for them before the
     // first barrier; the rest, turned round from step 1 on, by waves 6 and 7, which wait before the second.
-    // F13: waves 4 and 5 first fetch the 1x1 weights, four of the eight fragments each - lane (ln, g) holds
-    // W1x[32 ct + ln][16 kk + 8 g .. + 7] of fragment (ct, kk) - and put them into LDS once they are there
-    V8 wx[4];
-    if (F13 && hh < 2) {
+    // F13: waves 6 and 7, whose rows are needed last, first fetch the 1x1 weights, four of the eight fragments
+    // each - lane (ln, g) holds W1x[32 ct + ln][16 kk + 8 g .. + 7] of fragment (ct, kk) - and put them into LDS
+    if (F13 && hh >= 2) {
       const T* W1g = reinterpret_cast<const T*>(p.w1x);
+      V8 wx[4];
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
-        const int c1 = 32 * hh + ln, c0 = 16 * kk + 8 * g;
+        const int c1 = 32 * (hh - 2) + ln, c0 = 16 * kk + 8 * g;
         V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
         if (c1 < p.Cm && c0 < p.C0) v = *reinterpret_cast<const V8*>(W1g + (long long)c1 * p.C0 + c0);
         wx[kk] = v;
       }
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) *reinterpret_cast<V8*>(w1x + ((4 * (hh - 2) + kk) * 64 + lane) * 16) = wx[kk];
     }
     if (hh < 2) {
       if (4 + hh < nin) issue_row(4 + hh);
@@ -194,14 +202,14 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
     }
     const int j = lane & 15, kg = lane >> 4;
     // A operand: lane (m, kg) holds W2[64 hh + 16 ct + m][32 ks + 8 kg .. + 7]
-    V8 w2f[NCT][2];
+    V8 w2f[NCT][NKS];
     {
       const T* W2g = reinterpret_cast<const T*>(p.w2);
 #pragma unroll
       for (int ct = 0; ct < NCT; ++ct)
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-          const int c2 = cb + 16 * ct + j, k0 = 32 * ks + 8 * kg;
+        for (int ks = 0; ks < NKS; ++ks) {
+          const int c2 = cb + 16 * ct + j, k0 = 32 * (ks0 + ks) + 8 * kg;
           V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
           if (F13) {  // row c2 of the identity
 #pragma unroll
@@ -213,19 +221,16 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
         }
     }
     if (F13) {
-      if (hh < 2) {
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NI) : "memory");  // (at most the row's loads are still on their way)
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) *reinterpret_cast<V8*>(w1x + ((4 * hh + kk) * 64 + lane) * 16) = wx[kk];
-      }
-      lds_barrier();  // the 1x1 weights are in LDS
+      lds_barrier();  // the 1x1 weights are in LDS, and rows 0 .. 3 (the other waves have waited for them)
+      // the second pixel tile of rows 0 .. 3, next to the other waves' first
+      if (ntile == 2 && hh < nin) transpose_row(hh, 1, 2);
     }
     // The band's output pixels, row after row, are one contiguous run of every channel plane.  After step s the
     // wave stores the pixels up to the last whole 128-byte line of what is computed (the rest waits for the next
     // step; with rows of 112 bytes every other line would else be written in two halves, 3 us apart, and go out to
     // memory twice), in windows of 128 pixels: MFMA column j of tile t is pixel w0 + 8 j + t of the band, so a
     // lane ends with 8 consecutive pixels of each of its 4 channels and 16 lanes write 256 contiguous bytes.
-    // The pixel lives in the intermediate buffer of its own step (slot SJ t + jj, chunk XORed with (jj >> 1) & 7),
+    // The pixel lives in the intermediate buffer of its own step (slot SJ t + jj, chunk XORed with (jj >> 1) & 7 and t),
     // this step's or the one before: three buffers.
     const int WB = 2 * Wi;                       // pixels of a step
     const int align = WB >= 64 ? 64 : 8;         // window ends on whole lines where a step spans one
@@ -255,11 +260,12 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
         const int jj = (qc - sq * WB) >> 3;
         const char* const mr = mid + (sq % 3) * MIDBUF + jj * 128;
         const int b_x = (jj >> 1) & 7;
-        V8 bf[2][8];
+        V8 bf[NKS][8];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+        for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
-          for (int t = 0; t < 8; ++t) bf[ks][t] = *reinterpret_cast<const V8*>(mr + SJ * t * 128 + (((4 * ks + kg) ^ b_x) << 4));
+          for (int t = 0; t < 8; ++t)
+            bf[ks][t] = *reinterpret_cast<const V8*>(mr + SJ * t * 128 + (((4 * (ks0 + ks) + kg) ^ b_x ^ (F13 ? t : 0)) << 4));
         const unsigned y_lane = (unsigned)((cb + 4 * kg) * (int)plane * 2 + (A0 + qc) * 2);
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct) {
@@ -268,8 +274,10 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
           const f32x4 z = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int t = 0; t < 8; ++t) o[t] = Elem<T>::mfma16(w2f[ct][0], bf[0][t], z);
+          if (NKS == 2) {
 #pragma unroll
-          for (int t = 0; t < 8; ++t) o[t] = Elem<T>::mfma16(w2f[ct][1], bf[1][t], o[t]);
+            for (int t = 0; t < 8; ++t) o[t] = Elem<T>::mfma16(w2f[ct][NKS - 1], bf[NKS - 1][t], o[t]);
+          }
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const V2 q0 = cvt2<T>(o[0][i], o[1][i]), q1 = cvt2<T>(o[2][i], o[3][i]);
@@ -308,8 +316,9 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
     for (int st = 0; st < NSTEP; ++st) w1f[st] = *reinterpret_cast<const V8*>(w + st * 2048);
   }
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NSTEP) : "memory");  // the row (issued ahead of the W1 fragments) has landed
-  if (F13) lds_barrier();  // waves 4 and 5 have put the 1x1 weights into LDS
-  if (wave < nin) transpose_row(wave, 0, 1);  // rows 0 .. 3: what step 0 reads
+  if (F13) lds_barrier();  // waves 6 and 7 have put the 1x1 weights into LDS
+  // rows 0 .. 3: what step 0 reads (F13: a second pixel tile is the other waves')
+  if (wave < nin) transpose_row(wave, 0, F13 ? 2 : 1);
 
   // pixel tiles pt = 0, 1: column ln of the MFMA is pixel 32 pt + ln of the row; pixels past the row read pixel 0.
   // Ring rows are whole multiples of 128 bytes, so a fragment's address is (row + xb) ^ (chunk << 4) with
@@ -328,7 +337,9 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
     }
     // pixel of the step: slot SJ t + j with 8 j + t = W rho + px
     const int pp = Wi * rho + pxc, jj = pp >> 3, tt = pp & 7;
-    mb[pt] = (SJ * tt + jj) * 128 | (((jj >> 1) & 7) << 4) | 8 * g;
+    // (the chunk index is XORed with tt as well: the 8 lanes of one jj then write 8 different chunk columns
+    // instead of the same banks of 8 slots that lie a multiple of 128 bytes apart)
+    mb[pt] = (SJ * tt + jj) * 128 | ((((jj >> 1) & 7) ^ (F13 ? tt : 0)) << 4) | 8 * g;
   }
   for (int k = 0; k <= nsteps; ++k) {
     lds_barrier();  // the transposed rows of step k are there; the buffer of step k - 2 has been read
