@@ -248,6 +248,23 @@ def test_row_pipeline_conv1x1_conv3x3(oracle, case, dtype, monkeypatch):
         assert mx <= MAX_ABS and rel <= REL_L2, (relu_mid, relu_out, mx, rel)
         again = run_conv(X, W1, W2, dtype, 0, 1, inter, relu_out, None, None, 1)
         assert np.array_equal(again, got)
+    # prepared weights: same bits as the one-call form; without the workspace the prepared form is refused
+    desc = chain.conv_chain_desc(x, w1, w2, y, 0, 1, 1, 1, "relu", True)
+    ws = chain.prepare_conv_chain(desc, w1, w2)
+    y1 = torch.full_like(y, float("nan"))
+    chain.run_conv_chain(x, w1, w2, y1, desc=desc, workspace=ws, prepared=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(y1.float().cpu().numpy(), got)
+    # a 1x1 weight tensor that is only element-aligned: the one-call form runs the general kernel instead
+    w1_off = torch.empty(w1.numel() + 1, device=x.device, dtype=w1.dtype)[1:].view_as(w1).copy_(w1)
+    assert w1_off.data_ptr() % 16 != 0
+    y3 = torch.full_like(y, float("nan"))
+    chain.run_conv_chain(x, w1_off, w2, y3, 0, 1, 1, 1, "relu", True)
+    torch.cuda.synchronize()
+    mx, rel = errors(y3.float().cpu().numpy(), got)
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
+    with pytest.raises(ValueError):  # ... and the prepared form, whose weights are in this kernel's layout, reports it
+        chain.run_conv_chain(x, w1_off, w2, y3, desc=desc, workspace=ws, prepared=True)
     monkeypatch.setenv("DITTO_CONV_ROWS", "0")
     assert chain.select_tile(chain.conv_chain_desc(x, w1, w2, y, 0, 1, 1, 1, "relu", False)).variant // 100 == 36
     other = run_conv(X, W1, W2, dtype, 0, 1, "relu", True, None, None, 1)
