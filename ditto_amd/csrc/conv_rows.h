@@ -320,21 +320,24 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
   // rows 0 .. 3: what step 0 reads (F13: a second pixel tile is the other waves')
   if (wave < nin) transpose_row(wave, 0, F13 ? 2 : 1);
 
-  // pixel tiles pt = 0, 1: column ln of the MFMA is pixel 32 pt + ln of the row; pixels past the row read pixel 0.
+  // pixel tiles pt = 0, 1: column ln of the MFMA is pixel 32 pt + ln of the row.
   // Ring rows are whole multiples of 128 bytes, so a fragment's address is (row + xb) ^ (chunk << 4) with
-  // xb = column * 128 | swizzle << 4; likewise the intermediate pixel's chunk is at (buffer + mb) ^ (chunk << 4)
-  int xb[2][3], mb[2];
+  // xb = column * 128 | swizzle << 4; likewise the intermediate pixel's chunk is at (buffer + mb) ^ (chunk << 4).
+  // Column + 32 has the same swizzle, so the second tile's fragment lies 4096 bytes behind the first one's (an
+  // immediate offset); its pixels past the row read whatever follows the ring row - the next one or the
+  // intermediate buffers, inside the allocation - and their MFMA columns are dropped.
+  int xb[3], mb[2];
   bool px_ok[2];
+#pragma unroll
+  for (int ds = 0; ds < 3; ++ds) {
+    const int col = (ln < Wi ? ln : 0) + ds;
+    xb[ds] = col * 128 | (((col >> 1) & 7) << 4);
+  }
 #pragma unroll
   for (int pt = 0; pt < 2; ++pt) {
     const int px = 32 * pt + ln;
     px_ok[pt] = px < Wi;
     const int pxc = px_ok[pt] ? px : 0;
-#pragma unroll
-    for (int ds = 0; ds < 3; ++ds) {
-      const int col = pxc + ds;
-      xb[pt][ds] = col * 128 | (((col >> 1) & 7) << 4);
-    }
     // pixel of the step: slot SJ t + j with 8 j + t = W rho + px
     const int pp = Wi * rho + pxc, jj = pp >> 3, tt = pp & 7;
     // (the chunk index is XORed with tt as well: the 8 lanes of one jj then write 8 different chunk columns
@@ -365,7 +368,7 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
       const int tap = st >> 2, kk = st & 3, dr = tap / 3, ds = tap - 3 * dr;
 #pragma unroll
       for (int pt = 0; pt < 2; ++pt)
-        xf[st][pt] = *reinterpret_cast<const V8*>(Xt + ((rowoff[dr] + xb[pt][ds]) ^ ((2 * kk + g) << 4)));
+        xf[st][pt] = *reinterpret_cast<const V8*>(Xt + ((rowoff[dr] + xb[ds]) ^ ((2 * kk + g) << 4)) + 4096 * pt);
     };
 #pragma unroll
     for (int st = 0; st < kAhead; ++st) fetch(st);
