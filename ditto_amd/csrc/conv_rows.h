@@ -172,6 +172,11 @@ __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs 
 
   if (wave >= 4) {
     // ======================= second convolution / stores =======================
+    // F13: these waves' short instruction streams (the 1x1 stage of a pixel tile, a window of stores) share a SIMD
+    // with an MFMA loop that leaves them about one issue slot in ten cycles; with a raised priority they get
+    // through in two thirds of the time (5 % of the kernel).  With the 3x3 first the same setting delays the first
+    // convolution's start-up and costs 10 %.
+    if (F13) __builtin_amdgcn_s_setprio(2);
     const int hh = wave - 4;  // output channels 64 hh .. 64 hh + 63 (F13: 16 hh .. 16 hh + 15)
     // (F13: the identity's rows 16 hh .. + 15 are zero outside the 32-channel block hh / 2: one k step)
     constexpr int NCT = F13 ? 1 : 4, NKS = F13 ? 1 : 2;
