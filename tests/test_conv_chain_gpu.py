@@ -273,6 +273,41 @@ def test_row_pipeline_conv1x1_conv3x3(oracle, case, dtype, monkeypatch):
     assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
 
 
+def test_row_pipeline_conv1x1_conv3x3_at_benchmark_size(oracle, monkeypatch):
+    """The benchmark's shape, 32 x 64 x 56 x 56 -> 64 -> 64 (one band per CU): three images against the oracle, all
+    of them against the kernel that keeps W2 in LDS, and the chain's linearity in x (no ReLU: f(2x) = 2 f(x); a power
+    of two only shifts exponents, so the two differ only where an intermediate value is subnormal in fp16)."""
+    N, C0, H, W, C1, C2 = 32, 64, 56, 56, 64, 64
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, 1, 3, "float16", seed=77, w_std=0.05)
+    x, w1, w2 = to_dev(X, "float16"), to_dev(W1, "float16"), to_dev(W2, "float16")
+    y = torch.full((N, C2, H, W), float("nan"), device=x.device, dtype=torch.float16)
+    desc = chain.conv_chain_desc(x, w1, w2, y, 0, 1, 1, 1, "relu", True)
+    assert chain.select_tile(desc).variant == 3807
+    chain.run_conv_chain(x, w1, w2, y, desc=desc)
+    torch.cuda.synchronize()
+    got = y.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    for n in (0, 17, 31):
+        want = oracle.conv_chain_f32(X[n:n + 1], W1, W2, 0, 1, 1, 1, relu_mid=True, relu_out=True, round_mid="float16")
+        mx, rel = errors(got[n:n + 1], oracle.np_round_to(want, "float16"))
+        assert mx <= MAX_ABS and rel <= REL_L2, (n, mx, rel)
+    ya, yb = torch.empty_like(y), torch.empty_like(y)
+    chain.run_conv_chain(x, w1, w2, ya, 0, 1, 1, 1, "cast", False)
+    chain.run_conv_chain(x * 2, w1, w2, yb, 0, 1, 1, 1, "cast", False)
+    torch.cuda.synchronize()
+    mx, rel = errors((ya * 2).float().cpu().numpy(), yb.float().cpu().numpy())
+    assert mx <= 1e-3 and rel <= 1e-5, (mx, rel)
+    monkeypatch.setenv("DITTO_CONV_ROWS", "0")
+    y2 = torch.full_like(y, float("nan"))
+    desc2 = chain.conv_chain_desc(x, w1, w2, y2, 0, 1, 1, 1, "relu", True)
+    assert chain.select_tile(desc2).variant // 100 == 36
+    chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
+    torch.cuda.synchronize()
+    monkeypatch.delenv("DITTO_CONV_ROWS")
+    mx, rel = errors(got, y2.float().cpu().numpy())
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
+
+
 def test_resident_conv_chain_over_several_rounds(oracle, monkeypatch):
     """More tiles than CUs: every persistent workgroup walks over more than one tile.  Checked against the
     general kernel (which streams W2 per workgroup) on the same inputs, both against the oracle on a slice."""
