@@ -70,13 +70,15 @@ __host__ __device__ constexpr int conv_rows_band_max(int W) { return 2 * (48 / (
 // F13: the chain conv(1x1) -> cast|relu -> conv(3x3, pad 1) with at most 64 channels everywhere (the reference's
 // benchmark/chimera/cuda/conv1x1_conv3x3_cuda.py row).  The 3x3 convolution takes the place of the pipeline's first
 // convolution, so its input - the 1x1 convolution's result - is what the ring of transposed rows has to hold:
-// instead of only turning a raw row round, waves 0..3 multiply the transposed fragments by the 1x1 weights
-// (fragments in LDS, 8 MFMAs 32x32x16 per 32 pixels) and write the cast result into the ring; rows outside the
-// image arrive as zeros and stay zeros, which is the 3x3 convolution's padding.  The pipeline's second stage
+// instead of only turning a raw row round, the transposing stage multiplies the transposed fragments by the 1x1
+// weights (fragments in LDS, 8 MFMAs 32x32x16 per 32 pixels) and writes the cast result into the ring; rows outside
+// the image arrive as zeros and stay zeros, which is the 3x3 convolution's padding.  The pipeline's second stage
 // has no convolution left: waves 4..7 take 16 output channels each and multiply by an identity fragment, which
 // leaves the values as they are (one 16-bit rounding, done where the 3x3 result is cast) and gives the
 // 8-consecutive-pixel store layout.  (A non-finite output value turns the other channels of its pixel that share
-// the fragment into NaN: 0 x inf.)
+// the fragment into NaN: 0 x inf.)  With so little left to do there, waves 4..7 also run the transposing stage -
+// two waves per row, one per pixel tile of 32, next to the MFMA loop of waves 0..3 (for rows 0..3, which are needed
+// first, all eight waves share it) - at a raised wave priority.
 template <typename T, int NI, bool F13>
 __global__ __launch_bounds__(64 * kCvrWaves) void conv_rows_kernel(ConvRowsArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
