@@ -32,12 +32,20 @@
 #pragma once
 #include "bmm_chain_fp8.h"
 
+#ifndef DITTO_M16_PHASES
+#define DITTO_M16_PHASES 1
+#endif
+
 namespace ditto {
 
 template <int D>
 __host__ __device__ constexpr int bmm_chain8m16_lds_bytes() {
   // B tiles as loaded [4], raw C tiles [2 or 4], fragment-major C tiles [2]
+#ifdef DITTO_M16_NCR4
+  return (4 + 4 + 2) * kBN * D * 2;
+#else
   return (4 + (D == 64 ? 4 : 2) + 2) * kBN * D * 2;
+#endif
 }
 
 template <typename V8>
@@ -118,6 +126,13 @@ __device__ __forceinline__ float quad_sum(float x) {
   return pair_sum(a + b);
 }
 
+template <bool B>
+struct BoolC {
+  static constexpr bool value = B;
+};
+// a lane's partial row sum above which the optimistic walk lowers the row's scale (2^32)
+constexpr float kSumLimit = 4294967296.f;
+
 template <typename T, int D, int INTER>
 __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -125,6 +140,12 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   typedef typename Elem<T>::v4 V4;
   typedef typename Elem<T>::v2 V2;
   constexpr int NW = 8, BM = NW * 32;
+#ifdef DITTO_M16_NO_OPTIMISTIC
+  constexpr bool kOptimistic = false;
+#else
+  // bf16 only: an fp16 probability overflows 2^16, far below what a tile's scores may climb between two votes
+  constexpr bool kOptimistic = INTER == kInterSoftmax && Elem<T>::is_bf16;
+#endif
   constexpr int TB = kBN * D * 2;     // bytes per tile
   constexpr int B_RB = D * 2;         // bytes per LDS row of a B tile ([L][K])
   constexpr int B_CPR = B_RB / 16;
@@ -136,7 +157,11 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   constexpr int NLD = TB / 1024 / NW; // direct loads per wave per tile
   constexpr int NTR = NFRAG / NW;     // fragments each wave transposes per tile
   static_assert(NLD >= 1 && NTR >= 1, "tile too small for eight waves");
+#ifdef DITTO_M16_NCR4
+  constexpr int NCR = 4;
+#else
   constexpr int NCR = D == 64 ? 4 : 2;
+#endif
   constexpr int B_LOAD = 0;                   // [4] row-read layout
   constexpr int C_RAW = 4 * TB;               // [NCR]
   constexpr int C_FRAG = C_RAW + NCR * TB;    // [2]
@@ -357,16 +382,47 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
     }
   };
 
+  // The optimistic walk (bf16): no maximum is taken per half tile.  The row's reference exponent is the maximum of
+  // its first 32 scores, and what is watched is the row SUM: a probability is never larger than the sum it went
+  // into, so while a lane's partial sum stays below 2^kSumLimitLog2 no probability has come near the end of the
+  // fp32 / bf16 range.  Once per tile a lane votes when its sum has passed the limit; the row's reference is then
+  // raised by a whole number of binary orders (scaling by a power of two is exact) and sums and accumulators follow.
+  // A row whose scores climb by more than the range within one tile overflows before the vote: its sum ends up
+  // infinite or NaN, which the end of the walk detects, and the workgroup then walks the keys again the exact way
+  // (maximum per half tile before any exponential).
+  auto sum_rescale = [&]() __attribute__((always_inline)) {
+    const bool vote = fmaxf(lsum[0], lsum[1]) > kSumLimit;
+    if (__builtin_amdgcn_ballot_w64(vote) != 0) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float sref = quad_max(lsum[j]);  // the same in the four lanes of a row
+        // (an infinite or NaN sum is left as it is: that is what the end of the walk looks for)
+        const int e = (sref > kSumLimit && sref < INFINITY) ? ((__builtin_bit_cast(int, sref) >> 23) & 255) - 127 : 0;
+        const float alpha = __builtin_bit_cast(float, (127 - e) << 23);  // 2^-e, 32 <= e <= 127
+        mrow[j] += (float)e;
+        lsum[j] *= alpha;
+#pragma unroll
+        for (int t = 0; t < NTN; ++t) acc_scale(2 * t + j, alpha, o);
+      }
+    }
+  };
+  // reference exponent of a fresh row: the maximum of its first half tile (finite: key 0 exists and is not masked)
+  auto init_max = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) mrow[j] = quad_max(mloc[j]);
+  };
+
   // One half step: consumes `cur` (half hh of tile it), produces `nxt` (the following half).  Fragment
   // groups: 2 NS of the first contraction (16-row tile i of the next half x k step), then NTN of the second
   // (column tile t); each fragment feeds the two row tiles.
   constexpr int kAhead = 3;
   constexpr int NGS = 2 * NS, NG = NGS + NTN;
-  auto half_step = [&](Half& cur, Half& nxt, int it, auto j_c, auto hh_c) __attribute__((always_inline)) {
+  auto half_step = [&](Half& cur, Half& nxt, int it, auto j_c, auto hh_c, auto safe_c) __attribute__((always_inline)) {
     constexpr int J = decltype(j_c)::value, hh = decltype(hh_c)::value;
+    constexpr bool SAFE = decltype(safe_c)::value;
     constexpr int BNX = B_LOAD + (hh ? (J + 1) % 4 : J) * TB;  // B tile of the next half
     constexpr int CF = C_FRAG + (J & 1) * TB;
-    if constexpr (INTER == kInterSoftmax) maybe_rescale();
+    if constexpr (INTER == kInterSoftmax && SAFE) maybe_rescale();
     V8 fr[NG];
     auto fetch = [&](int k) __attribute__((always_inline)) {
       // first contraction: k = st * 2 + i (the two 16-row tiles of the half alternate: four accumulators in turn)
@@ -375,10 +431,31 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
 #pragma unroll
     for (int k = 0; k < kAhead; ++k) fetch(k);
     V8 pf[2];
+#if DITTO_M16_PHASES
+    // vector phase first, all of it, then the MFMAs of both contractions back to back
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (INTER == kInterSoftmax) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) exp_unit(cur, u);
+    }
+    make_p(cur, 0, pf[0]);
+    make_p(cur, 1, pf[1]);
+    asm volatile("" : "+v"(pf[0]), "+v"(pf[1]));
+    __builtin_amdgcn_sched_barrier(0);
+#endif
 #pragma unroll
     for (int k = 0; k < NG; ++k) {
       if (k + kAhead < NG) fetch(k + kAhead);
       __builtin_amdgcn_sched_barrier(0);
+#ifdef DITTO_M16_SPREAD
+      // the step's direct loads go out among the MFMAs, C in the first half step and B in the second (the waits
+      // count them in that order), not all at once behind the barrier where the whole workgroup's loads queue up
+      if (k == DITTO_M16_SPREAD) {
+        if (hh == 0) load_c(it + C_AHEAD, NCR == 4 ? (J + 3) % 4 : (J & 1));
+        else load_b(it + B_AHEAD, (J + 3) % 4);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#endif
       if (k < NGS) {
         const int i = k & 1, st = k >> 1;
 #pragma unroll
@@ -387,6 +464,7 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
           else nxt.v[i][j] = Mfma16<T>::run(fr[k], af[j][st], nxt.v[i][j]);
         }
         // the four exponential units of `cur` are spread over the first contraction's groups
+#if !DITTO_M16_PHASES
         if constexpr (INTER == kInterSoftmax) {
           if (NGS >= 4) {
             if (k % (NGS / 4) == 0 && k / (NGS / 4) < 4) exp_unit(cur, k / (NGS / 4));
@@ -399,6 +477,7 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
           make_p(cur, 0, pf[0]);
           make_p(cur, 1, pf[1]);
         }
+#endif
       } else {
         const int t = k - NGS;
 #pragma unroll
@@ -409,26 +488,39 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
     if constexpr (INTER == kInterSoftmax) {
       const int nt = hh ? it + 1 : it;  // tile of the next half
       if (ragged && nt == ntiles - 1) mask_tail(nxt, nt * kBN + 32 * (hh ^ 1));
-      local_max(nxt);
+      if constexpr (SAFE) local_max(nxt);
     }
   };
-  auto tile_step = [&](int it, auto j_c) __attribute__((always_inline)) {
+  auto tile_step = [&](int it, auto j_c, auto safe_c) __attribute__((always_inline)) {
     constexpr int J = decltype(j_c)::value;
+    constexpr bool SAFE = decltype(safe_c)::value;
     constexpr int PAR = J & 1;
     V8 xc[NTR];
     // C first: the wait at the end of the step can then leave the (younger) B loads in flight
+#ifndef DITTO_M16_SPREAD
     load_c(it + C_AHEAD, NCR == 4 ? (J + 3) % 4 : PAR);
     load_b(it + B_AHEAD, (J + 3) % 4);
+#endif
+#ifndef DITTO_ABL_NOTR
     tr_read_c(C_RAW + (NCR == 4 ? (J + 1) % 4 : (PAR ^ 1)) * TB, xc);
-    half_step(sa, sb, it, j_c, IntC<0>{});
+#endif
+    half_step(sa, sb, it, j_c, IntC<0>{}, safe_c);
+#ifndef DITTO_ABL_NOTR
     tr_write(C_FRAG + (PAR ^ 1) * TB, xc);
-    half_step(sb, sa, it, j_c, IntC<1>{});
+#endif
+    half_step(sb, sa, it, j_c, IntC<1>{}, safe_c);
+    if constexpr (INTER == kInterSoftmax && !SAFE) sum_rescale();
+#ifndef DITTO_ABL_NOBAR
     if (NCR == 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLD) : "memory");
     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
     __syncthreads();
+#endif
   };
 
-  // ---- prologue: first tiles in flight, first transposition, scores of the very first half
+  // ---- one walk over the keys: prologue (first tiles in flight, first transposition, scores of the very first
+  // half), then the tile loop
+  auto walk = [&](auto safe_c) __attribute__((always_inline)) {
+  constexpr bool SAFE = decltype(safe_c)::value;
   load_b(0, 0);
   load_b(1, 1);
   load_c(0, 0);
@@ -456,14 +548,48 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   if constexpr (INTER == kInterSoftmax) {
     if (ragged && ntiles == 1) mask_tail(sa, 0);
     local_max(sa);
+    if constexpr (!SAFE) init_max();
   }
   __syncthreads();
 
   for (int it = 0; it < ntiles; it += 4) {
-    tile_step(it, IntC<0>{});
-    if (it + 1 < ntiles) tile_step(it + 1, IntC<1>{});
-    if (it + 2 < ntiles) tile_step(it + 2, IntC<2>{});
-    if (it + 3 < ntiles) tile_step(it + 3, IntC<3>{});
+    tile_step(it, IntC<0>{}, safe_c);
+    if (it + 1 < ntiles) tile_step(it + 1, IntC<1>{}, safe_c);
+    if (it + 2 < ntiles) tile_step(it + 2, IntC<2>{}, safe_c);
+    if (it + 3 < ntiles) tile_step(it + 3, IntC<3>{}, safe_c);
+  }
+  };  // walk
+
+  if constexpr (kOptimistic) {
+    walk(BoolC<false>{});
+    // a sum that is not finite (or NaN) in any lane of the workgroup sends all of it through the exact walk:
+    // the tiles are a workgroup's common property.  The flag lives in the fragment-major region, which no direct
+    // load writes; loads of tiles past the last one may still be landing elsewhere.
+    const bool bad = !(lsum[0] < INFINITY) || !(lsum[1] < INFINITY);
+    int* const flag = reinterpret_cast<int*>(smem_raw + C_FRAG);
+    if (tid == 0) *flag = 0;
+    wg_sync();
+    if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0) *flag = 1;
+    wg_sync();
+    const int again = __builtin_amdgcn_readfirstlane(*flag);
+    if (again) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      wg_sync();
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        acc_pin(i, o[i]);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        mrow[j] = -INFINITY;
+        lsum[j] = 0.f;
+        mloc[j] = -INFINITY;
+      }
+      walk(BoolC<true>{});
+    }
+  } else {
+    walk(BoolC<true>{});
   }
 
   // ---- epilogue: normalise (softmax), cast, store: by rows through LDS (free by now) where the output allows

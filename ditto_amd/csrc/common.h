@@ -34,6 +34,7 @@ struct Elem;
 
 template <>
 struct Elem<f16> {
+  static constexpr bool is_bf16 = false;
   typedef f16x8 v8;
   typedef f16x4 v4;
   typedef f16x2 v2;
@@ -54,6 +55,7 @@ struct Elem<f16> {
 
 template <>
 struct Elem<bf16> {
+  static constexpr bool is_bf16 = true;
   typedef bf16x8 v8;
   typedef bf16x4 v4;
   typedef bf16x2 v2;

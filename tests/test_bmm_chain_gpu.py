@@ -24,6 +24,14 @@ REL_L2 = 1e-3
 # figure from the rounding floor); bound = that + 10 %.  bf16 cast / relu chains meet the stated 1e-3
 # against the checker that rounds where they round (measured: at most 1.1e-4).
 REL_L2_BF16_QUANT = 2.6e-3
+# the same chains with an fp32 output: only the probabilities are rounded to bf16, which costs 1.66e-3 on
+# N(0,1) data (tests/test_oracle.py::test_rounding_floor_of_the_16_bit_types); bound = that floor + 5 %, so a
+# kernel error of a few 1e-4 cannot hide under the allowance meant for the rounded output
+REL_L2_BF16_P_ONLY = 1.75e-3
+
+
+def bf16_softmax_bound(out_dtype):
+    return REL_L2_BF16_P_ONLY if out_dtype == "float32" else REL_L2_BF16_QUANT
 
 
 def variants(K, N, b_layout="LK"):
@@ -76,7 +84,7 @@ def test_softmax_chain_vs_oracle(oracle, shape, dtype, b_layout):
             if dtype == "bfloat16":
                 report("softmax bf16 %s %s variant %d out %s" % (shape, b_layout, variant, out_dtype), mx, rel)
             assert mx <= MAX_ABS, (variant, mx, rel)
-            assert rel <= (REL_L2 if dtype == "float16" else REL_L2_BF16_QUANT), (variant, mx, rel)
+            assert rel <= (REL_L2 if dtype == "float16" else bf16_softmax_bound(out_dtype)), (variant, out_dtype, mx, rel)
 
 
 CAST_SHAPES = [
@@ -205,7 +213,8 @@ def test_running_maximum_paths(oracle, variant, dtype):
     """What the lazily raised row maximum has to survive: every score far below zero from the first key on (the
     maximum starts negative), and keys sorted so that every tile of 64 brings a row maximum far above the last
     (a rescale per tile), with ragged M and L.  (The fp16 kernel that pre-scales A keeps scores relative to the
-    maximum; the others subtract it per score.)"""
+    maximum; the others subtract it per score; the bf16 kernel on the 16x16x32 MFMA takes no maximum per half
+    tile but lowers a row's scale when its sum has grown, and repeats the walk with maxima when a sum overflowed.)"""
     batch, M, N, K, L = 2, 200, 64, 64, 456
     rng = np.random.default_rng(5)
     A = rng.standard_normal((batch, M, K)).astype(np.float32)
@@ -222,13 +231,24 @@ def test_running_maximum_paths(oracle, variant, dtype):
     Bf = B.copy()
     Bf[:, 0, :] = np.linspace(20.0, -20.0, L)         # and the other way: later tiles far below the maximum
     cases["falling"] = Bf
+    # a jump of 120 in the exponent from one key to the next, and a short spike of 200 inside the first tile:
+    # more than an fp32 (or bf16) probability taken relative to the keys before can hold, so a kernel that
+    # watches the row sums instead of taking maxima has to notice and walk the keys again the exact way
+    Bs = B.copy()
+    Bs[:, 0, :] = -15.0
+    Bs[:, 0, 300:] = 15.0
+    cases["step up"] = Bs
+    Bp = B.copy()
+    Bp[:, 0, :] = -25.0
+    Bp[:, 0, 40:44] = 25.0
+    cases["spike in the first tile"] = Bp
     for name, Bx in cases.items():
         Ar, Bxr, Cr = (oracle.np_round_to(t, dtype) for t in (A, Bx, C))
         got = run_chain(Ar, Bxr, Cr, dtype, "softmax", 1.0, "LK", "float32", variant)
         want = oracle.bmm_chain_f64(Ar, Bxr, Cr, inter="softmax", scale=1.0)
         mx, rel = errors(got, want)
         assert np.isfinite(got).all(), name
-        assert mx <= MAX_ABS and rel <= (REL_L2_BF16_QUANT if dtype == "bfloat16" else REL_L2), (name, mx, rel)
+        assert mx <= MAX_ABS and rel <= (REL_L2_BF16_P_ONLY if dtype == "bfloat16" else REL_L2), (name, mx, rel)
 
 
 def test_reference_semantics_on_reference_inputs(oracle):
