@@ -23,8 +23,9 @@ from ... import _lib, chain
 from ...hardware import query_hw_param
 
 # kernel codes of the fp16/bf16 chain: four waves x 32 | 64 rows, eight waves x 32 rows (staggered phases,
-# software pipelined, on the 16x16x32 MFMA: the library refuses that one unless B is stored [L][K])
-FP_VARIANT_CODES = (1, 2, 8, 9, 6)
+# software pipelined, on the 16x16x32 MFMA with 256-row workgroups, the same with 384-row workgroups for the
+# first row blocks: the library refuses the last two unless B is stored [L][K])
+FP_VARIANT_CODES = (1, 2, 8, 9, 6, 7)
 
 
 class TuneEntry:

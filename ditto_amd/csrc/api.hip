@@ -4,6 +4,9 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <vector>
+
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -58,8 +61,47 @@ int device_cus() {
 struct BmmPlan {
   int family;  // 0: fp16/bf16 register-resident chain, 1: fp32 chain, 2: int8 requant chain
   int d_pad, qt;  // fp chains: head pad and rows-per-wave code; int8 chain: row tiles and ring depth
+  int nb3 = 0, nb = 0;  // 16x16x32-MFMA kernel: row blocks of 384 rows / row blocks in all, per batch entry
   ditto_tile_param tile;
 };
+
+// Row blocks of 384 and of 256 rows for the kernel on the 16x16x32 MFMA.  A 384-row workgroup does half as much
+// work again as a 256-row one in about kBig3 of its time, but 384 seldom divides the rows evenly over the compute
+// units: every split (a blocks of 384, then blocks of 256 for the rest) is priced by dealing its workgroups out the
+// way the hardware does (an XCD takes the large blocks of all of its batch entries first, then the small ones, each
+// to the compute unit that is free first) and the shortest finish wins.  Returns a.
+constexpr double kBig3 = 1.43;
+int plan_rows_384(long long M, long long batch, int cus) {
+  thread_local long long last_m = -1, last_batch = -1;
+  thread_local int last_cus = -1, last_a = 0;
+  if (M == last_m && batch == last_batch && cus == last_cus) return last_a;
+  const long long amax = M / 384 + (M % 384 > 256 ? 1 : 0);
+  const bool split = batch % 8 == 0 && cus % 8 == 0;
+  const long long per = split ? batch / 8 : batch;
+  const int cu = split ? cus / 8 : cus;
+  int best_a = 0;
+  if (amax > 0 && per * (M / 256 + 2) > 4096) {
+    best_a = (int)(M / 384);  // so many workgroups that the finish does not matter
+  } else if (amax > 0) {
+    double best = 0;
+    std::vector<double> free_at(cu);
+    for (long long a = 0; a <= amax; ++a) {
+      if (a > 0 && a < amax - 16) continue;  // the finish is tuned by the last few blocks
+      const long long rest = M - 384 * a;
+      const long long b = rest > 0 ? (rest + 255) / 256 : 0;
+      std::fill(free_at.begin(), free_at.end(), 0.0);
+      auto deal = [&](long long n, double cost) {
+        for (long long i = 0; i < n; ++i) *std::min_element(free_at.begin(), free_at.end()) += cost;
+      };
+      deal(per * a, kBig3);
+      deal(per * b, 1.0);
+      const double finish = *std::max_element(free_at.begin(), free_at.end());
+      if (a == 0 || finish < best - 1e-9) best = finish, best_a = (int)a;
+    }
+  }
+  last_m = M, last_batch = batch, last_cus = cus, last_a = best_a;
+  return best_a;
+}
 
 int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
   if (!d) return fail(DITTO_EINVAL, "null descriptor");
@@ -152,15 +194,24 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     }
     if (d->tile_variant != 0) {
       const int q = d->tile_variant % 10;
-      if (d->tile_variant / 10 != plan->d_pad || (q != 1 && q != 2 && q != 8 && q != 9 && q != 6))
-        return fail(DITTO_EINVAL, "tile_variant %d cannot run this shape (head_pad %d; q must be 1, 2, 6, 8 or 9)",
+      if (d->tile_variant / 10 != plan->d_pad || (q != 1 && q != 2 && q != 8 && q != 9 && q != 6 && q != 7))
+        return fail(DITTO_EINVAL, "tile_variant %d cannot run this shape (head_pad %d; q must be 1, 2, 6, 7, 8 or 9)",
                     d->tile_variant, plan->d_pad);
-      if (q == 6 && d->b_layout != DITTO_B_LK)
+      if ((q == 6 || q == 7) && d->b_layout != DITTO_B_LK)
         return fail(DITTO_EINVAL, "tile_variant %d (16x16x32 MFMA kernel) takes B stored [L][K]", d->tile_variant);
       plan->qt = q;
     }
     const bool kl = d->b_layout == DITTO_B_KL;
-    const bool eight = plan->qt >= 6;  // 6, 8, 9: eight waves owning 32 rows each
+    const bool eight = plan->qt >= 6;  // 6, 8, 9: eight waves owning 32 rows each; 7: 48 rows each in some workgroups
+    const bool m16 = plan->qt == 6 || plan->qt == 7;
+    if (plan->qt == 6 && d->tile_variant == 0 && plan->d_pad == 128) {
+      // the planner's own choice between all-256-row blocks (6) and the mix (7)
+      if (plan_rows_384(d->M, d->batch, cus) > 0) plan->qt = 7;
+    }
+    if (plan->qt == 7) {
+      plan->nb3 = plan_rows_384(d->M, d->batch, cus);
+      if (plan->nb3 == 0 && d->M > 256) plan->nb3 = 1;  // asked for by tile_variant: at least one large block to show for it
+    }
     const int bm = eight ? 256 : 128 * plan->qt;
     ditto_tile_param& t = plan->tile;
     t.block_threads = eight ? 512 : 256;
@@ -168,14 +219,20 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     t.block_l = ditto::kBN;
     t.block_n = (int)d->N;
     t.head_pad = plan->d_pad;
-    if (plan->qt == 6)
+    if (m16)
       t.lds_bytes = plan->d_pad == 64 ? ditto::bmm_chain8m16_lds_bytes<64>() : ditto::bmm_chain8m16_lds_bytes<128>();
     else if (eight)
       t.lds_bytes = plan->d_pad == 64 ? (kl ? ditto::bmm_chain8_lds_bytes<64, true>() : ditto::bmm_chain8_lds_bytes<64, false>())
                                       : (kl ? ditto::bmm_chain8_lds_bytes<128, true>() : ditto::bmm_chain8_lds_bytes<128, false>());
     else
       t.lds_bytes = plan->d_pad == 64 ? ditto::bmm_chain_lds_bytes<64>() : ditto::bmm_chain_lds_bytes<128>();
-    t.grid_x = (int)(((d->M + bm - 1) / bm) * d->batch);
+    plan->nb = (int)((d->M + bm - 1) / bm);
+    if (plan->qt == 7) {
+      const long long rest = d->M - 384LL * plan->nb3;
+      plan->nb = plan->nb3 + (int)(rest > 0 ? (rest + 255) / 256 : 0);
+      if (plan->nb3 > 0) t.block_m = 384;  // the larger of the two block sizes
+    }
+    t.grid_x = (int)(plan->nb * d->batch);
     t.grid_y = t.grid_z = 1;
     t.variant = plan->d_pad * 10 + plan->qt;
     return DITTO_OK;
@@ -909,7 +966,8 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     args.K = (int)d->K;
     args.L = (int)d->L;
     args.batch = (int)d->batch;
-    args.mblocks = (int)((d->M + plan.tile.block_m - 1) / plan.tile.block_m);
+    args.mblocks = plan.nb;
+    args.mblocks3 = plan.nb3;
     args.scale_log2 = d->softmax_scale * 1.4426950408889634f;
     args.relu = d->inter_op == DITTO_INTER_RELU;
     args.relu_out = d->relu_out;

@@ -40,6 +40,7 @@ struct BmmChainArgs {
   int a_rs, b_rs, c_rs, f_rs;        // row strides, elements
   int M, N, K, L, batch;
   int mblocks;       // workgroups per batch entry
+  int mblocks3;      // 16x16x32-MFMA kernel: how many of them, the first ones, have 384 rows (the others 256)
   float scale_log2;  // softmax: scale * log2(e)
   int relu;          // inter = relu instead of cast (non-softmax kernels)
   int relu_out;      // ReLU on the second accumulator before the final cast (non-softmax kernels)

@@ -32,20 +32,12 @@
 #pragma once
 #include "bmm_chain_fp8.h"
 
-#ifndef DITTO_M16_PHASES
-#define DITTO_M16_PHASES 1
-#endif
-
 namespace ditto {
 
 template <int D>
 __host__ __device__ constexpr int bmm_chain8m16_lds_bytes() {
   // B tiles as loaded [4], raw C tiles [2 or 4], fragment-major C tiles [2]
-#ifdef DITTO_M16_NCR4
-  return (4 + 4 + 2) * kBN * D * 2;
-#else
   return (4 + (D == 64 ? 4 : 2) + 2) * kBN * D * 2;
-#endif
 }
 
 template <typename V8>
@@ -100,14 +92,23 @@ __device__ __forceinline__ void acc_pin(int i, f32x4& x) {
     case 13: asm volatile("" : "+{v[52:55]}"(x)); break;
     case 14: asm volatile("" : "+{v[56:59]}"(x)); break;
     case 15: asm volatile("" : "+{v[60:63]}"(x)); break;
+    case 16: asm volatile("" : "+{v[64:67]}"(x)); break;
+    case 17: asm volatile("" : "+{v[68:71]}"(x)); break;
+    case 18: asm volatile("" : "+{v[72:75]}"(x)); break;
+    case 19: asm volatile("" : "+{v[76:79]}"(x)); break;
+    case 20: asm volatile("" : "+{v[80:83]}"(x)); break;
+    case 21: asm volatile("" : "+{v[84:87]}"(x)); break;
+    case 22: asm volatile("" : "+{v[88:91]}"(x)); break;
+    case 23: asm volatile("" : "+{v[92:95]}"(x)); break;
   }
 }
+constexpr int kMaxAcc = 24;
 template <typename V8>
-__device__ __forceinline__ void acc_mfma(int i, V8 a, V8 b, f32x4 (&o)[16]) {
+__device__ __forceinline__ void acc_mfma(int i, V8 a, V8 b, f32x4 (&o)[kMaxAcc]) {
   o[i] = Mfma16<typename ElemOf<V8>::type>::run(a, b, o[i]);
   acc_pin(i, o[i]);
 }
-__device__ __forceinline__ void acc_scale(int i, float alpha, f32x4 (&o)[16]) {
+__device__ __forceinline__ void acc_scale(int i, float alpha, f32x4 (&o)[kMaxAcc]) {
   o[i] *= alpha;
   acc_pin(i, o[i]);
 }
@@ -133,13 +134,13 @@ struct BoolC {
 // a lane's partial row sum above which the optimistic walk lowers the row's scale (2^32)
 constexpr float kSumLimit = 4294967296.f;
 
-template <typename T, int D, int INTER>
-__global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
-#if defined(__HIP_DEVICE_COMPILE__)
+// One workgroup's walk: eight waves of RT 16-row tiles each, rows row0 .. row0 + 128 RT - 1 of batch entry bz.
+template <typename T, int D, int INTER, int RT>
+__device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* smem_raw, int row0, int bz) {
   typedef typename Elem<T>::v8 V8;
   typedef typename Elem<T>::v4 V4;
   typedef typename Elem<T>::v2 V2;
-  constexpr int NW = 8, BM = NW * 32;
+  constexpr int NW = 8;
 #ifdef DITTO_M16_NO_OPTIMISTIC
   constexpr bool kOptimistic = false;
 #else
@@ -157,18 +158,13 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   constexpr int NLD = TB / 1024 / NW; // direct loads per wave per tile
   constexpr int NTR = NFRAG / NW;     // fragments each wave transposes per tile
   static_assert(NLD >= 1 && NTR >= 1, "tile too small for eight waves");
-#ifdef DITTO_M16_NCR4
-  constexpr int NCR = 4;
-#else
   constexpr int NCR = D == 64 ? 4 : 2;
-#endif
   constexpr int B_LOAD = 0;                   // [4] row-read layout
   constexpr int C_RAW = 4 * TB;               // [NCR]
   constexpr int C_FRAG = C_RAW + NCR * TB;    // [2]
   constexpr int B_AHEAD = 3;
   constexpr int C_AHEAD = NCR == 4 ? 3 : 2;
 
-  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c16 = lane & 15, q = lane >> 4;
@@ -183,14 +179,11 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   // without the read; 32 is the matrix pipe's own time): about four register writes per MFMA pair are free,
   // each further one costs four cycles.  This kernel has the read and about 5.6 vector results per pair.
 
-  const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
-  const int mb = lid % p.mblocks;
-  const int bz = lid / p.mblocks;
   const int zo = bz / p.batch_inner, zi = bz - zo * p.batch_inner;
   const T* __restrict__ Ag = reinterpret_cast<const T*>(p.a) + zo * p.a_bs2 + zi * p.a_bs;
   const T* Bg = reinterpret_cast<const T*>(p.b) + zo * p.b_bs2 + zi * p.b_bs;
   const T* Cg = reinterpret_cast<const T*>(p.c) + zo * p.c_bs2 + zi * p.c_bs;
-  const int m_wave = mb * BM + wave * 32;
+  const int m_wave = row0 + wave * 16 * RT;
   const int M = p.M, N = p.N, K = p.K, L = p.L;
 
   const unsigned b_bytes = (unsigned)((long long)(L - 1) * p.b_rs + K) * 2u;
@@ -283,9 +276,9 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   };
 
   // ---- A fragments (B operand of the first contraction): lane holds A[16 j + c][32 st + 8 q .. + 7]
-  V8 af[2][NS];
+  V8 af[RT][NS];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < RT; ++j) {
     const int row = m_wave + 16 * j + c16;
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
@@ -297,21 +290,27 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   }
 
   // ---- accumulators of F^T: o[t][j][r] = F^T[16 t + 4 q + r][16 j + c]
-  // (flat: accumulator 2 t + j, pinned to v[4 (2 t + j) : +3], see acc_mfma)
-  static_assert(2 * NTN <= 16, "sixteen pinned accumulators");
-  f32x4 o[16];
+  // (flat: accumulator RT t + j, pinned to v[4 (RT t + j) : +3], see acc_mfma)
+  static_assert(RT * NTN <= kMaxAcc, "pinned accumulators");
+  f32x4 o[kMaxAcc];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < RT * NTN; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   // softmax state of the lane's two rows: running maximum (exp2 domain; the same in the four lanes of a
   // row), the lane's share of the row sum, and the lane's LOCAL scaled maximum of the half about to be consumed
-  float mrow[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f}, mloc[2] = {-INFINITY, -INFINITY};
+  float mrow[RT], lsum[RT], mloc[RT];
+#pragma unroll
+  for (int j = 0; j < RT; ++j) {
+    mrow[j] = -INFINITY;
+    lsum[j] = 0.f;
+    mloc[j] = -INFINITY;
+  }
   const float c2 = p.scale_log2;
   const int ntiles = (L + kBN - 1) / kBN;
   const bool ragged = (L % kBN) != 0;
 
   // A half tile of scores: sc[i][j] = 16-row tile i x row tile j
   struct Half {
-    f32x4 v[2][2];
+    f32x4 v[2][RT];
   };
   Half sa, sb;
   auto mask_tail = [&](Half& h, int l0) __attribute__((always_inline)) {
@@ -321,13 +320,13 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
         if (16 * i + r >= rem) {
-          h.v[i][0][r] = -INFINITY;
-          h.v[i][1][r] = -INFINITY;
+#pragma unroll
+          for (int j = 0; j < RT; ++j) h.v[i][j][r] = -INFINITY;
         }
   };
   auto local_max = [&](const Half& h) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < RT; ++j) {
       float mx = h.v[0][j][0];
 #pragma unroll
       for (int r = 1; r < 4; ++r) mx = fmaxf(mx, h.v[0][j][r]);
@@ -336,10 +335,9 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
       mloc[j] = mx * c2;
     }
   };
-  // probabilities of 16-row tile i (both rows): two registers' worth at a time would be finer, but four
-  // per call keeps the bookkeeping simple: unit u = 0..3 is (i = u / 2, j = u % 2)
+  // probabilities of 16-row tile i of the half, row tile j: unit u = 0 .. 2 RT - 1 is (i = u / RT, j = u % RT)
   auto exp_unit = [&](Half& h, int u) __attribute__((always_inline)) {
-    const int i = u >> 1, j = u & 1;
+    const int i = u / RT, j = u % RT;
 #pragma unroll
     for (int r = 0; r < 4; ++r) h.v[i][j][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(h.v[i][j][r], c2, -mrow[j]));
     // keep the unit where it is called, between the MFMAs of its group: statements with side effects keep
@@ -368,16 +366,18 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   // row's running maximum by more than 2^kLazy.  Only then are the row maxima exchanged (all rows of the
   // wave: a raised maximum must be the same in the four lanes of its row) and the accumulators rescaled.
   auto maybe_rescale = [&]() __attribute__((always_inline)) {
-    const bool vote = mloc[0] > mrow[0] + kLazy || mloc[1] > mrow[1] + kLazy;
+    bool vote = false;
+#pragma unroll
+    for (int j = 0; j < RT; ++j) vote = vote || mloc[j] > mrow[j] + kLazy;
     if (__builtin_amdgcn_ballot_w64(vote) != 0) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < RT; ++j) {
         const float mnew = fmaxf(mrow[j], quad_max(mloc[j]));
         const float alpha = __builtin_amdgcn_exp2f(mrow[j] - mnew);  // (-inf) - (-inf) does not occur: mnew is finite
         mrow[j] = mnew;
         lsum[j] *= alpha;
 #pragma unroll
-        for (int t = 0; t < NTN; ++t) acc_scale(2 * t + j, alpha, o);
+        for (int t = 0; t < NTN; ++t) acc_scale(RT * t + j, alpha, o);
       }
     }
   };
@@ -391,10 +391,12 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   // infinite or NaN, which the end of the walk detects, and the workgroup then walks the keys again the exact way
   // (maximum per half tile before any exponential).
   auto sum_rescale = [&]() __attribute__((always_inline)) {
-    const bool vote = fmaxf(lsum[0], lsum[1]) > kSumLimit;
-    if (__builtin_amdgcn_ballot_w64(vote) != 0) {
+    float smax = lsum[0];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+    for (int j = 1; j < RT; ++j) smax = fmaxf(smax, lsum[j]);
+    if (__builtin_amdgcn_ballot_w64(smax > kSumLimit) != 0) {
+#pragma unroll
+      for (int j = 0; j < RT; ++j) {
         const float sref = quad_max(lsum[j]);  // the same in the four lanes of a row
         // (an infinite or NaN sum is left as it is: that is what the end of the walk looks for)
         const int e = (sref > kSumLimit && sref < INFINITY) ? ((__builtin_bit_cast(int, sref) >> 23) & 255) - 127 : 0;
@@ -402,20 +404,20 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
         mrow[j] += (float)e;
         lsum[j] *= alpha;
 #pragma unroll
-        for (int t = 0; t < NTN; ++t) acc_scale(2 * t + j, alpha, o);
+        for (int t = 0; t < NTN; ++t) acc_scale(RT * t + j, alpha, o);
       }
     }
   };
   // reference exponent of a fresh row: the maximum of its first half tile (finite: key 0 exists and is not masked)
   auto init_max = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) mrow[j] = quad_max(mloc[j]);
+    for (int j = 0; j < RT; ++j) mrow[j] = quad_max(mloc[j]);
   };
 
   // One half step: consumes `cur` (half hh of tile it), produces `nxt` (the following half).  Fragment
   // groups: 2 NS of the first contraction (16-row tile i of the next half x k step), then NTN of the second
   // (column tile t); each fragment feeds the two row tiles.
-  constexpr int kAhead = 3;
+  constexpr int kAhead = RT == 3 ? 2 : 3;  // fragments in flight ahead of the MFMAs (three were no faster at RT = 3)
   constexpr int NGS = 2 * NS, NG = NGS + NTN;
   auto half_step = [&](Half& cur, Half& nxt, int it, auto j_c, auto hh_c, auto safe_c) __attribute__((always_inline)) {
     constexpr int J = decltype(j_c)::value, hh = decltype(hh_c)::value;
@@ -430,58 +432,34 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
     };
 #pragma unroll
     for (int k = 0; k < kAhead; ++k) fetch(k);
-    V8 pf[2];
-#if DITTO_M16_PHASES
+    V8 pf[RT];
     // vector phase first, all of it, then the MFMAs of both contractions back to back
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (INTER == kInterSoftmax) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) exp_unit(cur, u);
+      for (int u = 0; u < 2 * RT; ++u) exp_unit(cur, u);
     }
-    make_p(cur, 0, pf[0]);
-    make_p(cur, 1, pf[1]);
-    asm volatile("" : "+v"(pf[0]), "+v"(pf[1]));
+#pragma unroll
+    for (int j = 0; j < RT; ++j) {
+      make_p(cur, j, pf[j]);
+      asm volatile("" : "+v"(pf[j]));
+    }
     __builtin_amdgcn_sched_barrier(0);
-#endif
 #pragma unroll
     for (int k = 0; k < NG; ++k) {
       if (k + kAhead < NG) fetch(k + kAhead);
       __builtin_amdgcn_sched_barrier(0);
-#ifdef DITTO_M16_SPREAD
-      // the step's direct loads go out among the MFMAs, C in the first half step and B in the second (the waits
-      // count them in that order), not all at once behind the barrier where the whole workgroup's loads queue up
-      if (k == DITTO_M16_SPREAD) {
-        if (hh == 0) load_c(it + C_AHEAD, NCR == 4 ? (J + 3) % 4 : (J & 1));
-        else load_b(it + B_AHEAD, (J + 3) % 4);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-#endif
       if (k < NGS) {
         const int i = k & 1, st = k >> 1;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < RT; ++j) {
           if (st == 0) nxt.v[i][j] = Mfma16<T>::run(fr[k], af[j][st], f32x4{0.f, 0.f, 0.f, 0.f});
           else nxt.v[i][j] = Mfma16<T>::run(fr[k], af[j][st], nxt.v[i][j]);
         }
-        // the four exponential units of `cur` are spread over the first contraction's groups
-#if !DITTO_M16_PHASES
-        if constexpr (INTER == kInterSoftmax) {
-          if (NGS >= 4) {
-            if (k % (NGS / 4) == 0 && k / (NGS / 4) < 4) exp_unit(cur, k / (NGS / 4));
-          } else {  // two groups only (K = 32): two units behind each
-            exp_unit(cur, 2 * k);
-            exp_unit(cur, 2 * k + 1);
-          }
-        }
-        if (k == NGS - 1) {
-          make_p(cur, 0, pf[0]);
-          make_p(cur, 1, pf[1]);
-        }
-#endif
       } else {
         const int t = k - NGS;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc_mfma(2 * t + j, fr[k], pf[j], o);
+        for (int j = 0; j < RT; ++j) acc_mfma(RT * t + j, fr[k], pf[j], o);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -497,24 +475,16 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
     constexpr int PAR = J & 1;
     V8 xc[NTR];
     // C first: the wait at the end of the step can then leave the (younger) B loads in flight
-#ifndef DITTO_M16_SPREAD
     load_c(it + C_AHEAD, NCR == 4 ? (J + 3) % 4 : PAR);
     load_b(it + B_AHEAD, (J + 3) % 4);
-#endif
-#ifndef DITTO_ABL_NOTR
     tr_read_c(C_RAW + (NCR == 4 ? (J + 1) % 4 : (PAR ^ 1)) * TB, xc);
-#endif
     half_step(sa, sb, it, j_c, IntC<0>{}, safe_c);
-#ifndef DITTO_ABL_NOTR
     tr_write(C_FRAG + (PAR ^ 1) * TB, xc);
-#endif
     half_step(sb, sa, it, j_c, IntC<1>{}, safe_c);
     if constexpr (INTER == kInterSoftmax && !SAFE) sum_rescale();
-#ifndef DITTO_ABL_NOBAR
     if (NCR == 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLD) : "memory");
     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
     __syncthreads();
-#endif
   };
 
   // ---- one walk over the keys: prologue (first tiles in flight, first transposition, scores of the very first
@@ -540,7 +510,7 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
     for (int i = 0; i < 2; ++i) {
       const V8 bf = b_frag(B_LOAD, i, st);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < RT; ++j) {
         if (st == 0) sa.v[i][j] = Mfma16<T>::run(bf, af[j][st], f32x4{0.f, 0.f, 0.f, 0.f});
         else sa.v[i][j] = Mfma16<T>::run(bf, af[j][st], sa.v[i][j]);
       }
@@ -565,7 +535,9 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
     // a sum that is not finite (or NaN) in any lane of the workgroup sends all of it through the exact walk:
     // the tiles are a workgroup's common property.  The flag lives in the fragment-major region, which no direct
     // load writes; loads of tiles past the last one may still be landing elsewhere.
-    const bool bad = !(lsum[0] < INFINITY) || !(lsum[1] < INFINITY);
+    bool bad = false;
+#pragma unroll
+    for (int j = 0; j < RT; ++j) bad = bad || !(lsum[j] < INFINITY);
     int* const flag = reinterpret_cast<int*>(smem_raw + C_FRAG);
     if (tid == 0) *flag = 0;
     wg_sync();
@@ -576,12 +548,12 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       wg_sync();
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
+      for (int i = 0; i < RT * NTN; ++i) {
         o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
         acc_pin(i, o[i]);
       }
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < RT; ++j) {
         mrow[j] = -INFINITY;
         lsum[j] = 0.f;
         mloc[j] = -INFINITY;
@@ -597,25 +569,30 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   const bool by_rows = !p.out_f32 && (N & 7) == 0 && (p.f_rs & 7) == 0 && (p.f_bs & 7) == 0 && (p.f_bs2 & 7) == 0 &&
                        (reinterpret_cast<size_t>(p.f) & 15) == 0;  // wave-uniform
   constexpr int kRowBytes = tile_row_bytes<D>();
-  static_assert(8 * (32) * tile_row_bytes<D>() <= bmm_chain8m16_lds_bytes<D>(), "the parked rows need the staged tiles' LDS");
+  static_assert(8 * (16 * RT) * tile_row_bytes<D>() <= bmm_chain8m16_lds_bytes<D>(), "the parked rows need the staged tiles' LDS");
   if (by_rows) {
     // every wave is done with the staged tiles, and the direct loads still in flight (the tiles past the last one:
     // zeros) have landed -- they would otherwise fall on the rows parked below
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     wg_sync();
   }
-  char* const tw = smem_raw + wave * 32 * kRowBytes;
+  char* const tw = smem_raw + wave * 16 * RT * kRowBytes;
+  // lane coordinates taken afresh: values kept from the prologue for this would sit in registers (or spill)
+  // through the whole walk
+  int lane_e = threadIdx.x & 63;
+  asm volatile("" : "+v"(lane_e));
+  const int c16e = lane_e & 15, qe = lane_e >> 4;
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < RT; ++j) {
     float inv = 1.f;
     if constexpr (INTER == kInterSoftmax) inv = 1.f / quad_sum(lsum[j]);
-    const int row = m_wave + 16 * j + c16;
+    const int row = m_wave + 16 * j + c16e;
     if (!by_rows && row >= M) continue;
 #pragma unroll
     for (int t = 0; t < NTN; ++t) {
-      const int n = 16 * t + 4 * q;
+      const int n = 16 * t + 4 * qe;
       if (!by_rows && n >= N) continue;
-      float v0 = o[2 * t + j][0] * inv, v1 = o[2 * t + j][1] * inv, v2 = o[2 * t + j][2] * inv, v3 = o[2 * t + j][3] * inv;
+      float v0 = o[RT * t + j][0] * inv, v1 = o[RT * t + j][1] * inv, v2 = o[RT * t + j][2] * inv, v3 = o[RT * t + j][3] * inv;
       if (INTER != kInterSoftmax && p.relu_out) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); v2 = fmaxf(v2, 0.f); v3 = fmaxf(v3, 0.f); }
       const long long off = zo * p.f_bs2 + zi * p.f_bs + (long long)row * p.f_rs + n;
       if (p.out_f32) {
@@ -624,14 +601,41 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
       } else {
         V2 a0 = cvt2<T>(v0, v1), a1 = cvt2<T>(v2, v3);
         V4 w = {a0[0], a0[1], a1[0], a1[1]};
-        if (by_rows) *reinterpret_cast<V4*>(tw + (16 * j + c16) * kRowBytes + n * 2) = w;
+        if (by_rows) *reinterpret_cast<V4*>(tw + (16 * j + c16e) * kRowBytes + n * 2) = w;
         else *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.f) + off) = w;
       }
     }
   }
   if (by_rows)
-    store_tile_rows<T, D, 32>(tw, reinterpret_cast<T*>(p.f) + zo * p.f_bs2 + zi * p.f_bs + (long long)m_wave * p.f_rs, p.f_rs,
-                              M - m_wave, N, lane);
+    store_tile_rows<T, D, 16 * RT>(tw, reinterpret_cast<T*>(p.f) + zo * p.f_bs2 + zi * p.f_bs + (long long)m_wave * p.f_rs, p.f_rs,
+                              M - m_wave, N, lane_e);
+}
+
+// Workgroups come in two sizes: the first p.mblocks3 row blocks of a batch entry have 384 rows (three 16-row tiles
+// per wave: an operand fragment read from LDS feeds three MFMAs, and the per-tile overheads - direct loads,
+// transposition, barrier - are spread over half as many MFMAs again), the others 256.  The split lets a row count
+// that 384 does not divide fill the device evenly: 4096 rows on four compute units are 2 x 384 + 256 each.  Ids are
+// dealt so that every XCD first gets the large blocks of all of its batch entries, then the small ones (longest
+// first: the small blocks fill the gaps at the end).
+template <typename T, int D, int INTER>
+__global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  const int nb3 = p.mblocks3, nb2 = p.mblocks - p.mblocks3;
+  int x = 0, idx = blockIdx.x, per = p.batch;  // XCD, position in the XCD's dispatch order, batch entries per XCD
+  if (gridDim.x % 8 == 0 && p.batch % 8 == 0) {
+    x = blockIdx.x & 7;
+    idx = blockIdx.x >> 3;
+    per = p.batch >> 3;
+  }
+  if (idx < per * nb3) {
+    const int e = idx / nb3, mb = idx - e * nb3;
+    bmm_chain8m16_body<T, D, INTER, 3>(p, smem_raw, 384 * mb, x * per + e);
+  } else {
+    const int r = idx - per * nb3;
+    const int e = r / nb2, mb = r - e * nb2;
+    bmm_chain8m16_body<T, D, INTER, 2>(p, smem_raw, 384 * nb3 + 256 * mb, x * per + e);
+  }
 #else
   (void)p;
 #endif

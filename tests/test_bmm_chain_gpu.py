@@ -37,9 +37,10 @@ def bf16_softmax_bound(out_dtype):
 def variants(K, N, b_layout="LK"):
     """0 (the library's own choice) and every kernel variant that can run the head size:
     four waves x 32 rows, four waves x 64 rows, eight waves x 32 rows (staggered phases; software
-    pipelined; on the 16x16x32 MFMA, which takes B stored [L][K] only)."""
+    pipelined; on the 16x16x32 MFMA, which takes B stored [L][K] only, with 256-row workgroups and with
+    384-row ones for the first row blocks)."""
     pad = 64 if max(K, N) <= 64 else 128
-    return [0] + [pad * 10 + q for q in ((1, 2, 8, 9, 6) if b_layout == "LK" else (1, 2, 8, 9))]
+    return [0] + [pad * 10 + q for q in ((1, 2, 8, 9, 6, 7) if b_layout == "LK" else (1, 2, 8, 9))]
 
 
 def run_chain(A, B, C, dtype, inter, scale=1.0, b_layout="KL", out_dtype=None, variant=0):
@@ -207,7 +208,7 @@ def test_softmax_invariants_on_gpu(oracle, variant):
     assert np.isfinite(hot).all() and errors(hot, want)[0] <= MAX_ABS
 
 
-@pytest.mark.parametrize("variant", [0, 641, 642, 648, 649, 646])
+@pytest.mark.parametrize("variant", [0, 641, 642, 648, 649, 646, 647])
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
 def test_running_maximum_paths(oracle, variant, dtype):
     """What the lazily raised row maximum has to survive: every score far below zero from the first key on (the
@@ -296,7 +297,7 @@ MAX_ABS_BF16_LONG, REL_L2_BF16_LONG = 1.0e-3, 2.6e-3
 MAX_ABS_FP16_LONG, REL_L2_FP16_LONG = 1.4e-4, 3.25e-4
 
 
-@pytest.mark.parametrize("variant", [0, 1282, 1288, 1289, 1286])
+@pytest.mark.parametrize("variant", [0, 1282, 1288, 1289, 1286, 1287])
 def test_attention_full_size_fp16_long_sequence(oracle, variant):
     # the long-sequence shape in fp16, where the stated bar (1e-2 / 1e-3) is reachable: 64 online-softmax
     # steps per row, every variant; three whole heads and a row block of every head against the closed form
@@ -339,7 +340,7 @@ def test_attention_full_size_fp16_long_sequence(oracle, variant):
     assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
 
 
-@pytest.mark.parametrize("variant", [0, 1282, 1288, 1289, 1286])
+@pytest.mark.parametrize("variant", [0, 1282, 1288, 1289, 1286, 1287])
 def test_attention_full_size_bf16_long_sequence(oracle, variant):
     # the bf16 configuration at its full size (64 heads of 4096 x 128).  The CPU closed form over
     # all of it would take minutes, so: every row of three heads chosen across the batch, one
