@@ -36,8 +36,8 @@ namespace ditto {
 
 template <int D>
 __host__ __device__ constexpr int bmm_chain8m16_lds_bytes() {
-  // B tiles as loaded [4], raw C tiles [2 or 4], fragment-major C tiles [2]
-  return (4 + (D == 64 ? 4 : 2) + 2) * kBN * D * 2;
+  // B tiles as loaded [4], raw C tiles [4], fragment-major C tiles [2]
+  return (4 + 4 + 2) * kBN * D * 2;
 }
 
 template <typename V8>
@@ -158,12 +158,10 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
   constexpr int NLD = TB / 1024 / NW; // direct loads per wave per tile
   constexpr int NTR = NFRAG / NW;     // fragments each wave transposes per tile
   static_assert(NLD >= 1 && NTR >= 1, "tile too small for eight waves");
-  constexpr int NCR = D == 64 ? 4 : 2;
+  constexpr int NCR = 4;
   constexpr int B_LOAD = 0;                   // [4] row-read layout
   constexpr int C_RAW = 4 * TB;               // [NCR]
   constexpr int C_FRAG = C_RAW + NCR * TB;    // [2]
-  constexpr int B_AHEAD = 3;
-  constexpr int C_AHEAD = NCR == 4 ? 3 : 2;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -434,6 +432,7 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
     for (int k = 0; k < kAhead; ++k) fetch(k);
     V8 pf[RT];
     // vector phase first, all of it, then the MFMAs of both contractions back to back
+    auto vphase = [&]() __attribute__((always_inline)) {
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (INTER == kInterSoftmax) {
 #pragma unroll
@@ -445,6 +444,8 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
       asm volatile("" : "+v"(pf[j]));
     }
     __builtin_amdgcn_sched_barrier(0);
+    };
+    vphase();
 #pragma unroll
     for (int k = 0; k < NG; ++k) {
       if (k + kAhead < NG) fetch(k + kAhead);
@@ -474,16 +475,20 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
     constexpr bool SAFE = decltype(safe_c)::value;
     constexpr int PAR = J & 1;
     V8 xc[NTR];
-    // C first: the wait at the end of the step can then leave the (younger) B loads in flight
-    load_c(it + C_AHEAD, NCR == 4 ? (J + 3) % 4 : PAR);
-    load_b(it + B_AHEAD, (J + 3) % 4);
-    tr_read_c(C_RAW + (NCR == 4 ? (J + 1) % 4 : (PAR ^ 1)) * TB, xc);
+    tr_read_c(C_RAW + ((J + 1) % 4) * TB, xc);
     half_step(sa, sb, it, j_c, IntC<0>{}, safe_c);
     tr_write(C_FRAG + (PAR ^ 1) * TB, xc);
     half_step(sb, sa, it, j_c, IntC<1>{}, safe_c);
     if constexpr (INTER == kInterSoftmax && !SAFE) sum_rescale();
-    if (NCR == 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLD) : "memory");
-    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLD) : "memory");
+    // The direct loads of tile it + 3 go out here, at the END of the step, into the slot of tile it - 1 (last read
+    // before the previous barrier): a wave whose loads queue up behind the workgroup's others then waits where it
+    // would wait for the barrier anyway, and the waves reach this point at different times.  Issued behind the
+    // barrier, all at once, the same loads held every wave up at the start of its step (2 % of the launch).
+    // What must have landed before the barrier is tile it + 2 (transposed from the next step's first instruction
+    // on); the 2 NLD loads just issued may stay in flight.
+    load_c(it + 3, (J + 3) % 4);
+    load_b(it + 3, (J + 3) % 4);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLD) : "memory");
     __syncthreads();
   };
 
@@ -496,7 +501,7 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
   load_c(0, 0);
   load_c(1, 1);
   load_b(2, 2);
-  if (NCR == 4) load_c(2, 2);
+  load_c(2, 2);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   {
@@ -538,7 +543,9 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
     bool bad = false;
 #pragma unroll
     for (int j = 0; j < RT; ++j) bad = bad || !(lsum[j] < INFINITY);
-    int* const flag = reinterpret_cast<int*>(smem_raw + C_FRAG);
+    int* const flag = reinterpret_cast<int*>(smem_raw);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no direct load still on its way into LDS
+    wg_sync();
     if (tid == 0) *flag = 0;
     wg_sync();
     if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0) *flag = 1;
