@@ -586,13 +586,18 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
   char* const tw = smem_raw + wave * 32 * tile_row_bytes<D>();
   float inv = 1.f;
   if constexpr (INTER == kInterSoftmax) inv = 1.f / pair_sum(lsum);
-  const int row = m_wave + ln;
+  // lane coordinates taken afresh: values kept from the prologue for this would sit in registers (or spill)
+  // through the whole walk
+  int lane_e = threadIdx.x & 63;
+  asm volatile("" : "+v"(lane_e));
+  const int ln_e = lane_e & 31, g_e = lane_e >> 5;
+  const int row = m_wave + ln_e;
   if (by_rows || row < M) {
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
-        const int n = 32 * t + 8 * q4 + 4 * g;
+        const int n = 32 * t + 8 * q4 + 4 * g_e;
         if (!by_rows && n >= N) continue;
         float v0 = o[t][4 * q4 + 0] * inv, v1 = o[t][4 * q4 + 1] * inv;
         float v2 = o[t][4 * q4 + 2] * inv, v3 = o[t][4 * q4 + 3] * inv;
@@ -604,14 +609,14 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
         } else {
           V2 a0 = cvt2<T>(v0, v1), a1 = cvt2<T>(v2, v3);
           V4 w = {a0[0], a0[1], a1[0], a1[1]};
-          if (by_rows) *reinterpret_cast<V4*>(tw + ln * tile_row_bytes<D>() + n * 2) = w;
+          if (by_rows) *reinterpret_cast<V4*>(tw + ln_e * tile_row_bytes<D>() + n * 2) = w;
           else *reinterpret_cast<V4*>(reinterpret_cast<T*>(p.f) + off) = w;
         }
       }
   }
   if (by_rows)
     store_tile_rows<T, D, 32>(tw, reinterpret_cast<T*>(p.f) + zo * p.f_bs2 + zi * p.f_bs + (long long)m_wave * p.f_rs, p.f_rs,
-                              M - m_wave, N, lane);
+                              M - m_wave, N, lane_e);
 #else
   (void)p;
 #endif
