@@ -7,7 +7,7 @@ import ctypes
 import os
 import threading
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # error codes (include/ditto_chain.h)
 OK, EINVAL, EUNSUPPORTED, EHIP, EWORKSPACE = 0, -1, -2, -3, -4
@@ -79,6 +79,8 @@ class ConvChainDesc(ctypes.Structure):
         ("pad2", ctypes.c_int64),
         ("stride2", ctypes.c_int64),
         ("groups1", ctypes.c_int64),
+        ("tile_variant", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
     ]
 
 

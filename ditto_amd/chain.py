@@ -152,10 +152,12 @@ def run_bmm_chain(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=
 
 
 def conv_chain_desc(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op="cast", relu_out=False,
-                    groups1=1):
+                    groups1=1, tile_variant=0):
     """Fill a ``ditto_conv_chain_desc`` for X[N,C0,H,W], W1[C1,C0/groups1,R1,S1], W2[C2,C1,R2,S2] -> Y.
 
-    ``groups1``: 1 (dense first convolution) or C0 (depthwise, C1 / C0 outputs per input channel)."""
+    ``groups1``: 1 (dense first convolution) or C0 (depthwise, C1 / C0 outputs per input channel).
+    ``tile_variant``: 0 (the library's choice) or the kernel to force: a variant id ``select_tile`` reported or a
+    family id (3000, 3500, 3600, 3700, 3800, 4000; see ``include/ditto_chain.h``)."""
     for t, name in ((X, "X"), (W1, "W1"), (W2, "W2"), (Y, "Y")):
         if t.dim() != 4 or not t.is_contiguous():
             raise ValueError("%s must be a contiguous 4-D NCHW/KCRS tensor" % name)
@@ -185,6 +187,7 @@ def conv_chain_desc(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op
     d.C1, d.R1, d.S1, d.pad1, d.stride1 = C1, R1, S1, pad1, stride1
     d.C2, d.R2, d.S2, d.pad2, d.stride2 = C2, R2, S2, pad2, stride2
     d.groups1 = groups1
+    d.tile_variant = int(tile_variant)
     return d
 
 
@@ -226,7 +229,7 @@ def prepare_conv_chain(desc, W1, W2, workspace=None):
 
 
 def run_conv_chain(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op="cast", relu_out=False,
-                   desc=None, workspace=None, groups1=1, prepared=False):
+                   desc=None, workspace=None, groups1=1, prepared=False, tile_variant=0):
     """Y = conv2d(inter(conv2d(X, W1)), W2) on the current stream: one fused kernel, preceded by
     a small kernel that repacks W1 into ``workspace`` (a uint8 tensor of
     ``ditto_conv_chain_workspace_bytes``; None: a cached per-device buffer; False: no
@@ -238,7 +241,7 @@ def run_conv_chain(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op=
     lib = _lib.load()
     dev = _check_device(X, W1, W2, Y)
     if desc is None:
-        desc = conv_chain_desc(X, W1, W2, Y, pad1, stride1, pad2, stride2, inter_op, relu_out, groups1)
+        desc = conv_chain_desc(X, W1, W2, Y, pad1, stride1, pad2, stride2, inter_op, relu_out, groups1, tile_variant)
     ws_bytes = lib.ditto_conv_chain_workspace_bytes(ctypes.byref(desc))
     if workspace is None:
         ws = _workspace(dev, ws_bytes) if ws_bytes else None

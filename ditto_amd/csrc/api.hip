@@ -9,7 +9,6 @@
 
 #include <cstdarg>
 #include <cstdio>
-#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -30,20 +29,6 @@ int fail(int code, const char* fmt, ...) {
 }
 
 bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
-
-int elem_bytes(int dt) {
-  switch (dt) {
-    case DITTO_F16:
-    case DITTO_BF16:
-      return 2;
-    case DITTO_F32:
-    case DITTO_I32:
-      return 4;
-    case DITTO_I8:
-      return 1;
-  }
-  return 0;
-}
 
 // Number of compute units of the current device (cached per thread).
 int device_cus() {
@@ -352,17 +337,46 @@ struct ConvPlan {
 // dw_mode 5: the row-streaming kernel for multiplier 16 (dw16_rows.h): 3x3, pad 1, stride 1, an even number of at
 // most 32 input channels, at most 64 output channels, image rows of whole 16-byte vectors whose ring of row slots
 // fits beside the filters in LDS, 16-bit output.  DITTO_DW16_ROWS=0 keeps such shapes on the persistent kernel.
-bool dw_rows_off() {
-  const char* v = getenv("DITTO_DW_ROWS");
-  return v && v[0] == '0';
+// What a forced tile_variant allows (0: everything; see ditto_conv_chain_desc.tile_variant).
+struct ConvSteer {
+  int tv = 0;
+  bool rows = true;      // 3700 / 3800: the row pipelines
+  bool resident = true;  // 3600: the persistent kernel with W2 resident in LDS
+  bool dw_rows = true;   // 4024
+  bool dw16_rows = true; // 4025
+  bool persist = false;  // 3900: the persistent 3x3 -> 1x1 kernel (switched off)
+};
+int conv_steer(int tv, ConvSteer* st) {
+  *st = ConvSteer();
+  st->tv = tv;
+  if (tv == 0) return DITTO_OK;
+  if (tv < 0) return fail(DITTO_EINVAL, "tile_variant must be 0, a variant id or a family id");
+  const int fam = tv / 100 * 100;
+  st->rows = fam == 3700 || fam == 3800;
+  st->resident = fam == 3600;
+  st->dw_rows = tv == 4024;
+  st->dw16_rows = tv == 4025;
+  st->persist = fam == 3900;
+  if (!(fam == 3000 || fam == 3100 || fam == 3500 || fam == 3600 || fam == 3700 || fam == 3800 || fam == 3900 || fam == 4000))
+    return fail(DITTO_EINVAL, "tile_variant %d names no conv chain kernel family", tv);
+  return DITTO_OK;
 }
-bool dw16_rows_off() {
-  const char* v = getenv("DITTO_DW16_ROWS");
-  return v && v[0] == '0';
+// The plan that came out against the variant that was asked for: a family id (a multiple of 100; 3000 also stands
+// for the 16-channel-chunk form 31xx, 4000 for every depthwise kernel but the two row-streaming ones) or an exact id.
+int conv_steer_check(const ConvSteer& st, int got) {
+  if (st.tv == 0 || st.tv == got) return DITTO_OK;
+  if (st.tv % 100 == 0) {
+    const int fam = got / 100 * 100;
+    if (fam == st.tv || (st.tv == 3000 && fam == 3100)) {
+      if (st.tv != 4000 || (got != 4024 && got != 4025)) return DITTO_OK;
+    }
+  }
+  return fail(DITTO_EINVAL, "tile_variant %d cannot run this chain (the kernel that fits it under that constraint is %d)",
+              st.tv, got);
 }
 
-int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvPlan* plan, bool need_device,
-                 bool allow_dwv = true, int vec_cap = 8, bool allow_rows = true) {
+int plan_dw_conv(const ditto_conv_chain_desc* d, const ConvSteer& steer, long long P, long long Q, ConvPlan* plan,
+                 bool need_device, bool allow_dwv = true, int vec_cap = 8, bool allow_rows = true) {
   if (d->C1 % d->C0) return fail(DITTO_EINVAL, "depthwise: C1 must be a multiple of C0");
   const long long mult = d->C1 / d->C0;
   const long long RS = d->R1 * d->S1;
@@ -383,7 +397,7 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   if (d->C1 > 32768) return fail(DITTO_EUNSUPPORTED, "depthwise chain: at most 32768 intermediate channels");
   memset(plan, 0, sizeof(*plan));
   plan->dw = true;
-  if (allow_rows && vec_cap >= 8 && !dw_rows_off() && mult == 1 && d->R1 == 3 && d->S1 == 3 && d->pad1 == 1 &&
+  if (allow_rows && vec_cap >= 8 && steer.dw_rows && mult == 1 && d->R1 == 3 && d->S1 == 3 && d->pad1 == 1 &&
       d->stride1 == 1 && d->C0 <= ditto::kDwRowsC && d->C2 <= 64 && d->W % 8 == 0 && d->W <= 128 &&
       d->out_dtype != DITTO_F32 && d->H * d->W * 64 < 0x7fffffffLL) {
     // Bands of whole output rows, one workgroup each: all input rows of a band stay in LDS.  Among the
@@ -424,7 +438,7 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
       return DITTO_OK;
     }
   }
-  if (allow_rows && vec_cap >= 8 && !dw16_rows_off() && mult == 16 && d->R1 == 3 && d->S1 == 3 && d->pad1 == 1 &&
+  if (allow_rows && vec_cap >= 8 && steer.dw16_rows && mult == 16 && d->R1 == 3 && d->S1 == 3 && d->pad1 == 1 &&
       d->stride1 == 1 && d->C0 <= 32 && d->C0 % 2 == 0 && d->C2 <= 64 && d->W % 8 == 0 && d->W >= 8 &&
       ditto::dw16_rows_ni((int)d->C0, (int)d->W) <= 8 &&
       ditto::dw16_rows_lds_bytes((int)d->C0, (int)d->W) <= 160 * 1024 && d->out_dtype != DITTO_F32 &&
@@ -574,7 +588,7 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   a.relu_mid = d->inter_op == DITTO_INTER_RELU;
   a.relu_out = d->relu_out != 0;
   a.out_f32 = d->out_dtype == DITTO_F32;
-  if (dwv && !a.wide) return plan_dw_conv(d, P, Q, plan, need_device, false, vec_cap, false);  // that variant needs the wide stores
+  if (dwv && !a.wide) return plan_dw_conv(d, steer, P, Q, plan, need_device, false, vec_cap, false);  // that variant needs the wide stores
   plan->c2_tiles = c2t;
   ditto_tile_param& t = plan->tile;
   t.block_threads = 256 * groups;
@@ -599,26 +613,24 @@ int plan_dw_conv(const ditto_conv_chain_desc* d, long long P, long long Q, ConvP
   return DITTO_OK;
 }
 
-// DITTO_CONV_RESIDENT=0 keeps the 1x1 -> 3x3 chains on the general kernel (A/B runs, tests of that kernel)
-bool resident_off() {
-  const char* v = getenv("DITTO_CONV_RESIDENT");
-  return v && v[0] == '0';
-}
+int plan_conv_steered(const ditto_conv_chain_desc* d, const ConvSteer& steer, ConvPlan* plan, bool need_device,
+                      int dw_vec_cap, bool allow_resident, bool allow_dw_rows);
 
-// DITTO_CONV_ROWS=0 keeps the 3x3 -> 1x1 chains on the general kernel (A/B runs, tests of that kernel)
-bool conv_rows_off() {
-  const char* v = getenv("DITTO_CONV_ROWS");
-  return v && v[0] == '0';
-}
-
-bool persist_requested() {
-  const char* v = getenv("DITTO_CONV_PERSIST");
-  return v && v[0] == '1';
-}
-
+// allow_resident = false: the general kernels only (pointers the specialised ones cannot take);
+// allow_dw_rows: y takes 16-byte stores
 int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device = false, int dw_vec_cap = 8,
-              bool allow_resident = true, bool allow_dw_rows = true) {  // allow_dw_rows: y takes 16-byte stores
+              bool allow_resident = true, bool allow_dw_rows = true) {
   if (!d) return fail(DITTO_EINVAL, "null descriptor");
+  ConvSteer steer;
+  int rc = conv_steer(d->tile_variant, &steer);
+  if (rc != DITTO_OK) return rc;
+  rc = plan_conv_steered(d, steer, plan, need_device, dw_vec_cap, allow_resident, allow_dw_rows);
+  if (rc != DITTO_OK) return rc;
+  return conv_steer_check(steer, plan->tile.variant);
+}
+
+int plan_conv_steered(const ditto_conv_chain_desc* d, const ConvSteer& steer, ConvPlan* plan, bool need_device,
+                      int dw_vec_cap, bool allow_resident, bool allow_dw_rows) {
   if (d->abi_version != DITTO_CHAIN_ABI_VERSION)
     return fail(DITTO_EINVAL, "descriptor abi_version %d, library %d", d->abi_version, DITTO_CHAIN_ABI_VERSION);
   if (d->in_dtype != DITTO_F16 && d->in_dtype != DITTO_BF16)
@@ -651,7 +663,7 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
       d->H > 65535 || d->W > 65535 || d->N > 65535 || d->C0 > 65535 || d->C2 > 65535)
     return fail(DITTO_EINVAL, "tensor too large");
   // (a y that is not 16-byte aligned rules out both kernels that only store 16-byte vectors)
-  if (dw) return plan_dw_conv(d, P, Q, plan, need_device, allow_dw_rows, dw_vec_cap, allow_dw_rows);
+  if (dw) return plan_dw_conv(d, steer, P, Q, plan, need_device, allow_dw_rows, dw_vec_cap, allow_dw_rows);
   memset(plan, 0, sizeof(*plan));
   const int c1t = d->C1 <= 32 ? 1 : d->C1 <= 64 ? 2 : d->C1 <= 128 ? 4 : 8;
   const int pxw = c1t == 8 ? 1 : 2;
@@ -669,7 +681,7 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
     a.R2 = (int)d->R2; a.S2 = (int)d->S2; a.pad2 = (int)d->pad2; a.P2 = (int)P2; a.Q2 = (int)Q2;
     // 1x1 -> 3x3 (pad 1) with at most 64 channels everywhere, 16-bit output and image rows of whole 16-byte
     // vectors up to 64 pixels: the row pipeline with the 1x1 convolution in its transposing stage (conv_rows.h)
-    if (allow_resident && !conv_rows_off() && !resident_off() && d->R1 == 1 && d->S1 == 1 && d->pad1 == 0 &&
+    if (allow_resident && steer.rows && d->R1 == 1 && d->S1 == 1 && d->pad1 == 0 &&
         d->stride1 == 1 && d->R2 == 3 && d->S2 == 3 && d->pad2 == 1 && d->C0 <= ditto::kCvrC && d->C1 <= ditto::kCvrC &&
         d->C2 <= ditto::kCvrC && d->C0 % 8 == 0 && d->W % 8 == 0 && d->W <= 64 && d->out_dtype != DITTO_F32 &&
         d->C0 * d->H * d->W * 2 < 0x7fffffffLL) {
@@ -718,7 +730,7 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
     }
     // 1x1 -> 3x3 (pad 1) with at most 64 channels everywhere and rows that are whole 16-byte vectors: the
     // persistent kernel that keeps W2 in LDS (conv_chain_resident.h), tiles of whole output rows
-    if (allow_resident && !resident_off() && d->R1 == 1 && d->S1 == 1 && d->pad1 == 0 && d->stride1 == 1 && d->R2 == 3 &&
+    if (allow_resident && steer.resident && d->R1 == 1 && d->S1 == 1 && d->pad1 == 0 && d->stride1 == 1 && d->R2 == 3 &&
         d->S2 == 3 && d->pad2 == 1 && d->C0 <= ditto::kCrC && d->C1 <= ditto::kCrC && d->C2 <= ditto::kCrC &&
         d->C0 % 8 == 0 && d->W % 8 == 0 && d->W <= 256 &&
         d->C0 * d->H * d->W * 2 < 0x7fffffffLL) {
@@ -796,16 +808,17 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
   // 3x3 (pad 1, stride 1) -> 1x1 with at most 64 input and intermediate and 256 output channels, image rows of
   // whole 16-byte vectors up to 64 pixels, 16-bit output: the row pipeline (conv_rows.h).  Bands of whole
   // output rows, one workgroup each; a band's rows are all in flight at once, which bounds its height.
-  if (allow_resident && !conv_rows_off() && !persist_requested() && d->R1 == 3 && d->S1 == 3 && d->pad1 == 1 &&
+  if (allow_resident && steer.rows && !steer.persist && d->R1 == 3 && d->S1 == 3 && d->pad1 == 1 &&
       d->stride1 == 1 && d->C0 <= ditto::kCvrC && d->C1 <= ditto::kCvrC && d->C2 <= 256 && d->W % 8 == 0 && d->W <= 64 &&
       d->out_dtype != DITTO_F32 && d->C0 * d->H * d->W * 2 < 0x7fffffffLL && d->C2 * d->H * d->W * 2 < 0x7fffffffLL &&
       // where it pays (measured against the general kernel): the pipeline pads C0 and C1 to 64, and its gain is the
       // output stream under the compute - wide outputs - or, with few images, more workgroups than the general
       // kernel's tiles of 256 pixels (32 x 32 x 56 x 56 -> 32 -> 128: 16.4 against 12.3 us; 64 -> 64 -> 64: a tie;
       // one image 64 -> 64 -> 256: 8.9 against 15.6 us)
-      (d->C0 > 32 || d->C1 > 32) &&
+      (steer.tv / 100 == 37 ||
+       ((d->C0 > 32 || d->C1 > 32) &&
       (d->C2 >= 192 || d->N * ((P + (256 / d->W > 0 ? 256 / d->W : 1) - 1) / (256 / d->W > 0 ? 256 / d->W : 1)) <
-                           (need_device ? device_cus() : 256))) {
+                           (need_device ? device_cus() : 256))))) {
     const int cus = need_device ? device_cus() : 256;
     int band_max = ditto::conv_rows_band_max((int)d->W);
     if (band_max > d->H) band_max = (int)d->H;
@@ -849,10 +862,10 @@ int plan_conv(const ditto_conv_chain_desc* d, ConvPlan* plan, bool need_device =
   // CU walking over the tiles) is switched off: it waits for its prefetched halo tile with a hand-counted
   // `s_waitcnt vmcnt` over loads the compiler does not track, and it is slower than the kernel below
   // (33.5 against 30.5 us on 32 x 64 x 56 x 56 -> 64 -> 256).  Asking for it is refused, not ignored.
-  if (persist_requested())
+  if (steer.persist)
     return fail(DITTO_EUNSUPPORTED,
-                "DITTO_CONV_PERSIST=1: the persistent conv chain kernel is switched off (untracked prefetch loads; "
-                "slower than the default kernel); unset the variable");
+                "tile_variant %d: the persistent conv chain kernel is switched off (untracked prefetch loads; "
+                "slower than the default kernel)", steer.tv);
   a.TW = (int)(Q < slots ? Q : slots);
   a.TH = slots / a.TW;
   if (a.TH > P) a.TH = (int)P;
@@ -913,7 +926,7 @@ const char* ditto_last_error(void) { return g_err; }
 
 int ditto_bmm_chain_select_tile(const ditto_bmm_chain_desc* desc, ditto_tile_param* out) {
   BmmPlan plan;
-  int rc = plan_bmm(desc, &plan, false);
+  int rc = plan_bmm(desc, &plan, true);  // the current device's compute-unit count (256 where there is none)
   if (rc != DITTO_OK) return rc;
   if (!out) return fail(DITTO_EINVAL, "null output");
   *out = plan.tile;
@@ -1047,7 +1060,7 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
 
 int ditto_conv_chain_select_tile(const ditto_conv_chain_desc* desc, ditto_tile_param* out) {
   ConvPlan plan;
-  int rc = plan_conv(desc, &plan);
+  int rc = plan_conv(desc, &plan, true);  // the current device's compute-unit count (256 where there is none)
   if (rc != DITTO_OK) return rc;
   if (!out) return fail(DITTO_EINVAL, "null output");
   *out = plan.tile;
@@ -1056,11 +1069,14 @@ int ditto_conv_chain_select_tile(const ditto_conv_chain_desc* desc, ditto_tile_p
 
 size_t ditto_conv_chain_workspace_bytes(const ditto_conv_chain_desc* desc) {
   ConvPlan plan;
-  if (plan_conv(desc, &plan) != DITTO_OK) return 0;
+  if (plan_conv(desc, &plan, true) != DITTO_OK) return 0;
   size_t need = plan.w1p_bytes + plan.w2p_bytes;
-  if (plan.resident || plan.rows31 || plan.rows13) {  // a call with pointers these kernels cannot take falls back to the general one
+  if (plan.resident || plan.rows31 || plan.rows13) {
+    // a call with pointers these kernels cannot take falls back to the general one (tile_variant 0 only): the
+    // larger of the two figures, whatever the device's compute-unit count makes of the choice
     ConvPlan general;
-    if (plan_conv(desc, &general, false, 8, false) == DITTO_OK && general.w1p_bytes + general.w2p_bytes > need)
+    if (desc->tile_variant == 0 && plan_conv(desc, &general, true, 8, false) == DITTO_OK &&
+        general.w1p_bytes + general.w2p_bytes > need)
       need = general.w1p_bytes + general.w2p_bytes;
   }
   return need;
@@ -1324,7 +1340,7 @@ int static_workspace(void** out) {
 extern "C" int ditto_conv_chain_run_static(const ditto_conv_chain_desc* d, const void* x, const void* w1,
                                            const void* w2, void* y, void* stream) {
   ConvPlan plan;
-  int rc = plan_conv(d, &plan);
+  int rc = plan_conv(d, &plan, true);
   if (rc != DITTO_OK) return rc;
   const size_t need = plan.w1p_bytes + plan.w2p_bytes;
   if (need > (size_t)DITTO_STATIC_WORKSPACE_BYTES)

@@ -26,7 +26,8 @@
 extern "C" {
 #endif
 
-#define DITTO_CHAIN_ABI_VERSION 1
+/* 2: ditto_conv_chain_desc gained tile_variant (the kernel to force; run-time switches in the environment are gone) */
+#define DITTO_CHAIN_ABI_VERSION 2
 
 /* error codes */
 #define DITTO_OK 0
@@ -123,6 +124,20 @@ typedef struct ditto_conv_chain_desc {
                             (benchmark/chimera/cuda/depthwise3x3_conv1x1_small_channel_cuda.py:77-169,
                             `factor` = C1 / C0); then R1 * S1 <= 9, the second convolution is 1x1
                             and C1 / C0 is 1, 2, 4 or a multiple of 8 */
+  int32_t tile_variant;  /* 0: the library's per-shape rules pick the kernel; else the kernel to force, the
+                            counterpart of an explicit CUDATensorizeParam (hyper_fusion.cc:586-607): either a
+                            `ditto_tile_param.variant` id as ditto_conv_chain_select_tile reported it, or a
+                            family id (a multiple of 100) that leaves the tile inside the family to the library:
+                              3000 general kernel, 1x1 second convolution (31xx: 16-channel chunks)
+                              3500 general kernel, second convolution up to 3x3 through LDS
+                              3600 conv1x1 -> conv3x3, persistent workgroups, W2 resident in LDS
+                              3700 conv3x3 -> conv1x1 row pipeline        3800 conv1x1 -> conv3x3 row pipeline
+                              4000 depthwise -> conv1x1, tile kernels (40xx = 4000 + 10 * output tiles + mode)
+                              4024 / 4025 depthwise row-streaming kernels (multiplier 1 / 16)
+                            DITTO_EINVAL if that kernel cannot run the chain; with a forced kernel a call
+                            whose pointers or workspace the kernel cannot take fails instead of falling
+                            back to the general kernel */
+  int32_t reserved0;     /* 0 */
 } ditto_conv_chain_desc;
 
 /* Tile choice reported back to the host; the static per-shape table replaces
@@ -140,7 +155,11 @@ typedef struct ditto_tile_param {
                              q = 1|2: four waves owning 32*q rows each; eight waves owning
                              32 rows each: q = 8 (phases staggered between the two waves of a
                              SIMD), q = 9 (software pipelined), q = 6 (16x16x32 MFMA, B stored
-                             [L][K] only); other chains: see api.hip  */
+                             [L][K] only), q = 7 (the same kernel with 384-row workgroups, 48 rows
+                             per wave, for the first row blocks of a batch entry and 256-row ones
+                             for the rest; block_m reports 384); conv chains: the ids listed at
+                             ditto_conv_chain_desc.tile_variant; fp32 / fp64 1000 / 1001; int8
+                             8000 + 10 * (row tiles of 32) + ring depth */
 } ditto_tile_param;
 
 /* ---- entry points ------------------------------------------------------- */
@@ -152,7 +171,9 @@ int ditto_chain_abi_version(void);
 const char* ditto_last_error(void);
 
 /* Tile the library would use for this chain; also validates the descriptor.
- * Replaces the parameter choice of chimera_integrate.py:452-478. */
+ * Replaces the parameter choice of chimera_integrate.py:452-478.  Rules that weigh workgroups against
+ * compute units use the current device's count, as the run calls do (256 where the process has no
+ * device), so the answer is the kernel a run on this device takes. */
 int ditto_bmm_chain_select_tile(const ditto_bmm_chain_desc* desc, ditto_tile_param* out);
 int ditto_conv_chain_select_tile(const ditto_conv_chain_desc* desc, ditto_tile_param* out);
 

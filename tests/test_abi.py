@@ -125,10 +125,9 @@ def _conv_desc(**kw):
     return _lib.ConvChainDesc(**d)
 
 
-def test_conv_tile_choice_without_gpu(monkeypatch):
+def test_conv_tile_choice_without_gpu():
     lib = _lib.load()
     tile = _lib.TileParam()
-    monkeypatch.delenv("DITTO_CONV_PERSIST", raising=False)
     # the workload shape runs on the row pipeline: bands of 7 output rows, one workgroup per CU, seven waves
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc()), ctypes.byref(tile)) == _lib.OK
     assert (tile.variant, tile.grid_x, tile.grid_y, tile.block_threads) == (3707, 256, 7, 512)
@@ -137,7 +136,7 @@ def test_conv_tile_choice_without_gpu(monkeypatch):
     # W1 as MFMA fragments takes 9 * 64 * 64 * 2 bytes; the query covers the general kernel too, which a call
     # with less aligned pointers falls back to
     assert rows_ws == max(9 * 64 * 64 * 2, 2 * 9 * 64 * 40 * 2)
-    # fp32 output, wider rows or more channels stay on the general kernel, and so does everything with DITTO_CONV_ROWS=0
+    # fp32 output, wider rows or more channels stay on the general kernel, and so does everything with tile_variant 3000
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(out_dtype=_lib.F32)), ctypes.byref(tile)) == _lib.OK
     assert tile.variant == 3022
     # ... and narrow outputs with enough images to fill the CUs with the general kernel's tiles (measured slower there)
@@ -147,18 +146,28 @@ def test_conv_tile_choice_without_gpu(monkeypatch):
     assert tile.variant // 100 == 37
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C0=32, C1=32)), ctypes.byref(tile)) == _lib.OK
     assert tile.variant // 100 == 30
-    monkeypatch.setenv("DITTO_CONV_ROWS", "0")
-    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc()), ctypes.byref(tile)) == _lib.OK
-    assert tile.variant == 3022 and tile.grid_x == 32 * 14 and tile.lds_bytes <= 80 * 1024  # two workgroups per CU
-    default_ws = lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc()))
-    assert default_ws == 2 * 9 * 64 * 40 * 2  # two chunks of 32 input channels, [tap][c1][32 + 8]
-    monkeypatch.delenv("DITTO_CONV_ROWS")
-    # the opt-in persistent kernel is switched off: asking for it is refused, not silently ignored
-    monkeypatch.setenv("DITTO_CONV_PERSIST", "1")
-    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc()), ctypes.byref(tile)) == _lib.EUNSUPPORTED
+    for forced in (3000, 3022):  # the family, or the exact kernel
+        general = _conv_desc(tile_variant=forced)
+        assert lib.ditto_conv_chain_select_tile(ctypes.byref(general), ctypes.byref(tile)) == _lib.OK
+        assert tile.variant == 3022 and tile.grid_x == 32 * 14 and tile.lds_bytes <= 80 * 1024  # two workgroups per CU
+        default_ws = lib.ditto_conv_chain_workspace_bytes(ctypes.byref(general))
+        assert default_ws == 2 * 9 * 64 * 40 * 2  # two chunks of 32 input channels, [tap][c1][32 + 8]
+    # the row pipeline by family and by exact id; an id the planner does not arrive at is refused, and so are
+    # families that cannot run the chain and ids that name nothing
+    for forced in (3700, 3707):
+        assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(tile_variant=forced)), ctypes.byref(tile)) == _lib.OK
+        assert tile.variant == 3707
+    assert lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc(tile_variant=3707))) == 9 * 64 * 64 * 2
+    # (narrow outputs, where the library's own choice is the general kernel: the pipeline can still be asked for)
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C2=128, tile_variant=3700)), ctypes.byref(tile)) == _lib.OK
+    assert tile.variant == 3707
+    for bad in (3705, 3800, 3600, 3500, 4000, 4024, 1286, 17, -1):
+        assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(tile_variant=bad)), ctypes.byref(tile)) == _lib.EINVAL, bad
+        assert lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc(tile_variant=bad))) == 0
+    # the persistent 3x3 -> 1x1 kernel is switched off: asking for it is refused, not silently ignored
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(tile_variant=3900)), ctypes.byref(tile)) == _lib.EUNSUPPORTED
     assert b"switched off" in lib.ditto_last_error()
-    assert lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc())) == 0
-    monkeypatch.delenv("DITTO_CONV_PERSIST")
+    assert lib.ditto_conv_chain_workspace_bytes(ctypes.byref(_conv_desc(tile_variant=3900))) == 0
     # depthwise first convolution: persistent kernel with the matrix-core depthwise stage; at multiplier 1 the
     # row-streaming kernel (bands of 14 rows: one workgroup per CU, nine waves) for up to 32 -> 64 channels and
     # the persistent kernel with the vector-ALU stage beyond
@@ -167,17 +176,15 @@ def test_conv_tile_choice_without_gpu(monkeypatch):
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=512, **dw)), ctypes.byref(tile)) == _lib.OK
     assert (tile.variant, tile.grid_x, tile.grid_y, tile.block_threads) == (4025, 256, 14, 576)
     assert tile.lds_bytes <= 160 * 1024
-    monkeypatch.setenv("DITTO_DW16_ROWS", "0")
-    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=512, **dw)), ctypes.byref(tile)) == _lib.OK
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=512, tile_variant=4000, **dw)), ctypes.byref(tile)) == _lib.OK
     assert tile.variant == 4022 and tile.grid_x == 256
-    monkeypatch.delenv("DITTO_DW16_ROWS")
+    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=512, tile_variant=4024, **dw)), ctypes.byref(tile)) == _lib.EINVAL
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=32, **dw)), ctypes.byref(tile)) == _lib.OK
     assert (tile.variant, tile.grid_x, tile.grid_y, tile.block_threads) == (4024, 256, 14, 832)
     assert tile.lds_bytes <= 160 * 1024
-    monkeypatch.setenv("DITTO_DW_ROWS", "0")
-    assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=32, **dw)), ctypes.byref(tile)) == _lib.OK
-    assert tile.variant == 4023
-    monkeypatch.delenv("DITTO_DW_ROWS")
+    for forced in (4000, 4023):
+        assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=32, tile_variant=forced, **dw)), ctypes.byref(tile)) == _lib.OK
+        assert tile.variant == 4023
     dw = dict(C0=64, H=56, W=56, C2=128, groups1=64)
     assert lib.ditto_conv_chain_select_tile(ctypes.byref(_conv_desc(C1=64, **dw)), ctypes.byref(tile)) == _lib.OK
     assert tile.variant == 4043

@@ -14,7 +14,7 @@ MAX_ABS, REL_L2 = 1e-2, 1e-3
 
 
 def run_conv(X, W1, W2, dtype, pad1=1, stride1=1, inter="cast", relu_out=False, out_dtype=None, workspace=None,
-             pad2=0, groups1=1):
+             pad2=0, groups1=1, tile_variant=0):
     x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
     N, _, H, W = X.shape
     R, S = W1.shape[2:]
@@ -22,7 +22,7 @@ def run_conv(X, W1, W2, dtype, pad1=1, stride1=1, inter="cast", relu_out=False, 
     Q = (W + 2 * pad1 - S) // stride1 + 1 + 2 * pad2 - W2.shape[3] + 1
     y = torch.full((N, W2.shape[0], P, Q), float("nan"), device=x.device, dtype=TORCH_DTYPES[out_dtype or dtype])
     chain.run_conv_chain(x, w1, w2, y, pad1, stride1, pad2, 1, inter, relu_out, workspace=workspace,
-                         groups1=groups1)
+                         groups1=groups1, tile_variant=tile_variant)
     torch.cuda.synchronize()
     return y.float().cpu().numpy()
 
@@ -85,7 +85,7 @@ CASES_ROWS_PIPELINE = [
 
 @pytest.mark.parametrize("case", CASES_ROWS_PIPELINE)
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
-def test_conv_chain_row_pipeline(oracle, case, dtype, monkeypatch):
+def test_conv_chain_row_pipeline(oracle, case, dtype):
     """The row pipeline against the oracle and against the general kernel on the same inputs (different
     summation orders: held to the workload tolerance), through run and through prepare + run_prepared."""
     N, C0, H, W, C1, C2 = case
@@ -111,20 +111,18 @@ def test_conv_chain_row_pipeline(oracle, case, dtype, monkeypatch):
         chain.run_conv_chain(x, w1, w2, y1, desc=desc, workspace=ws, prepared=True)
         torch.cuda.synchronize()
         assert torch.equal(y1, y), relu
-        monkeypatch.setenv("DITTO_CONV_ROWS", "0")
         y2 = torch.full_like(y, float("nan"))
-        desc2 = chain.conv_chain_desc(x, w1, w2, y2, 1, 1, 0, 1, inter, relu)
-        assert chain.select_tile(desc2).variant // 100 != 37
+        desc2 = chain.conv_chain_desc(x, w1, w2, y2, 1, 1, 0, 1, inter, relu, tile_variant=3000)  # the general kernel
+        assert chain.select_tile(desc2).variant // 100 in (30, 31)
         chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
         torch.cuda.synchronize()
-        monkeypatch.delenv("DITTO_CONV_ROWS")
         mx, rel = errors(got, y2.float().cpu().numpy())
         assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
 
 
 # Enough tiles of whole output rows for two rounds of persistent workgroups (at least 512), 16-bit
 # output, at most 64 input / intermediate channels: the opt-in kernel with both weight tensors resident
-# on the CU (DITTO_CONV_PERSIST=1).
+# on the CU (tile_variant 3900).
 CASES_PERSISTENT = [
     # N, C0, H, W, C1, R, pad, stride, C2
     (520, 8, 8, 8, 16, 3, 1, 1, 32),      # one tile per image, 32-channel variants
@@ -143,18 +141,17 @@ PERSIST_OFF = ("the persistent conv chain kernel is switched off in the planner 
 @pytest.mark.skip(reason=PERSIST_OFF)
 @pytest.mark.parametrize("case", CASES_PERSISTENT)
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
-def test_persistent_conv_chain_vs_oracle(oracle, case, dtype, monkeypatch):
-    monkeypatch.setenv("DITTO_CONV_PERSIST", "1")
+def test_persistent_conv_chain_vs_oracle(oracle, case, dtype):
     N, C0, H, W, C1, R, pad, stride, C2 = case
     X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, R, 1, dtype, seed=C0 + C2, w_std=0.05)
     x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
     P, Q = (H + 2 * pad - R) // stride + 1, (W + 2 * pad - R) // stride + 1
     y = torch.empty((N, C2, P, Q), device=x.device, dtype=TORCH_DTYPES[dtype])
-    desc = chain.conv_chain_desc(x, w1, w2, y, pad, stride, 0, 1, "cast", False)
+    desc = chain.conv_chain_desc(x, w1, w2, y, pad, stride, 0, 1, "cast", False, tile_variant=3900)
     assert chain.select_tile(desc).variant // 100 == 39  # the persistent kernel
     for relu in (False, True):
         want32 = oracle.conv_chain_f32(X, W1, W2, pad, stride, 0, 1, relu_mid=relu, relu_out=relu, round_mid=dtype)
-        got = run_conv(X, W1, W2, dtype, pad, stride, "relu" if relu else "cast", relu)
+        got = run_conv(X, W1, W2, dtype, pad, stride, "relu" if relu else "cast", relu, tile_variant=3900)
         assert got.shape == want32.shape and np.isfinite(got).all()
         mx, rel = errors(got, oracle.np_round_to(want32, dtype))
         assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
@@ -229,7 +226,7 @@ CASES_ROWS13 = [
 
 @pytest.mark.parametrize("case", CASES_ROWS13)
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
-def test_row_pipeline_conv1x1_conv3x3(oracle, case, dtype, monkeypatch):
+def test_row_pipeline_conv1x1_conv3x3(oracle, case, dtype):
     """conv1x1 -> conv3x3 (pad 1) through the row pipeline: against the oracle, and against the kernel that keeps
     W2 in LDS on the same inputs."""
     N, C0, H, W, C1, C2 = case
@@ -265,15 +262,17 @@ def test_row_pipeline_conv1x1_conv3x3(oracle, case, dtype, monkeypatch):
     assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
     with pytest.raises(ValueError):  # ... and the prepared form, whose weights are in this kernel's layout, reports it
         chain.run_conv_chain(x, w1_off, w2, y3, desc=desc, workspace=ws, prepared=True)
-    monkeypatch.setenv("DITTO_CONV_ROWS", "0")
-    assert chain.select_tile(chain.conv_chain_desc(x, w1, w2, y, 0, 1, 1, 1, "relu", False)).variant // 100 == 36
-    other = run_conv(X, W1, W2, dtype, 0, 1, "relu", True, None, None, 1)
-    monkeypatch.delenv("DITTO_CONV_ROWS")
+    assert chain.select_tile(chain.conv_chain_desc(x, w1, w2, y, 0, 1, 1, 1, "relu", False,
+                                                   tile_variant=3600)).variant // 100 == 36
+    other = run_conv(X, W1, W2, dtype, 0, 1, "relu", True, None, None, 1, tile_variant=3600)
     mx, rel = errors(got, other)
+    # a forced kernel does not step aside: the element-aligned weights are refused
+    with pytest.raises(ValueError):
+        chain.run_conv_chain(x, w1_off, w2, y3, 0, 1, 1, 1, "relu", True, tile_variant=3800)
     assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
 
 
-def test_row_pipeline_conv1x1_conv3x3_at_benchmark_size(oracle, monkeypatch):
+def test_row_pipeline_conv1x1_conv3x3_at_benchmark_size(oracle):
     """The benchmark's shape, 32 x 64 x 56 x 56 -> 64 -> 64 (one band per CU): three images against the oracle, all
     of them against the kernel that keeps W2 in LDS, and the chain's linearity in x (no ReLU: f(2x) = 2 f(x); a power
     of two only shifts exponents, so the two differ only where an intermediate value is subnormal in fp16)."""
@@ -297,39 +296,34 @@ def test_row_pipeline_conv1x1_conv3x3_at_benchmark_size(oracle, monkeypatch):
     torch.cuda.synchronize()
     mx, rel = errors((ya * 2).float().cpu().numpy(), yb.float().cpu().numpy())
     assert mx <= 1e-3 and rel <= 1e-5, (mx, rel)
-    monkeypatch.setenv("DITTO_CONV_ROWS", "0")
     y2 = torch.full_like(y, float("nan"))
-    desc2 = chain.conv_chain_desc(x, w1, w2, y2, 0, 1, 1, 1, "relu", True)
+    desc2 = chain.conv_chain_desc(x, w1, w2, y2, 0, 1, 1, 1, "relu", True, tile_variant=3600)
     assert chain.select_tile(desc2).variant // 100 == 36
     chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
     torch.cuda.synchronize()
-    monkeypatch.delenv("DITTO_CONV_ROWS")
     mx, rel = errors(got, y2.float().cpu().numpy())
     assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
 
 
-def test_resident_conv_chain_over_several_rounds(oracle, monkeypatch):
+def test_resident_conv_chain_over_several_rounds(oracle):
     """More tiles than CUs: every persistent workgroup walks over more than one tile.  Checked against the
     general kernel (which streams W2 per workgroup) on the same inputs, both against the oracle on a slice."""
-    monkeypatch.setenv("DITTO_CONV_ROWS", "0")  # (else the shape runs on the row pipeline)
     N, C0, H, W, C1, C2 = 20, 64, 56, 56, 64, 64
     X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, 1, 3, "float16", seed=5, w_std=0.05)
     x, w1, w2 = to_dev(X, "float16"), to_dev(W1, "float16"), to_dev(W2, "float16")
     y = torch.full((N, C2, H, W), float("nan"), device=x.device, dtype=torch.float16)
-    desc = chain.conv_chain_desc(x, w1, w2, y, 0, 1, 1, 1, "relu", False)
+    desc = chain.conv_chain_desc(x, w1, w2, y, 0, 1, 1, 1, "relu", False, tile_variant=3600)  # (0: the row pipeline)
     tile = chain.select_tile(desc)
     assert tile.variant == 3604 and tile.block_threads == 512 and tile.lds_bytes <= 160 * 1024
     chain.run_conv_chain(x, w1, w2, y, desc=desc)
     torch.cuda.synchronize()
     got = y.float().cpu().numpy()
     assert np.isfinite(got).all()
-    monkeypatch.setenv("DITTO_CONV_RESIDENT", "0")
     y2 = torch.full_like(y, float("nan"))
-    desc2 = chain.conv_chain_desc(x, w1, w2, y2, 0, 1, 1, 1, "relu", False)
+    desc2 = chain.conv_chain_desc(x, w1, w2, y2, 0, 1, 1, 1, "relu", False, tile_variant=3500)
     assert chain.select_tile(desc2).variant // 100 == 35
     chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
     torch.cuda.synchronize()
-    monkeypatch.delenv("DITTO_CONV_RESIDENT")
     mx, rel = errors(got, y2.float().cpu().numpy())
     assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
     for n in (0, 13, 19):  # first, a middle and the last image (the last one is the second tile of its workgroup)
@@ -427,7 +421,7 @@ CASES_DW_ROWS = [
 
 @pytest.mark.parametrize("case", CASES_DW_ROWS)
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
-def test_row_streaming_depthwise_chain(oracle, case, dtype, monkeypatch):
+def test_row_streaming_depthwise_chain(oracle, case, dtype):
     """The row-streaming kernel against the oracle and against the persistent kernel on the same inputs
     (both accumulate in fp32 in different orders: held to the workload tolerance, not to the bits)."""
     N, C0, H, W, C2 = case
@@ -449,13 +443,11 @@ def test_row_streaming_depthwise_chain(oracle, case, dtype, monkeypatch):
         if dtype == "bfloat16" and relu:
             report("conv chain (wide second filter / depthwise) bf16 rows %s" % (case,), mx, rel)
         assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
-        monkeypatch.setenv("DITTO_DW_ROWS", "0")
         y2 = torch.full_like(y, float("nan"))
-        desc2 = chain.conv_chain_desc(x, w1, w2, y2, 1, 1, 0, 1, "relu" if relu else "cast", relu, C0)
+        desc2 = chain.conv_chain_desc(x, w1, w2, y2, 1, 1, 0, 1, "relu" if relu else "cast", relu, C0, tile_variant=4000)
         assert chain.select_tile(desc2).variant % 10 != 4
         chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
         torch.cuda.synchronize()
-        monkeypatch.delenv("DITTO_DW_ROWS")
         mx, rel = errors(got, y2.float().cpu().numpy())
         assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
 
@@ -474,7 +466,7 @@ CASES_DW16_ROWS = [
 
 @pytest.mark.parametrize("case", CASES_DW16_ROWS)
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
-def test_row_streaming_depthwise_chain_factor_16(oracle, case, dtype, monkeypatch):
+def test_row_streaming_depthwise_chain_factor_16(oracle, case, dtype):
     """The row-streaming kernel for sixteen outputs per input channel against the oracle and against the tiled
     kernel on the same inputs (the same MFMAs in the same order: the same bits)."""
     N, C0, H, W, C2 = case
@@ -499,13 +491,11 @@ def test_row_streaming_depthwise_chain_factor_16(oracle, case, dtype, monkeypatc
         if dtype == "bfloat16" and relu:
             report("conv chain (wide second filter / depthwise) bf16 rows x16 %s" % (case,), mx, rel)
         assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
-        monkeypatch.setenv("DITTO_DW16_ROWS", "0")
         y2 = torch.full_like(y, float("nan"))
-        desc2 = chain.conv_chain_desc(x, w1, w2, y2, 1, 1, 0, 1, "relu" if relu else "cast", relu, C0)
+        desc2 = chain.conv_chain_desc(x, w1, w2, y2, 1, 1, 0, 1, "relu" if relu else "cast", relu, C0, tile_variant=4000)
         assert chain.select_tile(desc2).variant % 10 == 2
         chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
         torch.cuda.synchronize()
-        monkeypatch.delenv("DITTO_DW16_ROWS")
         assert torch.equal(y, y2), (relu, errors(got, y2.float().cpu().numpy()))
 
 
@@ -638,15 +628,89 @@ def test_conv_chain_full_size_linearity(oracle):
     assert errors(s, got)[1] <= 1e-5
 
 
+def test_row_pipeline_conv3x3_conv1x1_at_benchmark_size(oracle):
+    """The benchmarked kernel of the conv3x3 -> conv1x1 configuration at its size (N = 32, fp16 output, variant 3707:
+    bands of 7 rows, one workgroup per compute unit): three images against the checker, all of them against the
+    general kernel on the same inputs, and linearity in W2 over all of them."""
+    N, C0, H, W, C1, C2 = 32, 64, 56, 56, 64, 256
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, 3, 1, "float16", seed=0)
+    x, w1, w2 = to_dev(X, "float16"), to_dev(W1, "float16"), to_dev(W2, "float16")
+    y = torch.full((N, C2, H, W), float("nan"), device=x.device, dtype=torch.float16)
+    desc = chain.conv_chain_desc(x, w1, w2, y, 1, 1, 0, 1, "cast", False)
+    assert chain.select_tile(desc).variant == 3707
+    chain.run_conv_chain(x, w1, w2, y, desc=desc)
+    torch.cuda.synchronize()
+    got = y.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    for n in (0, 13, 31):
+        want = oracle.conv_chain_f32(X[n:n + 1], W1, W2, round_mid="float16")
+        mx, rel = errors(got[n:n + 1], oracle.np_round_to(want, "float16"))
+        assert mx <= MAX_ABS and rel <= REL_L2, (n, mx, rel)
+    y2 = torch.full_like(y, float("nan"))
+    desc2 = chain.conv_chain_desc(x, w1, w2, y2, 1, 1, 0, 1, "cast", False, tile_variant=3000)
+    assert chain.select_tile(desc2).variant == 3022
+    chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
+    torch.cuda.synchronize()
+    mx, rel = errors(got, y2.float().cpu().numpy())  # two summation orders, both rounded to fp16 at the end
+    assert mx <= MAX_ABS and rel <= 5e-4, (mx, rel)
+    # W2 = W2a + W2b with both parts exact in fp16: the two outputs add up to the whole one but for their roundings
+    W2a = oracle.np_round_to(W2 * 0.5, "float16")
+    W2b = W2 - W2a
+    assert np.array_equal(oracle.np_round_to(W2b, "float16"), W2b)
+    ya, yb = torch.empty_like(y), torch.empty_like(y)
+    chain.run_conv_chain(x, w1, to_dev(W2a, "float16"), ya, desc=desc)
+    chain.run_conv_chain(x, w1, to_dev(W2b, "float16"), yb, desc=desc)
+    torch.cuda.synchronize()
+    mx, rel = errors(ya.float().cpu().numpy() + yb.float().cpu().numpy(), got)
+    assert rel <= 5e-4, (mx, rel)  # three fp16 roundings of O(1) values: 2^-11 / sqrt(3) each
+
+
+@pytest.mark.parametrize("mult,variant", [(1, 4024), (16, 4025)])
+def test_row_streaming_depthwise_chains_at_benchmark_size(oracle, mult, variant):
+    """The two depthwise workloads of the benchmark at their size (32 x 32 x 112 x 112 -> 64, multiplier 1 and 16):
+    the benchmarked row-streaming kernel on three images against the checker, on all of them against the tile kernel
+    (tile_variant 4000), and linear in x (a power of two only shifts exponents)."""
+    N, C0, H, W, C2 = 32, 32, 112, 112, 64
+    C1 = C0 * mult
+    rng = np.random.default_rng(40 + mult)
+    X = oracle.np_round_to(rng.standard_normal((N, C0, H, W)).astype(np.float32), "float16")
+    W1 = oracle.np_round_to(rng.standard_normal((C1, 1, 3, 3)).astype(np.float32) * 0.3, "float16")
+    W2 = oracle.np_round_to(rng.standard_normal((C2, C1, 1, 1)).astype(np.float32) * (0.2 if mult == 1 else 0.05), "float16")
+    x, w1, w2 = to_dev(X, "float16"), to_dev(W1, "float16"), to_dev(W2, "float16")
+    y = torch.full((N, C2, H, W), float("nan"), device=x.device, dtype=torch.float16)
+    desc = chain.conv_chain_desc(x, w1, w2, y, 1, 1, 0, 1, "relu", False, C0)
+    assert chain.select_tile(desc).variant == variant
+    chain.run_conv_chain(x, w1, w2, y, desc=desc)
+    torch.cuda.synchronize()
+    got = y.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    for n in (0, 18, 31):
+        want = oracle.conv_chain_f32(X[n:n + 1], W1, W2, 1, 1, 0, 1, relu_mid=True, round_mid="float16", groups1=C0)
+        mx, rel = errors(got[n:n + 1], oracle.np_round_to(want, "float16"))
+        assert mx <= MAX_ABS and rel <= REL_L2, (n, mx, rel)
+    y2 = torch.full_like(y, float("nan"))
+    desc2 = chain.conv_chain_desc(x, w1, w2, y2, 1, 1, 0, 1, "relu", False, C0, tile_variant=4000)
+    assert chain.select_tile(desc2).variant not in (4024, 4025)
+    chain.run_conv_chain(x, w1, w2, y2, desc=desc2)
+    torch.cuda.synchronize()
+    mx, rel = errors(got, y2.float().cpu().numpy())
+    assert mx <= MAX_ABS and rel <= 5e-4, (mx, rel)
+    ya, yb = torch.empty_like(y), torch.empty_like(y)
+    chain.run_conv_chain(x, w1, w2, ya, 1, 1, 0, 1, "cast", False, groups1=C0)
+    chain.run_conv_chain(x * 2, w1, w2, yb, 1, 1, 0, 1, "cast", False, groups1=C0)
+    torch.cuda.synchronize()
+    mx, rel = errors((ya * 2).float().cpu().numpy(), yb.float().cpu().numpy())
+    assert mx <= 1e-3 and rel <= 1e-5, (mx, rel)
+
+
 @pytest.mark.skip(reason=PERSIST_OFF)
-def test_persistent_conv_chain_full_size(oracle, monkeypatch):
+def test_persistent_conv_chain_full_size(oracle):
     # the full configuration through the opt-in persistent kernel: two images against the checker, all
     # of them against the default kernel (two summation orders, both rounded to fp16 at the end)
     N, C0, H, W, C1, C2 = 32, 64, 56, 56, 64, 256
     X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, 3, 1, "float16", seed=1)
     default = run_conv(X, W1, W2, "float16", inter="relu", relu_out=True)
-    monkeypatch.setenv("DITTO_CONV_PERSIST", "1")
-    got = run_conv(X, W1, W2, "float16", inter="relu", relu_out=True)
+    got = run_conv(X, W1, W2, "float16", inter="relu", relu_out=True, tile_variant=3900)
     sel = [0, 31]
     want = oracle.np_round_to(oracle.conv_chain_f32(X[sel], W1, W2, relu_mid=True, relu_out=True, round_mid="float16"),
                               "float16")
