@@ -155,6 +155,81 @@ def auto_schedule_bmm_chain_hip(key, log_file, A, B, C, F, inter_op="softmax", s
     return select_tile_variant(key, log_file, A, B, C, F, inter_op, softmax_scale).record["variant"]
 
 
+# ---- conv -> conv chains: the same measurement and log over the conv kernel families ------------
+# family ids of ``ditto_conv_chain_desc.tile_variant`` (include/ditto_chain.h): general kernel with a 1x1 second
+# convolution, general kernel with the second convolution through LDS, W2 resident in LDS, the two row pipelines;
+# depthwise: the tile kernels and the two row-streaming ones
+CONV_FAMILY_IDS = (3000, 3500, 3600, 3700, 3800, 4000, 4024, 4025)
+
+
+def make_conv_tile_variant_space(desc):
+    """Kernels of the library that can run the conv chain ``desc``: one tile description per family that accepts
+    it (the library refuses the others), each carrying the exact variant id the family resolves to."""
+    lib = _lib.load()
+    space, seen = [], set()
+    for fam in (0,) + CONV_FAMILY_IDS:
+        d = copy.copy(desc)
+        d.tile_variant = fam
+        t = _lib.TileParam()
+        if lib.ditto_conv_chain_select_tile(ctypes.byref(d), ctypes.byref(t)) == _lib.OK and t.variant not in seen:
+            seen.add(t.variant)
+            space.append(t.to_json())
+    return space
+
+
+def conv_workload_key(desc):
+    return "conv_chain/dt%d/o%d/i%d/r%d/n%d/c%d/h%d/w%d/c%d/k%d/p%d/s%d/c%d/k%d/p%d/g%d" % (
+        desc.in_dtype, desc.out_dtype, desc.inter_op, desc.relu_out, desc.N, desc.C0, desc.H, desc.W, desc.C1, desc.R1,
+        desc.pad1, desc.stride1, desc.C2, desc.R2, desc.pad2, max(1, desc.groups1))
+
+
+def select_conv_tile_variant(wkl_key, log_file, X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op="cast",
+                             relu_out=False, groups1=1, min_repeat_ms=50):
+    """Measure every kernel that can run this conv chain with its weights prepared once (the fused kernel alone is
+    timed, as the reference times a function whose weights the host has packed), append every measurement to
+    ``log_file`` and return the best ``TuneEntry``."""
+    import torch
+
+    desc = chain.conv_chain_desc(X, W1, W2, Y, pad1, stride1, pad2, stride2, inter_op, relu_out, groups1)
+    best = None
+    for tile in make_conv_tile_variant_space(desc):
+        d = copy.copy(desc)
+        d.tile_variant = tile["variant"]
+        ws = chain.prepare_conv_chain(d, W1, W2) if chain.conv_chain_workspace_bytes(d) else None
+        if ws is not None:
+            call = lambda: chain.run_conv_chain(X, W1, W2, Y, desc=d, workspace=ws, prepared=True)
+        else:
+            call = lambda: chain.run_conv_chain(X, W1, W2, Y, desc=d)
+        call()
+        torch.cuda.synchronize()
+        n = 1
+        while True:
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                call()
+            e1.record()
+            e1.synchronize()
+            ms = e0.elapsed_time(e1)
+            if ms >= min_repeat_ms or n >= 1 << 20:
+                break
+            n = max(n + 1, int(n * max(1.5, min_repeat_ms / max(ms, 1e-3) * 1.05)))
+        entry = TuneEntry(tile, ms / n)
+        _log(log_file, wkl_key, entry)
+        if best is None or entry.value < best.value:
+            best = entry
+    return best
+
+
+def auto_schedule_conv_chain_hip(key, log_file, X, W1, W2, Y, **kw):
+    """Tune once per key, then reuse the log: returns the variant id to pass as ``tile_variant``."""
+    known = best_variant(log_file, key, default=None)
+    if known is not None:
+        return known
+    return select_conv_tile_variant(key, log_file, X, W1, W2, Y, **kw).record["variant"]
+
+
 # ---- layer-level entry points (chimera_integrate.py:452-556 of the reference) -------------------
 class AttentionSchedule:
     """What scheduling a ``multi_head_attention_mma_layer`` yields: the layer, the module that runs

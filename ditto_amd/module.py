@@ -35,7 +35,10 @@ class ChainFunction:
     on it (use ``specialize`` for a second object).  ``specialize(W1, W2)`` returns a function bound
     to fixed weights whose repacking is done once, the counterpart of the reference's drivers being
     handed host-packed weights (conv3x3_conv1x1_cuda.py:99-103): its calls run the fused kernel
-    alone for as long as they are given those same weight tensors."""
+    alone for as long as they are given those same weight tensors with unchanged contents.  The function keeps
+    the two tensors alive (their addresses cannot be handed to other tensors) and remembers their version
+    counters: other tensors, or the same ones after an in-place update, are repacked at that call and become
+    the bound weights."""
 
     entry_name = "default_function"
 
@@ -53,7 +56,7 @@ class ChainFunction:
         self.tile_variant = int(sch.tile_variant if tile_variant is None else tile_variant)
         self._descs = {}        # argument layout -> filled descriptor
         self._workspaces = {}   # device -> uint8 tensor (conv chains)
-        self._prepared = None   # (w1 data_ptr, w2 data_ptr, device) the workspace holds repacked weights of
+        self._prepared = None   # (W1, W2, W1._version, W2._version): what the workspace holds the repacked form of
 
     def _check_args(self, args):
         if len(args) != len(self.tensors):
@@ -103,8 +106,19 @@ class ChainFunction:
         ws = f._workspace(desc, W1.device)
         if ws is not False:
             chain.prepare_conv_chain(desc, W1, W2, ws)
-            f._prepared = (W1.data_ptr(), W2.data_ptr(), W1.device)
+            f._prepared = (W1, W2, W1._version, W2._version)
         return f
+
+    def _is_prepared(self, W1, W2):
+        p = self._prepared
+        if p is None:
+            return False
+
+        def same(held, w):  # the held tensor itself, or another view of exactly its memory (views share the counter)
+            return held is w or (w.data_ptr() == held.data_ptr() and w.shape == held.shape and w.dtype == held.dtype
+                                 and w.device == held.device)
+
+        return same(p[0], W1) and same(p[1], W2) and p[2] == W1._version and p[3] == W2._version
 
     def __call__(self, *args):
         self._check_args(args)
@@ -122,7 +136,17 @@ class ChainFunction:
             X, W1, W2, Y = args
             desc = self._conv_desc(X, W1, W2, Y)
             ws = self._workspace(desc, X.device)
-            prepared = ws is not False and self._prepared == (W1.data_ptr(), W2.data_ptr(), X.device)
+            prepared = ws is not False and self._is_prepared(W1, W2)
+            if ws is not False and self._prepared is not None and not prepared:
+                # a specialised function handed other weights (or the bound ones after an in-place update):
+                # repack them now; they are the bound weights from here on
+                self._prepared = None
+                try:
+                    chain.prepare_conv_chain(desc, W1, W2, ws)
+                    self._prepared = (W1, W2, W1._version, W2._version)
+                    prepared = True
+                except ValueError:
+                    pass  # pointers the prepared form cannot take: the one-call form below decides
             chain.run_conv_chain(X, W1, W2, Y, desc=desc, workspace=ws, prepared=prepared)
         else:
             raise NotImplementedError("no kernel family for chain kind %r" % s.kind)

@@ -48,7 +48,9 @@ class GraphEngine:
     def __init__(self, graph, built_mods, dev="cuda:0", prepare_weights=True):
         self.graph = graph
         # conv chain layers with weights: repack the weights once per compile (set_weight compiles
-        # again) instead of on every run; weights changed in place afterwards need a new compile
+        # again) instead of on every run.  Weights changed in place afterwards are noticed through their
+        # version counters: the bound function repacks them at its next call, the graph-replay engine
+        # records its graph again
         self.prepare_weights = prepare_weights
         self.built_mods = built_mods  # {layer fingerprint: callable f(*inputs, *weights, *outputs)}
         self.dev = torch.device(dev)
@@ -114,6 +116,10 @@ class GraphEngine:
                 func = func.specialize(*self.weight_buffer[li])
             args = [*self.input_buffer[li], *self.weight_buffer[li], *self.output_buffer[li]]
             self._to_exe.append((func, args))
+        self._weight_versions = self._versions()
+
+    def _versions(self):
+        return [w._version for li in sorted(self.weight_buffer) for w in self.weight_buffer[li]]
 
     def run(self):
         if not self._to_exe:
@@ -149,7 +155,9 @@ class HipGraphEngine(GraphEngine):
         self._graph = g
 
     def run(self):
-        if not self._to_exe or getattr(self, "_graph", None) is None:
+        # (a recorded graph holds the repacked weights of compile time: weights updated in place since then
+        # need the repacking, and with it the recording, done again)
+        if not self._to_exe or getattr(self, "_graph", None) is None or self._versions() != self._weight_versions:
             self.compile()
         self._graph.replay()
 

@@ -760,3 +760,29 @@ def test_prepared_weights_give_the_same_bits(oracle, case):
     small = torch.empty(16, dtype=torch.uint8, device=x.device)
     with pytest.raises(ValueError):
         chain.prepare_conv_chain(desc, w1, w2, workspace=small)
+
+
+def test_conv_tile_variant_tuning_round_trip(tmp_path, oracle):
+    """The measurement-driven kernel choice for conv chains: every family that can run the shape is timed with
+    prepared weights, logged in the reference's JSON-lines format (chimera_integrate.py:326-333, 527-556), and
+    the logged winner is what a later call is steered to."""
+    from ditto_amd.auto_schedule.schedulers import chimera_integrate as ci
+
+    N, C0, H, W, C1, C2 = 4, 64, 56, 56, 64, 256
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, 3, 1, "float16", seed=9)
+    x, w1, w2 = to_dev(X, "float16"), to_dev(W1, "float16"), to_dev(W2, "float16")
+    y = torch.full((N, C2, H, W), float("nan"), device=x.device, dtype=torch.float16)
+    desc = chain.conv_chain_desc(x, w1, w2, y)
+    space = ci.make_conv_tile_variant_space(desc)
+    assert sorted(t["variant"] // 100 for t in space) == [30, 37]
+    log = str(tmp_path / "chimera_conv.log")
+    key = ci.conv_workload_key(desc)
+    best = ci.select_conv_tile_variant(key, log, x, w1, w2, y, min_repeat_ms=5)
+    assert len(open(log).read().strip().splitlines()) == len(space)
+    assert ci.load_best_records(log)[key]["record"]["variant"] == best.record["variant"] and 0 < best.value < 5.0
+    assert ci.auto_schedule_conv_chain_hip(key, log, x, w1, w2, y) == best.record["variant"]
+    chain.run_conv_chain(x, w1, w2, y, tile_variant=best.record["variant"])
+    torch.cuda.synchronize()
+    want = oracle.conv_chain_f32(X[:1], W1, W2, round_mid="float16")
+    mx, rel = errors(y[:1].float().cpu().numpy(), oracle.np_round_to(want, "float16"))
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)

@@ -227,6 +227,31 @@ def test_tile_variant_space_and_analytic_filter():
     assert ci.workload_key(big) != ci.workload_key(small)
 
 
+def test_conv_tile_variant_space():
+    """Kernel families that can run a conv chain, as the tuner enumerates them (no device needed)."""
+    import torch
+    from ditto_amd import chain
+    from ditto_amd.auto_schedule.schedulers import chimera_integrate as ci
+
+    def desc(N, C0, H, W, C1, R1, C2, R2, groups=1, dt=torch.float16):
+        x = torch.zeros(N, C0, H, W, dtype=dt)
+        w1 = torch.zeros(C1, C0 // groups, R1, R1, dtype=dt)
+        w2 = torch.zeros(C2, C1, R2, R2, dtype=dt)
+        y = torch.zeros(N, C2, H, W, dtype=dt)
+        return chain.conv_chain_desc(x, w1, w2, y, R1 // 2, 1, R2 // 2, 1, "cast", False, groups)
+
+    fams = lambda d: sorted(t["variant"] // 100 * 100 for t in ci.make_conv_tile_variant_space(d))
+    assert fams(desc(32, 64, 56, 56, 64, 3, 256, 1)) == [3000, 3700]          # conv3x3 -> conv1x1
+    assert fams(desc(32, 64, 56, 56, 64, 1, 64, 3)) == [3500, 3600, 3800]     # conv1x1 -> conv3x3
+    assert fams(desc(1, 128, 28, 28, 128, 3, 128, 3)) == [3500]               # conv3x3 -> conv3x3: the general kernel only
+    space = ci.make_conv_tile_variant_space(desc(32, 32, 112, 112, 32, 3, 64, 1, groups=32))
+    assert sorted(t["variant"] for t in space) == [4023, 4024]                 # depthwise, multiplier 1
+    space = ci.make_conv_tile_variant_space(desc(32, 32, 112, 112, 512, 3, 64, 1, groups=32))
+    assert sorted(t["variant"] for t in space) == [4022, 4025]                 # depthwise, multiplier 16
+    a, b = desc(32, 64, 56, 56, 64, 3, 256, 1), desc(16, 64, 56, 56, 64, 3, 256, 1)
+    assert ci.conv_workload_key(a) != ci.conv_workload_key(b)
+
+
 def test_attention_layer_task_extraction_and_binding():
     """bert_inference.py:88-92 -- tasks keyed by layer fingerprint, attention layers bound to the
     chimera scheduler (chimera/task_binding.py:6-20), everything else to ansor."""

@@ -241,3 +241,68 @@ def test_captured_conv_chain_survives_growth_of_the_shared_workspace(oracle):
         torch.cuda.synchronize()
         assert torch.equal(y, want), it
     del junk
+
+
+def test_specialised_conv_chain_notices_other_and_updated_weights(oracle):
+    """A function bound to fixed weights (``specialize``) runs the fused kernel alone on the repacked copy it made.
+    It must not take for its own (a) new weight tensors that the allocator placed at the addresses of the bound
+    ones, nor (b) the bound tensors after an in-place update; the graph-replay engine records again after (b)."""
+    import numpy as np
+
+    from ditto_amd import chimera
+    from ditto_amd.auto_compute.nn import functional as F
+    from tests.gpu_util import errors, to_dev
+
+    n, c0, hw_, c1, c2 = 4, 64, 28, 64, 256  # (a shape that runs on the row pipeline: repacked W1 in the workspace)
+    cins, couts = F.Conv3x3Conv1x1(n, c0, hw_, hw_, c1, c2)
+    cl = ac.layer([couts[0].op], inputs=[cins[0]], weights=cins[1:], name="conv_chain")
+    func = ditto.build(common.describe_layer(cl), cl.schedule_tensors, "hip")
+    X, W1, W2 = oracle.make_conv_chain_inputs(n, c0, hw_, hw_, c1, c2, 3, 1, "float16", seed=11)
+    W1b = oracle.np_round_to(W1 * 0.5, "float16")
+    ref = lambda w1: oracle.np_round_to(oracle.conv_chain_f32(X[:1], w1, W2, 1, 1, 0, 1, round_mid="float16"), "float16")
+    want_a, want_b = ref(W1), ref(W1b)
+    assert errors(want_a, want_b)[1] > 0.1  # the two weight sets are told apart easily
+    x = to_dev(X, "float16")
+    y = torch.empty(n, c2, hw_, hw_, device=x.device, dtype=torch.float16)
+
+    def check(f, w1, w2, want):
+        y.fill_(float("nan"))
+        f(x, w1, w2, y)
+        torch.cuda.synchronize()
+        mx, rel = errors(y[:1].float().cpu().numpy(), want)
+        assert mx <= 1e-2 and rel <= 1e-3, (mx, rel)
+
+    # (a) the bound tensors go out of the caller's hands; same-size tensors with other values take their place
+    w1, w2 = to_dev(W1, "float16"), to_dev(W2, "float16")
+    f = func.specialize(w1, w2)
+    check(f, w1, w2, want_a)
+    p1, p2 = w1.data_ptr(), w2.data_ptr()
+    del w1, w2
+    w1n, w2n = to_dev(W1b, "float16"), to_dev(W2, "float16")
+    # (the function keeps the bound tensors alive, so the allocator cannot hand their addresses out again)
+    assert w1n.data_ptr() != p1 and w2n.data_ptr() != p2
+    check(f, w1n, w2n, want_b)
+    check(f, w1n, w2n, want_b)  # bound to the new ones now: prepared path
+    assert f._is_prepared(w1n, w2n)
+    # (b) in-place update of the bound weights
+    w1n.copy_(to_dev(W1, "float16"))
+    assert not f._is_prepared(w1n, w2n)
+    check(f, w1n, w2n, want_a)
+    assert f._is_prepared(w1n, w2n)
+    # a view of the bound memory is the bound weights
+    assert f._is_prepared(w1n.view(c1, c0, 3, 3), w2n.detach())
+    # both engines, weights updated in place between runs
+    for make in (runtime.create_graph_engine, runtime.create_hip_graph_engine):
+        eng = make(runtime.Graph([cl]), {cl.fingerprint: func}, "cuda:0")
+        eng.set_inputs([x])
+        ew1, ew2 = to_dev(W1, "float16"), to_dev(W2, "float16")
+        eng.set_weight(cl, cl.weights[0], ew1)
+        eng.set_weight(cl, cl.weights[1], ew2)
+        eng.compile()
+        eng.run()
+        torch.cuda.synchronize()
+        assert errors(eng.get_outputs()[0][:1].float().cpu().numpy(), want_a)[1] <= 1e-3
+        ew1.mul_(0.5)  # exact in fp16: now W1b
+        eng.run()
+        torch.cuda.synchronize()
+        assert errors(eng.get_outputs()[0][:1].float().cpu().numpy(), want_b)[1] <= 1e-3, make.__name__
