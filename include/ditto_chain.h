@@ -241,7 +241,9 @@ int ditto_conv_chain_run_prepared(const ditto_conv_chain_desc* desc, const void*
  *   - DITTO_EWORKSPACE if ditto_conv_chain_workspace_bytes(desc) exceeds that size;
  *   - every call on one GPU shares that GPU's array: calls that overlap on one GPU (two streams,
  *     two threads) race; calls on one stream are ordered and safe;
- *   - the array keeps the last call's contents; each call rewrites all it reads.
+ *   - the array keeps the last call's contents; each call rewrites all it reads;
+ *   - the first call on a device takes the array's address and sets the kernels' LDS limits (host-side
+ *     set-up): make it outside any stream capture.  Later calls only launch kernels and can be captured.
  */
 #define DITTO_STATIC_WORKSPACE_BYTES (4u << 20)
 int ditto_conv_chain_run_static(const ditto_conv_chain_desc* desc, const void* x, const void* w1,

@@ -786,3 +786,44 @@ def test_conv_tile_variant_tuning_round_trip(tmp_path, oracle):
     want = oracle.conv_chain_f32(X[:1], W1, W2, round_mid="float16")
     mx, rel = errors(y[:1].float().cpu().numpy(), oracle.np_round_to(want, "float16"))
     assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
+
+
+def test_overflowed_outputs_of_the_conv1x1_conv3x3_row_pipeline():
+    """An fp16 output that overflows: the kernels that keep W2 in LDS (tile_variant 3600) and the general one (3500)
+    confine the infinity to its own channel, as the reference's chain does.  The row pipeline (38xx, the default
+    for this shape) passes the cast result through an identity MFMA on its way to the 8-pixel stores, where
+    0 x inf is NaN: the overflowed value itself comes out infinite, the other channels of the same pixel within
+    its block of 32 come out NaN instead of their finite values, and every other pixel is untouched.  A caller
+    that needs the exact semantics on overflowing data asks for tile_variant 3600."""
+    N, C0, H, W, C1, C2 = 1, 64, 16, 16, 64, 64
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(N, C0, H, W, generator=g) * 4).half().to(dev)
+    w1 = (torch.randn(C1, C0, 1, 1, generator=g) * 0.05).half().to(dev)
+    w2 = (torch.randn(C2, C1, 3, 3, generator=g) * 0.05).half().to(dev)
+    w2[5] *= 20000.0     # channel 5 of the output (standard deviation about 4e4) overflows fp16 at some pixels
+    outs = {}
+    for tv in (0, 3600, 3500):
+        y = torch.full((N, C2, H, W), float("nan"), device=dev, dtype=torch.float16)
+        desc = chain.conv_chain_desc(x, w1, w2, y, 0, 1, 1, 1, "cast", False, tile_variant=tv)
+        if tv == 0:
+            assert chain.select_tile(desc).variant // 100 == 38
+        chain.run_conv_chain(x, w1, w2, y, desc=desc)
+        torch.cuda.synchronize()
+        outs[tv] = y.float().cpu()
+    ref = torch.nn.functional.conv2d(torch.nn.functional.conv2d(x.float(), w1.float()).half().float(), w2.float(),
+                                     padding=1).half().float().cpu()
+    over = torch.isinf(ref[0, 5])
+    assert over.any() and not over.all() and not torch.isinf(ref[0, :5]).any() and not torch.isinf(ref[0, 6:]).any()
+    for tv in (3600, 3500):  # exact semantics: infinities where the reference has them, everything else finite and close
+        o = outs[tv]
+        assert torch.equal(torch.isinf(o), torch.isinf(ref)) and not torch.isnan(o).any(), tv
+        fin = ~torch.isinf(ref)
+        assert bool(((o[fin] - ref[fin]).abs() <= 2e-3 * ref[fin].abs() + 1e-2).all()), tv
+    o = outs[0]
+    assert torch.equal(torch.isinf(o[0, 5]), over)                      # the overflowed values themselves
+    clean = ~over                                                        # pixels without an overflow: untouched
+    assert not torch.isnan(o[0][:, clean]).any()
+    assert float((o[0, :5][:, clean] - ref[0, :5][:, clean]).abs().max()) <= 1e-2
+    assert not torch.isnan(o[0, 32:]).any()                              # the other block of 32 channels: untouched
+    assert torch.isnan(o[0, :32][:, over]).sum() > 0                     # the documented divergence

@@ -58,3 +58,37 @@ def test_static_workspace_entry_rejects_what_does_not_fit():
     rc = _lib.load().ditto_conv_chain_run_static(ctypes.byref(desc), x.data_ptr(), w1.data_ptr(), w2.data_ptr(),
                                                  y.data_ptr(), None)
     assert rc == _lib.EWORKSPACE and "static workspace" in _lib.last_error()
+
+
+def test_static_workspace_entry_under_graph_capture(oracle):
+    """The use the entry point is for: after one call outside any capture (which takes the array's address and
+    configures the kernels on this device), the call is recorded into a HIP graph -- an allocation inside it would
+    fail the capture -- and every replay gives the eager result."""
+    case, dtype = (2, 64, 56, 56, 64, 3, 1, 256, 1, 0), "float16"
+    N, C0, H, W, C1, R1, pad1, C2, R2, pad2 = case
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, R1, R2, dtype, seed=21, w_std=0.05)
+    x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
+    y = torch.full((N, C2, H, W), float("nan"), device=x.device, dtype=TORCH_DTYPES[dtype])
+    desc = chain.conv_chain_desc(x, w1, w2, y, pad1, 1, pad2, 1, "relu", True)
+    lib = _lib.load()
+
+    def call():
+        stream = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.ditto_conv_chain_run_static(ctypes.byref(desc), x.data_ptr(), w1.data_ptr(), w2.data_ptr(),
+                                                   y.data_ptr(), stream))
+
+    call()  # the first call on the device: outside the capture
+    torch.cuda.synchronize()
+    want = y.clone()
+    assert torch.isfinite(want).all()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        call()
+    for it in range(3):  # replays with eager work and synchronisations in between
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), it
+        call()
+        torch.cuda.synchronize()
