@@ -101,6 +101,8 @@ class TensorizeHyperFusionState:
 
     def __init__(self, layer: Layer, fuse_choice: FusionChoice, match_info: Dict[te.Operation, MatchInfo]):
         self.layer = layer
+        self.fuse_choice = fuse_choice
+        self.match_info = dict(match_info or {})
         self.first_op = fuse_choice.first_op
         self.second_op = fuse_choice.second_op
         if not fuse_choice.attach_pos < len(fuse_choice.ordered_iters):
@@ -253,7 +255,7 @@ class ChainSchedule:
     requant_scale: float = 1.0       # inter_op "requant": the scale of every column ...
     scale_tensor: bool = False       # ... unless a float32 scale[L] placeholder follows A, B, C
     tile_variant: int = 0            # 0: the library's per-shape table; else the variant id to force
-    target: str = "hip"              # "cpu" only from tensorize_cpu / FusionContext.run, which nothing can build
+    target: str = "hip"              # "cpu": from tensorize_cpu / FusionContext.run, built with target "llvm"
 
 
 def _kinds(ops):
@@ -334,20 +336,71 @@ def tensorize_cuda(layer, state, cuda_param=None, tensorize_param=None):
 
 @dataclass
 class CPUTensorizeParam:
-    """Loop tiling of the CPU fused nest (hyper_fusion.cc:609-642: per-op tiling factors and loop
-    orders chosen by ``buildCPUTensorizeParam``).  Kept as a record only: this build has no CPU
-    product path."""
+    """Loop tiling of the CPU fused nest (hyper_fusion.cc:609-642: per-op tiling factors and loop orders chosen by
+    ``buildCPUTensorizeParam``).  The nest of this build has two free factors, the ones the reference's search
+    spends its time on: ``m_block``, the rows of the chain one parallel task owns (the tiling of the second
+    contraction's outer spatial loop), and ``l_block``, the columns of the intermediate computed at the attach
+    position before the second contraction consumes them (the tiling of its outer reduce loop).  ``cost`` is the
+    analytic score the candidates are ranked by (seconds of a cache-traffic model; a rank, not a time)."""
     firstOpTilingFactor: tuple = ()
     firstOpLoopOrder: tuple = ()
     secondOpTilingFactor: tuple = ()
     secondOpLoopOrder: tuple = ()
     parallelism: int = 1
+    mi: int = 6
+    ni1: int = 16
+    ni2: int = 16
+    m_block: int = 6
+    l_block: int = 16
+    fusion_level: int = -1
+    cost: float = 0.0
 
 
-def build_cpu_tensorize_param(sfs, fusion_choice, hw_param, dtype):
-    """Identity tiling in the loop order of ``fusion_choice`` (reference: hyper_fusion.py:297-302)."""
+def cpu_tensorize_candidates(sfs, fusion_choice, hw_param, dtype, dims=None, mi=6, ni1=16, ni2=16):
+    """Every (m_block, l_block) tiling of the fused nest for a GEMM chain of extents ``dims`` = (batch, M, N, K, L),
+    ranked by a cache model in the spirit of the reference's (hyper_fusion_cpu.cc:1000-1500: footprint of the
+    fused tile against the cache sizes picks the level it lives in, bytes moved across that level over its
+    bandwidth price the candidate): per task the first contraction's tile, the panels of B and C it meets and its
+    rows of A and F must sit in one cache level; B and C are streamed once per task, so fewer, taller tasks move
+    fewer bytes but leave cores idle when there are fewer tasks than cores."""
     if dtype not in _DTYPE_BYTES:
         raise ValueError("unknown dtype %s" % dtype)
+    eb = _DTYPE_BYTES[dtype]
+    batch, M, N, K, L = dims
+    par = max(1, int(getattr(hw_param, "num_groups", 1) or 1))
+    caches = list(getattr(hw_param, "cacheSizes", None) or [32 * 16, 32 * 1024, 1024 * 1024, 32 * 1024 * 1024])
+    bws = list(getattr(hw_param, "bandwidth", None) or [293.72, 81.72, 38.54, 13.14])
+    all2 = sfs.second_op.axis + sfs.second_op.reduce_axis
+    order2 = tuple(next(i for i, v in enumerate(all2) if v is iv) for iv in fusion_choice.ordered_iters)
+    n1 = len(sfs.first_op.axis + sfs.first_op.reduce_axis)
+    out = []
+    mbs = sorted({min(-(-M // mi) * mi, mi * f) for f in (1, 2, 4, 8, 16, 32, 64)})
+    lbs = sorted({min(-(-L // ni1) * ni1, ni1 * f) for f in (1, 2, 4, 8, 16, 32, 64, 1 << 20)})
+    for mb in mbs:
+        for lb in lbs:
+            foot = (mb * lb + K * lb + lb * N + mb * K + mb * N) * eb
+            level = next((i for i, c in enumerate(caches) if foot <= c), len(caches) - 1)
+            tasks = batch * -(-M // mb)
+            rounds = -(-tasks // par)
+            moved = (K * L + L * N + mb * (K + N)) * eb          # per task, across the level the tile lives in
+            flops = 2.0 * mb * L * (K + N)
+            per_task = moved / (bws[min(level + 1, len(bws) - 1)] * 1e9) + flops / (32.0 * 2.5e9)
+            p = CPUTensorizeParam(firstOpTilingFactor=(1,) * n1, firstOpLoopOrder=tuple(range(n1)),
+                                  secondOpTilingFactor=(1, mb // mi, 1, max(1, lb // ni1)) + (1,) * max(0, len(all2) - 4),
+                                  secondOpLoopOrder=order2, parallelism=par, mi=mi, ni1=ni1, ni2=ni2, m_block=mb,
+                                  l_block=lb, fusion_level=level, cost=rounds * per_task)
+            out.append(p)
+    out.sort(key=lambda p: (p.cost, p.m_block, p.l_block))
+    return out
+
+
+def build_cpu_tensorize_param(sfs, fusion_choice, hw_param, dtype, dims=None):
+    """The best-ranked tiling (reference: hyper_fusion.py:297-302).  Without ``dims`` (a chain whose extents are not
+    known here) the identity tiling in the loop order of ``fusion_choice``."""
+    if dtype not in _DTYPE_BYTES:
+        raise ValueError("unknown dtype %s" % dtype)
+    if dims is not None:
+        return cpu_tensorize_candidates(sfs, fusion_choice, hw_param, dtype, dims)[0]
     op1, op2 = sfs.first_op, sfs.second_op
     n1, n2 = len(op1.axis + op1.reduce_axis), len(op2.axis + op2.reduce_axis)
     all2 = op2.axis + op2.reduce_axis
@@ -357,10 +410,17 @@ def build_cpu_tensorize_param(sfs, fusion_choice, hw_param, dtype):
 
 
 def tensorize_cpu(layer, state, cpu_param=None, tensorize_param=None):
-    """The reference lowers the chain to an x86 loop nest here (hyper_fusion.py:262-268,
-    hyper_fusion_cpu.cc:1553-1614).  This build is the gfx950 path only: the chain is recognised
-    (so descriptor errors surface as they do for the GPU flow) and a ``ChainSchedule`` marked for a
-    CPU target is returned, which ``ditto_amd.build`` refuses."""
+    """Bind a described GEMM chain to the CPU fused nest (reference: hyper_fusion.py:262-268,
+    hyper_fusion_cpu.cc:1553-1614): the chain is recognised exactly as for the GPU flow (descriptor errors
+    surface the same way) and the ``ChainSchedule`` comes back marked for the CPU target, carrying the tiling
+    (``tensorize_param``: a ``CPUTensorizeParam``; None: the nest's default) and the micro-kernel sources of the
+    state's match infos.  ``ditto_amd.build(sch, tensors, "llvm")`` turns it into a callable over host tensors.
+    fp32 / fp64 GEMM chains (cast, relu, softmax between the contractions) only, as in the reference."""
     sch = tensorize_hip(layer, state, cpu_param, None)
+    if sch.kind != "bmm_chain" or sch.in_dtype not in ("float32", "float64"):
+        raise ValueError("the CPU target runs fp32 / fp64 GEMM chains (got %s, %s)" % (sch.kind, sch.in_dtype))
+    if tensorize_param is not None and not isinstance(tensorize_param, CPUTensorizeParam):
+        raise TypeError("tensorize_param must be a CPUTensorizeParam")
+    sch.tensorize_param = tensorize_param
     sch.target = "cpu"
     return sch

@@ -121,12 +121,54 @@ def intrinsic_match(target: te.Tensor, packed_intrin: PackedIntrinsic, restricti
     return choices
 
 
+def _cpu_gemm_source(name, M, N, K, dtype):
+    """C source of the register-tile micro-kernel ``<name>_update``: ``c[M][N] += a[M][kc] . b[kc][N]`` on row-major
+    tiles, the M x N accumulators held in ymm registers over the whole k loop (one broadcast of ``a`` per row and
+    step against the vectors of a row of ``b``), and ``<name>_reset`` that clears a tile -- the two externs the
+    reference's generated kernels export (intrinsic.py:292-416 for the 6 x 16 fp32 tile, :646-674 for the calls).
+    ``K`` is the reduction extent the intrinsic was described with; the function takes the actual count."""
+    fp32 = dtype == "float32"
+    T, W = ("float", 8) if fp32 else ("double", 4)
+    V, sfx = ("__m256", "ps") if fp32 else ("__m256d", "pd")
+    bcast = "_mm256_broadcast_ss" if fp32 else "_mm256_broadcast_sd"
+    nv, tail = N // W, N % W
+    lines = ["#include <immintrin.h>",
+             "/* %d x %d x %d %s register tile (%d vector accumulators%s) */" % (
+                 M, N, K, dtype, M * nv, ", scalar tail of %d" % tail if tail else ""),
+             "void %s_update(const %s* a, long lda, const %s* b, long ldb, %s* c, long ldc, long kc) {" % (name, T, T, T)]
+    for r in range(M):
+        for v in range(nv):
+            lines.append("  %s acc%d_%d = _mm256_loadu_%s(c + %d * ldc + %d);" % (V, r, v, sfx, r, v * W))
+    lines.append("  for (long k = 0; k < kc; ++k) {")
+    for v in range(nv):
+        lines.append("    const %s b%d = _mm256_loadu_%s(b + k * ldb + %d);" % (V, v, sfx, v * W))
+    for r in range(M):
+        lines.append("    { const %s av = %s(a + %d * lda + k);" % (V, bcast, r))
+        for v in range(nv):
+            lines.append("      acc%d_%d = _mm256_fmadd_%s(av, b%d, acc%d_%d);" % (r, v, sfx, v, r, v))
+        lines.append("    }")
+    if tail:
+        lines.append("    for (int r = 0; r < %d; ++r) for (int j = %d; j < %d; ++j) c[r * ldc + j] += a[r * lda + k] * b[k * ldb + j];"
+                     % (M, nv * W, N))
+    lines.append("  }")
+    for r in range(M):
+        for v in range(nv):
+            lines.append("  _mm256_storeu_%s(c + %d * ldc + %d, acc%d_%d);" % (sfx, r, v * W, r, v))
+    lines.append("}")
+    lines.append("void %s_reset(%s* c, long ldc) {" % (name, T))
+    lines.append("  for (int r = 0; r < %d; ++r) for (int j = 0; j < %d; ++j) c[r * ldc + j] = 0;" % (M, N))
+    lines.append("}")
+    return "\n".join(lines) + "\n"
+
+
 def cpu_intrin(op, shape, isa, dtype, prefix=""):
-    """The CPU micro-kernel contract (reference: intrinsic.py:1675-1706): returns
-    ``(packed_intrinsic, code)``.  In the reference ``code`` is the C / assembly source of a 6 x 16
-    (AVX2) or 6 x 64 (AVX-512) register-tile kernel reached through ``call_extern("<prefix>_update")``
-    (:292-416, :646-674); here it is a one-line description, since this build has no CPU product
-    path -- the object only carries the tile shape through ``intrinsic_match`` / ``match_info``."""
+    """The CPU micro-kernel contract (reference: intrinsic.py:1675-1706): returns ``(packed_intrinsic, code)``.
+    ``code`` is the C source of the register-tile kernel for that shape, exporting ``<prefix>_update`` and
+    ``<prefix>_reset``; a chain built for the ``llvm`` target compiles it and runs its full tiles on it
+    (``ditto_amd.build``).  AVX2 code is generated for either ``isa``; a tile wider than the sixteen ymm registers
+    hold (more than twelve vector accumulators: the reference's 6 x 32 and 6 x 64 AVX-512 shapes) gets no code and
+    is run by the nest in column panels of its own kernel.  The ``exp`` intrinsics carry no code: the nest applies
+    the op between the contractions itself."""
     if op not in ("gemm", "gemm_noreshape", "conv", "exp", "exp_noreshape"):
         raise ValueError("unknown cpu intrinsic %r" % op)
     if isa not in ("avx2", "avx512"):
@@ -138,7 +180,9 @@ def cpu_intrin(op, shape, isa, dtype, prefix=""):
         K = 1
     else:
         M, N, K = (int(x) for x in shape[:3])
-    compute = TensorIntrin("%s_update" % (prefix or op), M, N, K, dtype, dtype, "global")
-    code = "// %s micro-kernel %s (%d x %d x %d, %s, %s): described, not generated" % (op, compute.name, M, N, K,
-                                                                                     isa, dtype)
+    name = prefix or op
+    compute = TensorIntrin("%s_update" % name, M, N, K, dtype, dtype, "global")
+    width = 8 if dtype == "float32" else 4
+    fits = op in ("gemm", "gemm_noreshape") and 1 <= M <= 6 and M * (N // width) <= 12 and N >= width
+    code = _cpu_gemm_source(name, M, N, K, dtype) if fits else ""
     return packed_intrinsic([], compute, None, ["global", "global"], "global", "global"), code

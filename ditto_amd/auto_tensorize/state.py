@@ -64,13 +64,14 @@ def validate(state):
 
 
 class FusionContext:
-    """What ``build_fusion_context`` returns in the reference: the ranked candidate schedules of the
-    CPU fused nest (state.py:34-78, hyper_fusion.cc:2182-2247).  Here a single candidate: the
-    fusion the layer's ``TensorizeHyperFusionState`` describes.  ``run`` yields a schedule marked
-    for a CPU target, which ``ditto_amd.build`` refuses -- this build has no CPU product path."""
+    """What ``build_fusion_context`` returns in the reference: the ranked candidate schedules of the CPU fused
+    nest (state.py:34-78, hyper_fusion.cc:2182-2247).  The candidates are the (m_block, l_block) tilings of the
+    nest ranked by the cache model of ``cpu_tensorize_candidates``; ``mode`` bounds how many are kept ("test": the
+    best one, "best": the best five, "survey": all), ``run(i, sch)`` returns candidate ``i`` as a schedule for the
+    CPU target, which ``ditto_amd.build(sch, tensors, "llvm")`` builds."""
 
     def __init__(self, sfs, layer, state, path, hw_param, searchType, mode, dtype):
-        from .hyper_fusion import _DTYPE_BYTES
+        from .hyper_fusion import _DTYPE_BYTES, _recognise, cpu_tensorize_candidates
 
         if searchType not in ("normal", "stochastic"):
             raise ValueError("searchType must be normal or stochastic")
@@ -81,7 +82,21 @@ class FusionContext:
         self.sfs, self.layer, self.state, self.path = sfs, layer, state, path
         self.hw_param, self.searchType, self.mode, self.dtype = hw_param, searchType, mode, dtype
         self.bytePerEle = _DTYPE_BYTES[dtype]
-        self.size = 1
+        info = _recognise(layer, state)
+        self.candidates = [None]
+        if info["kind"] == "bmm_chain" and info["in_dtype"] in ("float32", "float64"):
+            d = info["dims"]
+            mi, ni1, ni2 = 6, 16, 16
+            infos = getattr(state, "match_info", None) or {}
+            m1, m2 = infos.get(sfs.first_op), infos.get(sfs.second_op)
+            if m1 is not None and m2 is not None:
+                c1, c2 = m1.intrin.compute_intrinsic, m2.intrin.compute_intrinsic
+                mi, ni1, ni2 = c1.M, c1.N, c2.N
+            cands = cpu_tensorize_candidates(sfs, state.fuse_choice, hw_param, dtype,
+                                             (d["batch"], d["M"], d["N"], d["K"], d["L"]), mi, ni1, ni2)
+            keep = {"test": 1, "best": 5, "survey": len(cands)}[mode]
+            self.candidates = cands[:keep]
+        self.size = len(self.candidates)
 
     def _check(self, i):
         if not 0 <= i < self.size:
@@ -91,9 +106,10 @@ class FusionContext:
         from .hyper_fusion import tensorize_cpu
 
         self._check(i)
-        out = tensorize_cpu(self.layer, self.state, self.hw_param, None)
+        out = tensorize_cpu(self.layer, self.state, self.hw_param, self.candidates[i])
         if verbose:
             print(self.state.summary(verbose=True))
+            print(self.candidates[i])
         return out
 
     def getComputation(self, i):

@@ -13,6 +13,10 @@ import sys
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB = os.path.join(CSRC, "libditto_chain.so")
 OBJ_DIR = os.path.join(CSRC, "build")
+# the CPU target of the GEMM chain (build(..., target="llvm")): a library of its own, built with g++
+CPU_LIB = os.path.join(CSRC, "libditto_chain_cpu.so")
+CPU_SRC = os.path.join(CSRC, "cpu", "chain_cpu.cpp")
+CPU_FLAGS = ["-O3", "-std=c++17", "-mavx2", "-mfma", "-fopenmp", "-fPIC", "-fvisibility=hidden", "-shared"]
 
 # -packed-fp32-ops is switched off: packed fp32 VALU forms are not wanted in these kernels.
 HIPCC_FLAGS = [
@@ -78,9 +82,23 @@ def _compile(unit):
     return obj
 
 
+def build_cpu(verbose=True):
+    """The CPU target's library (host code only)."""
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if not cxx:
+        raise RuntimeError("g++ not found; the CPU target of the chain needs a host C++ compiler")
+    r = subprocess.run([cxx, *CPU_FLAGS, "-o", CPU_LIB, CPU_SRC], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building %s failed:\n%s" % (CPU_SRC, r.stderr))
+    if verbose:
+        print("built", CPU_LIB)
+    return CPU_LIB
+
+
 def build(verbose=True, jobs=None):
     """Compile every translation unit and link the shared library.  Always rebuilds."""
     os.makedirs(OBJ_DIR, exist_ok=True)
+    build_cpu(verbose)
     jobs = jobs or min(8, os.cpu_count() or 1)
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(_compile, UNITS))

@@ -46,8 +46,8 @@ class ChainFunction:
         if not isinstance(sch, ChainSchedule):
             raise TypeError("build expects the ChainSchedule returned by tensorize_cuda / tensorize_hip")
         if getattr(sch, "target", "hip") != "hip" or target in ("llvm", "cpu", "c"):
-            raise NotImplementedError("this build runs the fused chains on HIP devices only: there is no CPU "
-                                      "product path (target %r)" % (target if target != "hip" else sch.target))
+            raise ValueError("a schedule for the CPU target is built with target \"llvm\" (ditto_amd.build), and a "
+                             "schedule for HIP devices with \"hip\": got schedule %r, target %r" % (sch.target, target))
         if target not in ("hip", "rocm", "cuda"):
             raise ValueError("the fused chains are built for HIP devices only (target %r)" % target)
         self.sch = sch
@@ -181,6 +181,124 @@ class ChainFunction:
         return evaluator
 
 
+class CpuChainFunction:
+    """A GEMM chain built for the CPU target: ``f(A, B, C, F)`` over host tensors (torch CPU tensors or numpy
+    arrays, fp32 / fp64, rows contiguous), blocking like the reference's LLVM-target function.  The fused loop nest
+    is ``libditto_chain_cpu.so`` (``csrc/cpu/chain_cpu.cpp``); its tiling is the schedule's ``CPUTensorizeParam``
+    and its full register tiles run on the micro-kernels compiled from the sources ``cpu_intrin`` generated, where
+    the schedule's match infos carry any (reference flow: benchmark/chimera/cpu/bmm_bmm_cpu.py:118-276)."""
+
+    entry_name = "default_function"
+
+    def __init__(self, sch, tensors=None, name="default_function"):
+        from . import _cpu_lib
+        from .auto_tensorize.hyper_fusion import CPUTensorizeParam
+
+        if sch.kind != "bmm_chain" or sch.in_dtype not in ("float32", "float64"):
+            raise NotImplementedError("the CPU target runs fp32 / fp64 GEMM chains (got %s, %s)" % (sch.kind, sch.in_dtype))
+        if sch.inter_op not in ("cast", "relu", "softmax"):
+            raise NotImplementedError("no CPU nest for inter op %r" % sch.inter_op)
+        self.sch = sch
+        self.tensors = list(tensors) if tensors is not None else sch.layer.schedule_tensors
+        self.target = "llvm"
+        self.entry_name = name
+        self._lib = _cpu_lib.load()
+        p = sch.tensorize_param if isinstance(sch.tensorize_param, CPUTensorizeParam) else CPUTensorizeParam()
+        d = sch.dims
+        self.param = p
+        self._update = [None, None]
+        infos = getattr(sch.state, "match_info", {}) or {}
+        mi, ni1, ni2 = p.mi, p.ni1, p.ni2
+        for slot, op in enumerate((sch.state.first_op, sch.state.second_op)):
+            m = infos.get(op)
+            if m is not None and m.impl:
+                self._update[slot] = _cpu_lib.compile_kernel(m.impl, m.intrin.compute_intrinsic.name)
+                ci = m.intrin.compute_intrinsic
+                if slot == 0:
+                    mi, ni1 = ci.M, ci.N
+                else:
+                    ni2 = ci.N
+        desc = _cpu_lib.CpuChainDesc()
+        desc.abi_version = _cpu_lib.ABI_VERSION
+        desc.dtype = 2 if sch.in_dtype == "float32" else 5
+        desc.inter_op = {"cast": 0, "relu": 1, "softmax": 2}[sch.inter_op]
+        desc.relu_out = int(bool(sch.relu_out))
+        desc.batch, desc.M, desc.N, desc.K, desc.L = d["batch"], d["M"], d["N"], d["K"], d["L"]
+        desc.softmax_scale = float(sch.softmax_scale)
+        desc.mi, desc.ni1, desc.ni2 = mi, ni1, ni2
+        desc.m_block = max(mi, p.m_block // mi * mi) if p.m_block >= mi else mi
+        desc.l_block = max(1, p.l_block)
+        desc.threads = max(0, int(p.parallelism if p.parallelism > 1 else 0))
+        desc.update1, desc.update2 = self._update
+        desc.a_batch_stride, desc.a_row_stride = d["M"] * d["K"], d["K"]
+        desc.b_batch_stride, desc.b_row_stride = d["K"] * d["L"], d["L"]
+        desc.c_batch_stride, desc.c_row_stride = d["L"] * d["N"], d["N"]
+        desc.f_batch_stride, desc.f_row_stride = d["M"] * d["N"], d["N"]
+        self._desc = desc
+
+    @staticmethod
+    def _host(t):
+        import numpy as np
+
+        if isinstance(t, np.ndarray):
+            return t
+        if t.device.type != "cpu":
+            raise ValueError("the CPU target takes host tensors")
+        return t.numpy()
+
+    def __call__(self, *args):
+        if len(args) != len(self.tensors):
+            raise ValueError("expected %d tensors (inputs then outputs), got %d" % (len(self.tensors), len(args)))
+        arrs = [self._host(a) for a in args]
+        d = self.sch.dims
+        want = self.sch.in_dtype
+        total = {"A": d["batch"] * d["M"] * d["K"], "B": d["batch"] * d["K"] * d["L"], "C": d["batch"] * d["L"] * d["N"],
+                 "F": d["batch"] * d["M"] * d["N"]}
+        for a, name in zip(arrs, "ABCF"):
+            # the reference's CPU placeholders are the same row-major memory split into micro-kernel tiles
+            # ([batch, M / MI, MI, K / KI, KI], bmm_bmm_cpu.py:65-69): any contiguous array of the right size does
+            if str(a.dtype) != want or not a.flags["C_CONTIGUOUS"] or a.size != total[name]:
+                raise ValueError("%s must be a contiguous %s array of %d elements, got %s %s" % (name, want, total[name],
+                                                                                             a.dtype, a.shape))
+        import ctypes
+
+        desc = self._desc
+
+        rc = self._lib.ditto_cpu_bmm_chain_run(ctypes.byref(desc), *(a.ctypes.data for a in arrs))
+        if rc != 0:
+            raise ValueError(self._lib.ditto_cpu_last_error().decode("utf-8", "replace"))
+
+    def time_evaluator(self, func_name=None, ctx=None, number=1, repeat=1, min_repeat_ms=0, f_preproc=""):
+        """Mean seconds per call (wall clock; the call is blocking).  ``f_preproc="cache_flush_cpu_non_first_arg"``
+        streams a buffer larger than the last-level cache between measurements, as the reference's CPU drivers ask
+        of TVM (bmm_bmm_cpu.py:264-266)."""
+        import time
+
+        import numpy as np
+
+        flush = np.zeros(64 << 20, dtype=np.uint8) if f_preproc == "cache_flush_cpu_non_first_arg" else None
+
+        def evaluator(*args):
+            self(*args)
+            results = []
+            n = max(1, int(number))
+            for _ in range(max(1, int(repeat))):
+                while True:
+                    if flush is not None:
+                        np.add(flush, 1, out=flush)
+                    t0 = time.perf_counter()
+                    for _ in range(n):
+                        self(*args)
+                    dt = time.perf_counter() - t0
+                    if dt * 1e3 >= min_repeat_ms or n >= (1 << 20):
+                        break
+                    n = max(n + 1, int(n * max(1.5, min_repeat_ms / max(dt * 1e3, 1e-3) * 1.05)))
+                results.append(dt / n)
+            return TimeResult(results)
+
+        return evaluator
+
+
 class AttentionFunction:
     """The built ``multi_head_attention_mma_layer``: ``f(query_key_value, out)`` runs the fused
     BMM -> softmax -> BMM chain over the per-head views of the packed projection."""
@@ -205,4 +323,9 @@ def build(sch, tensors=None, target="hip", name="default_function", tile_variant
 
     if isinstance(sch, AttentionSchedule):
         return AttentionFunction(sch, tensors, target)
+    if target in ("llvm", "cpu", "c"):
+        # the reference's CPU flow ends in tvm.build(sch, tensors, name=...) on the LLVM target (bmm_bmm_cpu.py:251)
+        if getattr(sch, "target", "hip") != "cpu":
+            raise ValueError("target %r needs a schedule from tensorize_cpu / FusionContext.run" % target)
+        return CpuChainFunction(sch, tensors, name)
     return ChainFunction(sch, tensors, target, tile_variant)

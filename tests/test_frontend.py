@@ -400,42 +400,6 @@ def test_int8_chain_builder_and_recognition():
     assert at.tensorize_hip(layer, state, tile_variant=1288).tile_variant == 1288
 
 
-def test_cpu_side_names_describe_but_do_not_build():
-    # the flow of benchmark/chimera/cpu/bmm_bmm_cpu.py:118-276 up to the point where it would compile
-    ins, outs = F.BatchGemmGemm(1, 516, 64, 64, 64, "float32", "float32", MI=6, NI=16, KI=16)
-    layer = ac.layer([outs[0].op], inputs=ins)
-    sfs = at.build_serial_fusion_state(layer)
-    op1, op2 = sfs.first_op, sfs.second_op
-    packed, code = at.cpu_intrin(op="gemm_noreshape", shape=(6, 16, 16), isa="avx2", dtype="float32", prefix="gemm1")
-    assert packed.compute_intrinsic.name == "gemm1_update" and "6 x 16 x 16" in code and packed.store_intrinsic is None
-    assert str(packed).startswith("PackedIntrinsic(")
-    with pytest.raises(ValueError):
-        at.cpu_intrin("gemm", (6, 16, 16), "avx2", "float16")  # the micro-kernels are fp32 / fp64
-    infos = {}
-    for op, prefix in ((op1, "gemm1"), (op2, "gemm2")):
-        pk, cd = at.cpu_intrin("gemm_noreshape", (6, 16, 16), "avx2", "float32", prefix)
-        infos[op] = at.match_info(at.intrinsic_match(op.output(0), pk, ["SameRange"])[0], pk, cd)
-    sfs.register_tensorize_axes(list(infos[op1].axis) + list(infos[op2].axis))
-    cpu = hw.hardware_param(num_groups=16, cacheSizes=[32 * 16, 32 * 1024, 1024 * 1024, 11264 * 1024],
-                            bandwidth=[293.72, 81.72, 38.54, 13.14], coresPerCacheLevel=[1.0, 1.0, 1.0, 16.0],
-                            tensorWeight=[1.0, 2.0, 1.0, 1.0, 1.0], platform="CPU")
-    fc = at.build_fusion_choice(sfs, hw_param=cpu, dtype="float32", simple_mode=-1)
-    state = at.tensorize_hyper_fusion_state(layer, fc, infos)
-    param = at.build_cpu_tensorize_param(sfs, fc, cpu, "float32")
-    assert param.parallelism == 16 and len(param.secondOpLoopOrder) == 7
-    ctx = at.build_fusion_context(sfs, layer, state, "", hw_param=cpu, dtype="float32", searchType="stochastic",
-                                  mode="survey")
-    assert ctx.size == 1 and ctx.getComputation(0) == 516 * 64 * 64 * 2
-    # D_frag's tile under the fused loops (b, mo, no): 6 x 64 fp32 = 1.5 KB -> the 32 KB level
-    assert ctx.getFusionLevel(0) == 1
-    sch = ctx.run(0, None)
-    assert sch.target == "cpu" and sch.kind == "bmm_chain"
-    with pytest.raises(NotImplementedError, match="no CPU product path"):
-        ditto.build(sch, layer.schedule_tensors, "llvm")
-    with pytest.raises(IndexError):
-        ctx.run(1, None)
-
-
 def test_graph_fusion_folds_relu_layers_into_the_producing_chain():
     from ditto_amd import chimera, runtime
 
