@@ -80,6 +80,31 @@ def Conv3x3Conv1x1(batch, in_channel, H, W, out_channel1, out_channel2, stride1=
                       in_dtype, acc_dtype)
 
 
+def Conv1x1Conv1x1(batch, in_channel, H, W, out_channel1, out_channel2, stride1=1, stride2=1,
+                   in_dtype="float16", acc_dtype="float32", relu=False):
+    """conv1x1 -> cast | relu -> conv1x1; argument list of benchmark/chimera/cuda/conv1x1_conv1x1_cuda.py:77-88
+    (``relu=True``: conv1x1_relu_conv1x1.py, the ReLU on the first accumulator, :146-153 of its 3x3 sibling)."""
+    assert stride2 == 1
+    return conv_chain(batch, in_channel, H, W, out_channel1, 1, 1, out_channel2, 1, 1, 0, 0, stride1, stride2,
+                      in_dtype, acc_dtype, relu=relu)
+
+
+def Conv3x3ReluConv1x1(batch, in_channel, H, W, out_channel1, out_channel2, stride1=1, stride2=1,
+                       in_dtype="float16", acc_dtype="float32"):
+    """conv3x3 (pad 1) -> relu -> conv1x1 (benchmark/chimera/cuda/conv3x3_relu_conv1x1.py:77-172)."""
+    assert stride2 == 1
+    return conv_chain(batch, in_channel, H, W, out_channel1, 3, 3, out_channel2, 1, 1, 1, 0, stride1, stride2,
+                      in_dtype, acc_dtype, relu=True)
+
+
+def Conv1x1ReluConv3x3(batch, in_channel, H, W, out_channel1, out_channel2, stride1=1, stride2=1,
+                       in_dtype="float16", acc_dtype="float32"):
+    """conv1x1 -> relu -> conv3x3 (pad 1) (benchmark/chimera/cuda/conv1x1_relu_conv3x3_cuda.py:77-200)."""
+    assert stride2 == 1
+    return conv_chain(batch, in_channel, H, W, out_channel1, 1, 1, out_channel2, 3, 3, 0, 1, stride1, stride2,
+                      in_dtype, acc_dtype, relu=True)
+
+
 def Conv1x1Conv3x3(batch, in_channel, H, W, out_channel1, out_channel2, stride1=1, stride2=1,
                    in_dtype="float16", acc_dtype="float32"):
     """conv1x1 -> cast -> conv3x3 (pad 1, zero padding of the intermediate); argument list of

@@ -55,6 +55,11 @@ CONV3X3_CONV1X1_SHAPES = [
 CONV1X1_CONV3X3_SHAPES = [
     (64, 56, 56, 64, 64, 1, 1),  # ResNet-50
 ]
+# (C, H, W, K1, K2, stride1, stride2): conv1x1_conv1x1_cuda.py:315-318 (and conv1x1_relu_conv1x1.py:326-329)
+CONV1X1_CONV1X1_SHAPES = [
+    (64, 56, 56, 64, 64, 1, 1),  # modified ResNet-50
+    (256, 56, 56, 256, 64, 1, 1),  # modified ResNet-50
+]
 # (C, H, W, K, stride1, stride2): depthwise3x3_conv1x1_small_channel_cuda.py:340-346
 DEPTHWISE3X3_CONV1X1_SHAPES = [
     (32, 112, 112, 64, 1, 1),  # mobilenet-v1
@@ -198,3 +203,67 @@ def check_dtypes(args, int8_ok=False):
     if not ok:
         print(f"Data type not supported: sm_{args.sm}, in_dtype={args.in_dtype}, out_dtype={args.acc_dtype}.")
     return ok
+
+
+def conv_cal_ai(batch, C, H, W, K1, K2, stride1, stride2):
+    """Arithmetic intensity of the two convolutions as the reference's conv drivers print it (--ai)."""
+    return (batch * (H // stride1) * (W // stride1) * K1 / (batch * (H // stride1) * (W // stride1) + K1),
+            batch * (H // stride1 // stride2) * (W // stride1 // stride2) * K2
+            / (batch * (H // stride1 // stride2) * (W // stride1 // stride2) + K2))
+
+
+def conv_chain_main(builder, batch, in_channel, H, W, out_channel1, out_channel2, stride1=1, stride2=1,
+                    in_dtype="float16", acc_dtype="float32", sm="gfx950", only_once=False):
+    """``main`` of a conv -> conv driver: describe the chain the way the reference's drivers do (serial fusion state,
+    the [b, no, p, mo] fusion of the second convolution, one matrix intrinsic per convolution, the tensorize
+    parameters of conv3x3_conv1x1_cuda.py:266-278), build it and measure; failures give the sentinel cost."""
+    from ditto_amd import auto_compute as ac
+    from ditto_amd import auto_tensorize as at
+    from ditto_amd import hardware as hw
+
+    try:
+        ins, outs = builder(batch, in_channel, H, W, out_channel1, out_channel2, stride1, stride2, in_dtype, acc_dtype)
+        layer = ac.layer([outs[0].op], inputs=[ins[0]], weights=ins[1:])
+        sfs = at.build_serial_fusion_state(layer)
+        ok, why = at.validate(sfs)
+        if not ok:
+            raise ValueError(why)
+        conv1, conv2 = sfs.first_op, sfs.second_op
+        n, k, p, q = conv2.axis
+        fuse_choice = at.fusion_choice(conv1, conv2, [n, p, q, k] + list(conv2.reduce_axis), 2)
+        mfma = at.hip_mfma(32, 32, 16, in_dtype, acc_dtype)
+        state = at.tensorize_hyper_fusion_state(layer, fuse_choice, {
+            conv1: at.match_info([conv1.axis[3], conv1.axis[1], conv1.reduce_axis[0]], mfma),
+            conv2: at.match_info([conv2.axis[3], conv2.axis[1], conv2.reduce_axis[0]], mfma)})
+        param = at.cuda_tensorize_param(warp_size=32, ty_size=2, tz_size=2, input_vector_len=8, serial_y=2,
+                                        serial_z=2, block_rx=1, warp_rx=2, block_ry=1, warp_ry=2, unroll_steps=64)
+        sch = at.tensorize_cuda(layer, state, hw.query_hw_param(DEVICES[sm]), param)
+    except Exception as error:
+        print("chain failed:", type(error).__name__, error)
+        return SENTINEL_COST
+    args = random_args(layer, in_dtype, 1)
+    args[1] = args[1] * 0.05
+    args[2] = args[2] * 0.05
+    return evaluate(sch, layer, args, only_once)
+
+
+def conv_chain_cli(main, shapes, example_text):
+    """The command line the reference's conv drivers share: --batch, --begin / --num over the shape table, --ai,
+    the CSV with one cost (ms) per row."""
+    parser = base_parser(example_text, len(shapes))
+    parser.add_argument("--batch", type=int, default=1)
+    args = parser.parse_args()
+    if args.ai:
+        for ss in shapes[args.begin: args.begin + args.num]:
+            print(ss, *conv_cal_ai(args.batch, *ss))
+    elif check_dtypes(args):
+        costs = []
+        for ss in shapes[args.begin: args.begin + args.num]:
+            C, H, W, K1, K2, stride1, stride2 = ss
+            costs.append((ss, main(args.batch, C, H, W, K1, K2, stride1, stride2, args.in_dtype, args.acc_dtype,
+                                   args.sm, args.only_once)))
+        print("batch,C,H,W,K1,K2,stride1,stride2,in_dtype,acc_dtype,sm,cost")
+        for cc in costs:
+            print(f"{args.batch}," + ",".join(map(str, cc[0])) + f",{args.in_dtype},{args.acc_dtype},{args.sm},{cc[1]}")
+        for cc in costs:
+            print(cc[1])

@@ -1,8 +1,6 @@
 """conv3x3 -> conv1x1 chain driver (reference: benchmark/chimera/cuda/conv3x3_conv1x1_cuda.py).
 Takes plain NCHW tensors where the reference's driver takes its packed, pre-padded layout."""
 from ditto_amd import auto_compute as ac
-from ditto_amd import auto_tensorize as at
-from ditto_amd import hardware as hw
 
 from . import common
 
@@ -11,59 +9,14 @@ example_text = """
     python -m ditto_amd.drivers.conv3x3_conv1x1 --in_dtype float16 --acc_dtype float32 --begin 0 --num 1
 """
 shapes = common.CONV3X3_CONV1X1_SHAPES
-
-
-def cal_ai(batch, C, H, W, K1, K2, stride1, stride2):
-    return (batch * (H // stride1) * (W // stride1) * K1 / (batch * (H // stride1) * (W // stride1) + K1),
-            batch * (H // stride1 // stride2) * (W // stride1 // stride2) * K2
-            / (batch * (H // stride1 // stride2) * (W // stride1 // stride2) + K2))
+cal_ai = common.conv_cal_ai
 
 
 def main(batch, in_channel, H, W, out_channel1, out_channel2, stride1=1, stride2=1, in_dtype="float16",
          acc_dtype="float32", sm="gfx950", only_once=False):
-    try:
-        ins, outs = ac.nn.functional.Conv3x3Conv1x1(batch, in_channel, H, W, out_channel1, out_channel2,
-                                                    stride1, stride2, in_dtype, acc_dtype)
-        layer = ac.layer([outs[0].op], inputs=[ins[0]], weights=ins[1:])
-        sfs = at.build_serial_fusion_state(layer)
-        ok, why = at.validate(sfs)
-        if not ok:
-            raise ValueError(why)
-        conv1, conv2 = sfs.first_op, sfs.second_op
-        n, k, p, q = conv2.axis
-        # the reference fuses [b, no, p, mo] of the second convolution (conv3x3_conv1x1_cuda.py:211)
-        fuse_choice = at.fusion_choice(conv1, conv2, [n, p, q, k] + list(conv2.reduce_axis), 2)
-        mfma = at.hip_mfma(32, 32, 16, in_dtype, acc_dtype)
-        state = at.tensorize_hyper_fusion_state(layer, fuse_choice, {
-            conv1: at.match_info([conv1.axis[3], conv1.axis[1], conv1.reduce_axis[0]], mfma),
-            conv2: at.match_info([conv2.axis[3], conv2.axis[1], conv2.reduce_axis[0]], mfma)})
-        param = at.cuda_tensorize_param(warp_size=32, ty_size=2, tz_size=2, input_vector_len=8, serial_y=2,
-                                        serial_z=2, block_rx=1, warp_rx=2, block_ry=1, warp_ry=2, unroll_steps=64)
-        sch = at.tensorize_cuda(layer, state, hw.query_hw_param(common.DEVICES[sm]), param)
-    except Exception as error:
-        print("chain failed:", type(error).__name__, error)
-        return common.SENTINEL_COST
-    args = common.random_args(layer, in_dtype, 1)
-    args[1] = args[1] * 0.05
-    args[2] = args[2] * 0.05
-    return common.evaluate(sch, layer, args, only_once)
+    return common.conv_chain_main(ac.nn.functional.Conv3x3Conv1x1, batch, in_channel, H, W, out_channel1, out_channel2,
+                                  stride1, stride2, in_dtype, acc_dtype, sm, only_once)
 
 
 if __name__ == "__main__":
-    parser = common.base_parser(example_text, len(shapes))
-    parser.add_argument("--batch", type=int, default=1)
-    args = parser.parse_args()
-    if args.ai:
-        for ss in shapes[args.begin: args.begin + args.num]:
-            print(ss, *cal_ai(args.batch, *ss))
-    elif common.check_dtypes(args):
-        costs = []
-        for ss in shapes[args.begin: args.begin + args.num]:
-            C, H, W, K1, K2, stride1, stride2 = ss
-            costs.append((ss, main(args.batch, C, H, W, K1, K2, stride1, stride2, args.in_dtype, args.acc_dtype,
-                                   args.sm, args.only_once)))
-        print("batch,C,H,W,K1,K2,stride1,stride2,in_dtype,acc_dtype,sm,cost")
-        for cc in costs:
-            print(f"{args.batch}," + ",".join(map(str, cc[0])) + f",{args.in_dtype},{args.acc_dtype},{args.sm},{cc[1]}")
-        for cc in costs:
-            print(cc[1])
+    common.conv_chain_cli(main, shapes, example_text)

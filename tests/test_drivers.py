@@ -5,7 +5,8 @@ import sys
 
 import pytest
 
-from ditto_amd.drivers import (bmm_bmm, bmm_softmax_bmm, common, conv1x1_conv3x3, conv3x3_conv1x1,
+from ditto_amd.drivers import (bmm_bmm, bmm_softmax_bmm, common, conv1x1_conv1x1, conv1x1_conv3x3,
+                               conv1x1_relu_conv1x1, conv1x1_relu_conv3x3, conv3x3_conv1x1, conv3x3_relu_conv1x1,
                                depthwise3x3_conv1x1)
 
 
@@ -16,6 +17,9 @@ def test_shape_tables_match_reference():
     assert common.BMM_SHAPES[9] == (1, 512, 64, 64, 256)       # Mixer-Small/32-S: uround(49, 16)
     assert common.CONV3X3_CONV1X1_SHAPES[2] == (64, 56, 56, 128, 64, 1, 1)
     assert common.DEPTHWISE3X3_CONV1X1_SHAPES[3] == (16, 224, 224, 32, 2, 1)
+    assert conv1x1_conv1x1.shapes == conv1x1_relu_conv1x1.shapes == [(64, 56, 56, 64, 64, 1, 1), (256, 56, 56, 256, 64, 1, 1)]
+    assert conv3x3_relu_conv1x1.shapes is common.CONV3X3_CONV1X1_SHAPES
+    assert conv1x1_relu_conv3x3.shapes == [(64, 56, 56, 64, 64, 1, 1)]
     assert common.cal_ai(12, 512, 64, 64, 512) == (256.0, 512 * 64 / 576)
 
 
@@ -45,6 +49,13 @@ def test_drivers_run_one_row_each(capsys):
     C, H, W, K1, K2, s1, s2 = common.CONV1X1_CONV3X3_SHAPES[0]
     cost = conv1x1_conv3x3.main(1, C, H, W, K1, K2, s1, s2)
     assert 0 < cost < 5.0
+    # the sibling drivers of the conv chains (ReLU between the convolutions; conv1x1 -> conv1x1)
+    for drv in (conv1x1_conv1x1, conv1x1_relu_conv1x1, conv3x3_relu_conv1x1, conv1x1_relu_conv3x3):
+        C, H, W, K1, K2, s1, s2 = drv.shapes[-1 if drv is conv1x1_relu_conv3x3 else 0]
+        if drv is conv3x3_relu_conv1x1:
+            C, H, W, K1, K2, s1, s2 = drv.shapes[2]
+        cost = drv.main(1, C, H, W, K1, K2, s1, s2)
+        assert 0 < cost < 5.0, drv.__name__
     for C, H, W, K, s1, s2 in common.DEPTHWISE3X3_CONV1X1_SHAPES:
         cost = depthwise3x3_conv1x1.main(1, C, H, W, K, 16, s1, s2)
         assert 0 < cost < 5.0

@@ -453,3 +453,18 @@ def test_graph_fusion_folds_relu_layers_into_the_producing_chain():
     cl = ac.layer([couts[0].op], inputs=[cins[0]], weights=cins[1:], name="conv_chain")
     g5 = chimera.graph_fusion(runtime.Graph([cl, relu_layer([2, 48, 16, 16])], edges={(1, 0): (0, 0)}))
     assert len(g5.layers) == 1 and g5.layers[0].ops[0].kind == "relu_cast" and len(g5.layers[0].weights) == 2
+
+
+def test_the_reference_import_name_resolves():
+    """``from ditto import auto_compute as ac`` etc. (the first lines of the reference's drivers) give the modules of
+    this package."""
+    import ditto
+    import ditto.auto_tensorize as at_ref
+    from ditto import auto_compute as ac_ref
+    from ditto.auto_compute.nn.functional import BatchGemmSoftmaxGemmMMA  # noqa: F401
+    from ditto.hardware.hw_param import hardware_param
+
+    import ditto_amd
+    assert ac_ref is ditto_amd.auto_compute and at_ref is ditto_amd.auto_tensorize
+    assert hardware_param is ditto_amd.hardware.hardware_param and ditto.build is ditto_amd.build
+    assert ditto.chimera is ditto_amd.chimera and ditto.runtime.Graph is ditto_amd.runtime.Graph
