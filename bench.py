@@ -32,29 +32,23 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "i8": 5000.0, "f32": 157.3}
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a copy kernel of known
-# size (FETCH_SIZE reads half of a plain copy's bytes on this device: scale factor 2.00; WRITE_SIZE all of
-# them); the summaries are under profiles/.  Each figure belongs to the kernel variant it was measured on
-# (``tile.variant``): when the library picks another variant for the workload the figure is stale and
-# ``roofline.traffic`` is reported as null.
-MEASURED_TRAFFIC = {
-    # workload: (FETCH MiB, WRITE MiB, tile variant measured)
-    "attn_bf16_b64_s4096_d128": (192.28, 64.00, 1286),
-    "gemm_chain_bf16_b64_4096x128x4096x128": (192.30, 64.00, 1282),
-    "attn_f16_b96_s512_d64": (18.21, 6.00, 649),
-    "conv_chain_f16_n32_c64_56x56_k64_k256": (13.30, 50.00, 3707),
-    "gemm_chain_i8_8192x1024x256x1024": (12.15, 32.00, 8014),
-    "conv1x1_conv3x3_f16_n32_c64_56x56_k64_k64": (13.10, 12.50, 3807),
-    "dw3x3_conv1x1_f16_n32_c32_112x112_f16_k64": (29.18, 49.50, 4025),
-    "dw3x3_conv1x1_f16_n32_c32_112x112_x1_k64": (24.64, 49.00, 4024),
-}
-
-
+# HBM bytes per launch come from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/ (each counter
+# scaled by what it reads for a plain copy of known size in the same run: FETCH_SIZE reads half of a copy's bytes on
+# this device, factor 2.00, WRITE_SIZE all of them).  A summary belongs to the kernel variant named in its header
+# ("tile variant N"): when the library picks another variant for the workload, or no summary exists, the figure
+# would be stale and ``roofline.traffic`` is null.
 def measured_traffic(name, variant):
-    rec = MEASURED_TRAFFIC.get(name)
-    if rec is None or rec[2] != variant:
-        return None
-    return int((rec[0] + rec[1]) * 2 ** 20)
+    import glob
+    import re
+
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*__%s.txt" % name))):
+        text = open(path).read()
+        m = re.search(r"tile variant (\d+)", text)
+        f = re.search(r"^FETCH_SIZE: .* scaled ([0-9.]+) MiB per launch", text, re.M)
+        w = re.search(r"^WRITE_SIZE: .* scaled ([0-9.]+) MiB per launch", text, re.M)
+        if m and f and w and int(m.group(1)) == int(variant):
+            return int((float(f.group(1)) + float(w.group(1))) * 2 ** 20)
+    return None
 
 
 WORKLOADS = {
