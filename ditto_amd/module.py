@@ -61,9 +61,50 @@ class ChainFunction:
     def _check_args(self, args):
         if len(args) != len(self.tensors):
             raise ValueError("expected %d tensors (inputs then outputs), got %d" % (len(self.tensors), len(args)))
+        if self.sch.kind == "conv_chain" and args[0].dim() == 5:
+            return  # the reference's packed placeholders: checked in _call_packed
         for a, t in zip(args, self.tensors):
             if tuple(a.shape) != tuple(t.shape):
                 raise ValueError("argument for %s has shape %s, expected %s" % (t.name, tuple(a.shape), t.shape))
+
+    def _call_packed(self, img_p, w1_p, w2_p, out_p):
+        """The reference's calling convention for conv chains: packed, pre-padded tensors
+        (conv3x3_conv1x1_cuda.py:90-105; ``ditto_amd.layout``).  The padded image is unpacked to NCHW and the first
+        convolution runs over it without padding (the border is the caller's, as in the reference); the weights are
+        unpacked once per pair of weight tensors (kept like ``specialize`` keeps its weights: by identity and
+        version); the result is packed into ``out_p``.  Stride 1."""
+        from . import layout
+
+        d = self.sch.dims
+        if d["stride1"] != 1 or d["stride2"] != 1:
+            raise NotImplementedError("packed placeholders are taken for stride 1 chains")
+        N, C0, H, W = d["N"], d["C0"], d["H"], d["W"]
+        pad1 = d["pad1"]
+        Q = (W + 2 * pad1 - d["S1"]) + 1 + 2 * d["pad2"] - d["S2"] + 1
+        P = (H + 2 * pad1 - d["R1"]) + 1 + 2 * d["pad2"] - d["R2"] + 1
+        if tuple(img_p.shape[:3]) != (N, C0 // 16, H + 2 * pad1) or img_p.shape[3] < W + 2 * pad1 or C0 % 16:
+            raise ValueError("packed image must be [%d, %d, %d, >= %d, 16], got %s"
+                             % (N, C0 // 16, H + 2 * pad1, W + 2 * pad1, tuple(img_p.shape)))
+        x = layout.unpack_image(img_p, W + 2 * pad1)
+        cache = getattr(self, "_packed_weights", None)
+        if not (cache and cache[0] is w1_p and cache[1] is w2_p and cache[2] == (w1_p._version, w2_p._version)):
+            cache = (w1_p, w2_p, (w1_p._version, w2_p._version), layout.unpack_weight(w1_p), layout.unpack_weight(w2_p))
+            self._packed_weights = cache
+        w1, w2 = cache[3], cache[4]
+        want1 = (d["C1"], C0 // d.get("groups1", 1), d["R1"], d["S1"])
+        if tuple(w1.shape) != want1 or tuple(w2.shape) != (d["C2"], d["C1"], d["R2"], d["S2"]):
+            raise ValueError("packed weights do not match the chain: %s, %s" % (tuple(w1_p.shape), tuple(w2_p.shape)))
+        f = getattr(self, "_packed_fn", None)
+        if f is None:  # the same chain with the first padding taken out of the kernel's hands
+            import copy
+
+            sch = copy.copy(self.sch)
+            sch.dims = dict(d, H=H + 2 * pad1, W=W + 2 * pad1, pad1=0)
+            f = self._packed_fn = ChainFunction(sch, [None] * 4, self.target, self.tile_variant)
+            f._check_args = lambda args: None
+        y = torch.empty((N, d["C2"], P, Q), device=x.device, dtype=out_p.dtype)
+        f(x, w1, w2, y)
+        layout.pack_output_into(y, out_p)
 
     @staticmethod
     def _layout(args):
@@ -134,6 +175,8 @@ class ChainFunction:
             chain.run_bmm_chain(A, B, C, F, aux=aux, desc=desc)
         elif s.kind == "conv_chain":
             X, W1, W2, Y = args
+            if X.dim() == 5:
+                return self._call_packed(X, W1, W2, Y)
             desc = self._conv_desc(X, W1, W2, Y)
             ws = self._workspace(desc, X.device)
             prepared = ws is not False and self._is_prepared(W1, W2)

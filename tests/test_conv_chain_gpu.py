@@ -827,3 +827,64 @@ def test_overflowed_outputs_of_the_conv1x1_conv3x3_row_pipeline():
     assert float((o[0, :5][:, clean] - ref[0, :5][:, clean]).abs().max()) <= 1e-2
     assert not torch.isnan(o[0, 32:]).any()                              # the other block of 32 channels: untouched
     assert torch.isnan(o[0, :32][:, over]).sum() > 0                     # the documented divergence
+
+
+@pytest.mark.parametrize("first", ["3x3", "1x1"])
+def test_packed_placeholders_of_the_reference(oracle, first):
+    """The reference's calling convention for its GPU conv drivers: packed, pre-padded tensors
+    (conv3x3_conv1x1_cuda.py:90-105 and :164-170; conv1x1_conv3x3_cuda.py:90-105).  The built function takes them as they
+    are; the index maps are restated here with plain loops-free numpy against the NCHW result of the checker,
+    including a border the caller filled with something other than zeros (which the reference's index expression
+    reads like any other pixel)."""
+    import ditto_amd as ditto
+    from ditto_amd import auto_compute as ac, layout
+    from ditto_amd.drivers import common
+
+    N, C0, H, W, C1, C2 = 2, 32, 12, 16, 64, 48
+    Fn = ac.nn.functional
+    if first == "3x3":
+        ins, outs = Fn.Conv3x3Conv1x1(N, C0, H, W, C1, C2)
+        R1, R2, pad1, pad2 = 3, 1, 1, 0
+    else:
+        ins, outs = Fn.Conv1x1Conv3x3(N, C0, H, W, C1, C2)
+        R1, R2, pad1, pad2 = 1, 3, 0, 1
+    layer = ac.layer([outs[0].op], inputs=[ins[0]], weights=ins[1:])
+    func = ditto.build(common.describe_layer(layer), layer.schedule_tensors, "hip")
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, R1, R2, "float16", seed=31, w_std=0.05)
+    rng = np.random.default_rng(2)
+    # the packed image as the reference's host code lays it out: [N, C/16, H + 2 pad, W + 2 pad + 1, 16], border NOT zero
+    Xp = rng.standard_normal((N, C0, H + 2 * pad1, W + 2 * pad1)).astype(np.float32)
+    Xp = oracle.np_round_to(Xp, "float16")
+    Xp[:, :, pad1:pad1 + H, pad1:pad1 + W] = X
+    img_np = np.zeros((N, C0 // 16, H + 2 * pad1, W + 2 * pad1 + 1, 16), np.float32)
+    img_np[:, :, :, :W + 2 * pad1, :] = Xp.reshape(N, C0 // 16, 16, H + 2 * pad1, W + 2 * pad1).transpose(0, 1, 3, 4, 2)
+    w1_np = W1.reshape(C1 // 16, 16, C0 // 16, 16, R1, R1).transpose(4, 5, 2, 0, 3, 1)      # [r, s, co, ko, ci, ki]
+    w2_np = W2.reshape(C2 // 16, 16, C1 // 16, 16, R2, R2).transpose(4, 5, 2, 0, 3, 1)
+    if R1 == 1:
+        w1_np = w1_np[0, 0]
+    if R2 == 1:
+        w2_np = w2_np[0, 0]
+    img_p, w1_p, w2_p = (to_dev(np.ascontiguousarray(t), "float16") for t in (img_np, w1_np, w2_np))
+    out_p = torch.full((N, C2 // 16, H, W, 16), float("nan"), device=img_p.device, dtype=torch.float16)
+    func(img_p, w1_p, w2_p, out_p)
+    torch.cuda.synchronize()
+    # the checker on the padded image without further padding of the first convolution
+    want = oracle.conv_chain_f32(Xp, W1, W2, 0, 1, pad2, 1, round_mid="float16")
+    got = out_p.float().cpu().numpy().transpose(0, 1, 4, 2, 3).reshape(N, C2, H, W)
+    mx, rel = errors(got, oracle.np_round_to(want, "float16"))
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
+    # the layout helpers are each other's inverses, and agree with the maps written out above
+    assert torch.equal(layout.pack_weight(layout.unpack_weight(w1_p)), w1_p)
+    assert torch.equal(layout.unpack_image(img_p, W + 2 * pad1).float().cpu(), torch.from_numpy(Xp))
+    assert torch.equal(layout.pack_image(to_dev(X, "float16"), pad1, 1)[:, :, pad1:pad1 + H, pad1:pad1 + W],
+                       img_p[:, :, pad1:pad1 + H, pad1:pad1 + W])
+    # a second call with the same packed weights reuses their unpacked form; updated weights are unpacked again
+    cached = func._packed_weights[3]
+    func(img_p, w1_p, w2_p, out_p)
+    assert func._packed_weights[3] is cached
+    w1_p.mul_(0.5)
+    func(img_p, w1_p, w2_p, out_p)
+    torch.cuda.synchronize()
+    got2 = out_p.float().cpu().numpy().transpose(0, 1, 4, 2, 3).reshape(N, C2, H, W)
+    want2 = oracle.conv_chain_f32(Xp, W1 * 0.5, W2, 0, 1, pad2, 1, round_mid="float16")
+    assert errors(got2, oracle.np_round_to(want2, "float16"))[1] <= REL_L2
