@@ -14,6 +14,7 @@
 
 #include "bmm_chain_fp8.h"
 #include "bmm_chain_fp8m16.h"
+#include "bmm_chain_fp4m16.h"
 #include "chain_kernels.h"
 
 namespace {
@@ -162,14 +163,15 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     // CUs.  From there on eight waves (two per SIMD) win, in their software-pipelined form (9) at every
     // size measured.  Once there are two workgroups per CU the chip runs at its power limit and the
     // kernel on the 16x16x32 MFMA (6; B stored [L][K] only), which needs less energy per flop, is ahead
-    // (64 x 4096 x 4096 x 128 bf16: 464 vs 484 us with the softmax, 410 vs 443 us without); the
-    // exception is head_pad 64 with the softmax (306 vs 314 us).  With B stored [K][L] and no softmax
-    // (nothing for a second wave per SIMD to overlap) the four-wave, 256-row kernel stays (429 vs 443 us).
+    // (64 x 4096 x 4096 x 128 bf16: 464 vs 484 us with the softmax, 410 vs 443 us without); at
+    // head_pad 64 the pipelined kernel stays (32 x 4096 x 4096 x 64 without softmax 127.9 vs 130.0 us).
+    // With B stored [K][L] and no softmax (nothing for a second wave per SIMD to overlap) the four-wave,
+    // 256-row kernel stays (429 vs 443 us).
     const long long n8 = ((d->M + 255) / 256) * d->batch;
     const bool sm = d->inter_op == DITTO_INTER_SOFTMAX;
     if (n8 >= 2LL * cus) {
       if (d->b_layout == DITTO_B_LK)
-        plan->qt = (sm && plan->d_pad == 64) ? 9 : 6;
+        plan->qt = plan->d_pad == 64 ? 9 : 6;
       else
         plan->qt = sm ? 9 : 2;
     } else if (n8 * 4 >= 3LL * cus) {
@@ -177,16 +179,39 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     } else {
       plan->qt = 1;
     }
+    // Head size up to 64 with B stored [L][K]: the four-wave kernels with 64-row workgroups (4: a wave owns 16 rows
+    // and all keys; 5: 32 rows and half the keys of every tile, half the LDS reads per MFMA for a merge at the end,
+    // ahead from 1024 keys on).  Measured, fp16 and bf16, us per launch in a graph replay, best other variant ->
+    // best of 4 | 5: softmax 96 x 512 x 512 13.2 -> 11.5, 12 x 512 x 512 9.9 -> 6.9, 8 x 1024 x 1024 15.5 -> 9.9,
+    // 16 x 512 x 2048 26.3 -> 15.5, 768 x 512 x 512 84.5 -> 78.1, 96 x 2048 x 2048 fp16 119.3 -> 116.7; bf16 at that
+    // size and beyond stays on the eight-wave 16x16x32 kernel (115.6 against 120.1; 32 x 4096 x 4096 139.9 against
+    // 150.6).  Without the softmax they are ahead below two 256-row workgroups per CU (96 x 512 x 512 11.2 -> 10.7,
+    // 16 x 512 x 2048 17.0 -> 14.6) and behind from there on (384 x 512 x 512 38.9 against 39.3); where the 64-row
+    // workgroups make one and a half rounds of the CUs and the 128-row ones fit in one, the latter stay
+    // (48 x 512 x 512 7.5 against 8.2).
+    if (plan->d_pad == 64 && d->b_layout == DITTO_B_LK) {
+      const long long n64 = ((d->M + 63) / 64) * d->batch, n128 = ((d->M + 127) / 128) * d->batch;
+      bool rows64;
+      if (sm)
+        rows64 = !(in == DITTO_BF16 && n8 >= 2LL * cus && d->L >= 2048);
+      else
+        rows64 = n8 < 2LL * cus && !(n64 > cus && n128 <= cus);
+      if (rows64) plan->qt = d->L >= 1024 ? 5 : 4;
+      else if (sm && n8 >= 2LL * cus) plan->qt = 6;
+    }
     if (d->tile_variant != 0) {
       const int q = d->tile_variant % 10;
-      if (d->tile_variant / 10 != plan->d_pad || (q != 1 && q != 2 && q != 8 && q != 9 && q != 6 && q != 7))
-        return fail(DITTO_EINVAL, "tile_variant %d cannot run this shape (head_pad %d; q must be 1, 2, 6, 7, 8 or 9)",
+      if (d->tile_variant / 10 != plan->d_pad || (q != 1 && q != 2 && q != 4 && q != 5 && q != 8 && q != 9 && q != 6 && q != 7))
+        return fail(DITTO_EINVAL, "tile_variant %d cannot run this shape (head_pad %d; q must be 1, 2, 4, 5, 6, 7, 8 or 9)",
                     d->tile_variant, plan->d_pad);
-      if ((q == 6 || q == 7) && d->b_layout != DITTO_B_LK)
+      if ((q == 4 || q == 5 || q == 6 || q == 7) && d->b_layout != DITTO_B_LK)
         return fail(DITTO_EINVAL, "tile_variant %d (16x16x32 MFMA kernel) takes B stored [L][K]", d->tile_variant);
+      if ((q == 4 || q == 5) && plan->d_pad != 64)
+        return fail(DITTO_EINVAL, "tile_variant %d: the 64-row kernel serves head_pad 64 only", d->tile_variant);
       plan->qt = q;
     }
     const bool kl = d->b_layout == DITTO_B_KL;
+    const bool four16 = plan->qt == 4 || plan->qt == 5;  // four waves, 64-row workgroups
     const bool eight = plan->qt >= 6;  // 6, 8, 9: eight waves owning 32 rows each; 7: 48 rows each in some workgroups
     const bool m16 = plan->qt == 6 || plan->qt == 7;
     if (plan->qt == 6 && d->tile_variant == 0 && plan->d_pad == 128) {
@@ -197,14 +222,16 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
       plan->nb3 = plan_rows_384(d->M, d->batch, cus);
       if (plan->nb3 == 0 && d->M > 256) plan->nb3 = 1;  // asked for by tile_variant: at least one large block to show for it
     }
-    const int bm = eight ? 256 : 128 * plan->qt;
+    const int bm = four16 ? 64 : eight ? 256 : 128 * plan->qt;
     ditto_tile_param& t = plan->tile;
     t.block_threads = eight ? 512 : 256;
     t.block_m = bm;
     t.block_l = ditto::kBN;
     t.block_n = (int)d->N;
     t.head_pad = plan->d_pad;
-    if (m16)
+    if (four16)
+      t.lds_bytes = ditto::bmm_chain4m16_lds_bytes<64>();
+    else if (m16)
       t.lds_bytes = plan->d_pad == 64 ? ditto::bmm_chain8m16_lds_bytes<64>() : ditto::bmm_chain8m16_lds_bytes<128>();
     else if (eight)
       t.lds_bytes = plan->d_pad == 64 ? (kl ? ditto::bmm_chain8_lds_bytes<64, true>() : ditto::bmm_chain8_lds_bytes<64, false>())

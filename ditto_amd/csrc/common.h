@@ -160,6 +160,17 @@ __device__ __forceinline__ void lds_dma_16(i32x4 rsrc, unsigned voffset, unsigne
       : "v"(voffset), "s"(rsrc), "s"(lds_base)
       : "memory", "m0");
 }
+// The same with the LDS address given as a wave-uniform base plus a constant known once the call is inlined: a
+// kernel that fills many tile slots keeps one base register instead of one address register per slot and load.
+__device__ __forceinline__ void lds_dma_16_at(i32x4 rsrc, unsigned voffset, unsigned lds_base, int const_off) {
+  asm volatile(
+      "s_add_u32 m0, %2, %3\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %0, %1, 0 offen lds"
+      :
+      : "v"(voffset), "s"(rsrc), "s"(lds_base), "i"(const_off)
+      : "memory", "m0", "scc");
+}
 // raw buffer resource (stride 0, range checked against `bytes`) as four dwords
 __device__ __forceinline__ i32x4 make_rsrc(const void* base, unsigned bytes) {
   const unsigned long long a = reinterpret_cast<unsigned long long>(base);
@@ -207,7 +218,9 @@ __device__ __forceinline__ void wg_sync() {
 template <int D>
 __host__ __device__ constexpr int tile_row_bytes() { return 2 * D + 16; }
 
-template <typename T, int D, int ROWS>
+// WT: the stores are written through (see kStoreWriteThrough): for a kernel whose only stores come at its very end,
+// so that no dirty lines are left for the release at the end of the dispatch to write back.
+template <typename T, int D, int ROWS, bool WT = false>
 __device__ __forceinline__ void store_tile_rows(const char* tw, T* f0, long long f_rs, int rows_valid, int N, int lane) {
   typedef typename Elem<T>::v8 V8;
   constexpr int CPR = D / 8;  // 16-byte chunks per row
@@ -216,7 +229,11 @@ __device__ __forceinline__ void store_tile_rows(const char* tw, T* f0, long long
   for (int i = 0; i < ROWS * CPR / 64; ++i) {
     const int v = 64 * i + lane, r = v / CPR, ch = v - r * CPR;
     const V8 x = *reinterpret_cast<const V8*>(tw + r * tile_row_bytes<D>() + ch * 16);
-    if (r < rows_valid && 8 * ch < N) *reinterpret_cast<V8*>(f0 + (long long)r * f_rs + 8 * ch) = x;
+    if (r < rows_valid && 8 * ch < N) {
+      V8* const dst = reinterpret_cast<V8*>(f0 + (long long)r * f_rs + 8 * ch);
+      if (WT) asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(dst), "v"(x) : "memory");
+      else *dst = x;
+    }
   }
 }
 

@@ -70,18 +70,27 @@ def test_select_tile_and_validation_without_gpu():
     lib = _lib.load()
     tile = _lib.TileParam()
     assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc()), ctypes.byref(tile)) == _lib.OK
-    assert tile.block_threads in (256, 512) and tile.block_m in (128, 256, 384) and tile.head_pad == 64
-    assert tile.grid_x == (512 // tile.block_m) * 96 and tile.lds_bytes <= 160 * 1024
+    # 96 heads of 512 rows, head size 64, keys stored [L][K]: 64-row workgroups, three per compute unit
+    assert (tile.variant, tile.block_threads, tile.block_m, tile.head_pad) == (644, 256, 64, 64)
+    assert tile.grid_x == (512 // tile.block_m) * 96 and 3 * tile.lds_bytes <= 160 * 1024
+    long_keys = _desc(L=2048, b_batch_stride=2048 * 64, c_batch_stride=2048 * 64)
+    assert lib.ditto_bmm_chain_select_tile(ctypes.byref(long_keys), ctypes.byref(tile)) == _lib.OK and tile.variant == 645
     # every fp variant can be forced through the descriptor; ids come back in tile.variant
-    for q, threads, bm in ((1, 256, 128), (2, 256, 256), (8, 512, 256), (9, 512, 256), (6, 512, 256), (7, 512, 384)):
+    for q, threads, bm in ((1, 256, 128), (2, 256, 256), (8, 512, 256), (9, 512, 256), (6, 512, 256), (7, 512, 384),
+                           (4, 256, 64), (5, 256, 64)):
         assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(tile_variant=640 + q)), ctypes.byref(tile)) == _lib.OK
         assert (tile.variant, tile.block_threads, tile.block_m) == (640 + q, threads, bm)
         assert tile.lds_bytes <= 160 * 1024
     assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(tile_variant=1288)), ctypes.byref(tile)) == _lib.EINVAL
     assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(tile_variant=643)), ctypes.byref(tile)) == _lib.EINVAL
     # the kernel on the 16x16x32 MFMA reads B stored [L][K] only
-    kl = _desc(tile_variant=646, b_layout=_lib.B_KL, b_row_stride=512)
-    assert lib.ditto_bmm_chain_select_tile(ctypes.byref(kl), ctypes.byref(tile)) == _lib.EINVAL
+    for v in (646, 644, 645):
+        kl = _desc(tile_variant=v, b_layout=_lib.B_KL, b_row_stride=512)
+        assert lib.ditto_bmm_chain_select_tile(ctypes.byref(kl), ctypes.byref(tile)) == _lib.EINVAL
+    # the 64-row kernels serve head sizes up to 64
+    wide = _desc(tile_variant=1284, N=128, K=128, a_row_stride=128, b_row_stride=128, c_row_stride=128, f_row_stride=128,
+                 a_batch_stride=512 * 128, b_batch_stride=512 * 128, c_batch_stride=512 * 128, f_batch_stride=512 * 128)
+    assert lib.ditto_bmm_chain_select_tile(ctypes.byref(wide), ctypes.byref(tile)) == _lib.EINVAL
     # the library's own choice: two 256-row workgroups per CU and B stored [L][K] -> that kernel, with eight of a
     # head's row blocks 384 rows tall and four 256 (4096 rows on four compute units: 2 x 384 + 256 each)
     big = _desc(in_dtype=_lib.BF16, out_dtype=_lib.BF16, batch=64, M=4096, L=4096, N=128, K=128, a_row_stride=128,

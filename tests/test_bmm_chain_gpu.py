@@ -38,9 +38,11 @@ def variants(K, N, b_layout="LK"):
     """0 (the library's own choice) and every kernel variant that can run the head size:
     four waves x 32 rows, four waves x 64 rows, eight waves x 32 rows (staggered phases; software
     pipelined; on the 16x16x32 MFMA, which takes B stored [L][K] only, with 256-row workgroups and with
-    384-row ones for the first row blocks)."""
+    384-row ones for the first row blocks), four waves with 64-row workgroups on the 16x16x32 MFMA (head
+    size up to 64, B stored [L][K]: a wave owns 16 rows and all keys, or 32 rows and half the keys)."""
     pad = 64 if max(K, N) <= 64 else 128
-    return [0] + [pad * 10 + q for q in ((1, 2, 8, 9, 6, 7) if b_layout == "LK" else (1, 2, 8, 9))]
+    codes = (1, 2, 8, 9, 6, 7) + ((4, 5) if pad == 64 else ())
+    return [0] + [pad * 10 + q for q in (codes if b_layout == "LK" else (1, 2, 8, 9))]
 
 
 def run_chain(A, B, C, dtype, inter, scale=1.0, b_layout="KL", out_dtype=None, variant=0):
@@ -183,7 +185,7 @@ def test_fused_cpu_nest_agrees_with_gpu(oracle):
     assert mx <= MAX_ABS and rel <= REL_L2
 
 
-@pytest.mark.parametrize("variant", [641, 642, 648, 649, 646])
+@pytest.mark.parametrize("variant", [641, 642, 648, 649, 646, 644, 645])
 def test_softmax_invariants_on_gpu(oracle, variant):
     batch, M, N, K, L = 2, 160, 64, 64, 264
     A, B, C = oracle.make_gemm_chain_inputs(batch, M, N, K, L, "float16", seed=9)
@@ -197,7 +199,7 @@ def test_softmax_invariants_on_gpu(oracle, variant):
                     "softmax", 0.125, "LK", "float32", variant)
     assert errors(got, base)[1] <= 5e-4
     # Q = 0 -> O = column means of V
-    zero = run_chain(np.zeros_like(A), B, C, "float16", "softmax", 0.125, "LK" if variant % 10 == 6 else "KL",
+    zero = run_chain(np.zeros_like(A), B, C, "float16", "softmax", 0.125, "LK" if variant % 10 in (4, 5, 6) else "KL",
                      "float32", variant)
     assert np.abs(zero - C.mean(axis=1, keepdims=True)).max() <= 1e-3
     # large scores do not overflow (the reference's exp-without-max form does)
@@ -208,7 +210,7 @@ def test_softmax_invariants_on_gpu(oracle, variant):
     assert np.isfinite(hot).all() and errors(hot, want)[0] <= MAX_ABS
 
 
-@pytest.mark.parametrize("variant", [0, 641, 642, 648, 649, 646, 647])
+@pytest.mark.parametrize("variant", [0, 641, 642, 648, 649, 646, 647, 644, 645])
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
 def test_running_maximum_paths(oracle, variant, dtype):
     """What the lazily raised row maximum has to survive: every score far below zero from the first key on (the
