@@ -673,11 +673,23 @@ int plan_conv_steered(const ditto_conv_chain_desc* d, const ConvSteer& steer, Co
   const bool dw = d->groups1 != 0 && d->groups1 != 1;
   if (dw && d->groups1 != d->C0) return fail(DITTO_EUNSUPPORTED, "groups1 must be 1 (dense) or C0 (depthwise)");
   const bool second_1x1 = d->R2 == 1 && d->S2 == 1 && d->pad2 == 0;
-  if (d->stride2 != 1) return fail(DITTO_EUNSUPPORTED, "the second convolution must have stride 1");
+  // A strided 1x1 second convolution keeps every stride2-th pixel of the intermediate image and nothing else: the
+  // chain is the same chain with the first convolution strided by stride1 * stride2 (output p of the second reads
+  // intermediate p * stride2, i.e. input rows from p * stride1 * stride2 - pad1 on; the number of outputs agrees,
+  // floor(floor(x / s1) / s2) = floor(x / (s1 s2))).  Planned and run that way.
+  ditto_conv_chain_desc folded;
+  if (second_1x1 && d->stride2 > 1) {
+    if (d->stride1 * d->stride2 > 0x7fff) return fail(DITTO_EINVAL, "strides too large");
+    folded = *d;
+    folded.stride1 = d->stride1 * d->stride2;
+    folded.stride2 = 1;
+    d = &folded;
+  }
+  if (dw && d->stride2 != 1) return fail(DITTO_EUNSUPPORTED, "depthwise chain: the second convolution must be 1x1");
   if (!dw) {
-    if (!second_1x1 && (d->R2 > 3 || d->S2 > 3 || d->C1 > 128))
-      return fail(DITTO_EUNSUPPORTED,
-                  "a second convolution larger than 1x1 takes filters up to 3x3 and at most 128 intermediate channels");
+    if (!second_1x1 && (d->R2 > 3 || d->S2 > 3))
+      return fail(DITTO_EUNSUPPORTED, "a second convolution larger than 1x1 takes filters up to 3x3");
+    if (!second_1x1 && d->stride2 > 4) return fail(DITTO_EUNSUPPORTED, "second convolution: strides up to 4");
     if (d->C1 % 8) return fail(DITTO_EINVAL, "C1 must be a multiple of 8");
     if (d->C1 > 256) return fail(DITTO_EUNSUPPORTED, "C1=%lld: at most 256 intermediate channels", (long long)d->C1);
   }
@@ -702,13 +714,16 @@ int plan_conv_steered(const ditto_conv_chain_desc* d, const ConvSteer& steer, Co
   if (!second_1x1) {
     // The first convolution produces the output tile grown by the second filter's halo (recomputed
     // per workgroup) into at most `slots` pixel slots; the second reads it from LDS.
-    const long long P2 = P + 2 * d->pad2 - d->R2 + 1, Q2 = Q + 2 * d->pad2 - d->S2 + 1;
+    const int s2 = (int)d->stride2;
+    if (P + 2 * d->pad2 < d->R2 || Q + 2 * d->pad2 < d->S2) return fail(DITTO_EINVAL, "empty convolution output");
+    const long long P2 = (P + 2 * d->pad2 - d->R2) / s2 + 1, Q2 = (Q + 2 * d->pad2 - d->S2) / s2 + 1;
     if (P2 <= 0 || Q2 <= 0) return fail(DITTO_EINVAL, "empty convolution output");
     if (d->N * d->C2 * P2 * Q2 > 0x7fffffffLL * 4) return fail(DITTO_EINVAL, "tensor too large");
     a.R2 = (int)d->R2; a.S2 = (int)d->S2; a.pad2 = (int)d->pad2; a.P2 = (int)P2; a.Q2 = (int)Q2;
+    a.stride2 = s2;
     // 1x1 -> 3x3 (pad 1) with at most 64 channels everywhere, 16-bit output and image rows of whole 16-byte
     // vectors up to 64 pixels: the row pipeline with the 1x1 convolution in its transposing stage (conv_rows.h)
-    if (allow_resident && steer.rows && d->R1 == 1 && d->S1 == 1 && d->pad1 == 0 &&
+    if (allow_resident && steer.rows && s2 == 1 && d->R1 == 1 && d->S1 == 1 && d->pad1 == 0 &&
         d->stride1 == 1 && d->R2 == 3 && d->S2 == 3 && d->pad2 == 1 && d->C0 <= ditto::kCvrC && d->C1 <= ditto::kCvrC &&
         d->C2 <= ditto::kCvrC && d->C0 % 8 == 0 && d->W % 8 == 0 && d->W <= 64 && d->out_dtype != DITTO_F32 &&
         d->C0 * d->H * d->W * 2 < 0x7fffffffLL) {
@@ -757,7 +772,7 @@ int plan_conv_steered(const ditto_conv_chain_desc* d, const ConvSteer& steer, Co
     }
     // 1x1 -> 3x3 (pad 1) with at most 64 channels everywhere and rows that are whole 16-byte vectors: the
     // persistent kernel that keeps W2 in LDS (conv_chain_resident.h), tiles of whole output rows
-    if (allow_resident && steer.resident && d->R1 == 1 && d->S1 == 1 && d->pad1 == 0 && d->stride1 == 1 && d->R2 == 3 &&
+    if (allow_resident && steer.resident && s2 == 1 && d->R1 == 1 && d->S1 == 1 && d->pad1 == 0 && d->stride1 == 1 && d->R2 == 3 &&
         d->S2 == 3 && d->pad2 == 1 && d->C0 <= ditto::kCrC && d->C1 <= ditto::kCrC && d->C2 <= ditto::kCrC &&
         d->C0 % 8 == 0 && d->W % 8 == 0 && d->W <= 256 &&
         d->C0 * d->H * d->W * 2 < 0x7fffffffLL) {
@@ -795,12 +810,14 @@ int plan_conv_steered(const ditto_conv_chain_desc* d, const ConvSteer& steer, Co
         return DITTO_OK;
       }
     }
+    // an output tile of TH2 x TW2 pixels needs the intermediate pixels (TH2 - 1) s2 + R2 by (TW2 - 1) s2 + S2
     a.TW2 = (int)Q2;
-    while ((a.TW2 + a.S2 - 1) * a.R2 > slots) a.TW2 = (a.TW2 + 1) / 2;
-    a.TW = a.TW2 + a.S2 - 1;
+    while (((a.TW2 - 1) * s2 + a.S2) * a.R2 > slots) a.TW2 = (a.TW2 + 1) / 2;
+    a.TW = (a.TW2 - 1) * s2 + a.S2;
     a.TH = slots / a.TW;
-    if (a.TH > P2 + a.R2 - 1) a.TH = (int)P2 + a.R2 - 1;
-    a.TH2 = a.TH - (a.R2 - 1);
+    if (a.TH > (P2 - 1) * s2 + a.R2) a.TH = (int)(P2 - 1) * s2 + a.R2;
+    a.TH2 = (a.TH - a.R2) / s2 + 1;
+    a.TH = (a.TH2 - 1) * s2 + a.R2;
     a.rows_in = (a.TH - 1) * a.stride + a.R;
     a.cols_in = (a.TW - 1) * a.stride + a.S;
     const int RS1 = a.R * a.S;

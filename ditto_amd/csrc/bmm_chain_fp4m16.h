@@ -456,7 +456,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     }
   }
   if (by_rows)
-    store_tile_rows<T, D, 16, true>(tw, reinterpret_cast<T*>(p.f) + zo * p.f_bs2 + zi * p.f_bs + (long long)m_tile * p.f_rs,
+    store_tile_rows<T, D, 16>(tw, reinterpret_cast<T*>(p.f) + zo * p.f_bs2 + zi * p.f_bs + (long long)m_tile * p.f_rs,
                                     p.f_rs, M - m_tile, N, lane);
 #else
   (void)p;

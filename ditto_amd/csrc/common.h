@@ -218,9 +218,10 @@ __device__ __forceinline__ void wg_sync() {
 template <int D>
 __host__ __device__ constexpr int tile_row_bytes() { return 2 * D + 16; }
 
-// WT: the stores are written through (see kStoreWriteThrough): for a kernel whose only stores come at its very end,
-// so that no dirty lines are left for the release at the end of the dispatch to write back.
-template <typename T, int D, int ROWS, bool WT = false>
+// The stores are written through (see kStoreWriteThrough): they come at the very end of a workgroup's life, and lines
+// left dirty in L2 would be written back by the release at the end of the dispatch, after the last wave (0.9 us of a
+// 12 us launch on 96 x 512 x 64; 0.4 % of the 430 us launch on 64 x 4096 x 128).
+template <typename T, int D, int ROWS>
 __device__ __forceinline__ void store_tile_rows(const char* tw, T* f0, long long f_rs, int rows_valid, int N, int lane) {
   typedef typename Elem<T>::v8 V8;
   constexpr int CPR = D / 8;  // 16-byte chunks per row
@@ -231,8 +232,7 @@ __device__ __forceinline__ void store_tile_rows(const char* tw, T* f0, long long
     const V8 x = *reinterpret_cast<const V8*>(tw + r * tile_row_bytes<D>() + ch * 16);
     if (r < rows_valid && 8 * ch < N) {
       V8* const dst = reinterpret_cast<V8*>(f0 + (long long)r * f_rs + 8 * ch);
-      if (WT) asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(dst), "v"(x) : "memory");
-      else *dst = x;
+      asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(dst), "v"(x) : "memory");
     }
   }
 }

@@ -43,13 +43,14 @@ struct ConvChainArgs {
   int tiles_h, tiles_w;
   int rows_in, cols_in;  // halo tile extent
   int relu_mid, relu_out, out_f32;
-  // second convolution larger than 1x1 (stride 1): then P, Q, TH, TW above describe the
+  // second convolution larger than 1x1: then P, Q, TH, TW above describe the
   // INTERMEDIATE tile (the output tile grown by the second filter's halo) and these the output
   const void* w2p;   // W2 repacked by pack_conv_w2
   int R2, S2, pad2;
   int P2, Q2;        // output extent
   int TH2, TW2;      // output tile per workgroup
   int wide2;         // 16-byte output stores through LDS: Q2 and TW2 multiples of 8, y 16-byte aligned, not fp32
+  int stride2;       // stride of the second convolution (the 1x1 second convolution is always run with stride 1)
 };
 
 // Input channels per staged chunk: 32 (two MFMA k steps per tap) or, where that does not fit in
@@ -102,7 +103,7 @@ __global__ void pack_conv_w1_kernel(const T* __restrict__ w1, T* __restrict__ ou
 }
 
 // PX2 = 0: the second convolution is 1x1 and consumes the first one's accumulators from registers;
-// PX2 = 1 | 2: it is R2 x S2 (stride 1) and reads the intermediate tile from LDS, PX2 tiles of 32
+// PX2 = 1 | 2: it is R2 x S2 (any stride) and reads the intermediate tile from LDS, PX2 tiles of 32
 // output pixels per wave.
 template <typename T, int C1T, int PXW, int CH, int PX2 = 0>
 __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
@@ -127,7 +128,7 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
   const int n = lid / tiles;
   const int th = (lid % tiles) / p.tiles_w, tw = (lid % tiles) % p.tiles_w;
   // origin of the tile the FIRST convolution produces (the intermediate tile when PX2 > 0)
-  const int p0 = PX2 ? th * p.TH2 - p.pad2 : th * p.TH, q0 = PX2 ? tw * p.TW2 - p.pad2 : tw * p.TW;
+  const int p0 = PX2 ? th * p.TH2 * p.stride2 - p.pad2 : th * p.TH, q0 = PX2 ? tw * p.TW2 * p.stride2 - p.pad2 : tw * p.TW;
   const int h0 = p0 * p.stride - p.pad, w0 = q0 * p.stride - p.pad;  // input coords of the halo origin
 
   const T* __restrict__ Xg = reinterpret_cast<const T*>(p.x) + (long long)n * p.C0 * p.H * p.W;
@@ -390,7 +391,7 @@ __global__ __launch_bounds__(256) void conv_chain_kernel(ConvChainArgs p) {
       const int oh = slot / p.TW2, ow = slot % p.TW2;
       valid2[j] = oh < p.TH2 && op0 + oh < p.P2 && oq0 + ow < p.Q2;
       const int ohc = valid2[j] ? oh : 0, owc = valid2[j] ? ow : 0;
-      moff[j] = (ohc * p.TW + owc) * MS + 8 * g;
+      moff[j] = (ohc * p.TW + owc) * p.stride2 * MS + 8 * g;
       opix2[j] = (long long)(op0 + ohc) * p.Q2 + oq0 + owc;
     }
     const long long plane2 = (long long)p.P2 * p.Q2;

@@ -24,12 +24,14 @@ hipError_t DITTO_PACK_NAME(int c1_tiles, int ch, const ConvChainArgs& args, void
   return launch_pack_conv_w1<DITTO_INST_T>(args, 32 * c1_tiles, ch, out, stream);
 }
 
-// second convolution larger than 1x1: c1_tiles in {1, 2, 4}, px2 in {1, 2} output-pixel tiles per wave
+// second convolution larger than 1x1: c1_tiles in {1, 2, 4, 8}, px2 in {1, 2} output-pixel tiles per wave (eight
+// tiles of intermediate channels leave 128 pixel slots: one output-pixel tile per wave)
 hipError_t DITTO_INST2_NAME(int c1_tiles, int px2, const ConvChainArgs& args, hipStream_t stream) {
   typedef DITTO_INST_T T;
   if (c1_tiles == 1) return px2 == 1 ? launch_conv_chain<T, 1, 2, 32, 1>(args, stream) : launch_conv_chain<T, 1, 2, 32, 2>(args, stream);
   if (c1_tiles == 2) return px2 == 1 ? launch_conv_chain<T, 2, 2, 32, 1>(args, stream) : launch_conv_chain<T, 2, 2, 32, 2>(args, stream);
   if (c1_tiles == 4) return px2 == 1 ? launch_conv_chain<T, 4, 2, 32, 1>(args, stream) : launch_conv_chain<T, 4, 2, 32, 2>(args, stream);
+  if (c1_tiles == 8 && px2 == 1) return launch_conv_chain<T, 8, 1, 32, 1>(args, stream);
   return hipErrorInvalidValue;
 }
 

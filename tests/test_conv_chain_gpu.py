@@ -14,14 +14,14 @@ MAX_ABS, REL_L2 = 1e-2, 1e-3
 
 
 def run_conv(X, W1, W2, dtype, pad1=1, stride1=1, inter="cast", relu_out=False, out_dtype=None, workspace=None,
-             pad2=0, groups1=1, tile_variant=0):
+             pad2=0, groups1=1, tile_variant=0, stride2=1):
     x, w1, w2 = to_dev(X, dtype), to_dev(W1, dtype), to_dev(W2, dtype)
     N, _, H, W = X.shape
     R, S = W1.shape[2:]
-    P = (H + 2 * pad1 - R) // stride1 + 1 + 2 * pad2 - W2.shape[2] + 1
-    Q = (W + 2 * pad1 - S) // stride1 + 1 + 2 * pad2 - W2.shape[3] + 1
+    P = ((H + 2 * pad1 - R) // stride1 + 1 + 2 * pad2 - W2.shape[2]) // stride2 + 1
+    Q = ((W + 2 * pad1 - S) // stride1 + 1 + 2 * pad2 - W2.shape[3]) // stride2 + 1
     y = torch.full((N, W2.shape[0], P, Q), float("nan"), device=x.device, dtype=TORCH_DTYPES[out_dtype or dtype])
-    chain.run_conv_chain(x, w1, w2, y, pad1, stride1, pad2, 1, inter, relu_out, workspace=workspace,
+    chain.run_conv_chain(x, w1, w2, y, pad1, stride1, pad2, stride2, inter, relu_out, workspace=workspace,
                          groups1=groups1, tile_variant=tile_variant)
     torch.cuda.synchronize()
     return y.float().cpu().numpy()
@@ -568,10 +568,47 @@ def test_conv_chain_rejects_what_it_cannot_fuse():
     with pytest.raises(NotImplementedError):  # 5x5 second filter
         chain.run_conv_chain(x, w1, torch.zeros(32, 32, 5, 5, device="cuda:0", dtype=torch.float16),
                              torch.zeros(1, 32, 14, 14, device="cuda:0", dtype=torch.float16), 0, 1, 2, 1)
-    w1b = torch.zeros(160, 16, 1, 1, device="cuda:0", dtype=torch.float16)
-    with pytest.raises(NotImplementedError):  # 3x3 second filter over more than 128 intermediate channels
-        chain.run_conv_chain(x, w1b, torch.zeros(32, 160, 3, 3, device="cuda:0", dtype=torch.float16),
-                             torch.zeros(1, 32, 14, 14, device="cuda:0", dtype=torch.float16), 0, 1, 1, 1)
+    with pytest.raises(NotImplementedError):  # second convolution with a stride beyond 4
+        chain.run_conv_chain(x, w1, torch.zeros(32, 32, 3, 3, device="cuda:0", dtype=torch.float16),
+                             torch.zeros(1, 32, 3, 3, device="cuda:0", dtype=torch.float16), 0, 1, 1, 5)
+
+
+CASES_STRIDED_SECOND = [
+    # N, C0, H, W, C1, R1, pad1, stride1, C2, R2, pad2, stride2, groups1
+    (2, 32, 30, 30, 64, 3, 1, 1, 64, 1, 0, 2, 1),     # 3x3 -> 1x1 keeping every second pixel
+    (1, 24, 29, 31, 40, 3, 1, 2, 48, 1, 0, 2, 1),     # both strided, odd extents
+    (1, 64, 56, 56, 64, 1, 0, 1, 128, 1, 0, 2, 1),    # 1x1 -> 1x1 stride 2 (a ResNet downsampling branch)
+    (2, 16, 28, 28, 16, 3, 1, 1, 32, 1, 0, 2, 16),    # depthwise first convolution
+    (1, 32, 29, 29, 64, 1, 0, 1, 64, 3, 1, 2, 1),     # 1x1 -> 3x3 stride 2
+    (2, 16, 20, 36, 32, 3, 1, 1, 40, 3, 0, 2, 1),     # 3x3 -> 3x3 stride 2 without padding
+    (1, 16, 33, 17, 24, 3, 1, 1, 32, 3, 1, 3, 1),     # stride 3
+    (1, 32, 14, 14, 192, 1, 0, 1, 64, 3, 1, 1, 1),    # 192 intermediate channels under a 3x3 second filter
+    (2, 64, 20, 24, 256, 1, 0, 1, 96, 3, 1, 1, 1),    # 256
+    (1, 32, 15, 15, 256, 1, 0, 1, 32, 3, 1, 2, 1),    # 256, strided
+]
+
+
+@pytest.mark.parametrize("case", CASES_STRIDED_SECOND)
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_strided_second_convolution_and_wide_intermediates(oracle, case, dtype):
+    """Second convolutions with a stride (a strided 1x1 is run as the chain whose first convolution carries both
+    strides; a strided 3x3 reads the intermediate tile in LDS with that stride) and 3x3 second convolutions over up
+    to 256 intermediate channels."""
+    N, C0, H, W, C1, R1, pad1, stride1, C2, R2, pad2, stride2, groups1 = case
+    X, W1, W2 = oracle.make_conv_chain_inputs(N, C0, H, W, C1, C2, R1, R2, dtype, seed=C0 + C2 + stride2, w_std=0.05)
+    if groups1 != 1:  # depthwise: one filter per channel
+        W1 = oracle.np_round_to(np.random.default_rng(C0).standard_normal((C1, 1, R1, R1)).astype(np.float32) * 0.3, dtype)
+    for relu in (False, True):
+        want32 = oracle.conv_chain_f32(X, W1, W2, pad1, stride1, pad2, stride2, relu_mid=relu, relu_out=relu,
+                                       round_mid=dtype, groups1=groups1)
+        got32 = run_conv(X, W1, W2, dtype, pad1, stride1, "relu" if relu else "cast", relu, "float32", None, pad2,
+                         groups1, 0, stride2)
+        assert got32.shape == want32.shape and np.isfinite(got32).all()
+        mx, rel = errors(got32, want32)
+        assert mx <= MAX_ABS and rel <= REL_L2, (relu, mx, rel)
+    got = run_conv(X, W1, W2, dtype, pad1, stride1, "relu", True, None, None, pad2, groups1, 0, stride2)
+    mx, rel = errors(got, oracle.np_round_to(want32, dtype))
+    assert mx <= MAX_ABS and rel <= REL_L2, (mx, rel)
 
 
 def test_conv_relu_conv_relu_vs_torch(oracle):
@@ -726,8 +763,6 @@ def test_conv_chain_rejects_unsupported():
     w1 = torch.zeros(16, 16, 3, 3, device=dev, dtype=torch.float16)
     w2 = torch.zeros(16, 16, 3, 3, device=dev, dtype=torch.float16)
     y = torch.zeros(1, 16, 8, 8, device=dev, dtype=torch.float16)
-    with pytest.raises(NotImplementedError, match="stride 1"):  # strided second convolution
-        chain.run_conv_chain(x, w1, w2, y[:, :, :4, :4].contiguous(), 1, 1, 1, 2)
     with pytest.raises(ValueError):
         chain.run_conv_chain(x, w1, w2[:, :, :1, :1].contiguous(), y[:, :8].contiguous(), 1, 1, 0, 1)
 
