@@ -96,9 +96,10 @@ def BatchGemmGemmMMA(A, B, C, MI=16, NI=16, KI=16, in_dtype="float16", acc_dtype
     int8 operands with an int32 accumulator (the ("80", "int8", "int32") row of
     bmm_bmm_cuda.py:273-288): the middle result goes back to int8 through a *requantise* op,
     ``saturate(round_to_nearest_even(acc * s))`` with ``s = requant_scale`` for every intermediate
-    column or ``scale[l]`` from a float32 placeholder ``scale[L]`` (the reference's chain wraps
-    with ``astype("int8")``, :116, which no kernel here implements), and ``F`` keeps the
-    accumulator type unless ``out_dtype`` says otherwise."""
+    column or ``scale[l]`` from a float32 placeholder ``scale[L]``, and ``F`` keeps the accumulator
+    type unless ``out_dtype`` says otherwise.  Without a scale the chain is the reference's own: the
+    middle result and ``F`` go back to int8 with ``astype("int8")`` (:116, :147), which keeps the low
+    byte of the int32 accumulator."""
     batch, M, K = A.shape
     _batch, _K, L = B.shape
     _batch2, _L, N = C.shape

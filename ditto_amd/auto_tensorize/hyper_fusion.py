@@ -310,9 +310,12 @@ def _recognise(layer, state):
                     requant_scale=1.0 if has_tensor else float(req.attrs["scale"]), scale_tensor=has_tensor)
     if inter in (["cast"], ["relu"]) and (epi == ["unpack_cast"] or relu_out):
         if A.dtype == "int8":
-            raise NotImplementedError(
-                "the int8 chain is built with a requantised middle result (BatchGemmGemm(..., requant_scale=s)); "
-                "the wrapping astype(int8) of bmm_bmm_cuda.py:116 has no kernel here")
+            # the reference's own int8 chain (bmm_bmm_cuda.py:114-118, 145-149): astype("int8") of the int32
+            # accumulators keeps their low byte, for the middle result and (out_dtype int8) for the output
+            if first.output(0).dtype != "int32" or out_t.dtype not in ("int8", "int32") or relu_out:
+                raise ValueError("the int8 chain accumulates in int32 and outputs int8 or int32, without an output ReLU")
+            return dict(kind="bmm_chain", inter_op=inter[0], dims=dims, relu_out=False, in_dtype=A.dtype,
+                        acc_dtype="int32", out_dtype=out_t.dtype, softmax_scale=1.0)
         return dict(kind="bmm_chain", inter_op=inter[0], dims=dims, relu_out=relu_out, in_dtype=A.dtype,
                     acc_dtype=first.output(0).dtype, out_dtype=out_t.dtype, softmax_scale=1.0)
     raise ValueError("The fusion and tensorize decisions are not valid (inter path %s, epilogue %s)." % (inter, epi))

@@ -277,10 +277,11 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     return DITTO_OK;
   }
   if (in == DITTO_I8) {
-    if (d->acc_dtype != DITTO_I32 || d->out_dtype != DITTO_I32)
-      return fail(DITTO_EINVAL, "the int8 chain accumulates and outputs int32");
-    if (d->inter_op != DITTO_INTER_REQUANT)
-      return fail(DITTO_EUNSUPPORTED, "the int8 chain needs inter_op = DITTO_INTER_REQUANT");
+    if (d->acc_dtype != DITTO_I32 || (d->out_dtype != DITTO_I32 && d->out_dtype != DITTO_I8))
+      return fail(DITTO_EINVAL, "the int8 chain accumulates in int32 and outputs int32 or (the low byte) int8");
+    // requantised middle result, or the reference's wrapping cast (optionally behind a ReLU)
+    if (d->inter_op != DITTO_INTER_REQUANT && d->inter_op != DITTO_INTER_CAST && d->inter_op != DITTO_INTER_RELU)
+      return fail(DITTO_EUNSUPPORTED, "the int8 chain takes inter_op requant, cast (wrapping) or relu (then wrapping)");
     if (d->b_layout != DITTO_B_KL) return fail(DITTO_EUNSUPPORTED, "the int8 chain takes B as [K][L]");
     if (d->tile_variant != 0) return fail(DITTO_EINVAL, "the int8 chain has a single variant (tile_variant must be 0)");
     if (d->K % 16 || d->L % 16 || d->N % 16)
@@ -1079,6 +1080,9 @@ int ditto_bmm_chain_run(const ditto_bmm_chain_desc* d, const void* a, const void
     args.d = static_cast<const int8_t*>(c);
     args.scale = static_cast<const float*>(aux);
     args.scale_uniform = d->requant_scale;
+    args.wrap = d->inter_op != DITTO_INTER_REQUANT;
+    args.relu = d->inter_op == DITTO_INTER_RELU;
+    args.out_i8 = d->out_dtype == DITTO_I8;
     args.e = static_cast<int32_t*>(f);
     args.a_bs = d->a_batch_stride;
     args.b_bs = d->b_batch_stride;

@@ -11,6 +11,9 @@ struct I8ChainArgs {
   const int8_t* d;
   const float* scale;   // [L] or null
   float scale_uniform;  // used when scale == null
+  int wrap;             // middle result = the accumulator's low byte (the wrapping astype("int8")) instead of requantised
+  int relu;             // wrap only: max(acc, 0) first
+  int out_i8;           // e is int8: the low byte of every result (the chain's closing astype("int8"))
   int32_t* e;
   long long a_bs, b_bs, d_bs, e_bs;  // batch strides, elements
   int a_rs, b_rs, d_rs, e_rs;        // row strides, elements

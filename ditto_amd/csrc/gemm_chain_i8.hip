@@ -1,4 +1,6 @@
 // int8 GEMM -> requantise -> GEMM chain on gfx950:  E = sat_i8(rne((A.B) * scale[l])) . D
+// (and the reference's own middle step, E = wrap_i8(A.B) . D, optionally with a ReLU in front of the wrap: the
+// accumulator's low byte, benchmark/chimera/cuda/bmm_bmm_cuda.py:114-118)
 //
 // The reference declares int8 -> int32 for its GEMM chain (benchmark/chimera/cuda/
 // bmm_bmm_cuda.py:273-288) and casts the middle result with a wrapping astype("int8")
@@ -255,10 +257,19 @@ __global__ __launch_bounds__(64 * i8::NW) void gemm_chain_i8_kernel(I8ChainArgs 
           const f32x4 s4 = *reinterpret_cast<const f32x4*>(sc + l);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
-            const int b0 = requant_i8(acc[lt][mt][4 * q + 0], s4[0]);
-            const int b1 = requant_i8(acc[lt][mt][4 * q + 1], s4[1]);
-            const int b2 = requant_i8(acc[lt][mt][4 * q + 2], s4[2]);
-            const int b3 = requant_i8(acc[lt][mt][4 * q + 3], s4[3]);
+            int b0, b1, b2, b3;
+            if (p.wrap) {  // (uniform) the packing below keeps the low byte of each
+              const int floor_at = p.relu ? 0 : (int)0x80000000;
+              b0 = max(acc[lt][mt][4 * q + 0], floor_at);
+              b1 = max(acc[lt][mt][4 * q + 1], floor_at);
+              b2 = max(acc[lt][mt][4 * q + 2], floor_at);
+              b3 = max(acc[lt][mt][4 * q + 3], floor_at);
+            } else {
+              b0 = requant_i8(acc[lt][mt][4 * q + 0], s4[0]);
+              b1 = requant_i8(acc[lt][mt][4 * q + 1], s4[1]);
+              b2 = requant_i8(acc[lt][mt][4 * q + 2], s4[2]);
+              b3 = requant_i8(acc[lt][mt][4 * q + 3], s4[3]);
+            }
             const int packed = (b0 & 0xff) | ((b1 & 0xff) << 8) | ((b2 & 0xff) << 16) | ((unsigned)b3 << 24);
             *reinterpret_cast<int*>(mid + (32 * mt + ln) * MIDSTR + l) = packed;
           }
@@ -293,7 +304,21 @@ __global__ __launch_bounds__(64 * i8::NW) void gemm_chain_i8_kernel(I8ChainArgs 
       // acc[nt][mt][r] = E[m][n], m = m0 + 32mt + 8(r/4) + 4g + r%4, n = nc + 32(CTW*wave + nt) + ln:
       // the 32 lanes of a half-wave write 128 contiguous bytes of one output row
       const int nc = rot(ob, rot_nc, nnc) * WC;
-      if (m0 + BM <= M && nc + WC <= N) {
+      if (p.out_i8) {
+        // one byte per result: the 32 lanes of a half-wave write 32 contiguous bytes of one output row
+        int8_t* const E8 = reinterpret_cast<int8_t*>(p.e) + (long long)bz * p.e_bs;
+#pragma unroll
+        for (int nt = 0; nt < CTW; ++nt) {
+          const int n = nc + 32 * (CTW * wave + nt) + ln;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int m = m0 + 32 * mt + 8 * (r >> 2) + 4 * g + (r & 3);
+              if (n < N && m < M) E8[(long long)m * p.e_rs + n] = (int8_t)(acc[nt][mt][r] & 0xff);
+            }
+        }
+      } else if (m0 + BM <= M && nc + WC <= N) {
         // whole tile in range: the row of register r is a scalar offset, the lane part of the
         // address is constant, so a store costs no address arithmetic
         const int voff = (4 * g * p.e_rs + ln) * 4;

@@ -50,7 +50,8 @@ typedef enum ditto_dtype {
 /* The op on the single path between the two contractions
  * (reference: TensorizeHyperFusionState::inter_path, src/auto_tensorize/hyper_fusion.cc:51-216). */
 typedef enum ditto_inter_op {
-  DITTO_INTER_CAST = 0,    /* mid = cast_in(acc)                      bmm_bmm_cuda.py:114-118           */
+  DITTO_INTER_CAST = 0,    /* mid = cast_in(acc)                      bmm_bmm_cuda.py:114-118 (int8: the
+                              accumulator's low byte, what astype("int8") keeps)                    */
   DITTO_INTER_RELU = 1,    /* mid = cast_in(max(acc,0))               conv_relu_conv_relu_fuse_hw_cuda.py:134-142 */
   DITTO_INTER_SOFTMAX = 2, /* mid = softmax(scale*acc) over L, online  bmm_chain.py:63-103 (exp + ones column + divide) */
   DITTO_INTER_REQUANT = 3  /* mid = sat_i8(rne(acc * scale[col]))      int8 chain; not in the reference,

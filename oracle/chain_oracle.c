@@ -30,6 +30,9 @@
  *                             requantise step is NOT in the reference (its int8 chain does a
  *                             wrapping astype("int8"), bmm_bmm_cuda.py:116): it is specified
  *                             by this build's workload definition.
+ *   oracle_gemm_chain_i8_wrap the reference's own int8 chain: the int32 middle result goes back to
+ *                             int8 with astype("int8"), which keeps the low byte (two's complement
+ *                             wrap), optionally behind a ReLU (bmm_bmm_cuda.py:114-118).
  *   oracle_conv_chain_grouped_f32  the same with a grouped (depthwise) first convolution
  *   oracle_conv_chain_f32     conv -> inter -> conv on NCHW tensors, the chain of
  *                             benchmark/chimera/cuda/conv3x3_conv1x1_cuda.py:77-172 in the
@@ -386,6 +389,43 @@ ORACLE_API int32_t oracle_requant_shift(int32_t mid, int shift) {
 }
 
 ORACLE_API int32_t oracle_requant_scale(int32_t mid, float s) { return (int32_t)requant_f32(mid, s); }
+
+/* E = wrap_i8(relu?(A.B)) . D in exact integers (bmm_bmm_cuda.py:114-118: astype("int8") of the int32 product). */
+ORACLE_API void oracle_gemm_chain_i8_wrap(int batch, int M, int N, int K, int L, const int8_t* A,
+                                          const int8_t* B, const int8_t* D, int relu, int32_t* E,
+                                          int8_t* mid_out) {
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int b = 0; b < batch; ++b) {
+    for (int m = 0; m < M; ++m) {
+      int32_t* mid = (int32_t*)calloc((size_t)L, sizeof(int32_t));
+      int8_t* q = (int8_t*)malloc((size_t)L);
+      const int8_t* a = A + ((size_t)b * M + m) * K;
+      const int8_t* Bb = B + (size_t)b * K * L;
+      const int8_t* Db = D + (size_t)b * L * N;
+      for (int k = 0; k < K; ++k) {
+        const int32_t av = a[k];
+        const int8_t* brow = Bb + (size_t)k * L;
+        for (int l = 0; l < L; ++l) mid[l] += av * (int32_t)brow[l];
+      }
+      for (int l = 0; l < L; ++l) {
+        int32_t v = mid[l];
+        if (relu && v < 0) v = 0;
+        const uint32_t low = (uint32_t)v & 0xffu; /* the low byte, read back as a signed 8-bit value */
+        q[l] = (int8_t)(low >= 128u ? (int32_t)low - 256 : (int32_t)low);
+      }
+      if (mid_out) memcpy(mid_out + ((size_t)b * M + m) * L, q, (size_t)L);
+      int32_t* e = E + ((size_t)b * M + m) * N;
+      for (int n = 0; n < N; ++n) e[n] = 0;
+      for (int l = 0; l < L; ++l) {
+        const int32_t qv = q[l];
+        const int8_t* drow = Db + (size_t)l * N;
+        for (int n = 0; n < N; ++n) e[n] += qv * (int32_t)drow[n];
+      }
+      free(mid);
+      free(q);
+    }
+  }
+}
 
 ORACLE_API void oracle_gemm_chain_i8(int batch, int M, int N, int K, int L, const int8_t* A,
                                      const int8_t* B, const int8_t* D, const float* scale,

@@ -59,6 +59,8 @@ def lib():
         L.oracle_requant_shift.argtypes = [ctypes.c_int32, ci]
         L.oracle_requant_scale.restype = ctypes.c_int32
         L.oracle_requant_scale.argtypes = [ctypes.c_int32, ctypes.c_float]
+        L.oracle_gemm_chain_i8_wrap.restype = None
+        L.oracle_gemm_chain_i8_wrap.argtypes = [ci] * 5 + [i8p] * 3 + [ci, i32p, i8p]
         L.oracle_gemm_chain_i8.restype = None
         L.oracle_gemm_chain_i8.argtypes = [ci] * 5 + [i8p] * 3 + [fp, i32p, i8p]
         L.oracle_conv_chain_f32.restype = None
@@ -219,6 +221,25 @@ def np_bmm_chain(A, B, C, inter="cast", scale=1.0, round_mid=None, round_out=Non
 def np_requant(mid, scale):
     v = np.rint(mid.astype(np.float32) * np.asarray(scale, dtype=np.float32))
     return np.clip(v, -128, 127).astype(np.int8)
+
+
+def gemm_chain_i8_wrap(A, B, D, relu=False, return_mid=False):
+    """The reference's own int8 chain (bmm_bmm_cuda.py:114-118): the int32 middle result goes back to int8 with
+    astype("int8"), i.e. its low byte, optionally behind a ReLU.  A[b,M,K], B[b,K,L], D[b,L,N] int8."""
+    A = np.ascontiguousarray(A, dtype=np.int8)
+    B = np.ascontiguousarray(B, dtype=np.int8)
+    D = np.ascontiguousarray(D, dtype=np.int8)
+    if A.ndim == 2:
+        A, B, D = A[None], B[None], D[None]
+    batch, M, K = A.shape
+    L, N = B.shape[2], D.shape[2]
+    E = np.empty((batch, M, N), dtype=np.int32)
+    mid = np.empty((batch, M, L), dtype=np.int8)
+    i8p = ctypes.POINTER(ctypes.c_int8)
+    lib().oracle_gemm_chain_i8_wrap(batch, M, N, K, L, A.ctypes.data_as(i8p), B.ctypes.data_as(i8p),
+                                    D.ctypes.data_as(i8p), int(bool(relu)), E.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)),
+                                    mid.ctypes.data_as(i8p))
+    return (E, mid) if return_mid else E
 
 
 def np_gemm_chain_i8(A, B, D, scale):

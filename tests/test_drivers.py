@@ -64,7 +64,9 @@ def test_drivers_run_one_row_each(capsys):
 @pytest.mark.gpu
 def test_int8_driver_row():
     # the ("80", "int8", "int32") combination of bmm_bmm_cuda.py:273-288 (GEMM chain only)
-    cost = bmm_bmm.main(*common.BMM_SHAPES[1], in_dtype="int8", acc_dtype="int32")
+    cost = bmm_bmm.main(*common.BMM_SHAPES[1], in_dtype="int8", acc_dtype="int32")  # the reference's wrapping chain
+    assert 0 < cost < 5.0
+    cost = bmm_bmm.main(*common.BMM_SHAPES[1], in_dtype="int8", acc_dtype="int32", requant=True)
     assert 0 < cost < 5.0
     out = subprocess.run([sys.executable, "-m", "ditto_amd.drivers.bmm_bmm", "--in_dtype", "int8", "--acc_dtype",
                           "int32", "--begin", "9", "--num", "1", "--only_once"], capture_output=True, text=True,

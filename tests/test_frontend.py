@@ -389,11 +389,14 @@ def test_int8_chain_builder_and_recognition():
     layer, sfs, fc, state = _reference_flow(ins, outs, "int8", "int32")
     sch = at.tensorize_hip(layer, state)
     assert sch.scale_tensor and [t.name for t in layer.schedule_tensors] == ["A", "B", "C", "scale", "F"]
-    # the reference's wrapping astype("int8") has no kernel: refused when the chain is tensorized
-    ins, outs = F.BatchGemmGemm(1, 64, 64, 64, 64, "int8", "int32")
-    layer, sfs, fc, state = _reference_flow(ins, outs, "int8", "int32")
-    with pytest.raises(NotImplementedError, match="requant"):
-        at.tensorize_hip(layer, state)
+    # the reference's own int8 chain: astype("int8") for the middle result and for F (bmm_bmm_cuda.py:116, :147)
+    for relu in (False, True):
+        ins, outs = F.BatchGemmGemm(1, 64, 64, 64, 64, "int8", "int32", relu=relu)
+        assert outs[0].dtype == "int8"
+        layer, sfs, fc, state = _reference_flow(ins, outs, "int8", "int32")
+        sch = at.tensorize_hip(layer, state)
+        assert (sch.kind, sch.inter_op, sch.in_dtype, sch.acc_dtype, sch.out_dtype) == (
+            "bmm_chain", "relu" if relu else "cast", "int8", "int32", "int8")
     # tile_variant travels on the schedule
     ins, outs = F.BatchGemmGemm(64, 4096, 128, 128, 4096, "bfloat16", "float32")
     layer, sfs, fc, state = _reference_flow(ins, outs, "bfloat16")

@@ -39,6 +39,26 @@ def test_i8_chain_bit_exact(oracle, shape):
     assert np.array_equal(run_i8(A, B, D, None, uniform=2.0 ** -10), want)
 
 
+@pytest.mark.parametrize("shape", [(64, 64, 256, 256), (100, 96, 48, 80), (200, 1024, 256, 1024), (37, 16, 16, 16)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_i8_wrapping_chain_bit_exact(oracle, shape, relu):
+    """The reference's own int8 chain: the middle result (and, with an int8 output, the result) keeps the low byte
+    of its int32 accumulator (bmm_bmm_cuda.py:116, :147), optionally behind a ReLU."""
+    M, K, L, N = shape
+    A, B, D, _ = oracle.make_i8_chain_inputs(M, K, L, N, seed=M + N + 1)
+    want, mid = oracle.gemm_chain_i8_wrap(A, B, D, relu, return_mid=True)
+    assert (np.abs(A.astype(np.int64) @ B.astype(np.int64)) > 127).any()  # the wrap is exercised
+    dev = "cuda:0"
+    a, b, d = (torch.from_numpy(np.ascontiguousarray(x)).to(dev) for x in (A, B, D))
+    e32 = torch.full((M, N), -7, dtype=torch.int32, device=dev)
+    chain.run_bmm_chain(a, b, d, e32, "relu" if relu else "cast")
+    e8 = torch.full((M, N), -7, dtype=torch.int8, device=dev)
+    chain.run_bmm_chain(a, b, d, e8, "relu" if relu else "cast")
+    torch.cuda.synchronize()
+    assert np.array_equal(e32.cpu().numpy(), want[0])
+    assert np.array_equal(e8.cpu().numpy(), want[0].astype(np.int8))  # numpy's cast keeps the low byte too
+
+
 def test_i8_chain_per_column_scales_and_saturation(oracle):
     M, K, L, N = 96, 256, 64, 48
     A, B, D, _ = oracle.make_i8_chain_inputs(M, K, L, N, seed=5)
@@ -97,7 +117,7 @@ def test_i8_chain_rejects_bad_descriptors():
     d = torch.zeros(32, 64, dtype=torch.int8, device=dev)
     e = torch.zeros(64, 64, dtype=torch.int32, device=dev)
     with pytest.raises(NotImplementedError):
-        chain.run_bmm_chain(a, b, d, e, "cast")
+        chain.run_bmm_chain(a, b, d, e, "softmax")
     with pytest.raises(ValueError):
         chain.run_bmm_chain(a[:, :60], b[:60], d, e, "requant")
     with pytest.raises(ValueError):

@@ -217,6 +217,35 @@ def test_i8_chain_exact(oracle):
     assert np.array_equal(oracle.gemm_chain_i8(A, B, D, sc)[0], oracle.np_gemm_chain_i8(A, B, D, sc))
 
 
+def test_i8_wrap_chain_exact(oracle):
+    """The reference's own int8 chain (astype("int8") keeps the low byte): against the arithmetic definition of the
+    low byte (acc mod 256 taken to [-128, 128)), brute force, numpy's own wrapping cast, and the cases where it
+    reduces to the requantised chain (middle results inside int8: scale 1, no saturation, no wrap)."""
+    A, B, D, _ = oracle.make_i8_chain_inputs(37, 96, 40, 24, seed=3)
+    for relu in (False, True):
+        E, mid = oracle.gemm_chain_i8_wrap(A, B, D, relu, return_mid=True)
+        acc = A.astype(np.int64) @ B.astype(np.int64)
+        if relu:
+            acc = np.maximum(acc, 0)
+        low = ((acc + 128) % 256) - 128
+        assert abs(acc).max() > 127 and np.array_equal(mid[0], low) and (mid[0] != acc).any()
+        assert np.array_equal(mid[0], acc.astype(np.int32).astype(np.int8))
+        assert E.dtype == np.int32 and np.array_equal(E[0], low @ D.astype(np.int64))
+        m, n = 5, 7
+        tot = 0
+        for l in range(40):
+            d = sum(int(A[m, k]) * int(B[k, l]) for k in range(96))
+            d = max(d, 0) if relu else d
+            d &= 0xff
+            tot += (d - 256 if d >= 128 else d) * int(D[l, n])
+        assert E[0, m, n] == tot
+    # small operands: nothing wraps, and scale 1 requantises to the same bytes
+    rng = np.random.default_rng(0)
+    As, Bs = rng.integers(-2, 3, (16, 8), dtype=np.int8), rng.integers(-2, 3, (8, 16), dtype=np.int8)
+    Ds = rng.integers(-127, 128, (16, 16), dtype=np.int8)
+    assert np.array_equal(oracle.gemm_chain_i8_wrap(As, Bs, Ds), oracle.gemm_chain_i8(As, Bs, Ds, 1.0))
+
+
 # ---------------------------------------------------------------------------- conv chain
 def _torch_conv_chain(X, W1, W2, pad1, stride1, pad2, stride2, relu_mid, relu_out):
     x = torch.from_numpy(X).double()
