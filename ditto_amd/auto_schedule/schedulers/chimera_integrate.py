@@ -29,6 +29,10 @@ from ...hardware import query_hw_param
 FP_VARIANT_CODES = (1, 2, 8, 9, 6, 7, 4, 5)
 
 
+# int8 chain: 8000 + 10 * (row tiles of 32 per workgroup) + depth of the ring of staged weight chunks
+I8_VARIANTS = (8012, 8014, 8022, 8023)
+
+
 class TuneEntry:
     """One measurement: ``record`` (the tile description, JSON-able) and ``value`` (ms)."""
 
@@ -53,6 +57,13 @@ def make_tile_variant_space(desc):
         for q in FP_VARIANT_CODES:
             d = copy.copy(desc)
             d.tile_variant = tile.head_pad * 10 + q
+            t = _lib.TileParam()
+            if lib.ditto_bmm_chain_select_tile(ctypes.byref(d), ctypes.byref(t)) == _lib.OK:
+                space.append(t.to_json())
+    elif desc.in_dtype == _lib.I8:
+        for variant in I8_VARIANTS:
+            d = copy.copy(desc)
+            d.tile_variant = variant
             t = _lib.TileParam()
             if lib.ditto_bmm_chain_select_tile(ctypes.byref(d), ctypes.byref(t)) == _lib.OK:
                 space.append(t.to_json())

@@ -283,7 +283,6 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     if (d->inter_op != DITTO_INTER_REQUANT && d->inter_op != DITTO_INTER_CAST && d->inter_op != DITTO_INTER_RELU)
       return fail(DITTO_EUNSUPPORTED, "the int8 chain takes inter_op requant, cast (wrapping) or relu (then wrapping)");
     if (d->b_layout != DITTO_B_KL) return fail(DITTO_EUNSUPPORTED, "the int8 chain takes B as [K][L]");
-    if (d->tile_variant != 0) return fail(DITTO_EINVAL, "the int8 chain has a single variant (tile_variant must be 0)");
     if (d->K % 16 || d->L % 16 || d->N % 16)
       return fail(DITTO_EINVAL, "K, L and N must be multiples of 16 for the int8 chain");
     if (d->a_row_stride % 16 || d->b_row_stride % 16 || d->c_row_stride % 16 || d->a_batch_stride % 16 ||
@@ -307,6 +306,15 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     if (!fits(mt, nst)) nst = 2;
     if (!fits(mt, nst)) mt = 1, nst = 4;
     if (!fits(mt, nst)) nst = 2;
+    if (d->tile_variant != 0) {
+      // 8000 + 10 * (row tiles of 32) + ring depth, as select_tile reports it
+      const int fm = (d->tile_variant - 8000) / 10, fn = d->tile_variant % 10;
+      const bool built = (fm == 1 && (fn == 2 || fn == 4)) || (fm == 2 && (fn == 2 || fn == 3));
+      if (d->tile_variant < 8000 || !built || !fits(fm, fn))
+        return fail(DITTO_EINVAL, "tile_variant %d cannot run this int8 chain (8012, 8014, 8022 or 8023, within LDS)",
+                    d->tile_variant);
+      mt = fm, nst = fn;
+    }
     const int lds = ditto::i8_chain_lds_bytes_host((int)Lp, mt, nst);
     if (lds > 160 * 1024)
       return fail(DITTO_EUNSUPPORTED, "L=%lld: the requantised row block does not fit in LDS", (long long)d->L);

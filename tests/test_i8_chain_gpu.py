@@ -59,6 +59,26 @@ def test_i8_wrapping_chain_bit_exact(oracle, shape, relu):
     assert np.array_equal(e8.cpu().numpy(), want[0].astype(np.int8))  # numpy's cast keeps the low byte too
 
 
+def test_i8_chain_variants_agree(oracle):
+    """Every kernel variant (32 or 64 rows per workgroup, ring depth) can be forced and gives the same bits."""
+    M, K, L, N = 300, 256, 256, 512
+    A, B, D, scale = oracle.make_i8_chain_inputs(M, K, L, N, seed=9)
+    want = oracle.gemm_chain_i8(A, B, D, scale)[0]
+    dev = "cuda:0"
+    a, b, d = (torch.from_numpy(np.ascontiguousarray(x)).to(dev) for x in (A, B, D))
+    aux = torch.from_numpy(scale).to(dev)
+    for variant in (8012, 8014, 8022, 8023):
+        e = torch.full((M, N), -7, dtype=torch.int32, device=dev)
+        desc = chain.bmm_chain_desc(a, b, d, e, "requant", tile_variant=variant)
+        assert chain.select_tile(desc).variant == variant
+        chain.run_bmm_chain(a, b, d, e, aux=aux, desc=desc)
+        torch.cuda.synchronize()
+        assert np.array_equal(e.cpu().numpy(), want), variant
+    with pytest.raises(ValueError):
+        chain.bmm_chain_desc(a, b, d, e, "requant", tile_variant=8013) and chain.select_tile(
+            chain.bmm_chain_desc(a, b, d, e, "requant", tile_variant=8013))
+
+
 def test_i8_chain_per_column_scales_and_saturation(oracle):
     M, K, L, N = 96, 256, 64, 48
     A, B, D, _ = oracle.make_i8_chain_inputs(M, K, L, N, seed=5)
