@@ -24,8 +24,8 @@ from ...hardware import query_hw_param
 
 # kernel codes of the fp16/bf16 chain: four waves x 32 | 64 rows, eight waves x 32 rows (staggered phases,
 # software pipelined, on the 16x16x32 MFMA with 256-row workgroups, the same with 384-row workgroups for the
-# first row blocks: the library refuses the last two unless B is stored [L][K]), four waves with 64-row workgroups on
-# the 16x16x32 MFMA (a wave owns 16 rows and all keys | 32 rows and half the keys; head size up to 64, B [L][K])
+# first row blocks: the library refuses these two unless B is stored [L][K]), four waves with 64-row workgroups on
+# the 16x16x32 MFMA (a wave owns 16 rows and all keys | 32 rows and half the keys; head size up to 64)
 FP_VARIANT_CODES = (1, 2, 8, 9, 6, 7, 4, 5)
 
 

@@ -179,32 +179,39 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     } else {
       plan->qt = 1;
     }
-    // Head size up to 64 with B stored [L][K]: the four-wave kernels with 64-row workgroups (4: a wave owns 16 rows
-    // and all keys; 5: 32 rows and half the keys of every tile, half the LDS reads per MFMA for a merge at the end,
-    // ahead from 1024 keys on).  Measured, fp16 and bf16, us per launch in a graph replay, best other variant ->
-    // best of 4 | 5: softmax 96 x 512 x 512 13.2 -> 11.5, 12 x 512 x 512 9.9 -> 6.9, 8 x 1024 x 1024 15.5 -> 9.9,
+    // Head size up to 64: the four-wave kernels with 64-row workgroups (4: a wave owns 16 rows and all keys; 5: 32
+    // rows and half the keys of every tile, half the LDS reads per MFMA for a merge at the end, ahead from 1024 keys
+    // on).  Measured, fp16 and bf16, us per launch in a graph replay, best other variant -> best of 4 | 5, B stored
+    // [L][K]: softmax 96 x 512 x 512 13.2 -> 11.5, 12 x 512 x 512 9.9 -> 6.9, 8 x 1024 x 1024 15.5 -> 9.9,
     // 16 x 512 x 2048 26.3 -> 15.5, 768 x 512 x 512 84.5 -> 78.1, 96 x 2048 x 2048 fp16 119.3 -> 116.7; bf16 at that
     // size and beyond stays on the eight-wave 16x16x32 kernel (115.6 against 120.1; 32 x 4096 x 4096 139.9 against
     // 150.6).  Without the softmax they are ahead below two 256-row workgroups per CU (96 x 512 x 512 11.2 -> 10.7,
     // 16 x 512 x 2048 17.0 -> 14.6) and behind from there on (384 x 512 x 512 38.9 against 39.3); where the 64-row
     // workgroups make one and a half rounds of the CUs and the 128-row ones fit in one, the latter stay
-    // (48 x 512 x 512 7.5 against 8.2).
-    if (plan->d_pad == 64 && d->b_layout == DITTO_B_LK) {
+    // (48 x 512 x 512 7.5 against 8.2).  B stored [K][L] (its fragments come out of transposing reads): softmax
+    // 96 x 512 x 512 13.1 -> 11.8, 12 x 512 x 512 10.0 -> 7.3, 16 x 512 x 2048 26.9 -> 16.6, 768 x 512 x 512
+    // 83.8 -> 81.8, level at 96 x 2048 x 2048 (122.7 / 121.6) and 32 x 4096 x 4096 (153.1 / 154.7: stays); without
+    // the softmax only the grids that leave CUs empty gain (12 x 512 x 512 7.5 -> 7.0, 8 x 1024 x 1024 10.9 -> 10.0,
+    // 16 x 512 x 2048 17.9 -> 16.0; but 96 x 512 x 512 10.7 against 11.6, 48 x 512 x 512 7.5 against 9.0).
+    if (plan->d_pad == 64) {
+      const bool lk = d->b_layout == DITTO_B_LK;
       const long long n64 = ((d->M + 63) / 64) * d->batch, n128 = ((d->M + 127) / 128) * d->batch;
       bool rows64;
       if (sm)
-        rows64 = !(in == DITTO_BF16 && n8 >= 2LL * cus && d->L >= 2048);
-      else
+        rows64 = !((in == DITTO_BF16 || !lk) && n8 >= 2LL * cus && d->L >= 2048);
+      else if (lk)
         rows64 = n8 < 2LL * cus && !(n64 > cus && n128 <= cus);
+      else
+        rows64 = n64 <= cus;
       if (rows64) plan->qt = d->L >= 1024 ? 5 : 4;
-      else if (sm && n8 >= 2LL * cus) plan->qt = 6;
+      else if (sm && lk && n8 >= 2LL * cus) plan->qt = 6;
     }
     if (d->tile_variant != 0) {
       const int q = d->tile_variant % 10;
       if (d->tile_variant / 10 != plan->d_pad || (q != 1 && q != 2 && q != 4 && q != 5 && q != 8 && q != 9 && q != 6 && q != 7))
         return fail(DITTO_EINVAL, "tile_variant %d cannot run this shape (head_pad %d; q must be 1, 2, 4, 5, 6, 7, 8 or 9)",
                     d->tile_variant, plan->d_pad);
-      if ((q == 4 || q == 5 || q == 6 || q == 7) && d->b_layout != DITTO_B_LK)
+      if ((q == 6 || q == 7) && d->b_layout != DITTO_B_LK)
         return fail(DITTO_EINVAL, "tile_variant %d (16x16x32 MFMA kernel) takes B stored [L][K]", d->tile_variant);
       if ((q == 4 || q == 5) && plan->d_pad != 64)
         return fail(DITTO_EINVAL, "tile_variant %d: the 64-row kernel serves head_pad 64 only", d->tile_variant);

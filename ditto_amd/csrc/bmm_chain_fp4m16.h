@@ -19,8 +19,10 @@
 //      keys; the two halves of a row are merged once, at the end, through LDS (each wave of a pair finishes one of the
 //      pair's two row tiles).  A step is a tenth shorter, the merge costs about what six steps save.
 //
-// LDS: a ring of three B tiles ([64 l][D k] as loaded) and three C tiles ([64 l][D n] as loaded).  A wave reads its
-// C^T fragments from the raw tile with two transposing reads (ds_read_b64_tr_b16) per fragment.
+// LDS: a ring of three B tiles ([64 l][D k] as loaded, or [D k][64 l] when B is stored [K][L]) and three C tiles
+// ([64 l][D n] as loaded).  A wave reads its C^T fragments from the raw tile with two transposing reads
+// (ds_read_b64_tr_b16) per fragment, and its B fragments likewise when B is stored [K][L]: the contraction index of
+// a fragment then runs 4 q .. + 3, 16 + 4 q .. + 3 within a step of 32, and the A fragments are loaded in that order.
 //
 // Softmax: the optimistic walk of bmm_chain_fp8m16.h (the reference exponent of a row is the maximum of the wave's
 // first keys; the lane's partial row SUM is watched once per tile and the reference raised by whole binary orders
@@ -48,7 +50,7 @@ __host__ __device__ constexpr int bmm_chain4m16_lds_bytes() {
   return 2 * kRing4m16 * kBN * D * 2 + 64;  // the tiles and the flag of the optimistic walk
 }
 
-template <typename T, int D, int INTER, int KSPLIT>
+template <typename T, int D, int INTER, int KSPLIT, bool B_KL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void bmm_chain4m16_kernel(BmmChainArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef typename Elem<T>::v8 V8;
@@ -90,46 +92,68 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   const int m_wave = mb * 64 + rh * (16 * RT);  // (either way 16 RT rows per unit of rh)
   const int M = p.M, N = p.N, K = p.K, L = p.L;
 
-  const unsigned b_bytes = (unsigned)((long long)(L - 1) * p.b_rs + K) * 2u;
+  const unsigned b_bytes = (unsigned)(B_KL ? ((long long)(K - 1) * p.b_rs + L) : ((long long)(L - 1) * p.b_rs + K)) * 2u;
   const unsigned c_bytes = (unsigned)((long long)(L - 1) * p.c_rs + N) * 2u;
   const i32x4 b_rsrc = make_rsrc(Bg, b_bytes);
   const i32x4 c_rsrc = make_rsrc(Cg, c_bytes);
   const unsigned lds0 = (unsigned)(size_t)(DITTO_LDS char*)smem_raw;
 
   // ---- A fragments first (their loads are the oldest in the vector-memory queue): lane holds
-  // A[16 j + c][32 st + 8 q .. + 7]
+  // A[16 j + c][32 st + 8 q .. + 7]; with B stored [K][L] its fragments come out of transposing reads with the
+  // contraction index in the order 4 q .. + 3, 16 + 4 q .. + 3 (like the C fragments), and A follows:
+  // A[16 j + c][32 st + 4 q .. + 3] and A[16 j + c][32 st + 16 + 4 q .. + 3]
   V8 af[RT][NS];
 #pragma unroll
   for (int j = 0; j < RT; ++j) {
     const int row = m_wave + 16 * j + c16;
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
-      const int col = 32 * st + 8 * q;
-      V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (row < M && col < K) v = *reinterpret_cast<const V8*>(Ag + (long long)row * p.a_rs + col);
-      af[j][st] = v;
+      if (B_KL) {
+        const int col = 32 * st + 4 * q;
+        V4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+        if (row < M && col < K) lo = *reinterpret_cast<const V4*>(Ag + (long long)row * p.a_rs + col);
+        if (row < M && col + 16 < K) hi = *reinterpret_cast<const V4*>(Ag + (long long)row * p.a_rs + col + 16);
+        af[j][st] = concat4<V4, V8>(lo, hi);
+      } else {
+        const int col = 32 * st + 8 * q;
+        V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (row < M && col < K) v = *reinterpret_cast<const V8*>(Ag + (long long)row * p.a_rs + col);
+        af[j][st] = v;
+      }
     }
   }
 
   // ---- per-lane source offsets of the direct loads: load i of this wave fills LDS bytes [1024 (NLD wave + i), + 1024)
   // of a tile, lane -> (row, physical chunk) -> swizzled source chunk
   int b_voff[NLD], c_voff[NLD];
+  int b_col[NLD];  // B stored [K][L] only: first key (within the tile) the lane loads
 #pragma unroll
   for (int i = 0; i < NLD; ++i) {
     const int gi = NLD * wave + i;
     const int row = gi * (64 / CPR) + lane / CPR, pc = lane % CPR;
-    const int bl = pc ^ swz4m16_rows(row);  // rows are l, columns k
-    b_voff[i] = bl * 8 < K ? (row * p.b_rs + bl * 8) * 2 : (int)b_bytes;
+    if (B_KL) {
+      const int bl = pc ^ swz4m16_tr(row);  // rows are k, columns l
+      b_col[i] = bl * 8;
+      b_voff[i] = row < K ? (row * p.b_rs + bl * 8) * 2 : (int)b_bytes;
+    } else {
+      const int bl = pc ^ swz4m16_rows(row);  // rows are l, columns k
+      b_col[i] = 0;
+      b_voff[i] = bl * 8 < K ? (row * p.b_rs + bl * 8) * 2 : (int)b_bytes;
+    }
     const int cl = pc ^ swz4m16_tr(row);    // rows are l, columns n
     c_voff[i] = cl * 8 < N ? (row * p.c_rs + cl * 8) * 2 : (int)c_bytes;
   }
   // tiles past the last one are out of range and load zeros
   const unsigned lds_wave = lds0 + 1024 * NLD * wave;  // this wave's share of a tile slot
   auto load_tile = [&](int tile, int buf) __attribute__((always_inline)) {
-    int bo = tile * kBN * p.b_rs * 2, co = tile * kBN * p.c_rs * 2;
+    int bo = B_KL ? tile * kBN * 2 : tile * kBN * p.b_rs * 2, co = tile * kBN * p.c_rs * 2;
     asm volatile("" : "+s"(bo), "+s"(co));
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) lds_dma_16_at(b_rsrc, (unsigned)(b_voff[i] + bo), lds_wave, B_OFF + buf * TB + 1024 * i);
+    for (int i = 0; i < NLD; ++i) {
+      int vo = b_voff[i] + bo;
+      if (B_KL) vo = (tile * kBN + b_col[i] < L) ? vo : (int)b_bytes;  // keys past L lie inside the buffer (the next row)
+      lds_dma_16_at(b_rsrc, (unsigned)vo, lds_wave, B_OFF + buf * TB + 1024 * i);
+    }
 #pragma unroll
     for (int i = 0; i < NLD; ++i) lds_dma_16_at(c_rsrc, (unsigned)(c_voff[i] + co), lds_wave, C_OFF + buf * TB + 1024 * i);
   };
@@ -137,9 +161,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   // ---- per-lane LDS read addresses (bytes within a tile), loop invariant; the wave's key half is folded in
   // B fragment (16-row tile i of the key half, k step st): row 32 kh + 16 i + c, logical chunk 4 st + q; the swizzle
   // of that row does not depend on kh or i
-  int b_ad[NS];
+  // B stored [K][L]: the tile is [k][64 l] and a fragment (tile i, k step st) is read like a C^T fragment:
+  // rows 32 st + 4 q + {0..3} (and + 16) x columns 16 (2 kh + i) .. + 15
+  constexpr int NBA = B_KL ? NI : NS;
+  int b_ad[NBA];
+  if (B_KL) {
 #pragma unroll
-  for (int st = 0; st < NS; ++st) b_ad[st] = (32 * kh + c16) * RB + (((4 * st + q) ^ swz4m16_rows(c16)) * 16);
+    for (int i = 0; i < NI; ++i) {
+      const int row = 4 * q + (c16 >> 2);
+      const int chunk = 2 * (NI * kh + i) + ((c16 & 3) >> 1);
+      b_ad[i] = row * RB + ((chunk ^ swz4m16_tr(row)) * 16) + 8 * (c16 & 1);
+    }
+  } else {
+#pragma unroll
+    for (int st = 0; st < NS; ++st) b_ad[st] = (32 * kh + c16) * RB + (((4 * st + q) ^ swz4m16_rows(c16)) * 16);
+  }
   // C^T fragment (column tile t) of the key half: the 16 lanes of group q read rows 32 kh + 4 q + {0..3} (and + 16) x
   // columns 16 t .. + 15; lane s of the group points at row s / 4, 8 bytes at column 4 (s % 4).  The swizzle of a row
   // depends on row % 8 only.
@@ -151,7 +187,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     c_ad[t] = (32 * kh + row) * RB + ((chunk ^ swz4m16_tr(row)) * 16) + 8 * (c16 & 1) + C_OFF;
   }
   auto b_frag = [&](int buf, int i, int st) __attribute__((always_inline)) -> V8 {
-    return *reinterpret_cast<const V8*>(smem_raw + b_ad[st] + (B_OFF + buf * TB + 16 * i * RB));
+    if (B_KL) {
+      const char* a = smem_raw + b_ad[i % NBA] + (B_OFF + buf * TB + 32 * st * RB);
+      V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(a));
+      V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(a + 16 * RB));
+      return concat4<V4, V8>(lo, hi);
+    }
+    return *reinterpret_cast<const V8*>(smem_raw + b_ad[st % NBA] + (B_OFF + buf * TB + 16 * i * RB));
   };
   auto c_frag = [&](int buf, int h, int t) __attribute__((always_inline)) -> V8 {
     const char* a = smem_raw + c_ad[t] + (buf * TB + 32 * h * RB);
@@ -463,10 +505,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #endif
 }
 
-template <typename T, int D, int INTER, int KSPLIT>
+template <typename T, int D, int INTER, int KSPLIT, bool B_KL>
 hipError_t launch_bmm_chain4m16(const BmmChainArgs& args, hipStream_t stream) {
   constexpr int lds = bmm_chain4m16_lds_bytes<D>();
-  auto kern = bmm_chain4m16_kernel<T, D, INTER, KSPLIT>;
+  auto kern = bmm_chain4m16_kernel<T, D, INTER, KSPLIT, B_KL>;
   static thread_local int configured_dev = -1;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);

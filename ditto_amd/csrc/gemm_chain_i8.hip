@@ -226,7 +226,7 @@ __global__ __launch_bounds__(64 * i8::NW) void gemm_chain_i8_kernel(I8ChainArgs 
     int c_stage = 0;
     for (int ob = 0; ob < nlc; ++ob) {
       for (int ib = 0; ib < nk; ++ib) {
-        __syncthreads();
+        wg_sync();  // (explicit wait for this wave's own LDS accesses: the packed middle result of the last chunk)
         const char* st = smem_raw + c_stage * STAGE;
         c_stage = c_stage + 1 == NST ? 0 : c_stage + 1;
         // all fragments of the chunk first (one LDS round trip), then the MFMAs

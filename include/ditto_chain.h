@@ -159,7 +159,7 @@ typedef struct ditto_tile_param {
                              [L][K] only), q = 7 (the same kernel with 384-row workgroups, 48 rows
                              per wave, for the first row blocks of a batch entry and 256-row ones
                              for the rest; block_m reports 384); four waves on the 16x16x32 MFMA
-                             with 64-row workgroups (head_pad 64, B stored [L][K] only): q = 4 (a
+                             with 64-row workgroups (head_pad 64, either layout of B): q = 4 (a
                              wave owns 16 rows and all keys), q = 5 (32 rows and half the keys of
                              every tile); conv chains: the ids listed at
                              ditto_conv_chain_desc.tile_variant; fp32 / fp64 1000 / 1001; int8

@@ -84,9 +84,9 @@ def test_select_tile_and_validation_without_gpu():
     assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(tile_variant=1288)), ctypes.byref(tile)) == _lib.EINVAL
     assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(tile_variant=643)), ctypes.byref(tile)) == _lib.EINVAL
     # the kernel on the 16x16x32 MFMA reads B stored [L][K] only
-    for v in (646, 644, 645):
+    for v, rc in ((646, _lib.EINVAL), (647, _lib.EINVAL), (644, _lib.OK), (645, _lib.OK)):
         kl = _desc(tile_variant=v, b_layout=_lib.B_KL, b_row_stride=512)
-        assert lib.ditto_bmm_chain_select_tile(ctypes.byref(kl), ctypes.byref(tile)) == _lib.EINVAL
+        assert lib.ditto_bmm_chain_select_tile(ctypes.byref(kl), ctypes.byref(tile)) == rc
     # the 64-row kernels serve head sizes up to 64
     wide = _desc(tile_variant=1284, N=128, K=128, a_row_stride=128, b_row_stride=128, c_row_stride=128, f_row_stride=128,
                  a_batch_stride=512 * 128, b_batch_stride=512 * 128, c_batch_stride=512 * 128, f_batch_stride=512 * 128)
