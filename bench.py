@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused operator chains on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-also]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-also] [--no-zero]
 
 A "step" is one call of the fused chain on one batch of synthetic input that is already
 resident in HBM.  The headline workload is the long-sequence BMM -> softmax -> BMM chain
@@ -360,7 +360,7 @@ def config1_cpu(repeats=40):
                       "128 MiB streamed between calls" % repeats}
 
 
-def run_one(name, steps, warmup, dev, long_run=False):
+def run_one(name, steps, warmup, dev, long_run=False, zero_leg=True):
     w = WORKLOADS[name]
     wall_ms, ev_ms, gr_ms, tile, long_ms = time_gpu(w, steps, warmup, dev, long_run=long_run)
     fl, by = flops_of(w), bytes_of(w)
@@ -382,7 +382,7 @@ def run_one(name, steps, warmup, dev, long_run=False):
     roof["graph_replay_ms"] = gr_ms
     if long_ms is not None:
         roof["min_repeat_600ms_ms"] = long_ms
-    if long_run and w["bound"] == "mfma" and w["kind"] in ("softmax", "cast"):
+    if long_run and zero_leg and w["bound"] == "mfma" and w["kind"] in ("softmax", "cast"):
         # The same launch on all-zero operands: the same instruction stream without the switching activity of
         # real data.  The gap to kernel_ms is what the device's power management takes on N(0,1) operands.
         zcall, _ = make_call(w, dev, zero=True)
@@ -405,6 +405,9 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-also", action="store_true", help="skip the brief runs of the other configurations")
+    ap.add_argument("--no-zero", action="store_true",
+                    help="skip the launches on all-zero operands (a kernel trace of the run then averages the launches on "
+                         "N(0,1) operands only)")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="also launch one plain device copy of MIB MiB (read MIB, write MIB): a dispatch of known "
                          "traffic against which rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled")
@@ -427,7 +430,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    w, wall_ms, ev_ms, tile, roof = run_one(args.workload, args.steps, args.warmup, dev, long_run=True)
+    w, wall_ms, ev_ms, tile, roof = run_one(args.workload, args.steps, args.warmup, dev, long_run=True,
+                                            zero_leg=not args.no_zero)
     fl = flops_of(w)
     value = fl / (wall_ms * 1e-3) / 1e12
     short = SHORT[w["dtype"]]
