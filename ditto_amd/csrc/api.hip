@@ -162,18 +162,19 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
     // workgroups.  Below 3/4 of the CUs the four-wave kernel with 128-row workgroups spreads over more
     // CUs.  From there on eight waves (two per SIMD) win, in their software-pipelined form (9) at every
     // size measured.  Once there are two workgroups per CU the chip runs at its power limit and the
-    // kernel on the 16x16x32 MFMA (6; B stored [L][K] only), which needs less energy per flop, is ahead
+    // kernel on the 16x16x32 MFMA (6), which needs less energy per flop, is ahead
     // (64 x 4096 x 4096 x 128 bf16: 464 vs 484 us with the softmax, 410 vs 443 us without); at
     // head_pad 64 the pipelined kernel stays (32 x 4096 x 4096 x 64 without softmax 127.9 vs 130.0 us).
-    // With B stored [K][L] and no softmax (nothing for a second wave per SIMD to overlap) the four-wave,
-    // 256-row kernel stays (429 vs 443 us).
+    // With B stored [K][L] (B fragments through transposing reads on the 16x16x32 kernel) the softmax at
+    // head_pad 128 goes the same way (bf16 441 vs 503 us, fp16 482 vs 538), without softmax the four-wave,
+    // 256-row kernel stays (431 vs 430 us).
     const long long n8 = ((d->M + 255) / 256) * d->batch;
     const bool sm = d->inter_op == DITTO_INTER_SOFTMAX;
     if (n8 >= 2LL * cus) {
       if (d->b_layout == DITTO_B_LK)
         plan->qt = plan->d_pad == 64 ? 9 : 6;
       else
-        plan->qt = sm ? 9 : 2;
+        plan->qt = sm ? (plan->d_pad == 64 ? 9 : 6) : 2;
     } else if (n8 * 4 >= 3LL * cus) {
       plan->qt = 9;
     } else {
@@ -211,8 +212,6 @@ int plan_bmm(const ditto_bmm_chain_desc* d, BmmPlan* plan, bool need_device) {
       if (d->tile_variant / 10 != plan->d_pad || (q != 1 && q != 2 && q != 4 && q != 5 && q != 8 && q != 9 && q != 6 && q != 7))
         return fail(DITTO_EINVAL, "tile_variant %d cannot run this shape (head_pad %d; q must be 1, 2, 4, 5, 6, 7, 8 or 9)",
                     d->tile_variant, plan->d_pad);
-      if ((q == 6 || q == 7) && d->b_layout != DITTO_B_LK)
-        return fail(DITTO_EINVAL, "tile_variant %d (16x16x32 MFMA kernel) takes B stored [L][K]", d->tile_variant);
       if ((q == 4 || q == 5) && plan->d_pad != 64)
         return fail(DITTO_EINVAL, "tile_variant %d: the 64-row kernel serves head_pad 64 only", d->tile_variant);
       plan->qt = q;

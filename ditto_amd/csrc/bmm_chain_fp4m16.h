@@ -27,8 +27,8 @@
 // Softmax: the optimistic walk of bmm_chain_fp8m16.h (the reference exponent of a row is the maximum of the wave's
 // first keys; the lane's partial row SUM is watched once per tile and the reference raised by whole binary orders
 // when it passes a limit; a sum that ends up infinite or NaN sends the workgroup through the exact walk), for bf16
-// and for fp16: an fp16 probability overflows at 2^16, so the limit is 2^10 there and a row whose scores climb by
-// more than 2^6 within one tile takes the second walk.  fp16 also uses the pre-scaled form of the pipelined
+// and for fp16: an fp16 probability overflows at 2^16, so the limit is 2^8 there and a row whose scores climb by
+// more than 2^8 within one tile takes the second walk.  fp16 also uses the pre-scaled form of the pipelined
 // eight-wave kernel: A is multiplied by scale * log2(e) once and every score tile starts from minus the reference
 // exponent, so a score costs its v_exp_f32 and nothing else.
 #pragma once
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   constexpr bool kSoftmax = INTER == kInterSoftmax;
   constexpr bool PRE = kSoftmax && !Elem<T>::is_bf16;
   // a lane's partial row sum above which the reference exponent is raised
-  constexpr float kLimit = Elem<T>::is_bf16 ? 4294967296.f : 1024.f;
+  constexpr float kLimit = Elem<T>::is_bf16 ? kSumLimitBf16 : kSumLimitF16;
 
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   const int tid = threadIdx.x, lane = tid & 63;

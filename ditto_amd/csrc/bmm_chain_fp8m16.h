@@ -127,15 +127,31 @@ __device__ __forceinline__ float quad_sum(float x) {
   return pair_sum(a + b);
 }
 
+// XOR applied to the 16-byte chunk index of a 128-byte row ([k][64 l] tiles of a B stored [K][L]) for the
+// transposing read with lanes (c, q) -> row 4 q + c / 4: 2.3 cycles per instruction with eight waves reading, against
+// 4 under the swizzle of the once-per-tile transposition passes
+__device__ __forceinline__ int swz_kl_tr(int row) { return 2 * ((row >> 1) & 3); }
+
+// The lane's id within its wave, computed where it is called (from an asm the compiler neither hoists nor merges):
+// for code behind a long loop that would otherwise keep the id in a register through it.
+__device__ __forceinline__ int fresh_lane_id() {
+  int ln;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+  return ln;
+}
+
 template <bool B>
 struct BoolC {
   static constexpr bool value = B;
 };
 // a lane's partial row sum above which the optimistic walk lowers the row's scale (2^32)
-constexpr float kSumLimit = 4294967296.f;
+constexpr float kSumLimitBf16 = 4294967296.f;
+// fp16: a probability overflows at 2^16, so the scale is lowered from 2^8 on and a row whose scores climb by more
+// than 2^8 within one tile of 64 keys ends with an infinite sum (and takes the exact walk)
+constexpr float kSumLimitF16 = 256.f;
 
 // One workgroup's walk: eight waves of RT 16-row tiles each, rows row0 .. row0 + 128 RT - 1 of batch entry bz.
-template <typename T, int D, int INTER, int RT>
+template <typename T, int D, int INTER, int RT, bool B_KL>
 __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* smem_raw, int row0, int bz) {
   typedef typename Elem<T>::v8 V8;
   typedef typename Elem<T>::v4 V4;
@@ -144,11 +160,12 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
 #ifdef DITTO_M16_NO_OPTIMISTIC
   constexpr bool kOptimistic = false;
 #else
-  // bf16 only: an fp16 probability overflows 2^16, far below what a tile's scores may climb between two votes
-  constexpr bool kOptimistic = INTER == kInterSoftmax && Elem<T>::is_bf16;
+  constexpr bool kOptimistic = INTER == kInterSoftmax;
 #endif
+  constexpr float kSumLimit = Elem<T>::is_bf16 ? kSumLimitBf16 : kSumLimitF16;
   constexpr int TB = kBN * D * 2;     // bytes per tile
-  constexpr int B_RB = D * 2;         // bytes per LDS row of a B tile ([L][K])
+  // bytes per LDS row of a B tile: [L][K] as stored, or, with B stored [K][L], [K][64 l]
+  constexpr int B_RB = B_KL ? kBN * 2 : D * 2;
   constexpr int B_CPR = B_RB / 16;
   constexpr int C_RB = D * 2;
   constexpr int C_CPR = C_RB / 16;
@@ -184,7 +201,7 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
   const int m_wave = row0 + wave * 16 * RT;
   const int M = p.M, N = p.N, K = p.K, L = p.L;
 
-  const unsigned b_bytes = (unsigned)((long long)(L - 1) * p.b_rs + K) * 2u;
+  const unsigned b_bytes = (unsigned)(B_KL ? ((long long)(K - 1) * p.b_rs + L) : ((long long)(L - 1) * p.b_rs + K)) * 2u;
   const unsigned c_bytes = (unsigned)((long long)(L - 1) * p.c_rs + N) * 2u;
   const i32x4 b_rsrc = make_rsrc(Bg, b_bytes);
   const i32x4 c_rsrc = make_rsrc(Cg, c_bytes);
@@ -197,8 +214,13 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
     const int gi = NLD * wave + i;
     {
       const int row = gi * (64 / B_CPR) + lane / B_CPR, pc = lane % B_CPR;
-      const int cl = pc ^ swz_rowread<B_CPR>(row);  // rows are l, columns k
-      b_voff[i] = cl * 8 < K ? (row * p.b_rs + cl * 8) * 2 : (int)b_bytes;
+      if (B_KL) {
+        const int cl = pc ^ swz_kl_tr(row);  // rows are k, columns l
+        b_voff[i] = row < K ? (row * p.b_rs + cl * 8) * 2 : (int)b_bytes;
+      } else {
+        const int cl = pc ^ swz_rowread<B_CPR>(row);  // rows are l, columns k
+        b_voff[i] = cl * 8 < K ? (row * p.b_rs + cl * 8) * 2 : (int)b_bytes;
+      }
     }
     {
       const int row = gi * (64 / C_CPR) + lane / C_CPR, pc = lane % C_CPR;
@@ -207,11 +229,22 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
     }
   }
   auto load_b = [&](int tile, int buf) __attribute__((always_inline)) {
-    int soff = tile * kBN * p.b_rs * 2;
+    int soff = B_KL ? tile * kBN * 2 : tile * kBN * p.b_rs * 2;
     asm volatile("" : "+s"(soff));  // one add per load, not a hoisted address register per load and tile slot
+    // B stored [K][L]: the first column l (within the tile) the lane loads is the same for all of its loads (their rows
+    // differ by multiples of 8 and the swizzle looks at row % 8: lane / 8 here); taken from the lane id afresh rather
+    // than kept in a register through the walk
+    int b_col = 0;
+    if (B_KL) {
+      const int ln = fresh_lane_id();
+      b_col = 8 * ((ln & 7) ^ swz_kl_tr(ln >> 3));
+    }
 #pragma unroll
-    for (int i = 0; i < NLD; ++i)
-      lds_dma_16(b_rsrc, (unsigned)(b_voff[i] + soff), lds0 + B_LOAD + buf * TB + 1024 * (NLD * wave + i));
+    for (int i = 0; i < NLD; ++i) {
+      int vo = b_voff[i] + soff;
+      if (B_KL) vo = (tile * kBN + b_col < L) ? vo : (int)b_bytes;  // columns past L lie inside the buffer (the next row)
+      lds_dma_16(b_rsrc, (unsigned)vo, lds0 + B_LOAD + buf * TB + 1024 * (NLD * wave + i));
+    }
   };
   auto load_c = [&](int tile, int buf) __attribute__((always_inline)) {
     int soff = tile * kBN * p.c_rs * 2;
@@ -224,21 +257,41 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
   // ---- per-lane LDS read addresses (bytes within a tile), loop invariant
   // B fragment (i = 16-row tile of the 64-row L tile, st = k step): row 16 i + c, logical chunks 4 st + q
   // (256-byte rows: the swizzle of row 16 i + c does not depend on i, so the tile index is a constant offset)
-  constexpr int NBI = B_CPR == 16 ? 1 : 4;
-  int b_ad[NBI][NS];
+  // B stored [K][L]: the tile is [k][64 l], 128-byte rows, and fragment (i, st) comes out of two transposing reads
+  // like a C fragment does in the transposition pass: rows 32 st + 4 q + {0..3} (and + 16) x columns 16 i .. + 15,
+  // so its contraction index runs 4 q .. + 3, 16 + 4 q .. + 3 within the step and the A fragments are loaded in
+  // that order; the address depends on i (the swizzle on the row % 8 only), the k step is a constant offset
+  constexpr int NBI = B_KL ? 4 : B_CPR == 16 ? 1 : 4;
+  constexpr int NBS = B_KL ? 1 : NS;
+  int b_ad[NBI][NBS];
+  if (B_KL) {
 #pragma unroll
-  for (int i = 0; i < NBI; ++i)
+    for (int i = 0; i < NBI; ++i) {
+      const int row = 4 * q + (c16 >> 2);
+      const int chunk = 2 * i + ((c16 & 3) >> 1);
+      b_ad[i][0] = row * B_RB + ((chunk ^ swz_kl_tr(row)) * 16) + 8 * (c16 & 1);
+    }
+  } else {
 #pragma unroll
-    for (int st = 0; st < NS; ++st)
-      b_ad[i][st] = (16 * i + c16) * B_RB + (((4 * st + q) ^ swz_rowread<B_CPR>(16 * i + c16)) * 16);
+    for (int i = 0; i < NBI; ++i)
+#pragma unroll
+      for (int st = 0; st < NBS; ++st)
+        b_ad[i][st] = (16 * i + c16) * B_RB + (((4 * st + q) ^ swz_rowread<B_CPR>(16 * i + c16)) * 16);
+  }
   // Fragment-major and raw C tiles lie beyond the 64 KB an LDS instruction's offset field reaches: each
   // region gets ONE base register, kept opaque so that the compiler folds only the small remainder into the
   // instructions' offsets (it otherwise makes an address register per buffer and fragment, and spills)
   int frag_ad = lane * 16 + C_FRAG;
   asm volatile("" : "+v"(frag_ad));
   auto b_frag = [&](int off, int i, int st) __attribute__((always_inline)) -> V8 {
-    if (NBI == 1) return *reinterpret_cast<const V8*>(smem_raw + b_ad[0][st] + (off + 16 * i * B_RB));
-    return *reinterpret_cast<const V8*>(smem_raw + b_ad[i % NBI][st] + off);
+    if (B_KL) {
+      const char* a = smem_raw + b_ad[i % NBI][0] + (off + 32 * st * B_RB);
+      V4 lo = lds_read_tr4<T>(reinterpret_cast<const T*>(a));
+      V4 hi = lds_read_tr4<T>(reinterpret_cast<const T*>(a + 16 * B_RB));
+      return concat4<V4, V8>(lo, hi);
+    }
+    if (NBI == 1) return *reinterpret_cast<const V8*>(smem_raw + b_ad[0][st % NBS] + (off + 16 * i * B_RB));
+    return *reinterpret_cast<const V8*>(smem_raw + b_ad[i % NBI][st % NBS] + off);
   };
   auto frag_rd = [&](int off, int f) __attribute__((always_inline)) -> V8 {
     return *reinterpret_cast<const V8*>(smem_raw + frag_ad + (off - C_FRAG + 1024 * f));
@@ -280,10 +333,18 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
     const int row = m_wave + 16 * j + c16;
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
-      const int col = 32 * st + 8 * q;
-      V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (row < M && col < K) v = *reinterpret_cast<const V8*>(Ag + (long long)row * p.a_rs + col);
-      af[j][st] = v;
+      if (B_KL) {
+        const int col = 32 * st + 4 * q;
+        V4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+        if (row < M && col < K) lo = *reinterpret_cast<const V4*>(Ag + (long long)row * p.a_rs + col);
+        if (row < M && col + 16 < K) hi = *reinterpret_cast<const V4*>(Ag + (long long)row * p.a_rs + col + 16);
+        af[j][st] = concat4<V4, V8>(lo, hi);
+      } else {
+        const int col = 32 * st + 8 * q;
+        V8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (row < M && col < K) v = *reinterpret_cast<const V8*>(Ag + (long long)row * p.a_rs + col);
+        af[j][st] = v;
+      }
     }
   }
 
@@ -546,9 +607,11 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
     int* const flag = reinterpret_cast<int*>(smem_raw);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no direct load still on its way into LDS
     wg_sync();
-    if (tid == 0) *flag = 0;
+    // (B stored [K][L]: that instantiation has no register left to keep the lane id through the walk)
+    const int lane_f = B_KL ? fresh_lane_id() : lane;
+    if (B_KL ? (lane_f == 0 && wave == 0) : tid == 0) *flag = 0;
     wg_sync();
-    if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0) *flag = 1;
+    if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane_f == 0) *flag = 1;
     wg_sync();
     const int again = __builtin_amdgcn_readfirstlane(*flag);
     if (again) {
@@ -624,7 +687,7 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
 // that 384 does not divide fill the device evenly: 4096 rows on four compute units are 2 x 384 + 256 each.  Ids are
 // dealt so that every XCD first gets the large blocks of all of its batch entries, then the small ones (longest
 // first: the small blocks fill the gaps at the end).
-template <typename T, int D, int INTER>
+template <typename T, int D, int INTER, bool B_KL>
 __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -637,21 +700,21 @@ __global__ __launch_bounds__(512) void bmm_chain8m16_kernel(BmmChainArgs p) {
   }
   if (idx < per * nb3) {
     const int e = idx / nb3, mb = idx - e * nb3;
-    bmm_chain8m16_body<T, D, INTER, 3>(p, smem_raw, 384 * mb, x * per + e);
+    bmm_chain8m16_body<T, D, INTER, 3, B_KL>(p, smem_raw, 384 * mb, x * per + e);
   } else {
     const int r = idx - per * nb3;
     const int e = r / nb2, mb = r - e * nb2;
-    bmm_chain8m16_body<T, D, INTER, 2>(p, smem_raw, 384 * nb3 + 256 * mb, x * per + e);
+    bmm_chain8m16_body<T, D, INTER, 2, B_KL>(p, smem_raw, 384 * nb3 + 256 * mb, x * per + e);
   }
 #else
   (void)p;
 #endif
 }
 
-template <typename T, int D, int INTER>
+template <typename T, int D, int INTER, bool B_KL>
 hipError_t launch_bmm_chain8m16(const BmmChainArgs& args, hipStream_t stream) {
   constexpr int lds = bmm_chain8m16_lds_bytes<D>();
-  auto kern = bmm_chain8m16_kernel<T, D, INTER>;
+  auto kern = bmm_chain8m16_kernel<T, D, INTER, B_KL>;
   static thread_local int configured_dev = -1;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);

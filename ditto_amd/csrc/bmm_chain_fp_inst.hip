@@ -8,7 +8,7 @@
 namespace ditto {
 
 // q = 1 | 2: four-wave kernel, 32*q rows per wave; q = 8: eight-wave kernel; q = 9: eight-wave kernel,
-// software pipelined; q = 6 | 7: eight-wave kernel on the 16x16x32 MFMA (B stored [L][K] only; 7: args.mblocks3 of a
+// software pipelined; q = 6 | 7: eight-wave kernel on the 16x16x32 MFMA (7: args.mblocks3 of a
 // batch entry's row blocks have 384 rows); q = 4 | 5: four-wave kernel on the 16x16x32 MFMA, 64-row workgroups (head_pad 64;
 // 5: the waves split the keys of a tile as well as the rows)
 hipError_t DITTO_INST_NAME(int d_pad, int q, bool b_kl, const BmmChainArgs& args, hipStream_t stream) {
@@ -27,7 +27,8 @@ hipError_t DITTO_INST_NAME(int d_pad, int q, bool b_kl, const BmmChainArgs& args
     return b_kl ? launch_bmm_chain8<T, DP, I, true, true>(args, stream)    \
                 : launch_bmm_chain8<T, DP, I, false, true>(args, stream);
 #define DITTO_CASE6(DP)                                                    \
-  if (d_pad == DP && (q == 6 || q == 7)) return b_kl ? hipErrorInvalidValue : launch_bmm_chain8m16<T, DP, I>(args, stream);
+  if (d_pad == DP && (q == 6 || q == 7))                                   \
+    return b_kl ? launch_bmm_chain8m16<T, DP, I, true>(args, stream) : launch_bmm_chain8m16<T, DP, I, false>(args, stream);
   if (d_pad == 64 && q == 4)
     return b_kl ? launch_bmm_chain4m16<T, 64, I, 1, true>(args, stream) : launch_bmm_chain4m16<T, 64, I, 1, false>(args, stream);
   if (d_pad == 64 && q == 5)

@@ -155,8 +155,7 @@ typedef struct ditto_tile_param {
   int32_t variant;        /* kernel variant id: fp16/bf16 chains head_pad*10 + q, with
                              q = 1|2: four waves owning 32*q rows each; eight waves owning
                              32 rows each: q = 8 (phases staggered between the two waves of a
-                             SIMD), q = 9 (software pipelined), q = 6 (16x16x32 MFMA, B stored
-                             [L][K] only), q = 7 (the same kernel with 384-row workgroups, 48 rows
+                             SIMD), q = 9 (software pipelined), q = 6 (16x16x32 MFMA), q = 7 (the same kernel with 384-row workgroups, 48 rows
                              per wave, for the first row blocks of a batch entry and 256-row ones
                              for the rest; block_m reports 384); four waves on the 16x16x32 MFMA
                              with 64-row workgroups (head_pad 64, either layout of B): q = 4 (a

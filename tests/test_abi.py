@@ -83,10 +83,10 @@ def test_select_tile_and_validation_without_gpu():
         assert tile.lds_bytes <= 160 * 1024
     assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(tile_variant=1288)), ctypes.byref(tile)) == _lib.EINVAL
     assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(tile_variant=643)), ctypes.byref(tile)) == _lib.EINVAL
-    # the kernel on the 16x16x32 MFMA reads B stored [L][K] only
-    for v, rc in ((646, _lib.EINVAL), (647, _lib.EINVAL), (644, _lib.OK), (645, _lib.OK)):
+    # every kernel reads B in either layout
+    for v in (646, 647, 644, 645):
         kl = _desc(tile_variant=v, b_layout=_lib.B_KL, b_row_stride=512)
-        assert lib.ditto_bmm_chain_select_tile(ctypes.byref(kl), ctypes.byref(tile)) == rc
+        assert lib.ditto_bmm_chain_select_tile(ctypes.byref(kl), ctypes.byref(tile)) == _lib.OK and tile.variant == v
     # the 64-row kernels serve head sizes up to 64
     wide = _desc(tile_variant=1284, N=128, K=128, a_row_stride=128, b_row_stride=128, c_row_stride=128, f_row_stride=128,
                  a_batch_stride=512 * 128, b_batch_stride=512 * 128, c_batch_stride=512 * 128, f_batch_stride=512 * 128)
@@ -98,8 +98,10 @@ def test_select_tile_and_validation_without_gpu():
                 b_batch_stride=4096 * 128, c_batch_stride=4096 * 128, f_batch_stride=4096 * 128)
     assert lib.ditto_bmm_chain_select_tile(ctypes.byref(big), ctypes.byref(tile)) == _lib.OK and tile.variant == 1287
     assert (tile.block_m, tile.grid_x) == (384, 64 * 12)
-    big.b_layout, big.b_row_stride = _lib.B_KL, 4096
-    assert lib.ditto_bmm_chain_select_tile(ctypes.byref(big), ctypes.byref(tile)) == _lib.OK and tile.variant == 1289
+    big.b_layout, big.b_row_stride = _lib.B_KL, 4096   # keys stored [K][L]: the same kernel (transposing reads)
+    assert lib.ditto_bmm_chain_select_tile(ctypes.byref(big), ctypes.byref(tile)) == _lib.OK and tile.variant == 1287
+    big.inter_op = _lib.INTER_CAST                    # without the softmax: four waves, 256-row workgroups
+    assert lib.ditto_bmm_chain_select_tile(ctypes.byref(big), ctypes.byref(tile)) == _lib.OK and tile.variant == 1282
     assert lib.ditto_bmm_chain_select_tile(ctypes.byref(_desc(relu_out=2)), ctypes.byref(tile)) == _lib.EINVAL
     # the long-sequence configuration picks the 128-wide head tile
     big = _desc(in_dtype=_lib.BF16, out_dtype=_lib.BF16, batch=64, M=4096, L=4096, K=128, N=128,
