@@ -32,6 +32,13 @@ def _code(t):
         raise ValueError("unsupported tensor dtype %s" % t.dtype)
 
 
+def _raw_stream(index):
+    """Handle of torch's current stream on device ``index`` (what ``torch.cuda.current_stream(i).cuda_stream`` returns,
+    without building the Stream object)."""
+    get = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    return get(index) if get is not None else torch.cuda.current_stream(index).cuda_stream
+
+
 def _check_device(*tensors):
     dev = tensors[0].device
     if dev.type != "cuda":
@@ -143,11 +150,16 @@ def run_bmm_chain(A, B, C, F, inter_op="cast", softmax_scale=1.0, requant_scale=
         if aux.dtype != torch.float32 or not aux.is_contiguous() or aux.numel() != desc.L:
             raise ValueError("aux must be a contiguous fp32 tensor of L = %d scales" % desc.L)
         aux_ptr = aux.data_ptr()
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
+    if torch.cuda.current_device() == dev.index:
+        # (the common case, kept short: for the smallest chains the host's call path is longer than the kernel)
         rc = lib.ditto_bmm_chain_run(ctypes.byref(desc), A.data_ptr(), B.data_ptr(), C.data_ptr(), aux_ptr,
-                                     F.data_ptr(), None, 0, stream)
-    _lib.check(rc)
+                                     F.data_ptr(), None, 0, _raw_stream(dev.index))
+    else:
+        with torch.cuda.device(dev):
+            rc = lib.ditto_bmm_chain_run(ctypes.byref(desc), A.data_ptr(), B.data_ptr(), C.data_ptr(), aux_ptr,
+                                         F.data_ptr(), None, 0, _raw_stream(dev.index))
+    if rc:
+        _lib.check(rc)
     return F
 
 
@@ -249,11 +261,14 @@ def run_conv_chain(X, W1, W2, Y, pad1=1, stride1=1, pad2=0, stride2=1, inter_op=
         ws = None
     else:
         ws = workspace
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
-        fn = lib.ditto_conv_chain_run_prepared if prepared else lib.ditto_conv_chain_run
-        rc = fn(ctypes.byref(desc), X.data_ptr(), W1.data_ptr(), W2.data_ptr(),
-                Y.data_ptr(), ws.data_ptr() if ws is not None else None,
-                ws.numel() * ws.element_size() if ws is not None else 0, stream)
-    _lib.check(rc)
+    fn = lib.ditto_conv_chain_run_prepared if prepared else lib.ditto_conv_chain_run
+    args = (ctypes.byref(desc), X.data_ptr(), W1.data_ptr(), W2.data_ptr(), Y.data_ptr(),
+            ws.data_ptr() if ws is not None else None, ws.numel() * ws.element_size() if ws is not None else 0)
+    if torch.cuda.current_device() == dev.index:
+        rc = fn(*args, _raw_stream(dev.index))
+    else:
+        with torch.cuda.device(dev):
+            rc = fn(*args, _raw_stream(dev.index))
+    if rc:
+        _lib.check(rc)
     return Y
