@@ -502,7 +502,9 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
 #pragma unroll
     for (int j = 0; j < RT; ++j) {
       make_p(cur, j, pf[j]);
-      asm volatile("" : "+v"(pf[j]));
+      // (the row sum is named too: left free, its dots sink to the end of the tile, and the rounded pairs they read
+      // then have to be kept in a second set of registers next to the operand)
+      asm volatile("" : "+v"(pf[j]), "+v"(lsum[j]));
     }
     __builtin_amdgcn_sched_barrier(0);
     };
