@@ -234,10 +234,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int l = l0 + 8 * (r >> 2) + 4 * g + (r & 3);
-      if (l >= L) {
+      const int gone = (L - 1 - l) >> 31;  // all ones where l >= L
 #pragma unroll
-        for (int j = 0; j < QT; ++j) s[j][r] = -INFINITY;
-      }
+      for (int j = 0; j < QT; ++j) s[j][r] = neg_inf_where(s[j][r], gone);
     }
   };
   // scaled row maximum of a finished half tile (pair of half-waves combined)

@@ -276,11 +276,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (16 * i + r >= rem) {
+          for (int r = 0; r < 4; ++r) {
+            const int gone = (rem - (16 * i + r) - 1) >> 31;  // all ones where 16 i + r >= rem
 #pragma unroll
-              for (int j = 0; j < RT; ++j) s[i][j][r] = -INFINITY;
-            }
+            for (int j = 0; j < RT; ++j) s[i][j][r] = neg_inf_where(s[i][j][r], gone);
+          }
       }
       if (SAFE || it == 0) {
         float mx[RT];

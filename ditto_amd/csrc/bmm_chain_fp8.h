@@ -304,7 +304,7 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int l = it * kBN + 32 * i + 8 * (r >> 2) + 4 * g + (r & 3);
-            if (l >= L) s[i][r] = -INFINITY;
+            s[i][r] = neg_inf_where(s[i][r], (L - 1 - l) >> 31);  // l >= L
           }
       }
       float mx = s[0][0];
@@ -384,7 +384,7 @@ __global__ __launch_bounds__(512) void bmm_chain8_kernel(BmmChainArgs p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int l = l0 + 8 * (r >> 2) + 4 * g + (r & 3);
-      if (l >= L) sc[r] = -INFINITY;
+      sc[r] = neg_inf_where(sc[r], (L - 1 - l) >> 31);  // l >= L
     }
   };
   auto row_max = [&](const f32x16& sc) __attribute__((always_inline)) {

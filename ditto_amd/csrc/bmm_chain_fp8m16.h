@@ -377,11 +377,11 @@ __device__ __forceinline__ void bmm_chain8m16_body(const BmmChainArgs& p, char* 
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (16 * i + r >= rem) {
+      for (int r = 0; r < 4; ++r) {
+        const int gone = (rem - (16 * i + r) - 1) >> 31;  // all ones where 16 i + r >= rem
 #pragma unroll
-          for (int j = 0; j < RT; ++j) h.v[i][j][r] = -INFINITY;
-        }
+        for (int j = 0; j < RT; ++j) h.v[i][j][r] = neg_inf_where(h.v[i][j][r], gone);
+      }
   };
   auto local_max = [&](const Half& h) __attribute__((always_inline)) {
 #pragma unroll

@@ -118,6 +118,13 @@ __device__ __forceinline__ typename Elem<T>::v4 lds_read_tr4(const T* p) {
   return __builtin_bit_cast(typename Elem<T>::v4, r);
 }
 
+// x where `gone` is 0, -infinity where it is all ones (gone = (limit - 1 - index) >> 31 for "index >= limit").  A select
+// by integer arithmetic: the comparisons of a masked tile are otherwise all made first and their lane masks held in
+// scalar registers together, which the walks of the chain kernels do not have to spare (spills, a scratch segment).
+__device__ __forceinline__ float neg_inf_where(float x, int gone) {
+  return __builtin_bit_cast(float, (__builtin_bit_cast(int, x) & ~gone) | ((int)0xff800000 & gone));
+}
+
 template <typename V4, typename V8>
 __device__ __forceinline__ V8 concat4(V4 lo, V4 hi) {
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
