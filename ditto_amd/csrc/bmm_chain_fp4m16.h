@@ -202,18 +202,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     return concat4<V4, V8>(lo, hi);
   };
 
-  if constexpr (PRE) {
+  // The first tile's loads go out before anything waits for A: the wait the compiler puts in front of the first use of
+  // the A fragments covers every load issued so far, so with A's loads, that wait and only then the tile's loads, a
+  // workgroup started with two memory latencies in a row.  The fragments are used here (scaled, or merely named), so
+  // that the wait falls between the first and the second tile's loads and does not take the second tile in as well.
+  load_tile(0, 0);
 #pragma unroll
-    for (int j = 0; j < RT; ++j)
+  for (int j = 0; j < RT; ++j)
 #pragma unroll
-      for (int st = 0; st < NS; ++st)
+    for (int st = 0; st < NS; ++st) {
+      if constexpr (PRE) {
 #pragma unroll
         for (int e = 0; e < 8; e += 2) {
           const V2 q2 = cvt2<T>((float)af[j][st][e] * p.scale_log2, (float)af[j][st][e + 1] * p.scale_log2);
           af[j][st][e] = q2[0];
           af[j][st][e + 1] = q2[1];
         }
-  }
+      }
+      asm volatile("" : "+v"(af[j][st]));
+    }
+  load_tile(1, 1);
 
   // ---- accumulators of F^T over the wave's keys: o[t][j][r] = F^T[16 t + 4 q + r][16 j + c]
   f32x4 o[NTN][RT];
@@ -401,8 +409,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
       ls[j] = f32x4{0.f, 0.f, 0.f, 0.f};
       negm[j] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    load_tile(0, 0);
-    load_tile(1, 1);
+    // (tiles 0 and 1 are in flight: issued by the caller)
     for (int it = 0; it < ntiles; it += 3) {
       tile_step(it, IntC<0>{}, safe_c);
       if (it + 1 < ntiles) tile_step(it + 1, IntC<1>{}, safe_c);
@@ -424,7 +431,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   if (tid == 0) *flag = 0;
   walk(BoolC<false>{});
   if constexpr (kSoftmax) {
-    if (__builtin_amdgcn_readfirstlane(*flag)) walk(BoolC<true>{});
+    if (__builtin_amdgcn_readfirstlane(*flag)) {
+      load_tile(0, 0);
+      load_tile(1, 1);
+      walk(BoolC<true>{});
+    }
   }
 
   // ---- KSPLIT == 2, the two key halves of a row meet: each wave of a pair finishes ONE of the pair's two row tiles
