@@ -241,6 +241,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   V8 ones;
 #pragma unroll
   for (int e = 0; e < 8; ++e) ones[e] = (T)1.0f;
+  asm volatile("" : "+v"(ones));  // kept in vector registers: as a known constant it is rebuilt from scalar ones every tile
   auto row_part = [&](int j) __attribute__((always_inline)) -> float { return kSumMfma ? ls[j][0] : lsum[j]; };
   auto row_scale = [&](int j, float a) __attribute__((always_inline)) {
     if (kSumMfma) ls[j] *= a;
