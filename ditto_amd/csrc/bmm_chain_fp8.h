@@ -9,8 +9,11 @@
 // exponentials run under the other wave's MFMAs without any software pipelining.
 //
 // The price is LDS traffic: with 32 rows per wave every operand fragment read from LDS feeds
-// a single MFMA.  16-byte row reads sustain that (256 B/clk per CU), the transposing read
-// ds_read_b64_tr_b16 (about 100 B/clk) does not.  So every tile whose contraction index is
+// a single MFMA.  16-byte row reads sustain that (256 B/clk per CU); the transposing read
+// ds_read_b64_tr_b16 moves half as many bytes per instruction (128 B/clk under these tiles' swizzle,
+// 220 B/clk at best), so the same fragments cost twice the LDS instructions, and with every wave
+// reading its fragments that way the 16x16x32 kernel was 4.5 % slower than with the pass below.
+// So every tile whose contraction index is
 // the row index (C always, B in [K][L] layout) is transposed ONCE per workgroup: the wave
 // that owns a fragment reads it with the transposing read and writes it back "fragment
 // major" (1 KB per fragment, lane l at byte 16*l), after which all eight waves fetch it with
